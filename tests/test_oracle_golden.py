@@ -1,0 +1,327 @@
+"""Pins the CPU checker (oracle/) against the vectors the reference's own tests hold for the path,
+and its software transcendentals against libm within the bounds the reference asserts."""
+import math
+import struct
+
+import numpy as np
+import pytest
+
+from jaxjs_hip.alu import AluExp, AluOp, AluVar, DType, Kernel, Reduction, accessorGlobal
+from jaxjs_hip.shape import ShapeTracker, unravelAlu
+from oracle import oracle
+
+MODES = [oracle.MODE_CPU, oracle.MODE_WASM]
+
+
+def f32(*v):
+    return np.array(v, dtype=np.float32)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_simple_operations(mode):  # src/backend/backend.test.ts:37-85
+    shape = ShapeTracker.fromShape([3])
+    a, b = f32(1, 2, 3), f32(4, 5, 6)
+    g = AluVar.gidx
+    for lowered in (True, False):
+        if lowered:
+            x = accessorGlobal(DType.Float32, 0, shape, [g])
+            y = accessorGlobal(DType.Float32, 1, shape.flip([True]), [g])
+        else:
+            x = AluExp.globalView(DType.Float32, 0, shape, [g])
+            y = AluExp.globalView(DType.Float32, 1, shape.flip([True]), [g])
+        np.testing.assert_array_equal(oracle.run_kernel(Kernel(2, 3, AluExp.mul(x, y)), [a, b], mode), f32(6, 10, 12))
+        np.testing.assert_array_equal(oracle.run_kernel(Kernel(2, 3, AluExp.add(x, y)), [a, b], mode), f32(7, 7, 7))
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_array_from_index(mode):  # src/backend/backend.test.ts:190-218
+    out = oracle.run_kernel(Kernel(0, 200, AluExp.cast(DType.Float32, AluVar.gidx)), [], mode)
+    np.testing.assert_array_equal(out, np.arange(200, dtype=np.float32))
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_reduction_with_epilogue(mode):  # src/backend/backend.test.ts:248-286
+    a = f32(1, 1, 2, 3, 5, 7)
+    st = ShapeTracker.fromShape([3, 2])
+    exp = AluExp.globalView(DType.Float32, 0, st, [AluVar.gidx, AluVar.ridx])
+    k = Kernel(1, 3, exp, Reduction(DType.Float32, AluOp.Add, 2))
+    np.testing.assert_array_equal(oracle.run_kernel(k, [a], mode), f32(2, 5, 12))
+    re = Reduction(DType.Float32, AluOp.Add, 2, AluExp.add(AluVar.acc(DType.Float32), AluExp.f32(1)))
+    np.testing.assert_array_equal(oracle.run_kernel(Kernel(1, 3, exp, re), [a], mode), f32(3, 6, 13))
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_bitwise_tables(mode):  # src/backend/backend.test.ts:288-373
+    shape = ShapeTracker.fromShape([4])
+    g = AluVar.gidx
+    a = np.array([0xFF00FF00, 0x0F0F0F0F, 0xAAAAAAAA, 7], dtype=np.uint32)
+    b = np.array([0x00FF00FF, 0xF0F0F0F0, 0x55555555, 3], dtype=np.uint32)
+    x = accessorGlobal(DType.Uint32, 0, shape, [g])
+    y = accessorGlobal(DType.Uint32, 1, shape, [g])
+    want = {"and": [0, 0, 0, 3], "or": [0xFFFFFFFF] * 3 + [7], "xor": [0xFFFFFFFF] * 3 + [4]}
+    for m, w in want.items():
+        out = oracle.run_kernel(Kernel(2, 4, AluExp.bitCombine(x, y, m)), [a, b], mode)
+        np.testing.assert_array_equal(out, np.array(w, dtype=np.uint32))
+    ones, amt = np.array([1, 1, 1, 1], dtype=np.uint32), np.array([0, 1, 8, 16], dtype=np.uint32)
+    out = oracle.run_kernel(Kernel(2, 4, AluExp.bitShift(x, y, "shl")), [ones, amt], mode)
+    np.testing.assert_array_equal(out, np.array([1, 2, 256, 65536], dtype=np.uint32))
+    r = np.array([256, 65536, 0xFFFF0000, 8], dtype=np.uint32)
+    out = oracle.run_kernel(Kernel(2, 4, AluExp.bitShift(x, y, "shr")), [r, amt], mode)
+    np.testing.assert_array_equal(out, np.array([256, 32768, 0x00FFFF00, 0], dtype=np.uint32))
+
+
+def _matmul_kernel(M, N, K, dtype=DType.Float32, same_buffer=False, swap=False):
+    stA = ShapeTracker.fromShape([M, K]).reshape([M, 1, K]).expand([M, N, K])
+    stB = ShapeTracker.fromShape([K, N]).permute([1, 0]).reshape([1, N, K]).expand([M, N, K])
+    idx = unravelAlu([M, N], AluVar.gidx) + [AluVar.ridx]
+    ga = AluExp.globalView(dtype, 0, stA, idx)
+    gb = AluExp.globalView(dtype, 0 if same_buffer else 1, stB, idx)
+    exp = AluExp.mul(gb, ga) if swap else AluExp.mul(ga, gb)
+    return Kernel(1 if same_buffer else 2, M * N, exp, Reduction(dtype, AluOp.Add, K))
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_matmul_ones(mode):  # src/backend/backend.test.ts:375-464
+    n = 64
+    a = np.ones(n * n, dtype=np.float32)
+    out = oracle.run_kernel(_matmul_kernel(n, n, n, same_buffer=True), [a], mode)
+    np.testing.assert_array_equal(out, np.full(n * n, n, dtype=np.float32))
+    M, N, K = 16, 48, 24
+    for swap in (False, True):
+        out = oracle.run_kernel(_matmul_kernel(M, N, K, swap=swap), [np.ones(M * K, np.float32), np.ones(K * N, np.float32)], mode)
+        np.testing.assert_array_equal(out, np.full(M * N, K, dtype=np.float32))
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_matmul_integer_valued_exact(mode):  # test/numpy.test.ts:1510-1530 style: small integer cases are exact
+    A = np.array([[1, 2], [3, 4]], dtype=np.float32)
+    B = np.array([[5, 6], [7, 8]], dtype=np.float32)
+    out = oracle.run_kernel(_matmul_kernel(2, 2, 2), [A, B], mode).reshape(2, 2)
+    np.testing.assert_array_equal(out, np.array([[19, 22], [43, 50]], dtype=np.float32))
+    rng = np.random.default_rng(0)
+    A = rng.integers(-8, 9, size=(7, 13)).astype(np.float32)
+    B = rng.integers(-8, 9, size=(13, 5)).astype(np.float32)
+    out = oracle.run_kernel(_matmul_kernel(7, 5, 13), [A, B], mode).reshape(7, 5)
+    np.testing.assert_array_equal(out, (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32))
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_row_dependent_strided_reduction(mode):  # src/backend/backend.test.ts:466-507
+    M, N, K = 32, 128, 5
+    m, k, n = np.meshgrid(np.arange(M), np.arange(K), np.arange(N), indexing="ij")
+    inp = (m * 1000 + k * 10 + n).astype(np.float32).reshape(-1)
+    mi, ni = unravelAlu([M, N], AluVar.gidx)
+    st = ShapeTracker.fromShape([M, K, N])
+    exp = AluExp.globalView(DType.Float32, 0, st, [mi, AluVar.ridx, ni])
+    out = oracle.run_kernel(Kernel(1, M * N, exp, Reduction(DType.Float32, AluOp.Add, K)), [inp], mode).reshape(M, N)
+    mm, nn = np.meshgrid(np.arange(M), np.arange(N), indexing="ij")
+    np.testing.assert_array_equal(out, (K * (mm * 1000 + nn) + 10 * K * (K - 1) // 2).astype(np.float32))
+
+
+def _unary_kernel(build, dtype_in, n):
+    st = ShapeTracker.fromShape([n])
+    return Kernel(1, n, build(AluExp.globalView(dtype_in, 0, st, [AluVar.gidx])))
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_nan_compares(mode):  # src/frontend/array.test.ts:283-292: only != is true against NaN
+    a = f32(math.nan, 1.0, math.nan)
+    b = f32(1.0, math.nan, math.nan)
+    st = ShapeTracker.fromShape([3])
+    x = AluExp.globalView(DType.Float32, 0, st, [AluVar.gidx])
+    y = AluExp.globalView(DType.Float32, 1, st, [AluVar.gidx])
+    lt = oracle.run_kernel(Kernel(2, 3, AluExp.cmplt(x, y)), [a, b], mode)
+    ne = oracle.run_kernel(Kernel(2, 3, AluExp.cmpne(x, y)), [a, b], mode)
+    eq = oracle.run_kernel(Kernel(2, 3, AluExp.cmpne(x, y).not_()), [a, b], mode)
+    ge = oracle.run_kernel(Kernel(2, 3, AluExp.cmplt(x, y).not_()), [a, b], mode)  # the IR's >= is !(x<y)
+    assert lt.dtype == np.int32
+    np.testing.assert_array_equal(lt, [0, 0, 0])
+    np.testing.assert_array_equal(ne, [1, 1, 1])
+    np.testing.assert_array_equal(eq, [0, 0, 0])
+    np.testing.assert_array_equal(ge, [1, 1, 1])
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_saturating_casts(mode):  # src/frontend/array.test.ts:415-432
+    v = f32(1e20, -1e20, 3.9, -3.9, math.nan, math.inf, -math.inf)
+    out = oracle.run_kernel(_unary_kernel(lambda x: AluExp.cast(DType.Int32, x), DType.Float32, 7), [v], mode)
+    np.testing.assert_array_equal(out, np.array([2147483647, -2147483648, 3, -3, 0, 2147483647, -2147483648], dtype=np.int32))
+    out = oracle.run_kernel(_unary_kernel(lambda x: AluExp.cast(DType.Uint32, x), DType.Float32, 7), [v], mode)
+    np.testing.assert_array_equal(out, np.array([4294967295, 0, 3, 0, 0, 4294967295, 0], dtype=np.uint32))
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_bitcast_and_int_wrap(mode):  # src/alu.test.ts:174-200
+    out = oracle.run_kernel(_unary_kernel(lambda x: AluExp.bitcast(DType.Float32, x), DType.Int32, 2),
+                            [np.array([0x3F800000, 0x7F800000], dtype=np.int32)], mode)
+    np.testing.assert_array_equal(out, f32(1.0, math.inf))
+    out = oracle.run_kernel(_unary_kernel(lambda x: AluExp.bitcast(DType.Uint32, x), DType.Int32, 1),
+                            [np.array([-1], dtype=np.int32)], mode)
+    assert out[0] == 0xFFFFFFFF
+    out = oracle.run_kernel(_unary_kernel(lambda x: AluExp.mul(x, AluExp.i32(65537)), DType.Int32, 2),
+                            [np.array([65535, -2147483648], dtype=np.int32)], mode)
+    np.testing.assert_array_equal(out, np.array([(65535 * 65537) - (1 << 32), -2147483648], dtype=np.int64).astype(np.int32))
+    out = oracle.run_kernel(_unary_kernel(lambda x: AluExp.bitShift(x, AluExp.i32(28), "shr"), DType.Int32, 1),
+                            [np.array([-1], dtype=np.int32)], mode)
+    assert out[0] == 15  # logical shift even for int32 (src/alu.ts:1088-1091)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_idiv_mod_signs(mode):  # src/alu.test.ts:211-272
+    a = np.array([7, -7, 7, -7], dtype=np.int32)
+    b = np.array([3, 3, -3, -3], dtype=np.int32)
+    st = ShapeTracker.fromShape([4])
+    x = AluExp.globalView(DType.Int32, 0, st, [AluVar.gidx])
+    y = AluExp.globalView(DType.Int32, 1, st, [AluVar.gidx])
+    np.testing.assert_array_equal(oracle.run_kernel(Kernel(2, 4, AluExp.idiv(x, y)), [a, b], mode), [2, -2, -2, 2])
+    np.testing.assert_array_equal(oracle.run_kernel(Kernel(2, 4, AluExp.mod(x, y)), [a, b], mode), [1, -1, 1, -1])
+    fx = AluExp.globalView(DType.Float32, 0, ShapeTracker.fromShape([1]), [AluVar.gidx])
+    out = oracle.run_kernel(Kernel(1, 1, AluExp.mod(fx, AluExp.f32(-1.7))), [f32(5.5)], mode)
+    assert out[0] == pytest.approx(0.4, abs=1e-6)
+
+
+def test_threefry_known_answers():  # wasm/builtins.test.ts:222-232, test/random.test.ts:21-71
+    L = oracle.lib()
+    import ctypes
+    buf = (ctypes.c_uint32 * 2)()
+    L.jo_threefry2x32(ctypes.c_uint32(0), ctypes.c_uint32(0), ctypes.c_uint32(0), ctypes.c_uint32(0), buf)
+    assert (buf[0], buf[1]) == (1797259609, 2579123966)
+    # random.bits(key, shape) lowers to threefry2x32(k0, k1, 0, gidx % n) with the two output words
+    # xor-combined (src/frontend/jit.ts:698-714), and key(seed) is [0, seed] (src/library/random.ts:62-77).
+    # Known answers: bits(key(0)) == 4070199207 and bits(key(10), [4]) (test/random.test.ts:21-40).
+    z = AluExp.u32(0)
+    for mode in MODES:
+        out = oracle.run_kernel(Kernel(0, 1, AluExp.threefry2x32(z, z, z, z, "xor")), [], mode)
+        assert out[0] == 4070199207 == (1797259609 ^ 2579123966)
+        c1 = AluExp.mod(AluExp.cast(DType.Uint32, AluVar.gidx), AluExp.u32(4))
+        out = oracle.run_kernel(Kernel(0, 4, AluExp.threefry2x32(z, AluExp.u32(10), z, c1, "xor")), [], mode)
+        assert list(out) == [169096361, 1572511259, 2689743692, 2228103506]
+        w0 = oracle.run_kernel(Kernel(0, 1, AluExp.threefry2x32(z, z, z, z, 0)), [], mode)
+        w1 = oracle.run_kernel(Kernel(0, 1, AluExp.threefry2x32(z, z, z, z, 1)), [], mode)
+        assert (w0[0], w1[0]) == (1797259609, 2579123966)
+
+
+def test_erf_values():  # src/alu.test.ts:115-137
+    L = oracle.lib()
+    assert L.jo_js_erf(1.0) == pytest.approx(0.84270079, abs=1e-5)
+    assert L.jo_js_erf(-1.0) == pytest.approx(-0.84270079, abs=1e-5)
+    assert L.jo_js_erfc(1.0) == pytest.approx(0.15729921, abs=1e-5)
+    assert L.jo_js_erfc(-1.0) == pytest.approx(1.84270079, abs=1e-5)
+    assert L.jo_js_erfc(100.0) == pytest.approx(0.0, abs=1e-5)
+    # The Wasm build evaluates the same formula in f32 (wasm/builtins.test.ts:169-209: < 5e-7 of alu.erf).
+    for x in np.linspace(-4, 4, 81):
+        assert abs(oracle.wasm_builtin("erf", x) - L.jo_js_erf(float(np.float32(x)))) < 5e-7
+        assert abs(oracle.wasm_builtin("erfc", x) - L.jo_js_erfc(float(np.float32(x)))) < 5e-7
+
+
+def test_wasm_exp_bounds():  # wasm/builtins.test.ts:20-42: rel < 2e-7 on moderate inputs, edge cases
+    for x in [-10, -5, -2, -1, -0.5, 0, 0.5, 1, 2, 5, 10, 0.001, -0.001, 3.14159]:
+        got, want = oracle.wasm_builtin("exp", x), math.exp(float(np.float32(x)))
+        assert abs(got - want) / want < 2e-6, x
+    assert oracle.wasm_builtin("exp", 0.0) == 1.0
+    assert oracle.wasm_builtin("exp", 1000.0) == math.inf  # test/numpy.test.ts:2803-2830
+    assert oracle.wasm_builtin("exp", -1000.0) == 0.0
+    assert math.isnan(oracle.wasm_builtin("exp", math.nan))
+    xs = np.linspace(-80, 80, 4001).astype(np.float32)
+    rel = max(abs(oracle.wasm_builtin("exp", float(x)) - math.exp(float(x))) / math.exp(float(x)) for x in xs)
+    assert rel < 1e-5  # grows with |x| because k*ln2 is formed in f32
+
+
+def test_wasm_log_bounds():  # wasm/builtins.test.ts:44-64
+    for x in [0.001, 0.1, 0.5, 1, 2, 2.718281828, 10, 100, 1000, 1e10]:
+        got, want = oracle.wasm_builtin("log", x), math.log(float(np.float32(x)))
+        assert abs(got - want) <= 2e-5 * max(1.0, abs(want)), x
+    assert oracle.wasm_builtin("log", 1.0) == 0.0
+    assert oracle.wasm_builtin("log", 0.0) == -math.inf
+    assert math.isnan(oracle.wasm_builtin("log", -1.0))
+    assert oracle.wasm_builtin("log", math.inf) == math.inf
+    # Series truncated at t^7: the worst case is a mantissa just below 2 with exponent 0.
+    worst = max(abs(oracle.wasm_builtin("log", float(x)) - math.log(float(x))) / abs(math.log(float(x)))
+                for x in np.linspace(1.5, 1.999, 200).astype(np.float32))
+    assert 1e-6 < worst < 3e-5
+
+
+def test_wasm_sincos_atan_bounds():  # wasm/builtins.test.ts:66-167
+    for x in np.linspace(-10, 10, 401).astype(np.float32):
+        x = float(x)
+        assert abs(oracle.wasm_builtin("sin", x) - math.sin(x)) < 5e-6
+        assert abs(oracle.wasm_builtin("cos", x) - math.cos(x)) < 5e-6
+    for x in np.concatenate([np.linspace(-20, 20, 401), [1e3, -1e3, 1e6]]).astype(np.float32):
+        x = float(x)
+        want = math.atan(x)
+        assert abs(oracle.wasm_builtin("atan", x) - want) <= 2e-6 * max(abs(want), 1e-3) + 1e-7
+    for x in np.linspace(-1, 1, 101).astype(np.float32):
+        assert abs(oracle.wasm_builtin("asin", float(x)) - math.asin(float(x))) < 5e-6
+    assert oracle.wasm_builtin("sin", 0.0) == 0.0 and oracle.wasm_builtin("cos", 0.0) == 1.0
+
+
+def test_half_conversion_matches_numpy_exhaustively():
+    L = oracle.lib()
+    all_bits = np.arange(65536, dtype=np.uint16)
+    vals = all_bits.view(np.float16).astype(np.float64)
+    for b, v in zip(all_bits[::7], vals[::7]):
+        got = L.jo_half_to_double(int(b))
+        assert (math.isnan(got) and math.isnan(v)) or got == v
+    rng = np.random.default_rng(3)
+    xs = np.concatenate([rng.normal(0, 1, 4000), rng.normal(0, 1e-6, 2000), rng.normal(0, 3e4, 2000),
+                         [65504, 65519.99, 65520, 1e9, 2.0**-24, 2.0**-25, 2.0**-25 * 1.0001, 0.0, -0.0]])
+    with np.errstate(over="ignore"):
+        want = xs.astype(np.float16).view(np.uint16)
+    got = np.array([L.jo_double_to_half(float(x)) for x in xs], dtype=np.uint16)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_f16_sum_accumulates_in_f32():  # test/dtype-f16.test.ts:77-89: sum of f16 values accumulates wide
+    n = 4096
+    x = np.full(n, 2.443, dtype=np.float16)  # partial sums leave f16's exact-integer range quickly
+    st = ShapeTracker.fromShape([1, n])
+    exp = AluExp.globalView(DType.Float16, 0, st, [AluVar.gidx, AluVar.ridx])
+    k = Kernel(1, 1, exp, Reduction(DType.Float16, AluOp.Add, n))
+    want = np.float16(np.float64(x[0]) * n)
+    for mode in MODES:
+        out = oracle.run_kernel(k, [x], mode)
+        assert out.dtype == np.float16 and out[0] == want
+
+
+def test_multi_view_and_padding():  # src/shape.test.ts:354-399 through the kernel path
+    st = ShapeTracker.fromShape([2, 2]).pad([(1, 1), (1, 1)]).flip([False, True]).reshape([16])
+    assert len(st.views) == 2
+    base = f32(10, 11, 12, 13)
+    k = Kernel(1, 16, AluExp.globalView(DType.Float32, 0, st, [AluVar.gidx]))
+    want = np.zeros(16, dtype=np.float32)
+    want[[5, 6, 9, 10]] = [11, 10, 13, 12]
+    for mode in MODES:
+        out, oob = oracle.run_kernel(k, [base], mode, return_oob=True)
+        np.testing.assert_array_equal(out, want)
+        assert oob == 0
+
+
+def test_gidx_subset_and_oob_count():
+    k = Kernel(1, 8, AluExp.globalIndex(DType.Float32, 0, 4, AluVar.gidx))
+    out, oob = oracle.run_kernel(k, [f32(1, 2, 3, 4)], oracle.MODE_WASM, gidx=[1, 3, 6], return_oob=True)
+    np.testing.assert_array_equal(out, f32(2, 4, 1))  # out-of-range load reads element 0 (translation.ts:221-228)
+    assert oob == 1
+
+
+def test_wasm_port_matmul_matvec_against_f64():
+    import ctypes
+    L = oracle.lib()
+    rng = np.random.default_rng(5)
+    for (M, N, K) in [(64, 64, 64), (16, 48, 24), (130, 260, 100), (256, 128, 192)]:
+        A = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+        B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+        C = np.full((M, N), np.nan, dtype=np.float32)
+        rc = L.jo_wasm_matmul_f32(A.ctypes.data_as(ctypes.c_void_p), B.ctypes.data_as(ctypes.c_void_p),
+                                  C.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(M), ctypes.c_int64(N), ctypes.c_int64(K))
+        assert rc == 0
+        ref = A.astype(np.float64) @ B.astype(np.float64)
+        bound = 2 * K * np.finfo(np.float32).eps * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
+        assert np.all(np.abs(C - ref) <= bound + 1e-30)
+    M, K = 44, 128
+    W = rng.normal(0, 0.02, (M, K)).astype(np.float32)
+    x = rng.normal(0, 1, K).astype(np.float32)
+    y = np.zeros(M, dtype=np.float32)
+    assert L.jo_wasm_matvec_f32(W.ctypes.data_as(ctypes.c_void_p), x.ctypes.data_as(ctypes.c_void_p),
+                                y.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(M), ctypes.c_int64(K)) == 0
+    ref = W.astype(np.float64) @ x.astype(np.float64)
+    assert np.all(np.abs(y - ref) <= 2 * K * np.finfo(np.float32).eps * (np.abs(W).astype(np.float64) @ np.abs(x)))
