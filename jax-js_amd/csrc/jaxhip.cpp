@@ -1,0 +1,331 @@
+// jaxhip.cpp -- the C-ABI runtime declared in include/jaxhip.h.
+//
+// Thin by design: hipMalloc / hipMemcpyAsync / hiprtc / hipModuleLaunchKernel on one in-order
+// stream.  Slots, reference counting, the kernel cache and code generation live in the host-side
+// HipBackend; see the header for which reference interface each entry point stands in for.
+
+#include "jaxhip.h"
+
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+
+namespace {
+
+thread_local std::string g_last_error;
+
+struct Runtime {
+  bool ready = false;
+  int device = -1;
+  hipStream_t stream = nullptr;
+};
+Runtime g_rt;
+
+int fail(int code, const char *fmt, ...) {
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code ? code : -1;
+}
+
+#define JH_HIP(expr)                                                                      \
+  do {                                                                                    \
+    hipError_t e_ = (expr);                                                               \
+    if (e_ != hipSuccess) return fail((int)e_, "%s failed: %s", #expr, hipGetErrorString(e_)); \
+  } while (0)
+
+#define JH_NEED_INIT()                                                  \
+  do {                                                                  \
+    if (!g_rt.ready) return fail(-2, "jh_init has not been called");    \
+  } while (0)
+
+}  // namespace
+
+extern "C" {
+
+int jh_abi_version(void) { return 1; }
+
+const char *jh_last_error(void) { return g_last_error.c_str(); }
+
+int jh_init(int device) {
+  if (g_rt.ready) {
+    if (g_rt.device == device) return 0;
+    return fail(-3, "runtime already initialised on device %d", g_rt.device);
+  }
+  int count = 0;
+  JH_HIP(hipGetDeviceCount(&count));
+  if (device < 0 || device >= count) return fail(-4, "device %d out of range (%d visible)", device, count);
+  JH_HIP(hipSetDevice(device));
+  // Default priority on purpose: work on streams of different priorities has hung on this pool.
+  JH_HIP(hipStreamCreateWithFlags(&g_rt.stream, hipStreamNonBlocking));
+  g_rt.device = device;
+  g_rt.ready = true;
+  return 0;
+}
+
+int jh_shutdown(void) {
+  if (!g_rt.ready) return 0;
+  JH_HIP(hipStreamSynchronize(g_rt.stream));
+  JH_HIP(hipStreamDestroy(g_rt.stream));
+  g_rt = Runtime();
+  return 0;
+}
+
+int jh_get_device_info(jh_device_info *out) {
+  JH_NEED_INIT();
+  if (!out) return fail(-5, "null output");
+  hipDeviceProp_t p;
+  JH_HIP(hipGetDeviceProperties(&p, g_rt.device));
+  memset(out, 0, sizeof(*out));
+  snprintf(out->name, sizeof(out->name), "%s", p.name);
+  snprintf(out->arch, sizeof(out->arch), "%s", p.gcnArchName);
+  out->compute_units = p.multiProcessorCount;
+  out->wavefront_size = p.warpSize;
+  out->max_threads_per_block = p.maxThreadsPerBlock;
+  out->lds_bytes_per_block = (int32_t)p.sharedMemPerBlock;
+  out->total_mem_bytes = (int64_t)p.totalGlobalMem;
+  out->clock_khz = p.clockRate;
+  out->l2_bytes = p.l2CacheSize;
+  return 0;
+}
+
+int jh_malloc(size_t bytes, jh_devptr *out) {
+  JH_NEED_INIT();
+  if (!out) return fail(-5, "null output");
+  *out = nullptr;
+  if (bytes == 0) return 0;
+  JH_HIP(hipMalloc(out, bytes));
+  return 0;
+}
+
+int jh_free(jh_devptr ptr) {
+  JH_NEED_INIT();
+  if (!ptr) return 0;
+  // hipFree waits for the device, so a buffer still read by a queued kernel is safe to release.
+  JH_HIP(hipFree(ptr));
+  return 0;
+}
+
+int jh_memcpy_h2d(jh_devptr dst, const void *src, size_t bytes) {
+  JH_NEED_INIT();
+  if (bytes == 0) return 0;
+  if (!dst || !src) return fail(-5, "null pointer in h2d copy");
+  JH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_rt.stream));
+  // Pageable source memory: make sure the runtime is done reading it before the caller reuses it.
+  JH_HIP(hipStreamSynchronize(g_rt.stream));
+  return 0;
+}
+
+int jh_memcpy_d2h(void *dst, jh_devptr src, size_t offset, size_t bytes) {
+  JH_NEED_INIT();
+  if (bytes == 0) {
+    JH_HIP(hipStreamSynchronize(g_rt.stream));
+    return 0;
+  }
+  if (!dst || !src) return fail(-5, "null pointer in d2h copy");
+  JH_HIP(hipMemcpyAsync(dst, (const char *)src + offset, bytes, hipMemcpyDeviceToHost, g_rt.stream));
+  JH_HIP(hipStreamSynchronize(g_rt.stream));
+  return 0;
+}
+
+int jh_memcpy_d2h_async(void *dst, jh_devptr src, size_t offset, size_t bytes, jh_event *done) {
+  JH_NEED_INIT();
+  if (!done) return fail(-5, "null event output");
+  if (bytes != 0) {
+    if (!dst || !src) return fail(-5, "null pointer in d2h copy");
+    JH_HIP(hipMemcpyAsync(dst, (const char *)src + offset, bytes, hipMemcpyDeviceToHost, g_rt.stream));
+  }
+  hipEvent_t ev;
+  JH_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+  hipError_t e = hipEventRecord(ev, g_rt.stream);
+  if (e != hipSuccess) {
+    (void)hipEventDestroy(ev);
+    return fail((int)e, "hipEventRecord failed: %s", hipGetErrorString(e));
+  }
+  *done = (jh_event)ev;
+  return 0;
+}
+
+int jh_memcpy_d2d(jh_devptr dst, jh_devptr src, size_t bytes) {
+  JH_NEED_INIT();
+  if (bytes == 0) return 0;
+  if (!dst || !src) return fail(-5, "null pointer in d2d copy");
+  JH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, g_rt.stream));
+  return 0;
+}
+
+int jh_host_alloc(size_t bytes, void **out) {
+  JH_NEED_INIT();
+  if (!out) return fail(-5, "null output");
+  *out = nullptr;
+  if (bytes == 0) return 0;
+  JH_HIP(hipHostMalloc(out, bytes, hipHostMallocDefault));
+  return 0;
+}
+
+int jh_host_free(void *ptr) {
+  JH_NEED_INIT();
+  if (!ptr) return 0;
+  JH_HIP(hipHostFree(ptr));
+  return 0;
+}
+
+int jh_compile(const char *source, const char *name, const char *const *options, int num_options, void **code,
+               size_t *code_size, char *log, size_t log_size) {
+  if (!source || !code || !code_size) return fail(-5, "null argument to jh_compile");
+  *code = nullptr;
+  *code_size = 0;
+  if (log && log_size) log[0] = '\0';
+  hiprtcProgram prog;
+  hiprtcResult r = hiprtcCreateProgram(&prog, source, name ? name : "kernel.hip", 0, nullptr, nullptr);
+  if (r != HIPRTC_SUCCESS) return fail((int)r, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
+  r = hiprtcCompileProgram(prog, num_options, const_cast<const char **>(options));
+  size_t n = 0;
+  if (hiprtcGetProgramLogSize(prog, &n) == HIPRTC_SUCCESS && n > 1) {
+    std::string text(n, '\0');
+    if (hiprtcGetProgramLog(prog, &text[0]) == HIPRTC_SUCCESS) {
+      if (log && log_size) snprintf(log, log_size, "%s", text.c_str());
+      if (r != HIPRTC_SUCCESS) g_last_error = text;
+    }
+  }
+  if (r != HIPRTC_SUCCESS) {
+    hiprtcDestroyProgram(&prog);
+    if (g_last_error.empty()) g_last_error = hiprtcGetErrorString(r);
+    return (int)r;
+  }
+  size_t sz = 0;
+  r = hiprtcGetCodeSize(prog, &sz);
+  if (r != HIPRTC_SUCCESS || sz == 0) {
+    hiprtcDestroyProgram(&prog);
+    return fail((int)r ? (int)r : -6, "hiprtcGetCodeSize: %s", hiprtcGetErrorString(r));
+  }
+  void *buf = malloc(sz);
+  if (!buf) {
+    hiprtcDestroyProgram(&prog);
+    return fail(-7, "out of host memory for %zu byte code object", sz);
+  }
+  r = hiprtcGetCode(prog, (char *)buf);
+  hiprtcDestroyProgram(&prog);
+  if (r != HIPRTC_SUCCESS) {
+    free(buf);
+    return fail((int)r, "hiprtcGetCode: %s", hiprtcGetErrorString(r));
+  }
+  *code = buf;
+  *code_size = sz;
+  return 0;
+}
+
+void jh_code_free(void *code) { free(code); }
+
+int jh_module_load(const void *code, size_t code_size, jh_module *out) {
+  JH_NEED_INIT();
+  if (!code || !code_size || !out) return fail(-5, "null argument to jh_module_load");
+  hipModule_t m;
+  JH_HIP(hipModuleLoadData(&m, code));
+  *out = (jh_module)m;
+  return 0;
+}
+
+int jh_module_unload(jh_module module) {
+  JH_NEED_INIT();
+  if (!module) return 0;
+  JH_HIP(hipModuleUnload((hipModule_t)module));
+  return 0;
+}
+
+int jh_module_function(jh_module module, const char *kernel_name, jh_function *out) {
+  JH_NEED_INIT();
+  if (!module || !kernel_name || !out) return fail(-5, "null argument to jh_module_function");
+  hipFunction_t f;
+  JH_HIP(hipModuleGetFunction(&f, (hipModule_t)module, kernel_name));
+  *out = (jh_function)f;
+  return 0;
+}
+
+int jh_launch(jh_function fn, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, uint32_t by, uint32_t bz,
+              uint32_t shared_bytes, void **args) {
+  JH_NEED_INIT();
+  if (!fn) return fail(-5, "null kernel");
+  if (gx == 0 || gy == 0 || gz == 0) return 0;  // empty grid: nothing to do
+  if (bx == 0 || by == 0 || bz == 0 || (uint64_t)bx * by * bz > 1024)
+    return fail(-8, "invalid block %ux%ux%u", bx, by, bz);
+  JH_HIP(hipModuleLaunchKernel((hipFunction_t)fn, gx, gy, gz, bx, by, bz, shared_bytes, g_rt.stream, args, nullptr));
+  return 0;
+}
+
+int jh_launch_repeat(jh_function fn, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, uint32_t by, uint32_t bz,
+                     uint32_t shared_bytes, void **args, int count) {
+  for (int i = 0; i < count; i++) {
+    int rc = jh_launch(fn, gx, gy, gz, bx, by, bz, shared_bytes, args);
+    if (rc) return rc;
+  }
+  return 0;
+}
+
+int jh_sync(void) {
+  JH_NEED_INIT();
+  JH_HIP(hipStreamSynchronize(g_rt.stream));
+  return 0;
+}
+
+int jh_event_create(jh_event *out) {
+  JH_NEED_INIT();
+  if (!out) return fail(-5, "null output");
+  hipEvent_t ev;
+  JH_HIP(hipEventCreate(&ev));
+  *out = (jh_event)ev;
+  return 0;
+}
+
+int jh_event_record(jh_event ev) {
+  JH_NEED_INIT();
+  if (!ev) return fail(-5, "null event");
+  JH_HIP(hipEventRecord((hipEvent_t)ev, g_rt.stream));
+  return 0;
+}
+
+int jh_event_query(jh_event ev, int *done) {
+  JH_NEED_INIT();
+  if (!ev || !done) return fail(-5, "null argument");
+  hipError_t e = hipEventQuery((hipEvent_t)ev);
+  if (e == hipSuccess) {
+    *done = 1;
+    return 0;
+  }
+  if (e == hipErrorNotReady) {
+    *done = 0;
+    return 0;
+  }
+  return fail((int)e, "hipEventQuery failed: %s", hipGetErrorString(e));
+}
+
+int jh_event_sync(jh_event ev) {
+  JH_NEED_INIT();
+  if (!ev) return fail(-5, "null event");
+  JH_HIP(hipEventSynchronize((hipEvent_t)ev));
+  return 0;
+}
+
+int jh_event_elapsed_ms(jh_event start, jh_event stop, float *ms) {
+  JH_NEED_INIT();
+  if (!start || !stop || !ms) return fail(-5, "null argument");
+  JH_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+  return 0;
+}
+
+int jh_event_destroy(jh_event ev) {
+  JH_NEED_INIT();
+  if (!ev) return 0;
+  JH_HIP(hipEventDestroy((hipEvent_t)ev));
+  return 0;
+}
+
+}  // extern "C"

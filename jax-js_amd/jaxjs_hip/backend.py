@@ -1,0 +1,239 @@
+"""`HipBackend`: the `hip` device behind the reference's Backend interface.
+
+Mirrors `interface Backend` (reference: src/backend.ts:158-211) member for member -- `type`,
+`maxArgs`, `malloc`, `incRef`, `decRef`, `read`, `readSync`, `prepareKernel(Sync)`,
+`prepareRoutine(Sync)`, `dispatch` -- with the same ownership and error rules:
+
+* slots are caller-refcounted handles to untyped byte buffers; `malloc` returns refcount 1, the
+  buffer is released when `decRef` reaches 0, any use of an unknown or freed slot raises
+  `SlotError` (src/backend.ts:170-179, 222-226);
+* `malloc(size, initialData)` requires `len(initialData) == size` (src/backend/cpu.ts:22-24);
+  `malloc(0)` is legal;
+* `prepareKernel*` is idempotent and cached per kernel structure (the role of
+  `FpHash.hash(kernel)` in src/backend/wasm.ts:125-147); unsupported op/dtype pairs raise
+  `UnsupportedOpError` here, not at dispatch;
+* `dispatch` never blocks; work runs in dispatch order on one HIP stream and `read` of a slot
+  observes every earlier dispatch (src/backend.ts:203-210).
+
+Device memory, compilation and launches go through the C ABI of `include/jaxhip.h`; there is no
+host fallback for kernels.  Routines run on the host exactly as the reference's Wasm backend does
+(src/backend/wasm.ts:158-165, 216-220), through device->host->device copies.
+"""
+
+from __future__ import annotations
+
+import asyncio
+import ctypes
+from typing import Dict, List, Optional, Sequence
+
+from .alu import Kernel, byteWidth
+from .errors import HipRuntimeError, SlotError, UnsupportedRoutineError
+from .kernelgen import KernelSource, generate
+from .routine import Routine, runCpuRoutine
+from .runtime import Device, compile_source, pack_args
+
+
+class Executable:
+    """A prepared Kernel or Routine (src/backend.ts:213-220)."""
+
+    def __init__(self, source, data):
+        self.source = source
+        self.data = data
+
+
+class _Prepared:
+    """Backend-private payload of an Executable for a Kernel."""
+
+    def __init__(self, ks: KernelSource, functions: List[int], scratch: List[int], modules: List[int]):
+        self.ks = ks
+        self.functions = functions  # one per launch step
+        self.scratch = scratch      # device pointers owned by this executable
+        self.modules = modules
+
+
+_ALIGN = 256  # allocation granularity; also keeps every slot 128-bit-load aligned
+
+
+class HipBackend:
+    """MI355X backend.  `numerics="wasm"` evaluates transcendentals with the reference Wasm
+    backend's polynomials (bit-faithful to the parity oracle); `"native"` uses the device libm."""
+
+    type = "hip"
+    maxArgs = 64  # kernel parameters are plain pointers; same bound as the Wasm backend (src/backend/wasm.ts:38)
+
+    def __init__(self, device: int = 0, numerics: str = "wasm"):
+        if numerics not in ("wasm", "native"):
+            raise ValueError("numerics must be 'wasm' or 'native'")
+        self.numerics = numerics
+        self.dev = Device.get(device)
+        self._slots: Dict[int, dict] = {}
+        self._next_slot = 1
+        self._pool: Dict[int, List[int]] = {}   # rounded size -> free device pointers
+        self._pool_bytes = 0
+        self._pool_limit = 8 << 30
+        self._exes: Dict[tuple, Executable] = {}
+        self.trace: Optional[list] = None       # when a list: (label, start_event, stop_event) per dispatch
+
+    # -- memory -----------------------------------------------------------------------------------
+    @staticmethod
+    def _rounded(size: int) -> int:
+        return max(_ALIGN, (size + _ALIGN - 1) // _ALIGN * _ALIGN)
+
+    def _alloc(self, size: int) -> int:
+        if size == 0:
+            return 0
+        r = self._rounded(size)
+        free = self._pool.get(r)
+        if free:
+            self._pool_bytes -= r
+            return free.pop()
+        try:
+            return self.dev.malloc(r)
+        except HipRuntimeError:
+            self._trim_pool(0)
+            return self.dev.malloc(r)
+
+    def _release(self, ptr: int, size: int) -> None:
+        if not ptr:
+            return
+        r = self._rounded(size)
+        # Reuse is safe without a fence: every consumer of the old contents was queued on the same
+        # in-order stream before any later producer.
+        self._pool.setdefault(r, []).append(ptr)
+        self._pool_bytes += r
+        if self._pool_bytes > self._pool_limit:
+            self._trim_pool(self._pool_limit // 2)
+
+    def _trim_pool(self, target: int) -> None:
+        for r in sorted(self._pool, reverse=True):
+            free = self._pool[r]
+            while free and self._pool_bytes > target:
+                self.dev.free(free.pop())
+                self._pool_bytes -= r
+
+    def malloc(self, size: int, initialData=None) -> int:
+        size = int(size)
+        if size < 0:
+            raise ValueError("malloc size must be non-negative")
+        if initialData is not None:
+            mv = memoryview(initialData).cast("B")
+            if len(mv) != size:
+                raise ValueError("initialData size does not match buffer size")
+        ptr = self._alloc(size)
+        if initialData is not None and size:
+            self.dev.h2d(ptr, initialData)
+        slot = self._next_slot
+        self._next_slot += 1
+        self._slots[slot] = {"ptr": ptr, "size": size, "ref": 1}
+        return slot
+
+    def _get(self, slot: int) -> dict:
+        s = self._slots.get(slot)
+        if s is None:
+            raise SlotError(slot)
+        return s
+
+    def incRef(self, slot: int) -> None:
+        self._get(slot)["ref"] += 1
+
+    def decRef(self, slot: int) -> None:
+        s = self._get(slot)
+        s["ref"] -= 1
+        if s["ref"] == 0:
+            del self._slots[slot]
+            self._release(s["ptr"], s["size"])
+
+    def readSync(self, slot: int, start: Optional[int] = None, count: Optional[int] = None) -> bytearray:
+        s = self._get(slot)
+        start = 0 if start is None else int(start)
+        count = s["size"] - start if count is None else int(count)
+        if start < 0 or count < 0 or start + count > s["size"]:
+            raise ValueError(f"read range [{start}, {start + count}) outside buffer of {s['size']} bytes")
+        return self.dev.d2h(s["ptr"], start, count)
+
+    async def read(self, slot: int, start: Optional[int] = None, count: Optional[int] = None) -> bytearray:
+        # Single-threaded host like the reference; yield once so callers can overlap preparation.
+        await asyncio.sleep(0)
+        return self.readSync(slot, start, count)
+
+    def slotPointer(self, slot: int) -> int:
+        """Device address of a slot (for the benchmark harness)."""
+        return self._get(slot)["ptr"]
+
+    # -- kernels ----------------------------------------------------------------------------------
+    def prepareKernelSync(self, kernel: Kernel, **tune_opts) -> Executable:
+        key = (kernel.key(), self.numerics, tuple(sorted(tune_opts.items())))
+        exe = self._exes.get(key)
+        if exe is not None:
+            return exe
+        ks = generate(kernel, self.numerics, **tune_opts)
+        modules = [self.dev.load_module(compile_source(src, f"{ks.klass}.hip")) for src in ks.sources]
+        functions = [self.dev.function(modules[s.module], s.name) for s in ks.steps]
+        scratch = [self.dev.malloc(self._rounded(b)) for b in ks.scratch_bytes]
+        exe = Executable(kernel, _Prepared(ks, functions, scratch, modules))
+        self._exes[key] = exe
+        return exe
+
+    async def prepareKernel(self, kernel: Kernel) -> Executable:
+        return self.prepareKernelSync(kernel)
+
+    def prepareRoutineSync(self, routine: Routine) -> Executable:
+        from .routine import SUPPORTED_ROUTINES
+
+        if routine.name not in SUPPORTED_ROUTINES:
+            raise UnsupportedRoutineError(routine.name, "hip")
+        return Executable(routine, None)
+
+    async def prepareRoutine(self, routine: Routine) -> Executable:
+        return self.prepareRoutineSync(routine)
+
+    def dispatch(self, exe: Executable, inputs: Sequence[int], outputs: Sequence[int], repeat: int = 1) -> None:
+        ins = [self._get(s) for s in inputs]
+        outs = [self._get(s) for s in outputs]
+        if isinstance(exe.source, Routine):
+            host_in = [self.dev.d2h(s["ptr"], 0, s["size"]) for s in ins]
+            host_out = [bytearray(s["size"]) for s in outs]
+            runCpuRoutine(exe.source, host_in, host_out)
+            for s, data in zip(outs, host_out):
+                if s["size"]:
+                    self.dev.h2d(s["ptr"], data)
+            return
+
+        kernel: Kernel = exe.source
+        prep: _Prepared = exe.data
+        if len(outs) != 1:
+            raise ValueError("a Kernel has exactly one output")
+        if len(ins) < kernel.nargs:
+            raise ValueError(f"kernel takes {kernel.nargs} inputs, got {len(ins)}")
+        if outs[0]["size"] < kernel.bytes:
+            raise ValueError(f"output slot holds {outs[0]['size']} bytes, kernel writes {kernel.bytes}")
+        # The generated code relies on the extents the index analysis saw: refuse a launch whose
+        # buffers are smaller instead of letting a wave read past an allocation.
+        for gid, need in prep.ks.min_input_bytes.items():
+            if ins[gid]["size"] < need:
+                raise ValueError(f"input {gid} holds {ins[gid]['size']} bytes, kernel addresses {need}")
+        if kernel.size == 0:
+            return
+        for step, fn in zip(prep.ks.steps, prep.functions):
+            values = []
+            for kind, i in step.args:
+                if kind == "in":
+                    values.append(ins[i]["ptr"])
+                elif kind == "out":
+                    values.append(outs[0]["ptr"])
+                else:
+                    values.append(prep.scratch[i])
+            argv, keep = pack_args(values)
+            if self.trace is not None:
+                e0, e1 = self.dev.event(), self.dev.event()
+                self.dev.record(e0)
+                self.dev.launch(fn, step.grid, step.block, step.shared, argv, repeat)
+                self.dev.record(e1)
+                self.trace.append((f"{prep.ks.klass}:{step.name}", e0, e1))
+            else:
+                self.dev.launch(fn, step.grid, step.block, step.shared, argv, repeat)
+            del keep
+
+    def sync(self) -> None:
+        """Completion fence (what `read(slot, 0, 0)` stands for in src/frontend/array.ts:827)."""
+        self.dev.sync()

@@ -1,0 +1,287 @@
+"""Splice a tuned Kernel into the hand-written HIP templates of `csrc/templates/`.
+
+The counterpart of `pipelineSource` in the reference's WebGPU backend (src/backend/webgpu.ts:285-530):
+take the tuner's result, declare the buffer arguments, generate the fused expression body (and the
+reduction epilogue) and return complete source text plus the launch geometry.  One function per
+kernel class; the text of the classes themselves lives in the `.hip.inc` files.
+"""
+
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Tuple
+
+from .alu import AluExp, AluOp, AluVar, DType, Kernel, Reduction, byteWidth
+from .codegen import CTYPE, STORAGE_CTYPE, HipExpCodegen, const_literal, strip_parens
+from .errors import UnsupportedOpError
+from .tuner import TuneResult, tuneHip
+
+_TEMPLATE_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc", "templates")
+_templates: Dict[str, str] = {}
+
+
+def template(name: str) -> str:
+    if name not in _templates:
+        with open(os.path.join(_TEMPLATE_DIR, name), "r") as f:
+            _templates[name] = f.read()
+    return _templates[name]
+
+
+def fill(text: str, subs: Dict[str, object]) -> str:
+    for k, v in subs.items():
+        text = text.replace(f"@@{k}@@", str(v))
+    if "@@" in text:
+        start = text.index("@@")
+        raise KeyError(f"unfilled template field near: {text[start:start + 40]!r}")
+    return text
+
+
+@dataclass
+class LaunchStep:
+    """One kernel launch of a prepared executable."""
+
+    name: str
+    grid: Tuple[int, int, int]
+    block: Tuple[int, int, int]
+    shared: int
+    # ("in", gid) | ("out", 0) | ("scratch", index)
+    args: List[Tuple[str, int]]
+    module: int = 0  # index into KernelSource.sources
+
+
+@dataclass
+class KernelSource:
+    sources: List[str]
+    steps: List[LaunchStep]
+    scratch_bytes: List[int] = field(default_factory=list)
+    klass: str = ""
+    # Minimum byte size each input slot must have (from the lengths the index analysis assumed).
+    min_input_bytes: Dict[int, int] = field(default_factory=dict)
+    info: Dict[str, object] = field(default_factory=dict)
+
+
+def _used_args(nargs: int, *exps: Optional[AluExp]) -> List[Optional[DType]]:
+    used: List[Optional[DType]] = [None] * nargs
+    for e in exps:
+        if e is None:
+            continue
+        for n in e.collect(lambda x: x.op == AluOp.GlobalIndex):
+            used[n.arg[0]] = n.dtype
+    return used
+
+
+def _min_bytes(*exps: Optional[AluExp]) -> Dict[int, int]:
+    need: Dict[int, int] = {}
+    for e in exps:
+        if e is None:
+            continue
+        for n in e.collect(lambda x: x.op == AluOp.GlobalIndex):
+            gid, length = n.arg
+            need[gid] = max(need.get(gid, 0), length * byteWidth(n.dtype))
+    return need
+
+
+def _params(used: List[Optional[DType]], out_t: str, out_name: str = "out") -> Tuple[str, List[str]]:
+    names = [f"in{i}" for i in range(len(used))]
+    parts = [f"const {STORAGE_CTYPE[d or DType.Float32]}* __restrict__ {n}" for d, n in zip(used, names)]
+    parts.append(f"{out_t}* __restrict__ {out_name}")
+    return ", ".join(parts), names
+
+
+def _reduce_text(op: AluOp, dtype: DType) -> str:
+    ct = CTYPE[dtype]
+    if dtype == DType.Bool:
+        return "(a) || (b)" if op in (AluOp.Add, AluOp.Max) else "(a) && (b)"
+    if op in (AluOp.Add, AluOp.Mul):
+        sym = "+" if op == AluOp.Add else "*"
+        if dtype == DType.Int32:
+            return f"jh_{'add' if op == AluOp.Add else 'mul'}_i32((a), (b))"
+        if dtype == DType.Float16:
+            return f"(jh_f16)((a) {sym} (b))"
+        return f"(a) {sym} (b)"
+    lo = op == AluOp.Min
+    if dtype in (DType.Float32, DType.Float16, DType.Float64):
+        return f"jh_{'fmin' if lo else 'fmax'}<{ct}>((a), (b))"
+    return f"jh_{'min' if lo else 'max'}_{'i32' if dtype == DType.Int32 else 'u32'}((a), (b))"
+
+
+class _Body:
+    """Generates the three renderings of one expression a template needs: the hoisted vector /
+    uniform loads at lane 0, the per-lane body that consumes them, and a plain scalar body."""
+
+    def __init__(self, exp: AluExp, args: List[str], names: Dict[str, str], lane_sym: str, lane_base: str,
+                 V: int, classes: Dict[int, str], numerics: str, indent: str, tag: str = ""):
+        self.exp, self.args, self.names = exp, args, names
+        self.lane_sym, self.lane_base, self.V, self.classes = lane_sym, lane_base, V, classes
+        self.numerics, self.indent, self.tag = numerics, indent, tag
+
+    def hoisted(self) -> Tuple[str, Dict[int, str]]:
+        names0 = dict(self.names)
+        names0[self.lane_sym] = self.lane_base
+        cg = HipExpCodegen(self.args, names0, self.indent, prefix=f"h{self.tag}", numerics=self.numerics)
+        nodes = [n for n in self.exp.collect(lambda x: x.op == AluOp.GlobalIndex) if id(n) in self.classes]
+        for n in nodes:
+            cg.countReferences(n.src[0])
+        loads: Dict[int, str] = {}
+        for k, n in enumerate(nodes):
+            idx = strip_parens(cg.run(n.src[0]))
+            st = STORAGE_CTYPE[n.dtype]
+            ptr = self.args[n.arg[0]]
+            if self.classes[id(n)] == "vector":
+                var = f"v{self.tag}{k}"
+                cg.emit(f"const jh_pack<{st}, {self.V}> {var} = jh_vload<{st}, {self.V}>({ptr} + ({idx}));")
+                loads[id(n)] = f"{var}.v[lane]"
+            else:
+                var = f"u{self.tag}{k}"
+                cg.emit(f"const {st} {var} = {ptr}[{idx}];")
+                loads[id(n)] = var
+        return "\n".join(cg.take_lines()), loads
+
+    def lanes(self, loads: Dict[int, str]) -> Tuple[str, str]:
+        cg = HipExpCodegen(self.args, self.names, self.indent + "  ", prefix=f"l{self.tag}", numerics=self.numerics)
+        cg.loads = loads
+        cg.countReferences(self.exp)
+        value = strip_parens(cg.run(self.exp))
+        return "\n".join(cg.take_lines()), value
+
+    def scalar(self, indent: Optional[str] = None, prefix: str = "s") -> Tuple[str, str]:
+        cg = HipExpCodegen(self.args, self.names, indent or self.indent, prefix=f"{prefix}{self.tag}",
+                           numerics=self.numerics)
+        cg.countReferences(self.exp)
+        value = strip_parens(cg.run(self.exp))
+        return "\n".join(cg.take_lines()), value
+
+
+def _prelude(numerics: str) -> str:
+    return f"#define JH_WASM_NUMERICS {1 if numerics == 'wasm' else 0}\n" + template("prelude.hip.inc") + "\n"
+
+
+IDENT = {"gidx": "gidx", "ridx": "ridx"}
+
+
+def generate(kernel: Kernel, numerics: str = "wasm", tune: Optional[TuneResult] = None, name: str = "jh_kernel",
+             **tune_opts) -> KernelSource:
+    """Full source text and launch plan for a Kernel."""
+    if kernel.size >= (1 << 31) or (kernel.reduction is not None and kernel.reduction.size >= (1 << 31)):
+        raise ValueError("kernel extents must stay below 2^31 (indices are int32, src/alu.ts:1463-1464)")
+    t = tune or tuneHip(kernel, **tune_opts)
+    if t.klass == "map":
+        return _gen_map(kernel, t, numerics, name)
+    if t.klass == "reduce_row":
+        return _gen_reduce(kernel, t, numerics, name, row=True)
+    if t.klass == "reduce_col":
+        return _gen_reduce(kernel, t, numerics, name, row=False)
+    if t.klass == "gemm":
+        from .gemm import gen_gemm
+
+        return gen_gemm(kernel, t, numerics, name)
+    raise ValueError(f"unknown kernel class {t.klass}")
+
+
+def _gen_map(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelSource:
+    V, block, grid = t.params["V"], t.params["block"], t.params["grid"]
+    used = _used_args(kernel.nargs, t.exp)
+    out_t = STORAGE_CTYPE[kernel.dtype]
+    params, args = _params(used, out_t)
+    body = _Body(t.exp, args, IDENT, "gidx", "g0", V, t.vector_loads, numerics, "    ")
+    hoisted, loads = body.hoisted()
+    lane_body, lane_value = body.lanes(loads)
+    scalar_body, scalar_value = body.scalar("    ")
+    src = _prelude(numerics) + fill(template("map.hip.inc"), dict(
+        SIZE=kernel.size, V=V, BLOCK=block, NAME=name, PARAMS=params, OUT_T=out_t,
+        VECTOR_LOADS=hoisted, LANE_BODY=lane_body, LANE_VALUE=lane_value,
+        SCALAR_BODY=scalar_body, SCALAR_VALUE=scalar_value))
+    step = LaunchStep(name, (grid, 1, 1), (block, 1, 1), 0,
+                      [("in", i) for i in range(kernel.nargs)] + [("out", 0)])
+    return KernelSource([src], [step], [], "map", _min_bytes(t.exp), dict(t.params))
+
+
+def _gen_reduce(kernel: Kernel, t: TuneResult, numerics: str, name: str, row: bool) -> KernelSource:
+    re = kernel.reduction
+    assert re is not None and t.epilogue is not None
+    p = dict(t.params)
+    V, T, split = p["V"], p["T"], p.get("split", 1)
+    R, size = re.size, kernel.size
+    if re.dtype == DType.Bool:
+        split = 1
+    acc_t = CTYPE[re.dtype]
+    out_t = STORAGE_CTYPE[kernel.dtype]
+    used = _used_args(kernel.nargs, t.exp, t.epilogue if split == 1 else None)
+    ident = const_literal(re.dtype, re.identity)
+
+    if split > 1:
+        unit = T * V if row else T
+        slice_len = -(-R // split)
+        slice_len = -(-slice_len // unit) * unit
+        split = -(-R // slice_len)
+    if split <= 1:
+        split, slice_len = 1, R
+    p["split"] = split
+
+    params, args = _params(used, acc_t if split > 1 else out_t, "partial" if split > 1 else "out")
+
+    if row:
+        body = _Body(t.exp, args, IDENT, "ridx", "r0", V, t.vector_loads, numerics, "        ")
+        hoisted, loads = body.hoisted()
+        lane_body, lane_value = body.lanes(loads)
+        scalar_body, scalar_value = body.scalar("        ")
+        epi = _Body(t.epilogue, args, {"gidx": "gidx", "acc": "acc"}, "gidx", "gidx", 1, {}, numerics, "      ", "e")
+        epi_body, epi_value = epi.scalar("      ", "e") if split == 1 else ("", "0")
+        src = _prelude(numerics) + fill(template("reduce_row.hip.inc"), dict(
+            SIZE=size, R=R, V=V, T=T, BLOCK=p["block"], ROWS=p["rows"], SPLIT=split, SLICE=slice_len,
+            REDUCE=_reduce_text(re.op, re.dtype), NAME=name, PARAMS=params, ACC_T=acc_t, OUT_T=out_t,
+            IDENTITY=ident, VECTOR_LOADS=hoisted, LANE_BODY=lane_body, LANE_VALUE=lane_value,
+            SCALAR_BODY=scalar_body, SCALAR_VALUE=scalar_value, EPILOGUE_BODY=epi_body, EPILOGUE_VALUE=epi_value))
+        grid_x = p["grid"]
+        block = p["block"]
+    else:
+        body = _Body(t.exp, args, IDENT, "gidx", "g0", V, t.vector_loads, numerics, "        ")
+        hoisted, loads = body.hoisted()
+        lane_body, lane_value = body.lanes(loads)
+        scalar_body, scalar_value = body.scalar("      ")
+        epi = _Body(t.epilogue, args, {"gidx": "gidx", "acc": "accv"}, "gidx", "g0", V, t.epi_vector_loads,
+                    numerics, "      ", "e")
+        if split == 1:
+            epi_hoisted, epi_loads = epi.hoisted()
+            epi_body, epi_value = epi.lanes(epi_loads)
+            tail_body, tail_value = epi.scalar("    ", "te")
+        else:
+            epi_hoisted = epi_body = tail_body = ""
+            epi_value = tail_value = "0"
+        src = _prelude(numerics) + fill(template("reduce_col.hip.inc"), dict(
+            SIZE=size, R=R, V=V, T=T, LX=p["lx"], SPLIT=split, SLICE=slice_len,
+            REDUCE=_reduce_text(re.op, re.dtype), NAME=name, PARAMS=params, ACC_T=acc_t, OUT_T=out_t,
+            IDENTITY=ident, VECTOR_LOADS=hoisted, LANE_BODY=lane_body, LANE_VALUE=lane_value,
+            SCALAR_BODY=scalar_body, SCALAR_VALUE=scalar_value,
+            EPI_VECTOR_LOADS=epi_hoisted, EPILOGUE_BODY=epi_body, EPILOGUE_VALUE=epi_value,
+            TAIL_EPILOGUE_BODY=tail_body, TAIL_EPILOGUE_VALUE=tail_value))
+        grid_x = p["grid"]
+        block = p["lx"] * T
+
+    klass = "reduce_row" if row else "reduce_col"
+    need = _min_bytes(t.exp, t.epilogue)
+    if split == 1:
+        step = LaunchStep(name, (grid_x, 1, 1), (block, 1, 1), 0,
+                          [("in", i) for i in range(kernel.nargs)] + [("out", 0)])
+        return KernelSource([src], [step], [], klass, need, p)
+
+    # Two-stage: slices -> scratch[size*split] (reduction dtype), then a small second reduce over the
+    # slices that applies the caller's epilogue.  The second stage is itself a Kernel over the IR.
+    grid_x = max(1, min(grid_x, (256 * 16) // split + 1))
+    step1 = LaunchStep(name, (grid_x, split, 1), (block, 1, 1), 0,
+                       [("in", i) for i in range(kernel.nargs)] + [("scratch", 0)])
+    gid_partial = kernel.nargs
+    idx = AluExp.add(AluExp.mul(AluVar.gidx, AluExp.i32(split)), AluVar.ridx)
+    stage2 = Kernel(kernel.nargs + 1, size,
+                    AluExp.globalIndex(re.dtype, gid_partial, size * split, idx),
+                    Reduction(re.dtype, re.op, split, re.epilogue))
+    ks2 = generate(stage2, numerics, name=name + "_fold", allow_gemm=False, allow_split=False)
+    steps2 = []
+    for s in ks2.steps:
+        mapped = [("scratch", 0) if a == ("in", gid_partial) else a for a in s.args]
+        steps2.append(LaunchStep(s.name, s.grid, s.block, s.shared, mapped, module=s.module + 1))
+    p["stage2"] = ks2.info
+    need.update({g: b for g, b in ks2.min_input_bytes.items() if g != gid_partial})
+    return KernelSource([src] + ks2.sources, [step1] + steps2, [size * split * byteWidth(re.dtype)],
+                        klass + "+fold", need, p)

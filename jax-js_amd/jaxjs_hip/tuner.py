@@ -1,0 +1,388 @@
+"""Kernel tuning for gfx950: which kernel class runs a `Kernel`, and with which tile/wave shape.
+
+Sibling of the reference's `tuneNullopt` / `tuneWebgpu` (src/tuner.ts:219-240, 243-478).  The WebGPU
+heuristics (upcast/unroll/group sizes for 32-wide SIMD groups and a 65535-group grid) do not carry
+over; `tuneHip` instead classifies the lowered expression's memory accesses and picks one of the
+hand-written CDNA4 templates:
+
+  map         no reduction: grid-stride, V consecutive outputs per lane, 128-bit loads/stores
+  reduce_row  reduce axis contiguous in memory: T lanes walk one output's reduce axis with vector
+              loads, wave64 shuffle tree (+ LDS across waves) to combine; matvec W[M,K].x is this
+              class with one wave per row
+  reduce_col  output axis contiguous in memory: each lane owns V consecutive outputs and loops the
+              reduce axis, optionally split over the waves of a block and combined through LDS
+  (both reduce classes can additionally split the reduce axis over blocks; partials then go to a
+   scratch buffer and a second, tiny reduce kernel applies the epilogue -- deterministic, no atomics)
+  gemm        dense contraction `sum_k A*B` with strided single-view operands: MFMA tiles
+
+The choice between classes uses a small affine analysis (`lane_form`) of every buffer index with
+respect to `gidx` and `ridx`; nothing is decided from the source-level op that produced the kernel.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+from .alu import AluExp, AluGroup, AluOp, AluVar, DType, Kernel, Reduction, byteWidth, isFloatDtype
+from .shape import ShapeTracker, unravelAlu
+
+CU_COUNT = 256          # MI355X: 8 XCDs x 32 CUs
+WAVE = 64
+MAX_GRID_BLOCKS = CU_COUNT * 16
+GEMM_ENABLED = False   # flipped on once the MFMA template is in place
+
+
+@dataclass
+class TuneResult:
+    """Lowered expression pair plus launch geometry (cf. `TuneResult`, src/tuner.ts:29-59)."""
+
+    exp: AluExp
+    epilogue: Optional[AluExp]
+    klass: str = "map"
+    params: Dict[str, int] = field(default_factory=dict)
+    # Index nodes (by id) of `exp` that are read with one vector load per V lanes, or once per group.
+    vector_loads: Dict[int, str] = field(default_factory=dict)  # id(node) -> "vector" | "uniform"
+    epi_vector_loads: Dict[int, str] = field(default_factory=dict)
+    gemm: Optional[dict] = None
+
+
+def tuneNullopt(kernel: Kernel) -> TuneResult:
+    """Lower views and bind gidx/ridx ranges without any optimisation (src/tuner.ts:219-240)."""
+    exp = kernel.exp
+    vars_ = {"gidx": AluExp.special(DType.Int32, "gidx", max(kernel.size, 1))}
+    re = kernel.reduction
+    if re is not None:
+        vars_["ridx"] = AluExp.special(DType.Int32, "ridx", max(re.size, 1))
+        if exp.dtype != re.dtype:
+            exp = AluExp.cast(re.dtype, exp)
+    epilogue = None
+    if re is not None:
+        epilogue = re.epilogue.substitute({"gidx": vars_["gidx"]}).rewriteGlobalViews().simplify()
+    return TuneResult(exp=exp.substitute(vars_).rewriteGlobalViews().simplify(), epilogue=epilogue)
+
+
+# ------------------------------------------------------------------------------------------------
+# Affine lane analysis
+# ------------------------------------------------------------------------------------------------
+
+
+def _is_symbol(e: AluExp, name: str) -> bool:
+    return (e.op == AluOp.Special and e.arg[0] == name) or (e.op == AluOp.Variable and e.arg == name)
+
+
+def references(e: AluExp, name: str, memo: Optional[dict] = None) -> bool:
+    return e.some(lambda n: _is_symbol(n, name))
+
+
+def known_divisor(e: AluExp) -> int:
+    """An integer that provably divides e's value (0 means "e is 0", i.e. divisible by anything)."""
+    if e.op == AluOp.Const:
+        return abs(int(e.arg)) if float(e.arg).is_integer() else 1
+    if e.op == AluOp.Mul:
+        a, b = known_divisor(e.src[0]), known_divisor(e.src[1])
+        return a * b
+    if e.op in (AluOp.Add, AluOp.Sub):
+        return math.gcd(known_divisor(e.src[0]), known_divisor(e.src[1]))
+    if e.op == AluOp.Mod and e.src[1].op == AluOp.Const:
+        return math.gcd(known_divisor(e.src[0]), abs(int(e.src[1].arg)))
+    if e.op == AluOp.Where:
+        return math.gcd(known_divisor(e.src[1]), known_divisor(e.src[2]))
+    return 1
+
+
+def lane_form(e: AluExp, sym: str, V: int) -> Optional[Tuple[int, int]]:
+    """Describe e when `sym = V*q + lane`, lane in [0,V): returns (stride, align) such that
+    e == u + stride*lane with u independent of lane and u % align == 0 (align 0: u is 0), or None
+    if e is not affine in the lane.  Only index arithmetic (int32 +,-,*,/,% by constants) is
+    understood; everything else referencing `sym` is "unknown".
+    """
+    if not references(e, sym):
+        return (0, known_divisor(e))
+    if _is_symbol(e, sym):
+        return (1, V)
+    if e.dtype not in (DType.Int32, DType.Uint32):
+        return None
+    op = e.op
+    if op in (AluOp.Add, AluOp.Sub):
+        a, b = lane_form(e.src[0], sym, V), lane_form(e.src[1], sym, V)
+        if a is None or b is None:
+            return None
+        stride = a[0] + b[0] if op == AluOp.Add else a[0] - b[0]
+        return (stride, math.gcd(a[1], b[1]))
+    if op == AluOp.Mul:
+        for i in (0, 1):
+            c = e.src[i]
+            if c.op == AluOp.Const:
+                f = lane_form(e.src[1 - i], sym, V)
+                if f is None:
+                    return None
+                return (f[0] * int(c.arg), f[1] * abs(int(c.arg)))
+        return None
+    if op in (AluOp.Idiv, AluOp.Mod) and e.src[1].op == AluOp.Const:
+        C = int(e.src[1].arg)
+        inner = e.src[0]
+        f = lane_form(inner, sym, V)
+        if f is None or C <= 0 or inner.min < 0:
+            return None
+        stride, align = f
+        if stride == 0:
+            return (0, math.gcd(align, C) if op == AluOp.Mod else 1)
+        # (u + s*lane) with 0 <= s*lane < s*V: stays inside one period of C when C | u's alignment
+        # step, i.e. when both C and align are multiples of s*V.
+        if stride < 0:
+            return None
+        span = stride * V
+        if C % span == 0 and (align == 0 or align % span == 0):
+            if op == AluOp.Mod:
+                return (stride, math.gcd(align, C))
+            return (0, 1)
+        return None
+    return None
+
+
+def _load_nodes(exp: Optional[AluExp]) -> List[AluExp]:
+    return exp.collect(lambda n: n.op == AluOp.GlobalIndex) if exp is not None else []
+
+
+def _in_bounds(node: AluExp) -> bool:
+    idx = node.src[0]
+    return idx.min >= 0 and idx.max < node.arg[1]
+
+
+def classify_loads(exp: Optional[AluExp], sym: str, V: int) -> Dict[int, str]:
+    """id(GlobalIndex node) -> "vector" (V consecutive, aligned elements per lane group) or
+    "uniform" (same element for the whole group).  Loads needing a bounds guard stay scalar."""
+    out: Dict[int, str] = {}
+    if V <= 1:
+        return out
+    for node in _load_nodes(exp):
+        if not _in_bounds(node):
+            continue
+        f = lane_form(node.src[0], sym, V)
+        if f is None:
+            continue
+        stride, align = f
+        if stride == 0:
+            out[id(node)] = "uniform"
+        elif stride == 1 and (align == 0 or align % V == 0):
+            out[id(node)] = "vector"
+    return out
+
+
+def _pow2_floor(x: int) -> int:
+    return 1 << (max(int(x), 1).bit_length() - 1)
+
+
+def _elem_sizes(exp: Optional[AluExp]) -> List[int]:
+    return [byteWidth(n.dtype) for n in _load_nodes(exp)]
+
+
+def _pick_vector_width(kernel: Kernel, t: TuneResult, axis_len: int) -> int:
+    """Elements per lane so that the narrowest stream moves 128 bits."""
+    sizes = _elem_sizes(t.exp) + _elem_sizes(t.epilogue) + [byteWidth(kernel.dtype)]
+    smallest = min(sizes)
+    V = max(16 // smallest, 1)
+    if max(sizes) == 8:
+        V = min(V, 4)
+    while V > 1 and axis_len < V:
+        V //= 2
+    return V
+
+
+# ------------------------------------------------------------------------------------------------
+# GEMM recognition
+# ------------------------------------------------------------------------------------------------
+
+
+def _strip_float_casts(e: AluExp) -> AluExp:
+    while e.op == AluOp.Cast and isFloatDtype(e.dtype) and isFloatDtype(e.src[0].dtype):
+        e = e.src[0]
+    return e
+
+
+def match_gemm(kernel: Kernel) -> Optional[dict]:
+    """Recognise `sum_k A[..m..,k] * B[..n..,k]` over single-view, unmasked operands.
+
+    Same precondition the reference's WebGPU tuner checks before optimising a reduction
+    (src/tuner.ts:255-282): every GlobalView is indexed by `[unravel(gidx)..., ridx]`.  Axes of the
+    broadcast shape are then classified by the operands' strides into batch / M / N, adjacent axes
+    with compatible strides are merged, and exactly one M and one N axis must remain.
+    """
+    re = kernel.reduction
+    if re is None or re.op != AluOp.Add or re.dtype != DType.Float32:
+        return None
+    root = _strip_float_casts(kernel.exp)
+    if root.op != AluOp.Mul:
+        return None
+    a, b = _strip_float_casts(root.src[0]), _strip_float_casts(root.src[1])
+    if a.op != AluOp.GlobalView or b.op != AluOp.GlobalView or a.dtype != b.dtype:
+        return None
+    if a.dtype not in (DType.Float16, DType.Float32):
+        return None
+    sta, stb = a.arg[1], b.arg[1]
+    if len(sta.views) != 1 or len(stb.views) != 1:
+        return None
+    va, vb = sta.views[0], stb.views[0]
+    if va.mask is not None or vb.mask is not None or va.shape != vb.shape or len(va.shape) < 1:
+        return None
+    shape = list(va.shape)
+    if shape[-1] != re.size or math.prod(shape[:-1]) != kernel.size or kernel.size == 0 or re.size == 0:
+        return None
+    expected = [u.simplify() for u in unravelAlu(shape[:-1], AluVar.gidx)] + [AluVar.ridx]
+    for gv in (a, b):
+        if len(gv.src) != len(expected) or any(x.simplify() is not y for x, y in zip(gv.src, expected)):
+            return None
+    ska, skb = va.strides[-1], vb.strides[-1]
+    if shape[-1] > 1 and (ska == 0 or skb == 0):
+        return None
+    # Output strides: row-major over shape[:-1].
+    outs = [1] * (len(shape) - 1)
+    for i in range(len(outs) - 2, -1, -1):
+        outs[i] = outs[i + 1] * shape[i + 1]
+    axes = []  # (role, size, stride_a, stride_b, stride_out)
+    for i in range(len(shape) - 1):
+        n = shape[i]
+        if n == 1:
+            continue
+        sa, sb = va.strides[i], vb.strides[i]
+        role = "batch" if (sa != 0) == (sb != 0) else ("m" if sa != 0 else "n")
+        axes.append([role, n, sa, sb, outs[i]])
+    # Merge neighbours of equal role whose strides nest (outer == inner * inner_size).
+    merged: List[list] = []
+    for ax in axes:
+        if merged and merged[-1][0] == ax[0]:
+            p = merged[-1]
+            if all(p[k] == ax[k] * ax[1] for k in (2, 3, 4)):
+                merged[-1] = [p[0], p[1] * ax[1], ax[2], ax[3], ax[4]]
+                continue
+        merged.append(ax)
+    ms = [x for x in merged if x[0] == "m"]
+    ns = [x for x in merged if x[0] == "n"]
+    bs = [x for x in merged if x[0] == "batch"]
+    if len(ms) > 1 or len(ns) > 1 or len(bs) > 3:
+        return None
+    m = ms[0] if ms else ["m", 1, 0, 0, 0]
+    n = ns[0] if ns else ["n", 1, 0, 0, 0]
+    info = dict(
+        dtype=a.dtype, gid_a=a.arg[0], gid_b=b.arg[0],
+        M=m[1], N=n[1], K=shape[-1],
+        a_off=va.offset, a_sm=m[2], a_sk=ska,
+        b_off=vb.offset, b_sn=n[3], b_sk=skb,
+        c_sm=m[4], c_sn=n[4],
+        batch=[(x[1], x[2], x[3], x[4]) for x in bs],
+        a_len=va.dataRange()[1], b_len=vb.dataRange()[1],
+    )
+    # Negative strides (flipped views) are left to the generic path.
+    if min(info["a_sm"], info["a_sk"], info["b_sn"], info["b_sk"], info["a_off"], info["b_off"]) < 0:
+        return None
+    if any(min(x[1:]) < 0 for x in info["batch"]):
+        return None
+    return info
+
+
+# ------------------------------------------------------------------------------------------------
+# tuneHip
+# ------------------------------------------------------------------------------------------------
+
+
+def _grid_for(blocks_needed: int) -> int:
+    return max(1, min(int(blocks_needed), MAX_GRID_BLOCKS))
+
+
+def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True) -> TuneResult:
+    """Pick the kernel class and its parameters for one Kernel on MI355X."""
+    t = tuneNullopt(kernel)
+    re = kernel.reduction
+    size = kernel.size
+
+    if re is None:
+        V = _pick_vector_width(kernel, t, size)
+        t.klass = "map"
+        t.vector_loads = classify_loads(t.exp, "gidx", V)
+        groups = max(size // V, 1)
+        t.params = dict(V=V, block=256, grid=_grid_for((groups + 255) // 256))
+        return t
+
+    R = re.size
+    if allow_gemm and GEMM_ENABLED:
+        g = match_gemm(kernel)
+        if g is not None and _gemm_worthwhile(g):
+            t.klass = "gemm"
+            t.gemm = g
+            return t
+
+    loads = _load_nodes(t.exp)
+    Vr = _pick_vector_width(kernel, t, R)
+    along_r = classify_loads(t.exp, "ridx", Vr)
+    Vg = _pick_vector_width(kernel, t, size)
+    along_g = classify_loads(t.exp, "gidx", Vg)
+    n_row = sum(1 for v in along_r.values() if v == "vector")
+    n_col = sum(1 for v in along_g.values() if v == "vector")
+    # Which axis do the heavy streams walk at unit stride?  Weight every load by the bytes it can
+    # touch, so that a large matrix decides the orientation and a small broadcast vector does not.
+    w_row = w_col = 0
+    for node in loads:
+        weight = node.arg[1] * byteWidth(node.dtype)
+        fr = lane_form(node.src[0], "ridx", 1)
+        fg = lane_form(node.src[0], "gidx", 1)
+        if fr is not None and fr[0] == 1:
+            w_row += weight
+        elif fg is not None and fg[0] == 1:
+            w_col += weight
+
+    row_major = w_row >= w_col and w_row > 0 and R >= 8
+    if w_row == 0 and w_col == 0 and size < 4096 and R >= 1024:
+        row_major = True  # few outputs, long fold, no coalescing either way: spread the fold over lanes
+
+    if row_major:
+        V = Vr if n_row > 0 else 1
+        vec_iters = max(R // V, 1)
+        t_hi = min(_pow2_floor(vec_iters), 1024)
+        # Enough lanes per row that a wave reads long contiguous runs, then ~8 vector loads per lane.
+        T = max(min(t_hi, 16), min(_pow2_floor(max(vec_iters // 8, 1)), t_hi))
+        while T < t_hi and size * T < CU_COUNT * 512:
+            T *= 2
+        block = max(T, 256)
+        rows = block // T
+        split = 1
+        if allow_split:
+            lanes_busy = size * T
+            if lanes_busy < CU_COUNT * 512 and R // (T * V) >= 64:
+                want = (CU_COUNT * 1024) // max(lanes_busy, 1)
+                split = max(1, min(want, R // (T * V * 8), 1024))
+        t.klass = "reduce_row"
+        t.vector_loads = along_r if V > 1 else {}
+        t.params = dict(V=V, T=T, block=block, rows=rows, split=split)
+        nrb = (size + rows - 1) // rows
+        t.params["grid"] = _grid_for(nrb)
+        return t
+
+    V = Vg if n_col > 0 else 1
+    groups = max(size // V, 1)
+    lx = 64
+    # Split the fold over waves (and blocks) when there are too few output groups to fill the chip.
+    T = 1
+    while T < 16 and groups * T < CU_COUNT * 256 and R // (T * 2) >= 8:
+        T *= 2
+    split = 1
+    if allow_split and groups * T < CU_COUNT * 256 and R // T >= 64:
+        want = (CU_COUNT * 512) // max(groups * T, 1)
+        split = max(1, min(want, R // (T * 16), 1024))
+    t.klass = "reduce_col"
+    t.vector_loads = along_g if V > 1 else {}
+    t.params = dict(V=V, T=T, lx=lx, block=lx * T, split=split)
+    t.params["grid"] = _grid_for((groups + lx - 1) // lx)
+    t.epi_vector_loads = classify_loads(t.epilogue, "gidx", V) if V > 1 else {}
+    return t
+
+
+def _gemm_worthwhile(g: dict) -> bool:
+    """MFMA tiles only pay off for a real dense contraction; thin shapes stream better through
+    the row-reduce template (matvec and friends)."""
+    if g["M"] < 16 or g["N"] < 16 or g["K"] < 16:
+        return False
+    a_ok = g["a_sk"] == 1 or g["a_sm"] == 1
+    b_ok = g["b_sk"] == 1 or g["b_sn"] == 1
+    return a_ok and b_ok
