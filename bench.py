@@ -1,0 +1,205 @@
+#!/usr/bin/env python3
+"""Benchmark of the jax-js `hip` backend on one MI355X.
+
+Headline workload (`config.workload`): dense f16 GEMM 8192^3 (f32 accumulation, f16 result) lowered the
+way `np.matmul` lowers it, one dispatch per step, operands resident in HBM.  `value` is TFLOP/s with
+FLOPs = 2*M*N*K (the reference's own convention, website/src/routes/bench/matmul/+page.svelte:16).
+`roofline` is priced against the dense f16 MFMA peak; `cpu_baseline` times a single-core C restatement of
+the reference Wasm backend's tiled f32 matmul loop on a slice of the same problem (the Wasm backend has
+no f16 and is single-threaded in Node).  `extra` carries the other configurations: f16 matvec in both
+layouts and the four fused row-reduce kernels of the softmax/argmax configuration (HBM-bound, GB/s),
+an f32 elementwise map, the f32 1024^3 matmul and a GEMM sweep.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (os.path.join(ROOT, "jax-js_amd"), ROOT):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+import numpy as np  # noqa: E402
+
+PEAK_HBM_GBS = 8000.0
+PEAK_F16_TFLOPS = 2500.0
+PEAK_F32_MATRIX_TFLOPS = 157.3
+
+
+def timed(be, exe, ins, out, steps, warmup):
+    """W untimed + K timed dispatches; wall clock around a device fence and HIP events on the stream."""
+    dev = be.dev
+    for _ in range(warmup):
+        be.dispatch(exe, ins, [out])
+    dev.sync()
+    e0, e1 = dev.event(), dev.event()
+    t0 = time.perf_counter()
+    dev.record(e0)
+    for _ in range(steps):
+        be.dispatch(exe, ins, [out])
+    dev.record(e1)
+    dev.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ev_ms = dev.elapsed_ms(e0, e1) / steps
+    dev.destroy_event(e0)
+    dev.destroy_event(e1)
+    return wall_ms, ev_ms
+
+
+def upload(be, arr):
+    a = np.ascontiguousarray(arr)
+    return be.malloc(a.nbytes, a.tobytes())
+
+
+def cpu_baseline_matmul(n, seconds=12.0):
+    """Single-core Wasm-loop restatement on an M-row slice of the n^3 problem, f32 stand-in for f16."""
+    from oracle import oracle
+    from jaxjs_hip import hostrand
+
+    L = oracle.lib()
+    rows = 32
+    B = hostrand.uniform(1004 + 1, (n, n), dtype=np.float32, stream=1)
+    done_flops, spent = 0.0, 0.0
+    sample_rows = 0
+    while spent < seconds:
+        A = hostrand.uniform(1004, (rows, n), dtype=np.float32)
+        C = np.empty((rows, n), dtype=np.float32)
+        t0 = time.perf_counter()
+        rc = L.jo_wasm_matmul_f32(A.ctypes.data_as(ctypes.c_void_p), B.ctypes.data_as(ctypes.c_void_p),
+                                  C.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(rows), ctypes.c_int64(n), ctypes.c_int64(n))
+        dt = time.perf_counter() - t0
+        assert rc == 0
+        spent += dt
+        done_flops += 2.0 * rows * n * n
+        sample_rows += rows
+        rate = done_flops / spent
+        rows = int(min(512, max(32, (seconds - spent) * rate / (2.0 * n * n) // 32 * 32)))
+        if seconds - spent < 0.5:
+            break
+    return dict(value=done_flops / spent / 1e12, unit="TFLOP/s", cores=1, kind="port",
+                sample=f"{sample_rows} of {n} output rows of the same {n}^3 problem in f32 (Wasm has no f16), "
+                       f"{spent:.1f} s on one host core; {os.cpu_count()} cores present")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--size", type=int, default=8192, help="M=N=K of the headline GEMM")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    from jaxjs_hip import AluExp, AluOp, DType, ShapeTracker, getBackend, hostrand, init
+    from jaxjs_hip.lowering import mapKernel, matmulKernel, matvecKernel, reduceKernel
+
+    init("hip")
+    be = getBackend("hip")
+    n = args.size
+
+    # ---- headline: f16 GEMM n^3 -----------------------------------------------------------------
+    A = hostrand.uniform(1004, (n, n), dtype=np.float16)
+    B = hostrand.uniform(1005, (n, n), dtype=np.float16, stream=1)
+    kern = matmulKernel(n, n, n, DType.Float16)
+    exe = be.prepareKernelSync(kern)
+    a, b = upload(be, A), upload(be, B)
+    c = be.malloc(kern.bytes)
+    wall_ms, ev_ms = timed(be, exe, [a, b], c, args.steps, args.warmup)
+    flops = 2.0 * n * n * n
+    value = flops / (wall_ms * 1e-3) / 1e12
+    achieved = flops / (ev_ms * 1e-3) / 1e12
+    result = {
+        "metric": "matmul TFLOP/s + f16 matvec HBM GB/s (% MI355X roofline) vs Wasm CPU",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"dense GEMM f16 {n}x{n}x{n}, f32 accumulate, np.matmul lowering (B stored [K,N])",
+                   "kernel_class": exe.data.ks.klass, "tile": exe.data.ks.info},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": None},
+    }
+    for s in (a, b, c):
+        be.decRef(s)
+    del A, B
+
+    extra = {}
+    if not args.no_extra:
+        steps, warm = max(args.steps, 20), max(args.warmup, 5)
+
+        def run(name, kernel, bufs, work, unit, peak):
+            ex = be.prepareKernelSync(kernel)
+            slots = [upload(be, x) for x in bufs]
+            o = be.malloc(kernel.bytes)
+            w_ms, e_ms = timed(be, ex, slots, o, steps, warm)
+            for s in slots + [o]:
+                be.decRef(s)
+            rate = work / (e_ms * 1e-3) / (1e9 if unit == "GB/s" else 1e12)
+            extra[name] = {"class": ex.data.ks.klass, "ms": round(e_ms, 5), "wall_ms": round(w_ms, 5),
+                           "achieved": round(rate, 2), "unit": unit, "frac_of_peak": round(rate / peak, 4)}
+
+        M, K = 11008, 4096
+        W = hostrand.normal(1003, (M, K), 0.02, np.float16)
+        x = hostrand.normal(1003, (K,), 1.0, np.float16, stream=1)
+        mv_bytes = M * K * 2 + K * 2 + M * 2
+        run("matvec_f16_W[11008,4096]", matvecKernel(M, K, DType.Float16), [W, x], mv_bytes, "GB/s", PEAK_HBM_GBS)
+        run("matvec_f16_W^T[4096,11008]", matvecKernel(M, K, DType.Float16, w_transposed=True),
+            [np.ascontiguousarray(W.T), x], mv_bytes, "GB/s", PEAK_HBM_GBS)
+        del W
+
+        rows, L = 8192, 4096
+        X = hostrand.normal(1002, (rows, L), 1.0, np.float32)
+        st = ShapeTracker.fromShape([rows, L])
+        stm = ShapeTracker.fromShape([rows]).reshape([rows, 1]).expand([rows, L])
+        f = DType.Float32
+        kmax = reduceKernel([rows, L], [(f, st)], lambda v: v, AluOp.Max)
+        m = X.max(axis=1)
+
+        def body(v, mm):
+            xm = AluExp.add(v, AluExp.sub(AluExp.f32(0), mm))
+            sig = AluExp.reciprocal(AluExp.add(AluExp.exp(AluExp.sub(AluExp.f32(0), v)), AluExp.f32(1)))
+            return AluExp.mul(AluExp.exp(xm), sig)
+
+        ksum = reduceKernel([rows, L], [(f, st), (f, stm)], body, AluOp.Add)
+        star = ShapeTracker.fromShape([L]).reshape([1, L]).expand([rows, L])
+        karg = reduceKernel(
+            [rows, L], [(f, st), (f, stm), (DType.Int32, star)],
+            lambda v, mm, rev: AluExp.mul(AluExp.cast(DType.Int32, AluExp.cmpne(v, mm).not_()), rev), AluOp.Max,
+            epilogue=lambda acc: AluExp.sub(AluExp.i32(L), acc))
+        rev = np.arange(L, 0, -1, dtype=np.int32)
+        xb = rows * L * 4
+        run("c2_rowmax_f32[8192,4096]", kmax, [X], xb + rows * 4, "GB/s", PEAK_HBM_GBS)
+        run("c2_sum_exp_sigmoid", ksum, [X, m], xb + 2 * rows * 4, "GB/s", PEAK_HBM_GBS)
+        run("c2_argmax", karg, [X, m, rev], xb + 2 * rows * 4 + L * 4, "GB/s", PEAK_HBM_GBS)
+        kmap = mapKernel([rows, L], [(f, st)], lambda v: AluExp.mul(AluExp.exp(v), AluExp.f32(0.5)))
+        run("map_exp_f32[8192,4096]", kmap, [X], 2 * xb, "GB/s", PEAK_HBM_GBS)
+        del X
+
+        for (mm, nn, kk, dt, tag, peak) in [
+            (1024, 1024, 1024, DType.Float32, "c1_matmul_f32_1024", PEAK_F32_MATRIX_TFLOPS),
+            (2048, 2048, 2048, DType.Float16, "gemm_f16_2048", PEAK_F16_TFLOPS),
+            (4096, 4096, 4096, DType.Float16, "gemm_f16_4096", PEAK_F16_TFLOPS),
+            (128, 14336, 4096, DType.Float16, "gemm_f16_skinny_128x14336x4096", PEAK_F16_TFLOPS),
+            (4096, 4096, 4096, DType.Float32, "gemm_f32_4096", PEAK_F32_MATRIX_TFLOPS),
+        ]:
+            npdt = np.float16 if dt == DType.Float16 else np.float32
+            Am = hostrand.uniform(1004, (mm, kk), dtype=npdt)
+            Bm = hostrand.uniform(1005, (kk, nn), dtype=npdt, stream=1)
+            run(tag, matmulKernel(mm, nn, kk, dt), [Am, Bm], 2.0 * mm * nn * kk, "TFLOP/s", peak)
+        result["extra"] = extra
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline_matmul(n)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

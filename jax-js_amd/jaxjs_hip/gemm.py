@@ -1,0 +1,87 @@
+"""Source generation for kernel class (d): MFMA GEMM (templates `gemm_f16.hip.inc`, `gemm_f32.hip.inc`).
+
+The tuner's `match_gemm` has already reduced the Kernel to strides of a batched `C = A . B^T`-style
+contraction; this module chooses the block tile, renders the fused epilogue as a device function
+and fills the template.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, List
+
+from .alu import AluExp, AluOp, DType, Kernel, byteWidth
+from .codegen import CTYPE, STORAGE_CTYPE, HipExpCodegen, strip_parens
+from .kernelgen import KernelSource, LaunchStep, _min_bytes, _prelude, _used_args, fill, template
+from .tuner import CU_COUNT, TuneResult
+
+
+def choose_tile(g: dict) -> Dict[str, int]:
+    """256x256 tiles when they still give every CU work, else 128x128."""
+    nb = 1
+    for b in g["batch"]:
+        nb *= b[0]
+
+    def tiles(bm, bn):
+        return -(-g["M"] // bm) * -(-g["N"] // bn) * nb
+
+    if g["M"] >= 256 and g["N"] >= 256 and tiles(256, 256) >= (3 * CU_COUNT) // 4:
+        return dict(BM=256, BN=256)
+    if g["M"] >= 256 and tiles(256, 128) >= (3 * CU_COUNT) // 4:
+        return dict(BM=256, BN=128)
+    return dict(BM=128, BN=128)
+
+
+def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelSource:
+    g = t.gemm
+    re = kernel.reduction
+    assert g is not None and re is not None and t.epilogue is not None
+    tile = choose_tile(g)
+    BM, BN = tile["BM"], tile["BN"]
+    out_t = STORAGE_CTYPE[kernel.dtype]
+    in_t = STORAGE_CTYPE[g["dtype"]]
+
+    used = _used_args(kernel.nargs, t.epilogue)
+    used[g["gid_a"]] = g["dtype"]
+    used[g["gid_b"]] = g["dtype"]
+    names = [f"in{i}" for i in range(kernel.nargs)]
+    params = ", ".join(
+        [f"const {STORAGE_CTYPE[d or DType.Float32]}* __restrict__ {n}" for d, n in zip(used, names)]
+        + [f"{out_t}* __restrict__ out"])
+
+    # Fused epilogue as a device function of (acc, gidx, buffers...).
+    cg = HipExpCodegen(names, {"acc": "acc", "gidx": "gidx"}, "  ", prefix="e", numerics=numerics)
+    cg.countReferences(t.epilogue)
+    value = strip_parens(cg.run(t.epilogue))
+    epi_params = "".join(f", const {STORAGE_CTYPE[d or DType.Float32]}* __restrict__ {n}" for d, n in zip(used, names))
+    epi_fn = (f"static __device__ __forceinline__ {out_t} jh_epilogue(float acc, int gidx{epi_params}) {{\n"
+              + "\n".join(cg.take_lines()) + f"\n  return ({out_t})({value});\n}}")
+    epi_args = "".join(f", {n}" for n in names)
+
+    # Batch index decode, innermost batch axis last in g["batch"].
+    lines = ["  {", "    int rem = batch;"]
+    for k, (size, sa, sb, sc) in reversed(list(enumerate(g["batch"]))):
+        lines.append(f"    const int b{k} = rem % {size}; rem /= {size};")
+        lines.append(f"    a_base += (long long)b{k} * {sa}ll; b_base += (long long)b{k} * {sb}ll; c_base += (long long)b{k} * {sc}ll;")
+    lines.append("  }")
+    nbatch = 1
+    for b in g["batch"]:
+        nbatch *= b[0]
+
+    tmpl = "gemm_f16.hip.inc" if g["dtype"] == DType.Float16 else "gemm_f32.hip.inc"
+    src = _prelude(numerics) + fill(template(tmpl), dict(
+        M=g["M"], N=g["N"], K=g["K"], BM=BM, BN=BN,
+        A_KCONTIG=1 if g["a_sk"] == 1 or g["K"] == 1 else 0, B_KCONTIG=1 if g["b_sk"] == 1 or g["K"] == 1 else 0,
+        NBATCH=nbatch, EPILOGUE_FN=epi_fn, NAME=name, PARAMS=params,
+        A_OFF=g["a_off"], B_OFF=g["b_off"], BATCH_DECODE="\n".join(lines),
+        A_PTR=names[g["gid_a"]], B_PTR=names[g["gid_b"]],
+        A_SM=g["a_sm"], A_SK=g["a_sk"], B_SN=g["b_sn"], B_SK=g["b_sk"],
+        C_SM=g["c_sm"], C_SN=g["c_sn"], EPILOGUE_ARGS=epi_args))
+    tiles = -(-g["M"] // BM) * -(-g["N"] // BN) * nbatch
+    step = LaunchStep(name, (tiles, 1, 1), (256, 1, 1), 0, [("in", i) for i in range(kernel.nargs)] + [("out", 0)])
+    need = _min_bytes(t.epilogue)
+    eb = byteWidth(g["dtype"])
+    need[g["gid_a"]] = max(need.get(g["gid_a"], 0), g["a_len"] * eb)
+    need[g["gid_b"]] = max(need.get(g["gid_b"], 0), g["b_len"] * eb)
+    info = dict(BM=BM, BN=BN, BK=64, tiles=tiles, a_kcontig=g["a_sk"] == 1, b_kcontig=g["b_sk"] == 1,
+                M=g["M"], N=g["N"], K=g["K"], nbatch=nbatch)
+    return KernelSource([src], [step], [], "gemm", need, info)

@@ -31,7 +31,7 @@ from .shape import ShapeTracker, unravelAlu
 CU_COUNT = 256          # MI355X: 8 XCDs x 32 CUs
 WAVE = 64
 MAX_GRID_BLOCKS = CU_COUNT * 16
-GEMM_ENABLED = False   # flipped on once the MFMA template is in place
+GEMM_ENABLED = True
 
 
 @dataclass
@@ -379,10 +379,24 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
 
 
 def _gemm_worthwhile(g: dict) -> bool:
-    """MFMA tiles only pay off for a real dense contraction; thin shapes stream better through
-    the row-reduce template (matvec and friends)."""
-    if g["M"] < 16 or g["N"] < 16 or g["K"] < 16:
+    """MFMA tiles only pay off for a real dense contraction; thin shapes stream better through the
+    row-reduce template (matvec and friends).  The tile loaders move 128-bit vectors, so every
+    address they form must be a multiple of the vector: unit stride on k or on the row axis, all
+    other strides and offsets divisible by the vector length."""
+    if g["M"] < 32 or g["N"] < 32 or g["K"] < 32:
         return False
-    a_ok = g["a_sk"] == 1 or g["a_sm"] == 1
-    b_ok = g["b_sk"] == 1 or g["b_sn"] == 1
-    return a_ok and b_ok
+    if g["dtype"] != DType.Float16:
+        return False
+    vec = 8 if g["dtype"] == DType.Float16 else 4
+    bstr_a = [b[1] for b in g["batch"]]
+    bstr_b = [b[2] for b in g["batch"]]
+
+    def operand_ok(sk, srow, rows, off, bstr):
+        if sk == 1:
+            return g["K"] % vec == 0 and srow % vec == 0 and off % vec == 0 and all(x % vec == 0 for x in bstr)
+        if srow == 1:
+            return rows % vec == 0 and sk % vec == 0 and off % vec == 0 and all(x % vec == 0 for x in bstr)
+        return False
+
+    return (operand_ok(g["a_sk"], g["a_sm"], g["M"], g["a_off"], bstr_a)
+            and operand_ok(g["b_sk"], g["b_sn"], g["N"], g["b_off"], bstr_b))

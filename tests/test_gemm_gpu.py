@@ -1,0 +1,118 @@
+"""Kernel class (d): MFMA GEMM parity.  f16 operands / f32 accumulation; bars: integer-valued inputs exact,
+otherwise |gpu - f64| <= 2*K*eps32*sum|a||b| on the accumulator plus half an ulp of the f16 result."""
+import numpy as np
+import pytest
+
+from jaxjs_hip import AluExp, AluOp, AluVar, DType, Kernel, Reduction, ShapeTracker, unravelAlu
+from jaxjs_hip.lowering import matmulKernel, reduceKernel
+from gpu_util import device_run
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+RNG = np.random.default_rng(77)
+
+
+def _check(got, A, B, K, out_f16=True):
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    mag = np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)
+    bound = 2 * K * np.finfo(np.float32).eps * mag
+    if out_f16:
+        bound = bound + np.abs(ref) * 2.0**-11 + 2.0**-24
+    err = np.abs(got.astype(np.float64).reshape(ref.shape) - ref)
+    assert np.all(err <= bound), f"max excess {np.max(err - bound)}"
+
+
+SHAPES = [(128, 128, 64), (256, 256, 128), (200, 264, 136), (32, 32, 32), (512, 384, 1000 // 8 * 8), (96, 1024, 72),
+          (1024, 1024, 1024)]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES, ids=lambda v: str(v))
+@pytest.mark.parametrize("layout", ["NN", "NT", "TN"])
+def test_gemm_f16_layouts(M, N, K, layout):
+    A = RNG.uniform(-1, 1, (M, K)).astype(np.float16)
+    B = RNG.uniform(-1, 1, (K, N)).astype(np.float16)
+    if layout == "TN":
+        if M % 8:
+            pytest.skip("A stored [K,M] needs M % 8 == 0 for the vector loader; other shapes take the generic class")
+        full = [M, N, K]
+        stA = ShapeTracker.fromShape([K, M]).permute([1, 0]).reshape([M, 1, K]).expand(full)
+        stB = ShapeTracker.fromShape([K, N]).permute([1, 0]).reshape([1, N, K]).expand(full)
+        k = reduceKernel(full, [(DType.Float16, stA), (DType.Float16, stB)], lambda a, b: AluExp.mul(a, b), AluOp.Add)
+        bufs = [np.ascontiguousarray(A.T), B]
+    else:
+        k = matmulKernel(M, N, K, DType.Float16, b_transposed=(layout == "NT"))
+        bufs = [A, np.ascontiguousarray(B.T) if layout == "NT" else B]
+    got, ks = device_run(k, bufs)
+    if layout != "NN" or N % 8 == 0:
+        assert ks.klass == "gemm", ks.klass
+    _check(got, A, B, K)
+
+
+def test_gemm_integer_valued_is_exact():
+    """Products and partial sums of small integers are exact in f32 whatever the order (the
+    200-256-200 style cases of test/numpy.test.ts:1510-1660)."""
+    M, N, K = 200, 200, 256
+    A = RNG.integers(-4, 5, (M, K)).astype(np.float16)
+    B = RNG.integers(-4, 5, (K, N)).astype(np.float16)
+    got, ks = device_run(matmulKernel(M, N, K, DType.Float16), [A, B])
+    assert ks.klass == "gemm"
+    np.testing.assert_array_equal(got.reshape(M, N).astype(np.float64), A.astype(np.float64) @ B.astype(np.float64))
+    got, _ = device_run(matmulKernel(64, 64, 64, DType.Float16), [np.ones((64, 64), np.float16)] * 2)
+    np.testing.assert_array_equal(got, np.full(64 * 64, 64, np.float16))
+
+
+def test_gemm_matches_checker_small():
+    M, N, K = 64, 96, 64
+    A = RNG.uniform(-1, 1, (M, K)).astype(np.float16)
+    B = RNG.uniform(-1, 1, (K, N)).astype(np.float16)
+    k = matmulKernel(M, N, K, DType.Float16)
+    got, ks = device_run(k, [A, B])
+    assert ks.klass == "gemm"
+    want = oracle.run_kernel(k, [A, B], oracle.MODE_CPU)
+    np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64), rtol=1e-2, atol=1e-3)
+
+
+def test_gemm_batched_two_batch_axes():
+    """Attention-score layout: einsum("BLNH,BSNH->BNLS") has two batch axes that cannot be merged
+    (strides from src/library/numpy/einsum.ts:345-353)."""
+    Bt, Nh, L, S, H = 2, 3, 64, 96, 32
+    q = RNG.normal(0, 1, (Bt, L, Nh, H)).astype(np.float16)
+    kk = RNG.normal(0, 1, (Bt, S, Nh, H)).astype(np.float16)
+    full = [Bt, Nh, L, S, H]
+    stq = ShapeTracker.fromShape([Bt, L, Nh, H]).permute([0, 2, 1, 3]).reshape([Bt, Nh, L, 1, H]).expand(full)
+    stk = ShapeTracker.fromShape([Bt, S, Nh, H]).permute([0, 2, 1, 3]).reshape([Bt, Nh, 1, S, H]).expand(full)
+    k = reduceKernel(full, [(DType.Float16, stq), (DType.Float16, stk)], lambda a, b: AluExp.mul(a, b), AluOp.Add)
+    got, ks = device_run(k, [q, kk])
+    assert ks.klass == "gemm" and ks.info["nbatch"] == Bt * Nh
+    ref = np.einsum("blnh,bsnh->bnls", q.astype(np.float64), kk.astype(np.float64))
+    np.testing.assert_allclose(got.reshape(ref.shape).astype(np.float64), ref, rtol=2e-3, atol=2e-2)
+
+
+def test_gemm_fused_epilogue_bias_relu_f32_out():
+    """Epilogue reads another buffer at the output position and changes dtype (src/frontend/jit.ts:816-889)."""
+    M, N, K = 192, 320, 128
+    A = RNG.uniform(-1, 1, (M, K)).astype(np.float16)
+    B = RNG.uniform(-1, 1, (K, N)).astype(np.float16)
+    bias = RNG.uniform(-1, 1, N).astype(np.float32)
+    base = matmulKernel(M, N, K, DType.Float16)
+    acc = AluVar.acc(DType.Float32)
+    n_idx = unravelAlu([M, N], AluVar.gidx)[1]
+    b = AluExp.globalView(DType.Float32, 2, ShapeTracker.fromShape([N]), [n_idx])
+    epi = AluExp.max(AluExp.add(acc, b), AluExp.f32(0))
+    k = Kernel(3, M * N, base.exp_raw, Reduction(DType.Float32, AluOp.Add, K, epi))
+    got, ks = device_run(k, [A, B, bias])
+    assert ks.klass == "gemm" and got.dtype == np.float32
+    ref = np.maximum(A.astype(np.float64) @ B.astype(np.float64) + bias, 0)
+    np.testing.assert_allclose(got.reshape(M, N), ref, rtol=1e-4, atol=1e-4)
+
+
+def test_gemm_8192_cubed_sampled():
+    """Headline shape.  Full f64 verification would take minutes on the host; rows are independent, so a
+    sample of 24 rows spread over all tile rows (and every column) is compared with exact dot products."""
+    n = 8192
+    A = RNG.uniform(-1, 1, (n, n)).astype(np.float16)
+    B = RNG.uniform(-1, 1, (n, n)).astype(np.float16)
+    got, ks = device_run(matmulKernel(n, n, n, DType.Float16), [A, B])
+    assert ks.klass == "gemm"
+    rows = sorted(set(list(range(0, n, 353)) + [255, 256, n - 1]))
+    _check(got.reshape(n, n)[rows], A[rows], B, n)
