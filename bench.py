@@ -92,6 +92,8 @@ def main():
     ap.add_argument("--size", type=int, default=8192, help="M=N=K of the headline GEMM")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--only", choices=["all", "gemm", "copy"], default="all",
+                    help="gemm: headline kernel only; copy: a plain f32 copy kernel of known size (counter calibration)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -103,6 +105,19 @@ def main():
     init("hip")
     be = getBackend("hip")
     n = args.size
+    if args.only == "gemm":
+        args.no_extra = True
+    if args.only == "copy":
+        # 8192x4096 f32 copied once per step: 134,217,728 bytes read and as many written per launch.
+        rows, L = 8192, 4096
+        X = hostrand.normal(1002, (rows, L), 1.0, np.float32)
+        kcopy = mapKernel([rows, L], [(DType.Float32, ShapeTracker.fromShape([rows, L]))], lambda v: v)
+        ex = be.prepareKernelSync(kcopy)
+        src, dst = upload(be, X), be.malloc(kcopy.bytes)
+        w_ms, e_ms = timed(be, ex, [src], dst, args.steps, args.warmup)
+        print(json.dumps({"workload": "copy f32 [8192,4096]", "bytes_read": rows * L * 4, "bytes_written": rows * L * 4,
+                          "ms": e_ms, "GBps": 2 * rows * L * 4 / (e_ms * 1e-3) / 1e9}))
+        return
 
     # ---- headline: f16 GEMM n^3 -----------------------------------------------------------------
     A = hostrand.uniform(1004, (n, n), dtype=np.float16)

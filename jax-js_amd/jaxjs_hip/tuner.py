@@ -385,8 +385,6 @@ def _gemm_worthwhile(g: dict) -> bool:
     other strides and offsets divisible by the vector length."""
     if g["M"] < 32 or g["N"] < 32 or g["K"] < 32:
         return False
-    if g["dtype"] != DType.Float16:
-        return False
     vec = 8 if g["dtype"] == DType.Float16 else 4
     bstr_a = [b[1] for b in g["batch"]]
     bstr_b = [b[2] for b in g["batch"]]

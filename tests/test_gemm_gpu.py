@@ -116,3 +116,43 @@ def test_gemm_8192_cubed_sampled():
     assert ks.klass == "gemm"
     rows = sorted(set(list(range(0, n, 353)) + [255, 256, n - 1]))
     _check(got.reshape(n, n)[rows], A[rows], B, n)
+
+
+F32_SHAPES = [(64, 64, 64), (128, 128, 64), (200, 264, 136), (1024, 1024, 1024), (96, 1028, 72), (512, 384, 100)]
+
+
+@pytest.mark.parametrize("M,N,K", F32_SHAPES, ids=lambda v: str(v))
+@pytest.mark.parametrize("layout", ["NN", "NT", "TN"])
+def test_gemm_f32_layouts(M, N, K, layout):
+    """Config 1/4 in f32 on v_mfma_f32_32x32x2_f32: |gpu - f64| <= 2*K*eps32*sum|a||b| (f32 rel 1e-5 class)."""
+    A = RNG.uniform(-1, 1, (M, K)).astype(np.float32)
+    B = RNG.uniform(-1, 1, (K, N)).astype(np.float32)
+    if layout == "TN":
+        if M % 4:
+            pytest.skip("A stored [K,M] needs M % 4 == 0 for the vector loader")
+        full = [M, N, K]
+        stA = ShapeTracker.fromShape([K, M]).permute([1, 0]).reshape([M, 1, K]).expand(full)
+        stB = ShapeTracker.fromShape([K, N]).permute([1, 0]).reshape([1, N, K]).expand(full)
+        k = reduceKernel(full, [(DType.Float32, stA), (DType.Float32, stB)], lambda a, b: AluExp.mul(a, b), AluOp.Add)
+        bufs = [np.ascontiguousarray(A.T), B]
+    else:
+        k = matmulKernel(M, N, K, DType.Float32, b_transposed=(layout == "NT"))
+        bufs = [A, np.ascontiguousarray(B.T) if layout == "NT" else B]
+    got, ks = device_run(k, bufs)
+    assert ks.klass == "gemm", ks.klass
+    _check(got, A, B, K, out_f16=False)
+
+
+def test_gemm_f32_integer_exact_and_checker():
+    M, N, K = 200, 256, 200
+    A = RNG.integers(-8, 9, (M, K)).astype(np.float32)
+    B = RNG.integers(-8, 9, (K, N)).astype(np.float32)
+    got, ks = device_run(matmulKernel(M, N, K, DType.Float32), [A, B])
+    assert ks.klass == "gemm"
+    np.testing.assert_array_equal(got.reshape(M, N), (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32))
+    A = RNG.uniform(-1, 1, (64, 96)).astype(np.float32)
+    B = RNG.uniform(-1, 1, (96, 64)).astype(np.float32)
+    k = matmulKernel(64, 64, 96, DType.Float32)
+    got, _ = device_run(k, [A, B])
+    want = oracle.run_kernel(k, [A, B], oracle.MODE_WASM)
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-5)
