@@ -36,7 +36,12 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     re = kernel.reduction
     assert g is not None and re is not None and t.epilogue is not None
     tile = choose_tile(g)
+    tile.update(t.params.get("gemm_tile") or {})
     BM, BN = tile["BM"], tile["BN"]
+    WM, WN = tile.get("WM", 2), tile.get("WN", 2)
+    if BM % (32 * WM) or BN % (32 * WN):
+        raise ValueError(f"tile {BM}x{BN} does not divide into {WM}x{WN} waves of 32x32 MFMA tiles")
+    nthreads = 64 * WM * WN
     out_t = STORAGE_CTYPE[kernel.dtype]
     in_t = STORAGE_CTYPE[g["dtype"]]
 
@@ -68,8 +73,20 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         nbatch *= b[0]
 
     tmpl = "gemm_f16.hip.inc" if g["dtype"] == DType.Float16 else "gemm_f32.hip.inc"
-    src = _prelude(numerics) + fill(template(tmpl), dict(
-        M=g["M"], N=g["N"], K=g["K"], BM=BM, BN=BN,
+    # Fast path: direct global->LDS loads need whole tiles (no bounds predicates) and 32-deep slabs.
+    full = g["M"] % BM == 0 and g["N"] % BN == 0 and g["K"] % 32 == 0 and BM >= 128 and BN >= 128
+    dlds = g["dtype"] == DType.Float16 and full and tile.get("DLDS", 1)
+    if dlds:
+        tmpl = "gemm_f16_dlds.hip.inc"
+    if dlds:
+        sched = dict(STAGES=tile.get("STAGES", 4), PIPE=tile.get("PIPE", 1), SGB=tile.get("SGB", 1), ASM_LOAD=tile.get("ASM", 1))
+    elif g["dtype"] == DType.Float16:
+        sched = dict(COMMIT_A=tile.get("CA", 2), COMMIT_B=tile.get("CB", 3), FETCH_A=tile.get("FA", 0),
+                     FETCH_B=tile.get("FB", 1), IGLP=tile.get("IGLP", -1), SCHED_FENCE=tile.get("FENCE", 0))
+    else:
+        sched = {}
+    src = _prelude(numerics) + fill(template(tmpl), dict(sched, 
+        M=g["M"], N=g["N"], K=g["K"], BM=BM, BN=BN, WM=WM, WN=WN,
         A_KCONTIG=1 if g["a_sk"] == 1 or g["K"] == 1 else 0, B_KCONTIG=1 if g["b_sk"] == 1 or g["K"] == 1 else 0,
         NBATCH=nbatch, EPILOGUE_FN=epi_fn, NAME=name, PARAMS=params,
         A_OFF=g["a_off"], B_OFF=g["b_off"], BATCH_DECODE="\n".join(lines),
@@ -77,11 +94,11 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         A_SM=g["a_sm"], A_SK=g["a_sk"], B_SN=g["b_sn"], B_SK=g["b_sk"],
         C_SM=g["c_sm"], C_SN=g["c_sn"], EPILOGUE_ARGS=epi_args))
     tiles = -(-g["M"] // BM) * -(-g["N"] // BN) * nbatch
-    step = LaunchStep(name, (tiles, 1, 1), (256, 1, 1), 0, [("in", i) for i in range(kernel.nargs)] + [("out", 0)])
+    step = LaunchStep(name, (tiles, 1, 1), (nthreads, 1, 1), 0, [("in", i) for i in range(kernel.nargs)] + [("out", 0)])
     need = _min_bytes(t.epilogue)
     eb = byteWidth(g["dtype"])
     need[g["gid_a"]] = max(need.get(g["gid_a"], 0), g["a_len"] * eb)
     need[g["gid_b"]] = max(need.get(g["gid_b"], 0), g["b_len"] * eb)
-    info = dict(BM=BM, BN=BN, BK=64, tiles=tiles, a_kcontig=g["a_sk"] == 1, b_kcontig=g["b_sk"] == 1,
+    info = dict(BM=BM, BN=BN, WM=WM, WN=WN, BK=32 if dlds else (64 if g["dtype"] == DType.Float16 else 16), direct_lds=bool(dlds), tiles=tiles, a_kcontig=g["a_sk"] == 1, b_kcontig=g["b_sk"] == 1,
                 M=g["M"], N=g["N"], K=g["K"], nbatch=nbatch)
     return KernelSource([src], [step], [], "gemm", need, info)

@@ -291,7 +291,8 @@ def _grid_for(blocks_needed: int) -> int:
     return max(1, min(int(blocks_needed), MAX_GRID_BLOCKS))
 
 
-def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True) -> TuneResult:
+def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True,
+            gemm_tile: Optional[tuple] = None) -> TuneResult:
     """Pick the kernel class and its parameters for one Kernel on MI355X."""
     t = tuneNullopt(kernel)
     re = kernel.reduction
@@ -311,6 +312,8 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
         if g is not None and _gemm_worthwhile(g):
             t.klass = "gemm"
             t.gemm = g
+            if gemm_tile:
+                t.params["gemm_tile"] = dict(gemm_tile)
             return t
 
     loads = _load_nodes(t.exp)
