@@ -16,7 +16,7 @@ from .tuner import CU_COUNT, TuneResult
 
 
 def choose_tile(g: dict) -> Dict[str, int]:
-    """256x256 tiles when they still give every CU work, else 128x128."""
+    """f16: 256x256 tiles when they still give every CU work, else 128x128; f32: 128x128 down to 64x64."""
     nb = 1
     for b in g["batch"]:
         nb *= b[0]
@@ -24,6 +24,14 @@ def choose_tile(g: dict) -> Dict[str, int]:
     def tiles(bm, bn):
         return -(-g["M"] // bm) * -(-g["N"] // bn) * nb
 
+    if g["dtype"] == DType.Float32:
+        # The f32 matrix pipe is 16x slower than the f16 one, so LDS traffic matters little and filling
+        # every CU matters most: take the largest tile that still yields two workgroups per CU (the
+        # second one hides the first one's staging latency).
+        for bm, bn in ((128, 128), (128, 64), (64, 64)):
+            if g["M"] >= bm and g["N"] >= bn and tiles(bm, bn) >= 2 * CU_COUNT:
+                return dict(BM=bm, BN=bn)
+        return dict(BM=64, BN=64)
     if g["M"] >= 256 and g["N"] >= 256 and tiles(256, 256) >= (3 * CU_COUNT) // 4:
         return dict(BM=256, BN=256)
     if g["M"] >= 256 and tiles(256, 128) >= (3 * CU_COUNT) // 4:

@@ -197,6 +197,11 @@ def _gen_map(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     return KernelSource([src], [step], [], "map", _min_bytes(t.exp), dict(t.params))
 
 
+def _partial_pitch(size: int, V: int) -> int:
+    """Row pitch of the slice-major partial buffer: the vector stores of each slice must stay aligned."""
+    return -(-size // max(V, 1)) * max(V, 1)
+
+
 def _gen_reduce(kernel: Kernel, t: TuneResult, numerics: str, name: str, row: bool) -> KernelSource:
     re = kernel.reduction
     assert re is not None and t.epilogue is not None
@@ -250,7 +255,7 @@ def _gen_reduce(kernel: Kernel, t: TuneResult, numerics: str, name: str, row: bo
             epi_hoisted = epi_body = tail_body = ""
             epi_value = tail_value = "0"
         src = _prelude(numerics) + fill(template("reduce_col.hip.inc"), dict(
-            SIZE=size, R=R, V=V, T=T, LX=p["lx"], SPLIT=split, SLICE=slice_len,
+            SIZE=size, R=R, V=V, T=T, LX=p["lx"], SPLIT=split, SLICE=slice_len, PITCH=_partial_pitch(size, V),
             REDUCE=_reduce_text(re.op, re.dtype), NAME=name, PARAMS=params, ACC_T=acc_t, OUT_T=out_t,
             IDENTITY=ident, VECTOR_LOADS=hoisted, LANE_BODY=lane_body, LANE_VALUE=lane_value,
             SCALAR_BODY=scalar_body, SCALAR_VALUE=scalar_value,
@@ -272,9 +277,15 @@ def _gen_reduce(kernel: Kernel, t: TuneResult, numerics: str, name: str, row: bo
     step1 = LaunchStep(name, (grid_x, split, 1), (block, 1, 1), 0,
                        [("in", i) for i in range(kernel.nargs)] + [("scratch", 0)])
     gid_partial = kernel.nargs
-    idx = AluExp.add(AluExp.mul(AluVar.gidx, AluExp.i32(split)), AluVar.ridx)
+    if row:  # partial[gidx][slice]
+        idx = AluExp.add(AluExp.mul(AluVar.gidx, AluExp.i32(split)), AluVar.ridx)
+        partial_len = size * split
+    else:  # partial[slice][gidx], rows padded to the vector width
+        pitch = _partial_pitch(size, V)
+        idx = AluExp.add(AluExp.mul(AluVar.ridx, AluExp.i32(pitch)), AluVar.gidx)
+        partial_len = pitch * split
     stage2 = Kernel(kernel.nargs + 1, size,
-                    AluExp.globalIndex(re.dtype, gid_partial, size * split, idx),
+                    AluExp.globalIndex(re.dtype, gid_partial, partial_len, idx),
                     Reduction(re.dtype, re.op, split, re.epilogue))
     ks2 = generate(stage2, numerics, name=name + "_fold", allow_gemm=False, allow_split=False)
     steps2 = []
@@ -283,5 +294,5 @@ def _gen_reduce(kernel: Kernel, t: TuneResult, numerics: str, name: str, row: bo
         steps2.append(LaunchStep(s.name, s.grid, s.block, s.shared, mapped, module=s.module + 1))
     p["stage2"] = ks2.info
     need.update({g: b for g, b in ks2.min_input_bytes.items() if g != gid_partial})
-    return KernelSource([src] + ks2.sources, [step1] + steps2, [size * split * byteWidth(re.dtype)],
+    return KernelSource([src] + ks2.sources, [step1] + steps2, [partial_len * byteWidth(re.dtype)],
                         klass + "+fold", need, p)

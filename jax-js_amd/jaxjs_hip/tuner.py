@@ -366,12 +366,15 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
     groups = max(size // V, 1)
     lx = 64
     # Split the fold over waves (and blocks) when there are too few output groups to fill the chip.
+    # Blocks stay small (at most 4 waves) when the fold may also be cut across blocks: many small
+    # blocks spread over all 256 CUs, a few 1024-thread blocks leave most of them without work.
+    t_max = 4 if allow_split else 16
     T = 1
-    while T < 16 and groups * T < CU_COUNT * 256 and R // (T * 2) >= 8:
+    while T < t_max and groups * T < CU_COUNT * 256 and R // (T * 2) >= 8:
         T *= 2
     split = 1
-    if allow_split and groups * T < CU_COUNT * 256 and R // T >= 64:
-        want = (CU_COUNT * 512) // max(groups * T, 1)
+    if allow_split and groups * T < CU_COUNT * 512 and R // T >= 64:
+        want = (CU_COUNT * 1024) // max(groups * T, 1)
         split = max(1, min(want, R // (T * 16), 1024))
     t.klass = "reduce_col"
     t.vector_loads = along_g if V > 1 else {}
