@@ -100,6 +100,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         A_OFF=g["a_off"], B_OFF=g["b_off"], BATCH_DECODE="\n".join(lines),
         A_PTR=names[g["gid_a"]], B_PTR=names[g["gid_b"]],
         A_SM=g["a_sm"], A_SK=g["a_sk"], B_SN=g["b_sn"], B_SK=g["b_sk"],
+        A_K0=g["a_k0"], A_SK1=g["a_sk1"], B_K0=g["b_k0"], B_SK1=g["b_sk1"],
         C_SM=g["c_sm"], C_SN=g["c_sn"], EPILOGUE_ARGS=epi_args))
     tiles = -(-g["M"] // BM) * -(-g["N"] // BN) * nbatch
     step = LaunchStep(name, (tiles, 1, 1), (nthreads, 1, 1), 0, [("in", i) for i in range(kernel.nargs)] + [("out", 0)])

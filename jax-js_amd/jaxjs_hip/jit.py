@@ -1,0 +1,858 @@
+"""The caller side of the backend: tracing to a Jaxpr and splitting it into Kernels.
+
+This restates the slice of the reference's front-end that decides WHICH Kernels reach a backend,
+so that whole programs (the fused softmax/argmax rows, the transformer block) present the same
+Kernel sequence to the `hip` backend that `jit()` would:
+
+  Jaxpr, JaxprEqn, Var, Lit, simplify     src/frontend/jaxpr.ts:40-255, 259-360
+  promoteAvals / weak types               src/frontend/core.ts:721-736, 1288-1300
+  jitRules (expression per primitive)     src/frontend/jit.ts:486-770
+  splitGraphDataflow (kernel boundaries)  src/frontend/jit.ts:792-1096
+  jitCompile (Kernel construction)        src/frontend/jit.ts:263-469
+  JitProgram.execute                      src/frontend/jit.ts:111-162
+
+Only the primitives whose lowering is a fused Kernel are covered (elementwise, Compare, Where,
+Reduce, Dot, Transpose/Reshape/Broadcast/Flip/Shrink/Pad); routines, Gather, RandomBits, Conv and
+Concatenate/Split are not traced here.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional, Sequence, Set, Tuple, Union
+
+from .alu import AluExp, AluOp, AluVar, DType, Kernel, Reduction, byteWidth, isFloatDtype
+from .shape import ShapeTracker, prod, unravelAlu
+
+# ---- abstract values ------------------------------------------------------------------------------
+
+_RANK = {DType.Bool: 0, DType.Uint32: 1, DType.Int32: 2, DType.Float16: 3, DType.Float32: 4, DType.Float64: 5}
+
+
+def promoteTypes(a: DType, b: DType) -> DType:
+    """src/alu.ts:68-83: the later dtype in bool < u32 < i32 < f16 < f32 < f64."""
+    return a if _RANK[a] >= _RANK[b] else b
+
+
+def generalBroadcast(a: Sequence[int], b: Sequence[int]) -> Tuple[int, ...]:
+    out = []
+    for i in range(max(len(a), len(b))):
+        x = a[len(a) - 1 - i] if i < len(a) else 1
+        y = b[len(b) - 1 - i] if i < len(b) else 1
+        if x != y and x != 1 and y != 1:
+            raise ValueError(f"incompatible shapes for broadcasting: {list(a)} and {list(b)}")
+        out.append(max(x, y) if min(x, y) != 0 else 0)
+    return tuple(reversed(out))
+
+
+@dataclass(frozen=True)
+class ShapedArray:
+    shape: Tuple[int, ...]
+    dtype: DType
+    weak: bool = False
+
+    @property
+    def ndim(self):
+        return len(self.shape)
+
+    @property
+    def size(self):
+        return prod(self.shape)
+
+
+def promoteAvals(a: ShapedArray, b: ShapedArray) -> ShapedArray:
+    """src/frontend/core.ts:721-736: a weak (Python-scalar) operand takes the strong one's dtype."""
+    shape = generalBroadcast(a.shape, b.shape)
+    if a.weak == b.weak:
+        dtype = promoteTypes(a.dtype, b.dtype)
+    elif a.weak:
+        dtype = promoteTypes(b.dtype, DType.Uint32)
+    else:
+        dtype = promoteTypes(a.dtype, DType.Uint32)
+    return ShapedArray(shape, dtype, a.weak and b.weak)
+
+
+class Var:
+    _next = 0
+
+    def __init__(self, aval: ShapedArray):
+        self.aval = aval
+        Var._next += 1
+        self.id = Var._next
+
+    def __repr__(self):
+        return f"v{self.id}:{self.aval.dtype.value}{list(self.aval.shape)}"
+
+
+class Lit:
+    def __init__(self, value, aval: ShapedArray):
+        self.value = value
+        self.aval = aval
+
+    @property
+    def dtype(self):
+        return self.aval.dtype
+
+    def __repr__(self):
+        return f"{self.value}:{self.aval.dtype.value}"
+
+
+Atom = Union[Var, Lit]
+
+
+def _is_lit(a: Atom, value=None) -> bool:
+    return isinstance(a, Lit) and (value is None or a.value == value)
+
+
+@dataclass
+class JaxprEqn:
+    primitive: str
+    inputs: List[Atom]
+    params: Dict[str, Any]
+    outBinders: List[Var]
+
+
+VIEW_PRIMITIVES = ("Transpose", "Broadcast", "Reshape", "Flip", "Shrink", "Pad")
+REDUCE_PRIMITIVES = ("Reduce", "Dot")
+UNARY_FUSABLE = ("Neg", "Reciprocal", "Floor", "Ceil", "StopGradient", "Cast", "Bitcast", "Sin", "Cos", "Asin", "Atan",
+                 "Exp", "Log", "Erf", "Erfc", "Sqrt")
+BINARY_FUSABLE = ("Add", "Mul", "Idiv", "Mod", "Min", "Max", "BitCombine", "BitShift")
+
+
+@dataclass
+class Jaxpr:
+    inBinders: List[Var]
+    eqns: List[JaxprEqn]
+    outs: List[Atom]
+
+    def simplify(self) -> "Jaxpr":
+        """Fold +0 / *1 / literal arithmetic and drop no-op movement ops and dead equations
+        (src/frontend/jaxpr.ts:259-360)."""
+        ctx: Dict[Var, Atom] = {}
+        new: List[JaxprEqn] = []
+        for e in self.eqns:
+            inputs = [ctx.get(x, x) if isinstance(x, Var) else x for x in e.inputs]
+            eqn = JaxprEqn(e.primitive, inputs, e.params, e.outBinders)
+            c = eqn.outBinders[0]
+            p = eqn.primitive
+            if p == "Add":
+                a, b = inputs
+                if _is_lit(a, 0):
+                    ctx[c] = b
+                elif _is_lit(b, 0):
+                    ctx[c] = a
+                elif _is_lit(a) and _is_lit(b):
+                    v = min(a.value + b.value, 1) if a.dtype == DType.Bool else a.value + b.value
+                    ctx[c] = Lit(v, promoteAvals(a.aval, b.aval))
+                else:
+                    new.append(eqn)
+            elif p == "Neg":
+                (a,) = inputs
+                if _is_lit(a):
+                    ctx[c] = Lit(-a.value, a.aval)
+                else:
+                    new.append(eqn)
+            elif p == "Mul":
+                a, b = inputs
+                if _is_lit(a, 1):
+                    ctx[c] = b
+                elif _is_lit(b, 1):
+                    ctx[c] = a
+                elif _is_lit(a) and _is_lit(b):
+                    ctx[c] = Lit(a.value * b.value, promoteAvals(a.aval, b.aval))
+                else:
+                    new.append(eqn)
+            elif p == "Idiv":
+                a, b = inputs
+                if _is_lit(b, 1) and not isFloatDtype(a.aval.dtype):
+                    ctx[c] = a
+                else:
+                    new.append(eqn)
+            elif ((p in ("Broadcast", "Reshape") and tuple(eqn.params["shape"]) == tuple(inputs[0].aval.shape))
+                  or (p == "Transpose" and all(q == i for i, q in enumerate(eqn.params["perm"])))
+                  or (p == "Flip" and len(eqn.params["axis"]) == 0)
+                  or (p == "Shrink" and all(s == 0 and e_ == inputs[0].aval.shape[i]
+                                            for i, (s, e_) in enumerate(eqn.params["slice"])))
+                  or (p == "Pad" and all(w0 == 0 and w1 == 0 for w0, w1 in eqn.params["width"]))):
+                ctx[c] = inputs[0]
+            else:
+                new.append(eqn)
+        outs = [ctx.get(x, x) if isinstance(x, Var) else x for x in self.outs]
+        used: Set[Var] = {x for x in outs if isinstance(x, Var)}
+        live: List[JaxprEqn] = []
+        for eqn in reversed(new):
+            if any(v in used for v in eqn.outBinders):
+                live.append(eqn)
+                used.update(v for v in eqn.inputs if isinstance(v, Var))
+        return Jaxpr(self.inBinders, list(reversed(live)), outs)
+
+    def __str__(self):
+        lines = ["{ lambda " + ", ".join(map(repr, self.inBinders)) + " ."]
+        for e in self.eqns:
+            ps = " ".join(f"{k}={v}" for k, v in e.params.items())
+            lines.append(f"  {', '.join(map(repr, e.outBinders))} = {e.primitive}[{ps}] " + " ".join(map(repr, e.inputs)))
+        lines.append("  in " + ", ".join(map(repr, self.outs)) + " }")
+        return "\n".join(lines)
+
+
+# ---- tracing ---------------------------------------------------------------------------------------
+
+class _Builder:
+    def __init__(self):
+        self.eqns: List[JaxprEqn] = []
+        self.consts: List[Tuple[Var, "ConstArray"]] = []
+        self._const_vars: Dict[int, Var] = {}
+
+    def const_var(self, c: "ConstArray") -> Var:
+        v = self._const_vars.get(id(c))
+        if v is None:
+            v = Var(ShapedArray(tuple(c.shape), c.dtype, False))
+            self._const_vars[id(c)] = v
+            self.consts.append((v, c))
+        return v
+
+
+_builders: List[_Builder] = []
+
+
+@dataclass
+class ConstArray:
+    """An array that exists before the traced function runs (the reference realises such closed-over
+    arrays and passes them as leading jit inputs, src/frontend/jaxpr.ts:1166-1169).  `exp` is its lazy
+    definition over `AluVar.idx`-free `gidx` (as arange/tri build them, src/frontend/array.ts:1570-1627);
+    `kernel()` is the nullary Kernel that realises it."""
+    shape: Tuple[int, ...]
+    dtype: DType
+    exp: AluExp
+
+    def kernel(self) -> Kernel:
+        return Kernel(0, prod(self.shape), self.exp)
+
+
+TracerValue = Union["Tracer", int, float, bool, ConstArray]
+
+
+class Tracer:
+    def __init__(self, atom: Atom):
+        self.atom = atom
+
+    @property
+    def aval(self) -> ShapedArray:
+        return self.atom.aval
+
+    @property
+    def shape(self):
+        return self.aval.shape
+
+    @property
+    def dtype(self):
+        return self.aval.dtype
+
+    @property
+    def ndim(self):
+        return len(self.shape)
+
+    # -- primitives as methods (src/frontend/core.ts:800-960) --
+    def add(self, o):
+        return add(self, o)
+
+    def mul(self, o):
+        return mul(self, o)
+
+    def sub(self, o):
+        return add(self, neg(o))  # core.ts:945-947
+
+    def div(self, o):
+        return mul(self, reciprocal(o)) if isFloatDtype(self.dtype) else bind1("Idiv", [self, o])  # :950-955
+
+    def astype(self, dtype: DType):
+        return self if self.dtype == dtype else bind1("Cast", [self], dict(dtype=dtype))
+
+    def reshape(self, shape):
+        return reshape(self, shape)
+
+    def transpose(self, perm=None):
+        return transpose(self, perm)
+
+    def sum(self, axis=None, keepdims=False):
+        return reduce(self, AluOp.Add, axis, keepdims)
+
+    def max(self, axis=None, keepdims=False):
+        return reduce(self, AluOp.Max, axis, keepdims)
+
+    def min(self, axis=None, keepdims=False):
+        return reduce(self, AluOp.Min, axis, keepdims)
+
+    def mean(self, axis=None, keepdims=False):
+        """f32 sum times 1/n, cast back for float inputs (core.ts:878-893)."""
+        ax = _normalize_axis(axis, self.ndim)
+        n = prod([self.shape[a] for a in ax])
+        if n == 0:
+            raise ValueError("mean: cannot compute mean over zero-length axis")
+        orig = self.dtype
+        out = reduce(self.astype(promoteTypes(orig, DType.Float32)), AluOp.Add, ax, keepdims).mul(1 / n)
+        return out.astype(orig) if isFloatDtype(orig) else out
+
+
+def _raise(x: TracerValue) -> Tracer:
+    if isinstance(x, Tracer):
+        return x
+    if isinstance(x, ConstArray):
+        return Tracer(_builders[-1].const_var(x))
+    if isinstance(x, bool):
+        return Tracer(Lit(int(x), ShapedArray((), DType.Bool, False)))  # core.ts:1291-1296
+    if isinstance(x, (int, float)):
+        return Tracer(Lit(float(x), ShapedArray((), DType.Float32, True)))
+    raise TypeError(f"Unknown value: {x!r}")
+
+
+def scalar(value, dtype: DType) -> Tracer:
+    """A strongly typed scalar literal (`array(5, {dtype})`, inlined by jaxpr.ts `_inlineLiterals`)."""
+    return Tracer(Lit(value, ShapedArray((), dtype, False)))
+
+
+def _normalize_axis(axis, ndim) -> List[int]:
+    if axis is None:
+        return list(range(ndim))
+    if isinstance(axis, int):
+        axis = [axis]
+    return sorted({a + ndim if a < 0 else a for a in axis})
+
+
+def _out_aval(prim: str, avals: List[ShapedArray], params: Dict[str, Any]) -> ShapedArray:
+    if prim in BINARY_FUSABLE:
+        return promoteAvals(avals[0], avals[1])
+    if prim == "Compare":
+        return ShapedArray(generalBroadcast(avals[0].shape, avals[1].shape), DType.Bool, False)
+    if prim == "Where":
+        xy = promoteAvals(avals[1], avals[2])
+        return ShapedArray(generalBroadcast(avals[0].shape, xy.shape), xy.dtype, xy.weak)
+    if prim in ("Cast", "Bitcast"):
+        return ShapedArray(avals[0].shape, params["dtype"], False)
+    if prim in UNARY_FUSABLE:
+        return avals[0]
+    if prim == "Reduce":
+        ax = params["axis"]
+        return ShapedArray(tuple(d for i, d in enumerate(avals[0].shape) if i not in ax), avals[0].dtype, avals[0].weak)
+    if prim == "Dot":
+        c = promoteAvals(avals[0], avals[1])
+        return ShapedArray(c.shape[:-1], c.dtype, c.weak)
+    if prim == "Transpose":
+        return ShapedArray(tuple(avals[0].shape[p] for p in params["perm"]), avals[0].dtype, avals[0].weak)
+    if prim in ("Reshape", "Broadcast"):
+        return ShapedArray(tuple(params["shape"]), avals[0].dtype, avals[0].weak)
+    if prim == "Flip":
+        return avals[0]
+    if prim == "Shrink":
+        return ShapedArray(tuple(e - s for s, e in params["slice"]), avals[0].dtype, avals[0].weak)
+    if prim == "Pad":
+        return ShapedArray(tuple(d + a + b for d, (a, b) in zip(avals[0].shape, params["width"])), avals[0].dtype, avals[0].weak)
+    raise NotImplementedError(f"jit: primitive {prim}")
+
+
+def bind1(prim: str, args: Sequence[TracerValue], params: Optional[Dict[str, Any]] = None) -> Tracer:
+    if not _builders:
+        raise RuntimeError("bind1 outside of a trace")
+    ts = [_raise(a) for a in args]
+    params = dict(params or {})
+    out = Var(_out_aval(prim, [t.aval for t in ts], params))
+    _builders[-1].eqns.append(JaxprEqn(prim, [t.atom for t in ts], params, [out]))
+    return Tracer(out)
+
+
+def add(x, y): return bind1("Add", [x, y])
+def mul(x, y): return bind1("Mul", [x, y])
+def neg(x): return bind1("Neg", [x])
+def reciprocal(x): return bind1("Reciprocal", [x])
+def exp(x): return bind1("Exp", [x])
+def log(x): return bind1("Log", [x])
+def sqrt(x): return bind1("Sqrt", [x])
+def erfc(x): return bind1("Erfc", [x])
+def stopGradient(x): return bind1("StopGradient", [x])
+def maximum(x, y): return bind1("Max", [x, y])
+def minimum(x, y): return bind1("Min", [x, y])
+def where(c, x, y): return bind1("Where", [c, x, y])
+def less(x, y): return bind1("Compare", [x, y], dict(op="Less"))
+def greater(x, y): return bind1("Compare", [y, x], dict(op="Less"))
+def equal(x, y): return bind1("Compare", [x, y], dict(op="Equal"))
+def notEqual(x, y): return bind1("Compare", [x, y], dict(op="NotEqual"))
+def lessEqual(x, y): return bind1("Compare", [x, y], dict(op="LessEqual"))
+def greaterEqual(x, y): return bind1("Compare", [y, x], dict(op="LessEqual"))  # core.ts:329-331
+
+
+def dot(x, y):
+    return bind1("Dot", [x, y])
+
+
+def transpose(x, perm=None):
+    x = _raise(x)
+    perm = list(reversed(range(x.ndim))) if perm is None else [p + x.ndim if p < 0 else p for p in perm]
+    return bind1("Transpose", [x], dict(perm=perm))
+
+
+def reshape(x, shape):
+    x = _raise(x)
+    shape = [shape] if isinstance(shape, int) else list(shape)
+    if -1 in shape:
+        known = prod([d for d in shape if d != -1])
+        shape[shape.index(-1)] = x.aval.size // max(known, 1)
+    if prod(shape) != x.aval.size:
+        raise ValueError(f"reshape: cannot reshape {list(x.shape)} into {shape}")
+    return bind1("Reshape", [x], dict(shape=tuple(shape)))
+
+
+def broadcast(x, shape, axis):
+    return bind1("Broadcast", [x], dict(shape=tuple(shape), axis=list(axis)))
+
+
+def shrink(x, slices):
+    """`x.slice(...)`: keep `[start, end)` per axis."""
+    return bind1("Shrink", [x], dict(slice=[tuple(s) for s in slices]))
+
+
+def reduce(x, op: AluOp, axis=None, keepdims=False):
+    """src/frontend/core.ts:271-289."""
+    x = _raise(x)
+    ax = _normalize_axis(axis, x.ndim)
+    original = x.shape
+    out = bind1("Reduce", [x], dict(op=op, axis=ax))
+    if keepdims:
+        out = out.reshape([1 if i in ax else d for i, d in enumerate(original)])
+    return out
+
+
+def trace(fn: Callable[..., Any], avals: Sequence[ShapedArray]) -> Tuple[Jaxpr, List[ConstArray]]:
+    """Run `fn` on tracers and return the simplified Jaxpr; closed-over ConstArrays come first in
+    `inBinders` (src/frontend/jaxpr.ts:707-720)."""
+    b = _Builder()
+    _builders.append(b)
+    try:
+        ins = [Var(a) for a in avals]
+        outs = fn(*[Tracer(v) for v in ins])
+        if isinstance(outs, Tracer):
+            outs = [outs]
+        out_atoms = [_raise(o).atom for o in outs]
+    finally:
+        _builders.pop()
+    jaxpr = Jaxpr([v for v, _ in b.consts] + ins, b.eqns, out_atoms).simplify()
+    return jaxpr, [c for _, c in b.consts]
+
+
+# ---- jit rules: one expression per primitive (src/frontend/jit.ts:486-770) -----------------------
+
+def reshapeViews(exp: AluExp, mapping: Callable[[ShapeTracker], Optional[ShapeTracker]], reduceAxis: bool = False) -> AluExp:
+    def visit(e: AluExp):
+        if e.op == AluOp.GlobalView:
+            gid, st = e.arg
+            new = mapping(st)
+            if new is not None:
+                if reduceAxis:
+                    indices = unravelAlu(new.shape[:-1], AluVar.gidx) + [AluVar.ridx]
+                else:
+                    indices = unravelAlu(new.shape, AluVar.gidx)
+                return AluExp.globalView(e.dtype, gid, new, indices)
+        elif e.op == AluOp.GlobalIndex:
+            raise RuntimeError("internal: reshapeViews() called with GlobalIndex op")
+        return None
+    return exp.rewrite(visit)
+
+
+def aluCompare(a: AluExp, b: AluExp, op: str) -> AluExp:
+    """src/frontend/array.ts:1786-1800."""
+    if op == "Less":
+        return AluExp.cmplt(a, b)
+    if op == "Equal":
+        return AluExp.cmpne(a, b).not_()
+    if op == "NotEqual":
+        return AluExp.cmpne(a, b)
+    if op == "LessEqual":
+        return AluExp.add(AluExp.cmplt(a, b), AluExp.cmpne(a, b).not_())
+    raise ValueError(op)
+
+
+def _broadcasted(fn, skipCastIdx=()):
+    def rule(exps, avals, params):
+        new = avals[0]
+        for a in avals[1:]:
+            new = promoteAvals(new, a)
+        newShape, newDtype = new.shape, new.dtype
+        if skipCastIdx:
+            rest = [a for i, a in enumerate(avals) if i not in skipCastIdx]
+            d = rest[0]
+            for a in rest[1:]:
+                d = promoteAvals(d, a)
+            newDtype = d.dtype
+        out = []
+        for i, e in enumerate(exps):
+            def mapping(st, _shape=newShape):
+                if tuple(st.shape) != tuple(_shape):
+                    return st.broadcast(list(_shape), list(range(len(_shape) - len(st.shape))))
+                return None
+            e = reshapeViews(e, mapping)
+            if e.dtype != newDtype and i not in skipCastIdx:
+                e = AluExp.cast(newDtype, e)
+            out.append(e)
+        return [fn(out, params)], None
+    return rule
+
+
+def _unop(fn):
+    return lambda exps, avals, params: ([fn(exps[0], params)], None)
+
+
+def _reshape_rule(fn):
+    return lambda exps, avals, params: ([reshapeViews(exps[0], lambda st: fn(st, params))], None)
+
+
+def _reduce_rule(exps, avals, params):
+    a, aval = exps[0], avals[0]
+    axis = params["axis"]
+    kept = [i for i in range(aval.ndim) if i not in axis]
+    shifted = [i for i in range(aval.ndim) if i in axis]
+    newShape = [aval.shape[i] for i in kept]
+    rsize = prod([aval.shape[i] for i in shifted])
+    newShape.append(rsize)
+    perm = kept + shifted
+    a = reshapeViews(a, lambda st: st.permute(perm).reshape(newShape), True)
+    return [a], Reduction(a.dtype, params["op"], rsize)
+
+
+def _dot_rule(exps, avals, params):
+    (c,), _ = JIT_RULES["Mul"](exps, avals, {})
+    cs = promoteAvals(avals[0], avals[1])
+    return _reduce_rule([c], [cs], dict(op=AluOp.Add, axis=[cs.ndim - 1]))
+
+
+def _flip_rule(st, params):
+    arg = [False] * len(st.shape)
+    for ax in params["axis"]:
+        arg[ax] = True
+    return st.flip(arg)
+
+
+JIT_RULES: Dict[str, Callable] = {
+    "Add": _broadcasted(lambda e, p: AluExp.add(e[0], e[1])),
+    "Mul": _broadcasted(lambda e, p: AluExp.mul(e[0], e[1])),
+    "Idiv": _broadcasted(lambda e, p: AluExp.idiv(e[0], e[1])),
+    "Mod": _broadcasted(lambda e, p: AluExp.mod(e[0], e[1])),
+    "Min": _broadcasted(lambda e, p: AluExp.min(e[0], e[1])),
+    "Max": _broadcasted(lambda e, p: AluExp.max(e[0], e[1])),
+    "Neg": _unop(lambda a, p: AluExp.sub(AluExp.const(a.dtype, 0), a)),
+    "Reciprocal": _unop(lambda a, p: AluExp.reciprocal(a)),
+    "Floor": _unop(lambda a, p: AluExp.floor(a)),
+    "Ceil": _unop(lambda a, p: AluExp.ceil(a)),
+    "StopGradient": _unop(lambda a, p: a),
+    "Cast": _unop(lambda a, p: AluExp.cast(p["dtype"], a)),
+    "Bitcast": _unop(lambda a, p: AluExp.bitcast(p["dtype"], a)),
+    "Sin": _unop(lambda a, p: AluExp.sin(a)),
+    "Cos": _unop(lambda a, p: AluExp.cos(a)),
+    "Asin": _unop(lambda a, p: AluExp.asin(a)),
+    "Atan": _unop(lambda a, p: AluExp.atan(a)),
+    "Exp": _unop(lambda a, p: AluExp.exp(a)),
+    "Log": _unop(lambda a, p: AluExp.log(a)),
+    "Erf": _unop(lambda a, p: AluExp.erf(a)),
+    "Erfc": _unop(lambda a, p: AluExp.erfc(a)),
+    "Sqrt": _unop(lambda a, p: AluExp.sqrt(a)),
+    "Reduce": _reduce_rule,
+    "Dot": _dot_rule,
+    "Compare": _broadcasted(lambda e, p: aluCompare(e[0], e[1], p["op"])),
+    "Where": _broadcasted(lambda e, p: AluExp.where(e[0], e[1], e[2]), skipCastIdx=(0,)),
+    "Transpose": _reshape_rule(lambda st, p: st.permute(p["perm"])),
+    "Broadcast": _reshape_rule(lambda st, p: st.broadcast(list(p["shape"]), list(p["axis"]))),
+    "Reshape": _reshape_rule(lambda st, p: st.reshape(list(p["shape"]))),
+    "Flip": _reshape_rule(_flip_rule),
+    "Shrink": _reshape_rule(lambda st, p: st.shrink([tuple(s) for s in p["slice"]])),
+    "Pad": _reshape_rule(lambda st, p: st.pad([tuple(w) for w in p["width"]])),
+}
+
+
+# ---- kernel boundaries (src/frontend/jit.ts:792-1096) ----------------------------------------------
+
+def splitGraphDataflow(jaxpr: Jaxpr, maxArgs: int) -> Set[Var]:
+    varToDefn: Dict[Var, int] = {}
+    varToUsages: Dict[Var, List[int]] = {}
+    for i, eqn in enumerate(jaxpr.eqns):
+        for v in eqn.outBinders:
+            varToDefn[v] = i
+        for x in eqn.inputs:
+            if isinstance(x, Var):
+                varToUsages.setdefault(x, []).append(i)
+
+    # Reduction epilogues: unary ops, and binary ops against a literal or an array that does not
+    # broadcast the reduction's output.
+    epilogueEqns: Set[int] = set()
+    endpointEqns: Set[int] = set()
+    for i, eqn in enumerate(jaxpr.eqns):
+        if eqn.primitive not in REDUCE_PRIMITIVES:
+            continue
+        head = i
+        while True:
+            epilogueEqns.add(head)
+            outVar = jaxpr.eqns[head].outBinders[0]
+            usages = varToUsages.get(outVar, [])
+            if outVar in jaxpr.outs or len(usages) != 1:
+                break
+            if usages[0] in epilogueEqns:
+                break
+            nxt = jaxpr.eqns[usages[0]]
+            if nxt.primitive in UNARY_FUSABLE:
+                head = usages[0]
+                continue
+            if nxt.primitive in BINARY_FUSABLE:
+                other = next(v for v in nxt.inputs if v is not outVar)
+                if isinstance(other, Lit) or generalBroadcast(other.aval.shape, outVar.aval.shape) == tuple(outVar.aval.shape):
+                    head = usages[0]
+                    continue
+            break
+        endpointEqns.add(head)
+
+    # A computed value that a Dot would broadcast (and so recompute per output) is materialised first.
+    materialized: Set[Var] = set()
+
+    def hasReuse(shape, promoted) -> bool:
+        offset = len(promoted) - len(shape)
+        for axis in range(len(promoted) - 1):
+            dim = 1 if axis < offset else shape[axis - offset]
+            if dim == 1 and promoted[axis] > 1:
+                return True
+        return False
+
+    def markNonViewProducer(v: Var) -> None:
+        cur = v
+        while True:
+            d = varToDefn.get(cur)
+            if d is None:
+                return
+            eqn = jaxpr.eqns[d]
+            if eqn.primitive not in VIEW_PRIMITIVES:
+                break
+            inp = next((x for x in eqn.inputs if isinstance(x, Var)), None)
+            if inp is None:
+                return
+            cur = inp
+        materialized.add(cur)
+
+    for eqn in jaxpr.eqns:
+        if eqn.primitive != "Dot":
+            continue
+        shapes = [eqn.inputs[0].aval.shape, eqn.inputs[1].aval.shape]
+        promoted = generalBroadcast(shapes[0], shapes[1])
+        for i, x in enumerate(eqn.inputs):
+            if isinstance(x, Var) and hasReuse(shapes[i], promoted):
+                markNonViewProducer(x)
+    for eqn in jaxpr.eqns:
+        if eqn.primitive == "Pad":  # Pad needs clean inputs
+            for x in eqn.inputs:
+                if isinstance(x, Var):
+                    markNonViewProducer(x)
+
+    # Backwards: a node is black when it is an output, a reduction endpoint, materialised, or when two
+    # different black nodes are reachable from it through non-black nodes.
+    black: Set[Var] = set()
+    nextBlack: Dict[Var, Var] = {}
+    for v in jaxpr.outs:
+        if isinstance(v, Var):
+            black.add(v)
+            nextBlack[v] = v
+    for i in range(len(jaxpr.eqns) - 1, -1, -1):
+        eqn = jaxpr.eqns[i]
+        if (i in endpointEqns or any(v in materialized for v in eqn.outBinders)
+                or any(v in black for v in eqn.outBinders)):
+            for v in eqn.outBinders:
+                black.add(v)
+                nextBlack[v] = v
+            continue
+        reach: List[Var] = []
+        for v in eqn.outBinders:
+            for j in varToUsages.get(v, []):
+                for o in jaxpr.eqns[j].outBinders:
+                    u = nextBlack.get(o)
+                    if u is not None and u not in reach:
+                        reach.append(u)
+        if len(reach) > 1:
+            for v in eqn.outBinders:
+                black.add(v)
+                nextBlack[v] = v
+        elif len(reach) == 1:
+            for v in eqn.outBinders:
+                nextBlack[v] = reach[0]
+
+    # Forwards: split further wherever a fused expression would read more than maxArgs buffers.
+    deps: Dict[Var, Set[Var]] = {v: {v} for v in jaxpr.inBinders}
+    idx = 0
+    while idx < len(jaxpr.eqns):
+        eqn = jaxpr.eqns[idx]
+        idx += 1
+        per_input: List[Set[Var]] = []
+        for x in eqn.inputs:
+            if isinstance(x, Var):
+                per_input.append({x} if x in black else deps[x])
+            else:
+                per_input.append(set())
+        counter: Dict[Var, int] = {}
+        for s in per_input:
+            for d in s:
+                counter[d] = counter.get(d, 0) + 1
+        if len(counter) > maxArgs:
+            best, which = 0, -1
+            for i, x in enumerate(eqn.inputs):
+                if isinstance(x, Var) and x in varToDefn:
+                    unique = sum(1 for d in per_input[i] if counter[d] == 1)
+                    if unique > best:
+                        best, which = unique, i
+            if which == -1:
+                raise RuntimeError(f"internal: maxArgs, no input found to mark as black in {eqn.primitive}")
+            idx = varToDefn[eqn.inputs[which]]
+            for out in jaxpr.eqns[idx].outBinders:
+                black.add(out)
+            idx += 1
+        else:
+            s = set(counter.keys())
+            for out in eqn.outBinders:
+                deps[out] = s
+    return black
+
+
+# ---- jitCompile / JitProgram (src/frontend/jit.ts:111-162, 263-469) ----------------------------------
+
+@dataclass
+class JitStep:
+    kind: str                      # "malloc" | "execute" | "free"
+    kernel: Optional[Kernel] = None
+    inputs: List[int] = field(default_factory=list)
+    output: int = -1
+    size: int = 0
+
+
+@dataclass
+class JitProgram:
+    steps: List[JitStep]
+    nargs: int
+    outputs: List[int]
+    consts: List[ConstArray]
+
+    @property
+    def kernels(self) -> List[Kernel]:
+        return [s.kernel for s in self.steps if s.kind == "execute"]
+
+    def execute(self, backend, inputs: Sequence[int], prepared: Optional[Dict[int, Any]] = None) -> List[int]:
+        """Run on `backend` with input slots (closed-over constants first).  Returns output slots owned
+        by the caller; inputs stay owned by the caller."""
+        if len(inputs) != self.nargs:
+            raise ValueError(f"jit program takes {self.nargs} inputs, got {len(inputs)}")
+        scope: Dict[int, int] = {i: s for i, s in enumerate(inputs)}
+        for k, step in enumerate(self.steps):
+            if step.kind == "malloc":
+                scope[step.output] = backend.malloc(step.size)
+            elif step.kind == "execute":
+                exe = prepared[k] if prepared is not None else backend.prepareKernelSync(step.kernel)
+                backend.dispatch(exe, [scope[i] for i in step.inputs], [scope[step.output]])
+            elif step.kind == "free":
+                backend.decRef(scope.pop(step.output))
+        outs = []
+        for o in self.outputs:
+            if o < self.nargs:
+                backend.incRef(scope[o])
+            outs.append(scope[o])
+        return outs
+
+    def prepare(self, backend) -> Dict[int, Any]:
+        return {k: backend.prepareKernelSync(s.kernel) for k, s in enumerate(self.steps) if s.kind == "execute"}
+
+
+def jitCompile(jaxpr: Jaxpr, consts: Sequence[ConstArray] = (), maxArgs: int = 64) -> JitProgram:
+    nargs = len(jaxpr.inBinders)
+    black = splitGraphDataflow(jaxpr, maxArgs)
+    steps: List[JitStep] = []
+    next_id = [nargs]
+
+    # ctx values: ("imm", id) | ("exp", exp, args) | ("red", exp, reduction, args)
+    ctx: Dict[Var, tuple] = {v: ("imm", i) for i, v in enumerate(jaxpr.inBinders)}
+    for eqn in jaxpr.eqns:
+        rule = JIT_RULES.get(eqn.primitive)
+        if rule is None:
+            raise NotImplementedError(f"JIT not implemented for primitive {eqn.primitive}")
+        inputExps: List[AluExp] = []
+        inputAvals: List[ShapedArray] = []
+        inputArgs: List[int] = []
+        inputReduction = None
+
+        def addArgs(args):
+            out = []
+            for a in args:
+                if a not in inputArgs:
+                    inputArgs.append(a)
+                out.append(inputArgs.index(a))
+            return out
+
+        for x in eqn.inputs:
+            if isinstance(x, Var):
+                jv = ctx[x]
+                if jv[0] == "exp":
+                    inputExps.append(jv[1].reindexGids(addArgs(jv[2])))
+                elif jv[0] == "imm":
+                    (gid,) = addArgs([jv[1]])
+                    st = ShapeTracker.fromShape(list(x.aval.shape))
+                    inputExps.append(AluExp.globalView(x.aval.dtype, gid, st, unravelAlu(st.shape, AluVar.gidx)))
+                else:
+                    if inputReduction is not None:
+                        raise RuntimeError("jit: unexpected, multiple red inputs")
+                    inputExps.append(jv[2].epilogue.reindexGids(addArgs(jv[3])))
+                    inputReduction = jv
+            else:
+                inputExps.append(AluExp.const(x.dtype, x.value))
+            inputAvals.append(x.aval)
+
+        if inputReduction is not None:
+            (newEpilogue,), _ = rule(inputExps, inputAvals, eqn.params)
+            jv = inputReduction
+            exps = [jv[1].reindexGids(addArgs(jv[3]))]
+            red = jv[2]
+            reduction = Reduction(red.dtype, red.op, red.size, newEpilogue)
+        else:
+            exps, reduction = rule(inputExps, inputAvals, eqn.params)
+
+        for i, outVar in enumerate(eqn.outBinders):
+            if outVar in black:
+                kernel = Kernel(len(inputArgs), outVar.aval.size, exps[i], reduction)
+                out_id = next_id[0]
+                next_id[0] += 1
+                steps.append(JitStep("malloc", output=out_id, size=kernel.bytes))
+                steps.append(JitStep("execute", kernel=kernel, inputs=list(inputArgs), output=out_id))
+                ctx[outVar] = ("imm", out_id)
+            elif reduction is not None:
+                ctx[outVar] = ("red", exps[i], reduction, list(inputArgs))
+            else:
+                ctx[outVar] = ("exp", exps[i], list(inputArgs))
+
+    outputs: List[int] = []
+    for out in jaxpr.outs:
+        if not isinstance(out, Var):
+            raise NotImplementedError("jit: literal outputs")
+        jv = ctx[out]
+        if jv[0] != "imm":
+            raise RuntimeError("internal: Expected imm, since outs are black nodes")
+        outputs.append(jv[1])
+
+    # Free every intermediate after its last use (JitProgramBuilder.insertFreeSteps).
+    last_use: Dict[int, int] = {}
+    for k, s in enumerate(steps):
+        if s.kind == "execute":
+            for i in s.inputs:
+                last_use[i] = k
+            last_use.setdefault(s.output, k)
+    final: List[JitStep] = []
+    for k, s in enumerate(steps):
+        final.append(s)
+        if s.kind == "execute":
+            for i in dict.fromkeys(s.inputs + [s.output]):
+                if i >= nargs and i not in outputs and last_use.get(i) == k:
+                    final.append(JitStep("free", output=i))
+    return JitProgram(final, nargs, outputs, list(consts))
+
+
+def jit(fn: Callable[..., Any], avals: Sequence[ShapedArray], maxArgs: int = 64) -> JitProgram:
+    """Trace `fn` at the given input avals and compile it to a Kernel program."""
+    jaxpr, consts = trace(fn, avals)
+    return jitCompile(jaxpr, consts, maxArgs)

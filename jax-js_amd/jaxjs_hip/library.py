@@ -1,0 +1,144 @@
+"""Library compositions over the tracing primitives, restating how the reference's numpy/nn/lax
+layers spell the operations the benchmark configurations use -- the spelling decides which Kernels
+the backend is handed, so it is kept literally:
+
+  square, sigmoid, tanh, gelu, softmax, standardize   src/library/numpy.ts:2579-2582, 3054-3060;
+                                                      src/library/nn.ts:65-67, 222-238, 291-301, 386-412
+  lax.dot / matmul / two-operand einsum               src/library/lax.ts:40-129; numpy.ts:1729-1747, 1935-1990
+  arange / tri (lazy constants)                       src/frontend/array.ts:1570-1627
+  argmax                                              src/library/numpy.ts:533-556
+  dotProductAttention                                 src/library/nn.ts:478-583
+"""
+
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence, Tuple
+
+from . import jit as J
+from .alu import AluExp, AluOp, AluVar, DType
+from .jit import ConstArray, Tracer
+from .shape import prod, unravelAlu
+
+
+def square(x):
+    return J.mul(x, x)
+
+
+def sigmoid(x):
+    return J.reciprocal(J.exp(J.neg(x)).add(1))
+
+
+def tanh(x):
+    """(e^{-2|x|} - 1) / (e^{-2|x|} + 1) * negsgn, avoiding overflow (numpy.ts:3054-3060)."""
+    negsgn = J.where(J.less(x, 0), 1, -1)
+    en2x = J.exp(x.mul(negsgn).mul(2))
+    return en2x.sub(1).div(en2x.add(1)).mul(negsgn)
+
+
+def gelu(x, approximate: bool = True):
+    if approximate:
+        c = math.sqrt(2 / math.pi)
+        return x.mul(0.5).mul(tanh(x.mul(x.mul(x).mul(0.044715).add(1)).mul(c)).add(1))
+    return x.mul(0.5).mul(J.erfc(J.neg(x.mul(math.sqrt(0.5)))))
+
+
+def softmax(x, axis: int = -1):
+    xMax = x.max(axis, keepdims=True)
+    unnormalized = J.exp(x.sub(J.stopGradient(xMax)))
+    return unnormalized.div(unnormalized.sum(axis, keepdims=True))
+
+
+def standardize(x, axis: int = -1, epsilon: float = 1e-5):
+    """Var[X] = E[X^2] - E[X]^2, like the reference (nn.ts:386-412)."""
+    mu = x.mean(axis, keepdims=True)
+    sigma2 = square(x).mean(axis, keepdims=True).sub(square(mu))
+    return x.sub(mu).div(J.sqrt(sigma2.add(epsilon)))
+
+
+def lax_dot(lhs: Tracer, rhs: Tracer, lc: Sequence[int], rc: Sequence[int], lb: Sequence[int] = (), rb: Sequence[int] = ()):
+    """General contraction: transpose to [batch, free, contract], reshape so the free axes of the two
+    operands interleave as size-1 axes, then one `Dot` (lax.ts:40-129)."""
+    norm = lambda ax, n: [a + n if a < 0 else a for a in ax]
+    lc, lb = norm(lc, lhs.ndim), norm(lb, lhs.ndim)
+    rc, rb = norm(rc, rhs.ndim), norm(rb, rhs.ndim)
+    lf = [a for a in range(lhs.ndim) if a not in lc and a not in lb]
+    rf = [a for a in range(rhs.ndim) if a not in rc and a not in rb]
+    lhs2 = lhs.transpose(lb + lf + lc)
+    rhs2 = rhs.transpose(rb + rf + rc)
+    if not lc:
+        return J.mul(lhs2.reshape([lhs.shape[a] for a in lb] + [lhs.shape[a] for a in lf] + [1] * len(rf)),
+                     rhs2.reshape([rhs.shape[a] for a in rb] + [1] * len(lf) + [rhs.shape[a] for a in rf]))
+    kx, ky = [lhs.shape[a] for a in lc], [rhs.shape[a] for a in rc]
+    if kx != ky:
+        raise ValueError(f"dot: shapes not aligned along contracting dims: {kx} != {ky}")
+    return J.dot(
+        lhs2.reshape([lhs.shape[a] for a in lb] + [lhs.shape[a] for a in lf] + [1] * len(rf) + [prod(kx)]),
+        rhs2.reshape([rhs.shape[a] for a in rb] + [1] * len(lf) + [rhs.shape[a] for a in rf] + [prod(ky)]))
+
+
+def matmul(x: Tracer, y: Tracer):
+    if y.ndim == 1:
+        return J.dot(x, y)
+    nb = min(max(x.ndim, 2), y.ndim) - 2
+    batch = list(range(-2 - nb, -2))
+    return lax_dot(x, y, [-1], [-2], batch, batch)
+
+
+def einsum(subscripts: str, a: Tracer, b: Tracer):
+    """Two-operand einsum without repeated or summed-alone indices: batch = shared kept indices,
+    contraction = shared dropped indices, then a transpose to the requested order
+    (numpy.ts:1935-1990)."""
+    lhs, out = subscripts.replace(" ", "").split("->")
+    ia, ib = lhs.split(",")
+    if len(set(ia)) != len(ia) or len(set(ib)) != len(ib):
+        raise NotImplementedError("einsum: repeated indices")
+    reduced = [c for c in ia if c in ib and c not in out]
+    if any((c not in out) and not (c in ia and c in ib) for c in ia + ib):
+        raise NotImplementedError("einsum: index summed over a single operand")
+    batch = [c for c in ia if c in ib and c not in reduced]
+    res = lax_dot(a, b, [ia.index(c) for c in reduced], [ib.index(c) for c in reduced],
+                  [ia.index(c) for c in batch], [ib.index(c) for c in batch])
+    order = batch + [c for c in ia if c not in ib] + [c for c in ib if c not in ia]
+    return res.transpose([order.index(c) for c in out])
+
+
+def arange_const(start: int, stop: int, step: int = 1, dtype: DType = DType.Int32, shape: Optional[Sequence[int]] = None) -> ConstArray:
+    """`arange(...)` (optionally reshaped): start + cast(idx)*step, realised by a nullary kernel."""
+    size = max(0, -(-(stop - start) // step)) if step > 0 else max(0, -((start - stop) // step))
+    exp = AluExp.add(AluExp.const(dtype, start), AluExp.mul(AluExp.cast(dtype, AluVar.gidx), AluExp.const(dtype, step)))
+    return ConstArray(tuple(shape) if shape is not None else (size,), dtype, exp)
+
+
+def tri_const(n: int, m: Optional[int] = None, k: int = 0) -> ConstArray:
+    """Boolean lower-triangular mask `rows.reshape([n,1]) >= cols` (array.ts:1614-1627)."""
+    m = n if m is None else m
+    r, c = unravelAlu([n, m], AluVar.gidx)
+    rows = AluExp.add(AluExp.i32(k), AluExp.mul(AluExp.cast(DType.Int32, r), AluExp.i32(1)))
+    cols = AluExp.add(AluExp.i32(0), AluExp.mul(AluExp.cast(DType.Int32, c), AluExp.i32(1)))
+    return ConstArray((n, m), DType.Bool, J.aluCompare(cols, rows, "LessEqual"))
+
+
+def argmax(a: Tracer, axis: int):
+    """First index of the maximum: max over isMax * (length - i), then length - that (numpy.ts:533-556)."""
+    axis = axis + a.ndim if axis < 0 else axis
+    n = a.shape[axis]
+    isMax = J.equal(a, a.max(axis, keepdims=True))
+    length = J.scalar(n, DType.Int32)
+    rev = arange_const(n, 0, -1, DType.Int32, shape=[n] + [1] * (a.ndim - axis - 1))
+    idx = isMax.astype(DType.Int32).mul(rev)
+    return length.sub(idx.max(axis))
+
+
+def dotProductAttention(query: Tracer, key: Tracer, value: Tracer, isCausal: bool = False, scale: Optional[float] = None):
+    """[B,L,N,H] attention with equal query and key/value head counts (nn.ts:478-583)."""
+    B, L, N, H = query.shape
+    S = key.shape[1]
+    if key.shape != value.shape or key.shape[0] != B or key.shape[3] != H or key.shape[2] != N:
+        raise ValueError("dotProductAttention: shape mismatch")
+    scale = 1 / math.sqrt(H) if scale is None else scale
+    scores = einsum("BLNH,BSNH->BNLS", query, key).mul(scale)
+    if isCausal:
+        scores = J.where(tri_const(L, S, 0), scores, -math.inf)
+    attn = softmax(scores, -1)
+    return einsum("BNLS,BSNH->BLNH", attn, value)

@@ -202,6 +202,59 @@ def _strip_float_casts(e: AluExp) -> AluExp:
     return e
 
 
+def _flatten_k_split(st) -> Optional[tuple]:
+    """(view, k0, sk1) describing the operand as ONE strided view over the broadcast shape.
+
+    A single-view tracker is returned as is (k0 = sk1 = 0).  Two views are accepted when the outer one
+    is a plain row-major reshape whose last axis K covers exactly the last two axes (K1, K0) of the
+    inner view and whose other axes map one-to-one onto the inner view's leading axes -- what
+    `x.transpose(..).reshape([.., K1*K0])` followed by a Dot produces (attention output [B,N,L,H] read
+    as [B,L,N*H]).  Then element k of the reduce axis lives at (k // K0) * sk1 + (k % K0) * sk0, and
+    the returned view carries sk0 as its last stride."""
+    if len(st.views) == 1:
+        return st.views[0], 0, 0
+    if len(st.views) != 2:
+        return None
+    inner, outer = st.views
+    if inner.mask is not None or outer.mask is not None or outer.offset != 0 or len(inner.shape) < 2:
+        return None
+    # The outer view must address the inner view's logical space row-major (stride-0 axes aside).
+    live = [(i, n) for i, n in enumerate(outer.shape) if n != 1 and outer.strides[i] != 0]
+    if not live or live[-1][0] != len(outer.shape) - 1:
+        return None
+    expect = 1
+    for i, n in reversed(live):
+        if outer.strides[i] != expect:
+            return None
+        expect *= n
+    lead = live[:-1]
+    if len(lead) != len(inner.shape) - 2 or any(n != inner.shape[j] for j, (_, n) in enumerate(lead)):
+        return None
+    K1, K0 = inner.shape[-2], inner.shape[-1]
+    if K1 * K0 != live[-1][1] or expect != math.prod(inner.shape):
+        return None
+    strides = [0] * len(outer.shape)
+    for j, (i, _) in enumerate(lead):
+        strides[i] = inner.strides[j]
+    strides[-1] = inner.strides[-1]
+    from .shape import View
+    flat = View(tuple(outer.shape), tuple(strides), inner.offset, None)
+    return flat, K0, inner.strides[-2]
+
+
+def _span(view, k0: int, sk1: int) -> int:
+    """One past the largest element index the operand can touch."""
+    hi = view.offset
+    dims = list(zip(view.shape, view.strides))
+    if k0:
+        K = view.shape[-1]
+        dims = dims[:-1] + [(k0, view.strides[-1]), (K // k0, sk1)]
+    for n, s in dims:
+        if n > 0 and s > 0:
+            hi += (n - 1) * s
+    return hi + 1
+
+
 def match_gemm(kernel: Kernel) -> Optional[dict]:
     """Recognise `sum_k A[..m..,k] * B[..n..,k]` over single-view, unmasked operands.
 
@@ -221,10 +274,10 @@ def match_gemm(kernel: Kernel) -> Optional[dict]:
         return None
     if a.dtype not in (DType.Float16, DType.Float32):
         return None
-    sta, stb = a.arg[1], b.arg[1]
-    if len(sta.views) != 1 or len(stb.views) != 1:
+    fa, fb = _flatten_k_split(a.arg[1]), _flatten_k_split(b.arg[1])
+    if fa is None or fb is None:
         return None
-    va, vb = sta.views[0], stb.views[0]
+    (va, ka0, ka1), (vb, kb0, kb1) = fa, fb
     if va.mask is not None or vb.mask is not None or va.shape != vb.shape or len(va.shape) < 1:
         return None
     shape = list(va.shape)
@@ -258,6 +311,12 @@ def match_gemm(kernel: Kernel) -> Optional[dict]:
                 merged[-1] = [p[0], p[1] * ax[1], ax[2], ax[3], ax[4]]
                 continue
         merged.append(ax)
+    # Several M (or N) axes that do not nest (rows of a transposed activation): keep the innermost as
+    # the tile axis and walk the outer ones like batch axes (the other operand's stride there is 0).
+    for role in ("m", "n"):
+        idx = [i for i, x in enumerate(merged) if x[0] == role]
+        for i in idx[:-1]:
+            merged[i][0] = "batch"
     ms = [x for x in merged if x[0] == "m"]
     ns = [x for x in merged if x[0] == "n"]
     bs = [x for x in merged if x[0] == "batch"]
@@ -268,11 +327,11 @@ def match_gemm(kernel: Kernel) -> Optional[dict]:
     info = dict(
         dtype=a.dtype, gid_a=a.arg[0], gid_b=b.arg[0],
         M=m[1], N=n[1], K=shape[-1],
-        a_off=va.offset, a_sm=m[2], a_sk=ska,
-        b_off=vb.offset, b_sn=n[3], b_sk=skb,
+        a_off=va.offset, a_sm=m[2], a_sk=ska, a_k0=ka0 or shape[-1], a_sk1=ka1,
+        b_off=vb.offset, b_sn=n[3], b_sk=skb, b_k0=kb0 or shape[-1], b_sk1=kb1,
         c_sm=m[4], c_sn=n[4],
         batch=[(x[1], x[2], x[3], x[4]) for x in bs],
-        a_len=va.dataRange()[1], b_len=vb.dataRange()[1],
+        a_len=_span(va, ka0, ka1), b_len=_span(vb, kb0, kb1),
     )
     # Negative strides (flipped views) are left to the generic path.
     if min(info["a_sm"], info["a_sk"], info["b_sn"], info["b_sk"], info["a_off"], info["b_off"]) < 0:
@@ -402,5 +461,10 @@ def _gemm_worthwhile(g: dict) -> bool:
             return rows % vec == 0 and sk % vec == 0 and off % vec == 0 and all(x % vec == 0 for x in bstr)
         return False
 
+    def split_ok(k0, sk, sk1):
+        # A two-level k axis is only loaded along unit-stride runs, and no k-slab may straddle two runs.
+        return k0 == g["K"] or (sk == 1 and k0 % 64 == 0 and sk1 % vec == 0 and sk1 > 0)
+
     return (operand_ok(g["a_sk"], g["a_sm"], g["M"], g["a_off"], bstr_a)
-            and operand_ok(g["b_sk"], g["b_sn"], g["N"], g["b_off"], bstr_b))
+            and operand_ok(g["b_sk"], g["b_sn"], g["N"], g["b_off"], bstr_b)
+            and split_ok(g["a_k0"], g["a_sk"], g["a_sk1"]) and split_ok(g["b_k0"], g["b_sk"], g["b_sk1"]))

@@ -1,0 +1,25 @@
+"""Helpers for replaying a traced JitProgram on a backend (the hip backend or the oracle one)."""
+import numpy as np
+
+from jaxjs_hip.alu import numpyDtype
+
+
+def run_program(backend, prog, arrays, out_dtypes_shapes=None):
+    """Realise the program's constants with their nullary kernels, upload `arrays`, execute, read back.
+    Returns one flat typed numpy array per program output; every slot is released again."""
+    const_slots = []
+    for c in prog.consts:
+        k = c.kernel()
+        s = backend.malloc(k.bytes)
+        backend.dispatch(backend.prepareKernelSync(k), [], [s])
+        const_slots.append(s)
+    in_slots = [backend.malloc(np.ascontiguousarray(a).nbytes, np.ascontiguousarray(a).tobytes()) for a in arrays]
+    outs = prog.execute(backend, const_slots + in_slots)
+    results = []
+    out_kernels = {s.output: s.kernel for s in prog.steps if s.kind == "execute"}
+    for slot, oid in zip(outs, prog.outputs):
+        raw = backend.readSync(slot)
+        results.append(np.frombuffer(raw, dtype=numpyDtype(out_kernels[oid].dtype)).copy())
+    for s in const_slots + in_slots + outs:
+        backend.decRef(s)
+    return results

@@ -1,0 +1,242 @@
+"""The restated tracing/jit layer: kernel boundaries follow the reference's rules
+(src/frontend/jit.ts:792-1096) and the library compositions reproduce the reference's own tables
+(test/nn.test.ts, test/numpy.test.ts, test/argreduce.test.ts) when replayed on the CPU oracle."""
+import math
+
+import numpy as np
+import pytest
+
+from jaxjs_hip import jit as J
+from jaxjs_hip import library as L
+from jaxjs_hip import workloads as W
+from jaxjs_hip.alu import AluOp, DType
+from jaxjs_hip.jit import ShapedArray
+from jit_util import run_program
+from oracle import oracle
+from oracle.backend import OracleBackend
+
+F32 = DType.Float32
+
+
+def run(fn, *arrays, dtype=F32):
+    prog = J.jit(fn, [ShapedArray(tuple(a.shape), dtype) for a in arrays])
+    be = OracleBackend()
+    outs = run_program(be, prog, arrays)
+    assert be.live_slots() == 0  # every intermediate, constant and output was released exactly once
+    return prog, outs
+
+
+def f32(x):
+    return np.asarray(x, dtype=np.float32)
+
+
+# ---- kernel boundaries ------------------------------------------------------------------------------
+
+def test_elementwise_chain_is_one_kernel():
+    prog, (y,) = run(lambda a, b: J.exp(a.mul(b).add(1)).mul(0.5), f32([1, 2, 3]), f32([4, 5, 6]))
+    assert len(prog.kernels) == 1 and prog.kernels[0].reduction is None
+    np.testing.assert_allclose(y, np.exp(f32([5, 11, 19])) * 0.5, rtol=1e-5)
+
+
+def test_reduction_fuses_unary_and_literal_epilogue():
+    """backend.test.ts:248-286 shape: a reduce followed by +1 stays one kernel with an epilogue."""
+    prog, (y,) = run(lambda a: J.neg(a.sum(-1).add(1)), f32([[1, 1], [2, 3], [4, 8]]))
+    assert len(prog.kernels) == 1
+    np.testing.assert_array_equal(y, f32([-3, -6, -13]))
+
+
+def test_reduction_epilogue_stops_at_broadcasting_operand_and_second_use():
+    # The keepdims reshape is a view op, so the epilogue ends at the sum; the division is a second kernel.
+    prog, (y,) = run(lambda a: a.div(a.sum(-1, keepdims=True)), f32([[1, 3], [2, 2]]))
+    assert [k.reduction is not None for k in prog.kernels] == [True, False]
+    np.testing.assert_allclose(y.reshape(2, 2), [[0.25, 0.75], [0.5, 0.5]], rtol=1e-6)
+
+
+def test_two_reductions_never_share_a_kernel():
+    prog, _ = run(lambda a: a.sum(-1).max(), f32([[1, 2], [3, 4]]))
+    assert len(prog.kernels) == 2
+
+
+def test_dot_operand_with_reuse_is_materialised():
+    """An activation feeding a matmul would be recomputed per output column; jit materialises it first."""
+    a, b = f32(np.arange(6).reshape(2, 3)), f32(np.arange(12).reshape(3, 4))
+    prog, (y,) = run(lambda x, w: L.matmul(J.exp(x), w), a, b)
+    assert len(prog.kernels) == 2 and prog.kernels[0].reduction is None
+    np.testing.assert_allclose(y.reshape(2, 4), np.exp(a) @ b, rtol=1e-5)
+    # A plain input needs no such copy.
+    prog, _ = run(lambda x, w: L.matmul(x, w), a, b)
+    assert len(prog.kernels) == 1
+
+
+def test_row_softmax_argmax_program_is_four_row_reductions_plus_one_constant():
+    prog = W.rowSoftmaxArgmaxProgram(16, 40)
+    assert len(prog.kernels) == 4 and all(k.reduction is not None and k.reduction.size == 40 for k in prog.kernels)
+    assert len(prog.consts) == 1 and prog.consts[0].shape == (40,)
+    x = np.random.default_rng(0).standard_normal((16, 40)).astype(np.float32)
+    x[3, 7] = x[3, 21] = 9.0  # a tie: the first index wins
+    y, idx = run_program(OracleBackend(), prog, [x])
+    x64 = x.astype(np.float64)
+    want = (np.exp(x64 - x64.max(-1, keepdims=True)) / (1 + np.exp(-x64))).sum(-1)
+    np.testing.assert_allclose(y, want, rtol=1e-5)
+    np.testing.assert_array_equal(idx, np.argmax(x, -1).astype(np.int32))
+    assert idx[3] == 7
+
+
+def test_max_args_splits_wide_expressions():
+    n = 6
+    arrays = [f32([i, i + 1]) for i in range(n)]
+
+    def f(*xs):
+        acc = xs[0]
+        for x in xs[1:]:
+            acc = acc.add(x)
+        return acc
+    jaxpr, consts = J.trace(f, [ShapedArray((2,), F32)] * n)
+    assert len(J.jitCompile(jaxpr, consts, maxArgs=64).kernels) == 1
+    prog = J.jitCompile(jaxpr, consts, maxArgs=3)
+    assert len(prog.kernels) > 1 and all(k.nargs <= 3 for k in prog.kernels)
+    (y,) = run_program(OracleBackend(), prog, arrays)
+    np.testing.assert_array_equal(y, sum(arrays))
+
+
+def test_jaxpr_simplify_folds_literals_and_noop_views():
+    def f(a):
+        return a.add(0).mul(1).reshape([2, 2]).transpose([0, 1]).add(J.neg(J.scalar(2.0, F32)))
+    jaxpr, _ = J.trace(f, [ShapedArray((2, 2), F32)])
+    assert [e.primitive for e in jaxpr.eqns] == ["Add"]
+    assert isinstance(jaxpr.eqns[0].inputs[1], J.Lit) and jaxpr.eqns[0].inputs[1].value == -2.0
+
+
+def test_weak_scalars_take_the_array_dtype():
+    jaxpr, _ = J.trace(lambda a: a.mul(0.5), [ShapedArray((4,), DType.Float16)])
+    assert jaxpr.outs[0].aval.dtype == DType.Float16
+    jaxpr, _ = J.trace(lambda a: a.mean(-1), [ShapedArray((4, 8), DType.Float16)])
+    assert jaxpr.outs[0].aval.dtype == DType.Float16
+    assert [e.primitive for e in jaxpr.eqns] == ["Cast", "Reduce", "Mul", "Cast"]
+
+
+# ---- library compositions against the reference's tables ---------------------------------------------
+
+def test_softmax_table():  # test/nn.test.ts:106-118
+    _, (y,) = run(lambda x: L.softmax(x), f32([[1, 2, 3], [4, 5, 6]]))
+    np.testing.assert_allclose(y.reshape(2, 3), [[0.09003057, 0.24472848, 0.66524094]] * 2, rtol=1e-5, atol=1e-7)
+
+
+GELU_X = [-10, -1, -0.3, 0, 0.1, 0.5, 3, 5, 500]
+GELU_Y = [-0, -0.158655, -0.114627, 0, 0.053983, 0.345731, 2.99595, 5, 500]
+
+
+def test_gelu_tables():  # test/nn.test.ts:86-103
+    _, (y,) = run(lambda x: L.gelu(x), f32(GELU_X))
+    np.testing.assert_allclose(y, GELU_Y, atol=1e-3)
+    _, (y,) = run(lambda x: L.gelu(x, approximate=False), f32(GELU_X))
+    np.testing.assert_allclose(y, GELU_Y, rtol=1e-5, atol=1e-5)  # the table itself carries 6 digits
+
+
+def test_tanh_matches_libm_and_saturates():
+    x = f32([-100, -3, -0.5, 0, 1e-3, 0.5, 3, 100])
+    _, (y,) = run(lambda v: L.tanh(v), x)
+    np.testing.assert_allclose(y, np.tanh(x.astype(np.float64)), rtol=2e-4, atol=1e-6)
+    assert y[0] == -1 and y[-1] == 1
+
+
+def test_standardize_table():  # test/nn.test.ts:217-229
+    _, (y,) = run(lambda x: L.standardize(x), f32([[1, 2, 3], [4, 5, 6]]))
+    np.testing.assert_allclose(y.reshape(2, 3), [[-1.22474487, 0, 1.22474487]] * 2, rtol=1e-4, atol=1e-5)
+
+
+def test_attention_tables():  # test/nn.test.ts:274-390
+    q = f32([[[[1, 0, 0, 0]], [[0, 1, 0, 0]]]])
+    v = f32([[[[1, 2, 3, 4]], [[5, 6, 7, 8]]]])
+    prog, (y,) = run(lambda a, b, c: L.dotProductAttention(a, b, c), q, q, v)
+    a, b = 0.62245935, 0.37754068
+    np.testing.assert_allclose(y.reshape(1, 2, 1, 4)[0, 0, 0], [a * 1 + b * 5, a * 2 + b * 6, a * 3 + b * 7, a * 4 + b * 8], atol=1e-5)
+    e = f32([[[[1, 0]], [[0, 1]]]])
+    _, (y,) = run(lambda a, b, c: L.dotProductAttention(a, b, c, scale=1.0), e, e, e)
+    np.testing.assert_allclose(y.reshape(1, 2, 1, 2)[0, 0, 0], [0.7310586, 0.26894143], atol=1e-5)
+
+
+def test_causal_attention_closed_form():  # test/nn.test.ts:371-390
+    q = f32([[[[1, 0]], [[0.2, 0.2]], [[1, 1]]]])
+    k = f32([[[[1, 0]], [[0, 1]], [[1, 1]]]])
+    v = f32([[[[1, 0]], [[0, 1]], [[0, 0]]]])
+    prog, (y,) = run(lambda a, b, c: L.dotProductAttention(a, b, c, isCausal=True), q, k, v)
+    y = y.reshape(1, 3, 1, 2)
+    np.testing.assert_allclose(y[0, 0, 0], [1, 0], rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(y[0, 1, 0], [0.5, 0.5], rtol=1e-5, atol=1e-7)
+    c = 1 / (2 + math.exp(math.sqrt(0.5)))
+    np.testing.assert_allclose(y[0, 2, 0], [c, c], rtol=1e-5, atol=1e-7)
+    assert len(prog.consts) == 1 and prog.consts[0].dtype == DType.Bool  # the triangular mask
+
+
+def test_matmul_integer_cases_are_exact():  # test/numpy.test.ts:1510-1560, 1696-1747
+    _, (y,) = run(lambda a, b: L.matmul(a, b), f32([[1, 2], [3, 4]]), f32([[5, 6], [7, 8]]))
+    np.testing.assert_array_equal(y.reshape(2, 2), [[19, 22], [43, 50]])
+    a = f32(np.arange(1 * 784).reshape(1, 784) % 7)
+    b = f32(np.ones((784, 10)))
+    _, (y,) = run(lambda p, q: L.matmul(p, q), a, b)
+    np.testing.assert_array_equal(y, np.full(10, a.sum()))
+    # stacked batch
+    a = f32(np.arange(2 * 3 * 3).reshape(2, 3, 3))
+    _, (y,) = run(lambda p, q: L.matmul(p, q), a, a)
+    np.testing.assert_array_equal(y.reshape(2, 3, 3), a @ a)
+
+
+def test_einsum_layouts_of_attention():
+    rng = np.random.default_rng(1)
+    B, Lq, N, H, S = 2, 3, 2, 4, 5
+    q = f32(rng.integers(-3, 4, (B, Lq, N, H)))
+    k = f32(rng.integers(-3, 4, (B, S, N, H)))
+    _, (y,) = run(lambda a, b: L.einsum("BLNH,BSNH->BNLS", a, b), q, k)
+    np.testing.assert_array_equal(y.reshape(B, N, Lq, S), np.einsum("BLNH,BSNH->BNLS", q, k))
+    p = f32(rng.integers(-3, 4, (B, N, Lq, S)))
+    _, (y,) = run(lambda a, b: L.einsum("BNLS,BSNH->BLNH", a, b), p, k)
+    np.testing.assert_array_equal(y.reshape(B, Lq, N, H), np.einsum("BNLS,BSNH->BLNH", p, k))
+
+
+# ---- transformer block ---------------------------------------------------------------------------------
+
+def block_reference(x, P, heads):
+    """float64 numpy restatement of the block, for a tolerance check of the whole program."""
+    def ln(v, g, b):
+        mu = v.mean(-1, keepdims=True)
+        var = (v * v).mean(-1, keepdims=True) - mu * mu
+        return (v - mu) / np.sqrt(var + 1e-5) * g + b
+    B, T, d = x.shape
+    H = d // heads
+    h = ln(x, P["ln1_g"], P["ln1_b"])
+    qkv = h @ P["w_qkv"] + P["b_qkv"]
+    q, k, v = (qkv[..., i * d:(i + 1) * d].reshape(B, T, heads, H) for i in range(3))
+    s = np.einsum("BLNH,BSNH->BNLS", q, k) / math.sqrt(H)
+    s = np.where(np.tril(np.ones((T, T), bool)), s, -np.inf)
+    p = np.exp(s - s.max(-1, keepdims=True))
+    p = p / p.sum(-1, keepdims=True)
+    a = np.einsum("BNLS,BSNH->BLNH", p, v).reshape(B, T, d)
+    x = x + a @ P["w_o"] + P["b_o"]
+    h = ln(x, P["ln2_g"], P["ln2_b"])
+    m = h @ P["w_fc1"] + P["b_fc1"]
+    m = 0.5 * m * (1 + np.tanh(math.sqrt(2 / math.pi) * (m + 0.044715 * m ** 3)))
+    return x + m @ P["w_fc2"] + P["b_fc2"]
+
+
+def block_inputs(batch, seq, d, d_ff, dtype, seed=5):
+    rng = np.random.default_rng(seed)
+    shapes = W.gpt2BlockShapes(batch, seq, d, d_ff)
+    arrs = {n: (rng.standard_normal(s) * (1.0 if n == "x" else 0.05)).astype(dtype) for n, s in shapes.items()}
+    arrs["ln1_g"] = (1 + arrs["ln1_g"]).astype(dtype)
+    arrs["ln2_g"] = (1 + arrs["ln2_g"]).astype(dtype)
+    return arrs
+
+
+def test_gpt2_block_program_structure_and_values_f32():
+    batch, seq, d, heads, d_ff = 2, 16, 32, 4, 64
+    prog = W.gpt2BlockProgram(batch, seq, d, heads, d_ff, dtype=F32)
+    # 6 contractions (QKV, QK^T, AV, out, fc1, fc2), 4 LayerNorm moment reductions, 2 softmax reductions,
+    # and the maps between them; one closed-over constant (the causal mask).
+    assert len(prog.kernels) == 18 and len(prog.consts) == 1
+    assert sum(1 for k in prog.kernels if k.reduction is not None) == 12
+    arrs = block_inputs(batch, seq, d, d_ff, np.float32)
+    order = ["x"] + list(W.GPT2_BLOCK_PARAMS)
+    (y,) = run_program(OracleBackend(), prog, [arrs[n] for n in order])
+    want = block_reference(arrs["x"].astype(np.float64), {n: arrs[n].astype(np.float64) for n in order[1:]}, heads)
+    np.testing.assert_allclose(y.reshape(batch, seq, d), want, rtol=2e-4, atol=2e-5)

@@ -1,0 +1,121 @@
+"""Whole traced programs on the hip backend: the row softmax/argmax pair and the GPT-2-small block.
+
+Every Kernel of a program is checked on its own (inputs taken from the oracle's replay of the program, so
+an error cannot hide behind a later kernel), then the program is replayed end to end on the GPU."""
+import math
+
+import numpy as np
+import pytest
+
+from gpu_util import WARM_ONLY, backend
+from jaxjs_hip import workloads as W
+from jaxjs_hip.alu import DType, numpyDtype
+from jit_util import run_program
+from oracle import oracle
+from oracle.backend import OracleBackend
+from test_jit import block_inputs, block_reference
+
+pytestmark = pytest.mark.gpu
+
+
+def warm(prog):
+    from jaxjs_hip.kernelgen import generate
+    from jaxjs_hip.runtime import compile_source
+    for k in prog.kernels + [c.kernel() for c in prog.consts]:
+        for src in generate(k).sources:
+            compile_source(src)
+    pytest.skip("warm-up run: compiled only")
+
+
+def replay_on_oracle(prog, arrays):
+    """id -> host array for every buffer of the program (constants, inputs, intermediates)."""
+    bufs = {}
+    for i, c in enumerate(prog.consts):
+        bufs[i] = oracle.run_kernel(c.kernel(), [], oracle.MODE_WASM)
+    for j, a in enumerate(arrays):
+        bufs[len(prog.consts) + j] = np.ascontiguousarray(a)
+    for s in prog.steps:
+        if s.kind == "execute":
+            bufs[s.output] = oracle.run_kernel(s.kernel, [bufs[i] for i in s.inputs], oracle.MODE_WASM)
+    return bufs
+
+
+def check_each_kernel(prog, bufs, f16_rtol=1e-2):
+    be = backend()
+    classes = []
+    for s in prog.steps:
+        if s.kind != "execute":
+            continue
+        k = s.kernel
+        exe = be.prepareKernelSync(k)
+        slots = [be.malloc(bufs[i].nbytes, bufs[i].tobytes()) for i in s.inputs]
+        out = be.malloc(k.bytes)
+        be.dispatch(exe, slots, [out])
+        got = np.frombuffer(be.readSync(out), dtype=numpyDtype(k.dtype))
+        for x in slots + [out]:
+            be.decRef(x)
+        want = bufs[s.output]
+        classes.append(exe.data.ks.klass)
+        msg = f"kernel -> buffer {s.output}, class {exe.data.ks.klass}, {exe.data.ks.info}"
+        if k.dtype in (DType.Int32, DType.Uint32, DType.Bool):
+            np.testing.assert_array_equal(got, want, err_msg=msg)
+        elif k.dtype == DType.Float16:
+            np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64), rtol=f16_rtol, atol=2e-3, equal_nan=True, err_msg=msg)
+        else:
+            R = k.reduction.size if k.reduction is not None else 1
+            np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64), rtol=1e-5 * max(1, math.sqrt(R)), atol=1e-6, equal_nan=True, err_msg=msg)
+    return classes
+
+
+def test_row_softmax_argmax_program():
+    prog = W.rowSoftmaxArgmaxProgram(256, 1000)
+    if WARM_ONLY:
+        warm(prog)
+    x = np.random.default_rng(3).standard_normal((256, 1000)).astype(np.float32)
+    x[5, 100] = x[5, 900] = 7.0
+    bufs = replay_on_oracle(prog, [x])
+    assert check_each_kernel(prog, bufs) == ["reduce_row"] * 4
+    y, idx = run_program(backend(), prog, [x])
+    np.testing.assert_array_equal(idx, np.argmax(x, -1).astype(np.int32))  # bit-exact, first index on ties
+    np.testing.assert_allclose(y, bufs[prog.outputs[0]], rtol=1e-5 * math.sqrt(1000))
+
+
+@pytest.mark.parametrize("heads,expect_out_proj", [(4, "reduce_row"), (2, "gemm")])
+def test_gpt2_block_small_f16(heads, expect_out_proj):
+    """d=128: with 4 heads (H=32) the out-projection reads the attention output through a two-level k axis
+    too short for MFMA slabs and takes the row-reduce class; with 2 heads (H=64) it is a GEMM."""
+    batch, seq, d, d_ff = 2, 64, 128, 512
+    prog = W.gpt2BlockProgram(batch, seq, d, heads, d_ff)
+    if WARM_ONLY:
+        warm(prog)
+    arrs = block_inputs(batch, seq, d, d_ff, np.float16)
+    order = ["x"] + list(W.GPT2_BLOCK_PARAMS)
+    arrays = [arrs[n] for n in order]
+    bufs = replay_on_oracle(prog, arrays)
+    classes = check_each_kernel(prog, bufs)
+    assert classes.count("gemm") == (6 if expect_out_proj == "gemm" else 5) and classes[11] == expect_out_proj
+    (y,) = run_program(backend(), prog, arrays)
+    np.testing.assert_allclose(y.astype(np.float64), bufs[prog.outputs[0]].astype(np.float64), rtol=2e-2, atol=2e-2)
+    want = block_reference(arrs["x"].astype(np.float64), {n: arrs[n].astype(np.float64) for n in order[1:]}, heads)
+    np.testing.assert_allclose(y.astype(np.float64).reshape(batch, seq, d), want, rtol=3e-2, atol=3e-2)
+
+
+def test_gpt2_block_full_size_f16_batch0_against_float64():
+    """The benchmark shape (batch 8, seq 1024, d 768, 12 heads, d_ff 3072).  The whole program runs on the GPU;
+    batch element 0 and 7 are compared with a float64 restatement (each kernel rounds its output to f16, so the
+    bound is a few f16 ulps of values of order 1)."""
+    batch, seq, d, heads, d_ff = 8, 1024, 768, 12, 3072
+    prog = W.gpt2BlockProgram(batch, seq, d, heads, d_ff)
+    if WARM_ONLY:
+        warm(prog)
+    arrs = block_inputs(batch, seq, d, d_ff, np.float16, seed=11)
+    order = ["x"] + list(W.GPT2_BLOCK_PARAMS)
+    be = backend()
+    (y,) = run_program(be, prog, [arrs[n] for n in order])
+    y = y.reshape(batch, seq, d).astype(np.float64)
+    assert np.isfinite(y).all()
+    P = {n: arrs[n].astype(np.float64) for n in order[1:]}
+    for b in (0, 7):
+        want = block_reference(arrs["x"][b:b + 1].astype(np.float64), P, heads)[0]
+        err = np.abs(y[b] - want)
+        assert err.max() < 6e-2 and err.mean() < 4e-3, (b, err.max(), err.mean())
