@@ -27,6 +27,9 @@ import numpy as np  # noqa: E402
 PEAK_HBM_GBS = 8000.0
 PEAK_F16_TFLOPS = 2500.0
 PEAK_F32_MATRIX_TFLOPS = 157.3
+# HBM bytes per launch of the 8192^3 f16 GEMM kernel from rocprofv3 FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 (factors from a
+# copy kernel of known size); the counters are collected in separate profiler runs, not in the timed run.
+GEMM_8192_HBM_BYTES = 1.750e9
 
 
 def timed(be, exe, ins, out, steps, warmup):
@@ -84,6 +87,70 @@ def cpu_baseline_matmul(n, seconds=12.0):
                        f"{spent:.1f} s on one host core; {os.cpu_count()} cores present")
 
 
+def bench_program_gpt2(be, hostrand, timed):
+    """GPT-2-small block forward (batch 8, seq 1024, d 768, 12 heads, d_ff 3072, f16) as the traced jit program:
+    every Kernel timed alone on the program's own buffers, and the whole program timed back to back."""
+    from jaxjs_hip import workloads as W
+
+    batch, seq, d, heads, d_ff = 8, 1024, 768, 12, 3072
+    prog = W.gpt2BlockProgram(batch, seq, d, heads, d_ff)
+    shapes = W.gpt2BlockShapes(batch, seq, d, d_ff)
+    order = ["x"] + list(W.GPT2_BLOCK_PARAMS)
+    bufs = {}
+    for i, c in enumerate(prog.consts):
+        k = c.kernel()
+        bufs[i] = be.malloc(k.bytes)
+        be.dispatch(be.prepareKernelSync(k), [], [bufs[i]])
+    for j, name in enumerate(order):
+        if name in ("ln1_g", "ln2_g"):
+            arr = np.ones(shapes[name], np.float16)
+        elif name in ("ln1_b", "ln2_b"):
+            arr = np.zeros(shapes[name], np.float16)
+        else:
+            arr = hostrand.normal(1005, shapes[name], 0.02, np.float16, stream=j)
+        bufs[len(prog.consts) + j] = upload(be, arr)
+    steps = [s for s in prog.steps if s.kind == "execute"]
+    exes = []
+    for s in steps:
+        bufs[s.output] = be.malloc(s.kernel.bytes)
+        exes.append(be.prepareKernelSync(s.kernel))
+
+    def whole():
+        for s, ex in zip(steps, exes):
+            be.dispatch(ex, [bufs[i] for i in s.inputs], [bufs[s.output]])
+
+    dev = be.dev
+    for _ in range(5):
+        whole()
+    dev.sync()
+    e0, e1 = dev.event(), dev.event()
+    reps = 10
+    dev.record(e0)
+    for _ in range(reps):
+        whole()
+    dev.record(e1)
+    dev.sync()
+    total_ms = dev.elapsed_ms(e0, e1) / reps
+    dev.destroy_event(e0)
+    dev.destroy_event(e1)
+    kernels = []
+    for s, ex in zip(steps, exes):
+        _, est = timed(be, ex, [bufs[i] for i in s.inputs], bufs[s.output], 3, 2)
+        n_steps = int(min(max(3.0 / max(est, 1e-4), 5), 2000))
+        _, ms = timed(be, ex, [bufs[i] for i in s.inputs], bufs[s.output], n_steps, max(n_steps // 2, 3))
+        k = s.kernel
+        row = {"class": ex.data.ks.klass, "out_elems": k.size, "reduce": k.reduction.size if k.reduction is not None else 0,
+               "ms": round(ms, 5)}
+        if ex.data.ks.klass == "gemm":
+            row["TFLOP/s"] = round(2.0 * k.size * k.reduction.size / (ms * 1e-3) / 1e12, 1)
+        kernels.append(row)
+    for sl in bufs.values():
+        be.decRef(sl)
+    flops = 1.417e11
+    return {"kernels_in_program": len(steps), "ms": round(total_ms, 4), "sum_of_kernel_ms": round(sum(r["ms"] for r in kernels), 4),
+            "model_flops": flops, "TFLOP/s": round(flops / (total_ms * 1e-3) / 1e12, 1), "per_kernel": kernels}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -138,7 +205,7 @@ def main():
         "config": {"workload": f"dense GEMM f16 {n}x{n}x{n}, f32 accumulate, np.matmul lowering (B stored [K,N])",
                    "kernel_class": exe.data.ks.klass, "tile": exe.data.ks.info},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": None},
+                     "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": GEMM_8192_HBM_BYTES if n == 8192 else None},
     }
     for s in (a, b, c):
         be.decRef(s)
@@ -212,6 +279,19 @@ def main():
             Am = hostrand.uniform(1004, (mm, kk), dtype=npdt)
             Bm = hostrand.uniform(1005, (kk, nn), dtype=npdt, stream=1)
             run(tag, matmulKernel(mm, nn, kk, dt), [Am, Bm], 2.0 * mm * nn * kk, "TFLOP/s", peak)
+        Am = hostrand.uniform(1004, (8192, 8192), dtype=np.float16)
+        Bm = hostrand.uniform(1005, (8192, 8192), dtype=np.float16, stream=1)
+        run("gemm_f16_8192_NT(B stored [N,K])", matmulKernel(8192, 8192, 8192, DType.Float16, b_transposed=True), [Am, Bm],
+            2.0 * 8192 ** 3, "TFLOP/s", PEAK_F16_TFLOPS)
+        del Am, Bm
+        for (mm, nn, kk, tag) in [(2048, 2048, 2048, "gemm_f32_2048"), (8192, 8192, 8192, "gemm_f32_8192"),
+                                  (128, 14336, 4096, "gemm_f32_skinny_128x14336x4096")]:
+            Am = hostrand.uniform(1004, (mm, kk), dtype=np.float32)
+            Bm = hostrand.uniform(1005, (kk, nn), dtype=np.float32, stream=1)
+            run(tag, matmulKernel(mm, nn, kk, DType.Float32), [Am, Bm], 2.0 * mm * nn * kk, "TFLOP/s", PEAK_F32_MATRIX_TFLOPS)
+        del Am, Bm
+
+        extra["c5_gpt2_block_b8_l1024_f16"] = bench_program_gpt2(be, hostrand, timed)
         result["extra"] = extra
 
     if not args.no_cpu:
