@@ -16,7 +16,7 @@ from .tuner import CU_COUNT, TuneResult
 
 
 def choose_tile(g: dict) -> Dict[str, int]:
-    """f16: 256x256 tiles when they still give every CU work, else 128x128; f32: 128x128 down to 64x64."""
+    """Block tile (and wave arrangement) for one GEMM: f16 by a small cost model, f32 128x128 down to 64x64."""
     nb = 1
     for b in g["batch"]:
         nb *= b[0]
@@ -32,19 +32,38 @@ def choose_tile(g: dict) -> Dict[str, int]:
             if g["M"] >= bm and g["N"] >= bn and tiles(bm, bn) >= 2 * CU_COUNT:
                 return dict(BM=bm, BN=bn)
         return dict(BM=64, BN=64)
-    if g["M"] >= 256 and g["N"] >= 256 and tiles(256, 256) >= (3 * CU_COUNT) // 4:
-        return dict(BM=256, BN=256)
-    if g["M"] >= 256 and tiles(256, 128) >= (3 * CU_COUNT) // 4:
-        return dict(BM=256, BN=128)
-    return dict(BM=128, BN=128)
+    # f16: estimated time = (tiles the busiest CU runs) x (tile area) x (K + fixed per-tile overhead) / efficiency.
+    # Efficiencies are measured rates of each tile shape relative to 256x256 on large problems (MI355X):
+    # 128x256 0.84, 256x128 0.79, 128x128 0.72 with two workgroups resident per CU (0.64 alone).  The fixed
+    # overhead (pipeline fill + epilogue) is about 100 k-steps.  This picks big tiles for big problems and
+    # smaller ones when 256x256 would leave the last round of CUs nearly empty (e.g. 288 tiles on 256 CUs).
+    if g["N"] <= 64 and g["M"] >= 128:
+        # A 128-wide tile would compute and store a half-empty block (attention's probabilities x V, N = head
+        # size 64): measured 30 % faster with 128x64 tiles, which is then bound by reading A.
+        return dict(BM=128, BN=64, WM=2, WN=2)
+    best = None
+    for bm, bn, eff, extra in ((256, 256, 1.00, dict()), (128, 256, 0.84, dict(WM=1, WN=4)), (256, 128, 0.79, dict()),
+                                (128, 128, 0.72, dict())):
+        if (bm > 128 and g["M"] < bm) or (bn > 128 and g["N"] < bn):
+            continue
+        per_cu = -(-tiles(bm, bn) // CU_COUNT)
+        if (bm, bn) == (128, 128) and per_cu < 2:
+            eff = 0.64
+        cost = per_cu * bm * bn * (g["K"] + 100) / eff
+        if best is None or cost < best[0]:
+            best = (cost, dict(BM=bm, BN=bn, **extra))
+    return best[1]
 
 
 def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelSource:
     g = t.gemm
     re = kernel.reduction
     assert g is not None and re is not None and t.epilogue is not None
-    tile = choose_tile(g)
-    tile.update(t.params.get("gemm_tile") or {})
+    override = dict(t.params.get("gemm_tile") or {})
+    tile = dict() if ("BM" in override or "BN" in override) else choose_tile(g)
+    tile.update(override)
+    if "BM" not in tile or "BN" not in tile:
+        raise ValueError("a tile override must give both BM and BN")
     BM, BN = tile["BM"], tile["BN"]
     WM, WN = tile.get("WM", 2), tile.get("WN", 2)
     if BM % (32 * WM) or BN % (32 * WN):
@@ -61,20 +80,37 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         [f"const {STORAGE_CTYPE[d or DType.Float32]}* __restrict__ {n}" for d, n in zip(used, names)]
         + [f"{out_t}* __restrict__ out"])
 
-    # Fused epilogue as a device function of (acc, gidx, buffers...).
-    cg = HipExpCodegen(names, {"acc": "acc", "gidx": "gidx"}, "  ", prefix="e", numerics=numerics)
-    cg.countReferences(t.epilogue)
-    value = strip_parens(cg.run(t.epilogue))
+    # Fused epilogue as a device function of (acc, row, col, batch coordinates, buffers...).  The kernel's
+    # epilogue is written over the flat output index; here that index is re-expressed through the tile's own
+    # coordinates and simplified, so `gidx % N` becomes `col` and a bias load no longer depends on the row
+    # (the compiler then hoists it out of the per-row loop instead of doing a division per element).
+    if len(g["batch"]) > 3:
+        raise ValueError("at most 3 batch axes")
+    I32 = DType.Int32
+    gexp = AluExp.add(AluExp.mul(AluExp.special(I32, "row", max(g["M"], 1)), AluExp.i32(g["c_sm"])),
+                      AluExp.mul(AluExp.special(I32, "col", max(g["N"], 1)), AluExp.i32(g["c_sn"])))
+    for k, (size, _sa, _sb, sc) in enumerate(g["batch"]):
+        gexp = AluExp.add(AluExp.mul(AluExp.special(I32, f"b{k}", size), AluExp.i32(sc)), gexp)
+
+    def _retarget(node):
+        if node.op == AluOp.Special and node.arg[0] == "gidx":
+            return gexp
+        return None
+    epilogue = t.epilogue.rewrite(_retarget).simplify()
+    cg = HipExpCodegen(names, {"acc": "acc", "row": "row", "col": "col", "b0": "b0", "b1": "b1", "b2": "b2"}, "  ",
+                       prefix="e", numerics=numerics)
+    cg.countReferences(epilogue)
+    value = strip_parens(cg.run(epilogue))
     epi_params = "".join(f", const {STORAGE_CTYPE[d or DType.Float32]}* __restrict__ {n}" for d, n in zip(used, names))
-    epi_fn = (f"static __device__ __forceinline__ {out_t} jh_epilogue(float acc, int gidx{epi_params}) {{\n"
+    epi_fn = (f"static __device__ __forceinline__ {out_t} jh_epilogue(float acc, int row, int col, int b0, int b1, int b2{epi_params}) {{\n"
               + "\n".join(cg.take_lines()) + f"\n  return ({out_t})({value});\n}}")
     epi_args = "".join(f", {n}" for n in names)
 
     # Batch index decode, innermost batch axis last in g["batch"].
     lines = ["  {", "    int rem = batch;"]
     for k, (size, sa, sb, sc) in reversed(list(enumerate(g["batch"]))):
-        lines.append(f"    const int b{k} = rem % {size}; rem /= {size};")
-        lines.append(f"    a_base += (long long)b{k} * {sa}ll; b_base += (long long)b{k} * {sb}ll; c_base += (long long)b{k} * {sc}ll;")
+        lines.append(f"    jh_b{k} = rem % {size}; rem /= {size};")
+        lines.append(f"    a_base += (long long)jh_b{k} * {sa}ll; b_base += (long long)jh_b{k} * {sb}ll; c_base += (long long)jh_b{k} * {sc}ll;")
     lines.append("  }")
     nbatch = 1
     for b in g["batch"]:
