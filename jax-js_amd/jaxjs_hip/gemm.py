@@ -11,8 +11,8 @@ from typing import Dict, List
 
 from .alu import AluExp, AluOp, DType, Kernel, byteWidth
 from .codegen import CTYPE, STORAGE_CTYPE, HipExpCodegen, strip_parens
-from .kernelgen import KernelSource, LaunchStep, _min_bytes, _prelude, _used_args, fill, template
-from .tuner import CU_COUNT, TuneResult
+from .kernelgen import KernelSource, LaunchStep, _Body, _min_bytes, _prelude, _used_args, fill, template
+from .tuner import CU_COUNT, TuneResult, classify_loads
 
 
 def choose_tile(g: dict) -> Dict[str, int]:
@@ -124,6 +124,20 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         tmpl = "gemm_f16_dlds.hip.inc"
     if dlds:
         sched = dict(STAGES=tile.get("STAGES", 4), PIPE=tile.get("PIPE", 1), SGB=tile.get("SGB", 1), ASM_LOAD=tile.get("ASM", 1))
+        # Vector epilogue: needs unit column stride and 8-element alignment of every row / batch start of C.
+        # It pays when the epilogue itself reads buffers (bias, residual): those become 128-bit loads.  A plain
+        # cast-and-store epilogue measures the same either way and keeps the simpler path.
+        has_loads = bool(epilogue.collect(lambda x: x.op == AluOp.GlobalIndex))
+        vec = (tile.get("VEPI", 1 if has_loads else 0) and g["c_sn"] == 1 and g["c_sm"] % 8 == 0 and all(b[3] % 8 == 0 for b in g["batch"])
+               and kernel.dtype != DType.Bool)
+        if vec:
+            vnames = {"acc": "acc", "row": "row", "col": "col", "b0": "b0", "b1": "b1", "b2": "b2"}
+            body = _Body(epilogue, names, vnames, "col", "c0", 8, classify_loads(epilogue, "col", 8), numerics, "      ", "e")
+            vhoist, vloads = body.hoisted()
+            vbody, vvalue = body.lanes(vloads)
+            sched.update(VEC_EPI=1, VEPI_LOADS=vhoist, VEPI_BODY=vbody, VEPI_VALUE=vvalue, OUT_T=out_t)
+        else:
+            sched.update(VEC_EPI=0, VEPI_LOADS="", VEPI_BODY="", VEPI_VALUE="0", OUT_T=out_t)
     elif g["dtype"] == DType.Float16:
         sched = dict(COMMIT_A=tile.get("CA", 2), COMMIT_B=tile.get("CB", 3), FETCH_A=tile.get("FA", 0),
                      FETCH_B=tile.get("FB", 1), IGLP=tile.get("IGLP", -1), SCHED_FENCE=tile.get("FENCE", 0))
