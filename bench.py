@@ -292,6 +292,32 @@ def main():
         del Am, Bm
 
         extra["c5_gpt2_block_b8_l1024_f16"] = bench_program_gpt2(be, hostrand, timed)
+
+        # Routines: sort / argsort of f32 [8192, 4096] rows (native bitonic network in LDS).
+        from jaxjs_hip.routine import Routine, Routines, RoutineType
+        rows, L = 8192, 4096
+        X = hostrand.normal(1006, (rows, L), 1.0, np.float32)
+        xs = upload(be, X)
+        for rname, nout in ((Routines.Sort, 1), (Routines.Argsort, 2)):
+            rt = Routine(rname, RoutineType([[rows, L]], [DType.Float32], [[rows, L]] * nout, [DType.Float32, DType.Int32][:nout]))
+            rexe = be.prepareRoutineSync(rt)
+            outs = [be.malloc(rows * L * 4) for _ in range(nout)]
+            for _ in range(5):
+                be.dispatch(rexe, [xs], outs)
+            be.dev.sync()
+            e0, e1 = be.dev.event(), be.dev.event()
+            be.dev.record(e0)
+            for _ in range(10):
+                be.dispatch(rexe, [xs], outs)
+            be.dev.record(e1)
+            be.dev.sync()
+            ms = be.dev.elapsed_ms(e0, e1) / 10
+            extra[f"routine_{rname.value.lower()}_f32[8192,4096]"] = {"class": "sort", "ms": round(ms, 4),
+                                                                        "Gelem/s": round(rows * L / (ms * 1e-3) / 1e9, 2)}
+            for o in outs:
+                be.decRef(o)
+        be.decRef(xs)
+        del X
         result["extra"] = extra
 
     if not args.no_cpu:

@@ -179,17 +179,56 @@ class HipBackend:
 
     def prepareRoutineSync(self, routine: Routine) -> Executable:
         from .routine import SUPPORTED_ROUTINES
+        from .routinegen import generateRoutine
 
         if routine.name not in SUPPORTED_ROUTINES:
             raise UnsupportedRoutineError(routine.name, "hip")
-        return Executable(routine, None)
+        ks = generateRoutine(routine, self.numerics)
+        if ks is None:
+            return Executable(routine, None)  # host path, as the reference's Wasm backend runs every routine
+        modules = [self.dev.load_module(compile_source(src, f"{ks.klass}.hip")) for src in ks.sources]
+        functions = [self.dev.function(modules[s.module], s.name) for s in ks.steps]
+        scratch = [self.dev.malloc(self._rounded(b)) for b in ks.scratch_bytes]
+        return Executable(routine, _Prepared(ks, functions, scratch, modules))
 
     async def prepareRoutine(self, routine: Routine) -> Executable:
         return self.prepareRoutineSync(routine)
 
+    def _dispatch_routine(self, exe: Executable, ins, outs) -> None:
+        """Launch a routine's native plan (several kernels on the one in-order stream)."""
+        routine: Routine = exe.source
+        prep: _Prepared = exe.data
+        t = routine.type
+        from .alu import byteWidth
+        from .shape import prod
+
+        if len(ins) != len(t.inputShapes) or len(outs) != len(t.outputShapes):
+            raise ValueError(f"{routine.name.value} takes {len(t.inputShapes)} inputs and {len(t.outputShapes)} outputs")
+        for what, slots, shapes, dtypes in (("input", ins, t.inputShapes, t.inputDtypes), ("output", outs, t.outputShapes, t.outputDtypes)):
+            for i, (s, shape, dt) in enumerate(zip(slots, shapes, dtypes)):
+                need = prod(shape) * byteWidth(dt)
+                if s["size"] < need:
+                    raise ValueError(f"{what} {i} holds {s['size']} bytes, the routine addresses {need}")
+        for step, fn in zip(prep.ks.steps, prep.functions):
+            values = []
+            for kind, i in step.args:
+                if kind == "in":
+                    values.append(ins[i]["ptr"])
+                elif kind == "out":
+                    values.append(outs[i]["ptr"])
+                elif kind == "scratch":
+                    values.append(prep.scratch[i])
+                else:
+                    values.append(int(i))
+            argv, keep = pack_args(values)
+            self.dev.launch(fn, step.grid, step.block, step.shared, argv, 1)
+
     def dispatch(self, exe: Executable, inputs: Sequence[int], outputs: Sequence[int], repeat: int = 1) -> None:
         ins = [self._get(s) for s in inputs]
         outs = [self._get(s) for s in outputs]
+        if isinstance(exe.source, Routine) and exe.data is not None:
+            self._dispatch_routine(exe, ins, outs)
+            return
         if isinstance(exe.source, Routine):
             host_in = [self.dev.d2h(s["ptr"], 0, s["size"]) for s in ins]
             host_out = [bytearray(s["size"]) for s in outs]

@@ -1,10 +1,11 @@
 """Routines: the non-fusable operations a backend is handed as a unit (reference: src/routine.ts).
 
 `Routine{name, type, params}` mirrors src/routine.ts:20-29 and `Routines` the enum at :32-102.
-The `hip` backend does what the reference's Wasm backend does for every routine
-(src/backend/wasm.ts:158-165, 216-220): copy the operands to the host, run the host
-implementation, copy the outputs back.  Host implementations here cover Sort, Argsort, Scatter,
-TriangularSolve and Cholesky (vectorised with numpy, same input/output contracts as
+Sort and Argsort have native GPU plans (`routinegen.py`, template `sort.hip.inc`) for 32-bit and
+f16 element types.  For the other routines the `hip` backend does what the reference's Wasm
+backend does for every routine (src/backend/wasm.ts:158-165, 216-220): copy the operands to the
+host, run the host implementation, copy the outputs back.  Host implementations here cover Sort,
+Argsort (also the checker of the native ones), Scatter, TriangularSolve and Cholesky (vectorised with numpy, same input/output contracts as
 src/routine.ts:185-362); LU, JacobiEigh and Fft are not provided yet and raise
 `UnsupportedRoutineError` at prepare time.
 """
