@@ -122,6 +122,20 @@ int jh_launch(jh_function fn, uint32_t grid_x, uint32_t grid_y, uint32_t grid_z,
 int jh_launch_repeat(jh_function fn, uint32_t grid_x, uint32_t grid_y, uint32_t grid_z, uint32_t block_x,
                      uint32_t block_y, uint32_t block_z, uint32_t shared_bytes, void **args, int count);
 
+/*
+ * Record a sequence of launches once and replay it with one call.  Everything queued with `jh_launch` between
+ * `jh_graph_begin` and `jh_graph_end` is captured into a HIP graph instead of running; `jh_graph_launch`
+ * then replays the whole sequence in order on the stream.  This is how a compiled jit program
+ * (`JitProgram.execute`, src/frontend/jit.ts:111-162: a fixed list of kernel dispatches over fixed
+ * buffers) is issued without per-kernel host work.  No allocation, copy or synchronisation call may be made
+ * while a capture is open; buffers the launches name must stay allocated for the graph's lifetime.
+ */
+typedef void *jh_graph;
+int jh_graph_begin(void);
+int jh_graph_end(jh_graph *out);
+int jh_graph_launch(jh_graph graph);
+int jh_graph_destroy(jh_graph graph);
+
 /* Wait for everything queued so far (the completion fence `read(slot, 0, 0)` stands for in
  * src/frontend/array.ts:827). */
 int jh_sync(void);

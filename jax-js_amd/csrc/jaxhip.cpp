@@ -270,6 +270,39 @@ int jh_launch_repeat(jh_function fn, uint32_t gx, uint32_t gy, uint32_t gz, uint
   return 0;
 }
 
+int jh_graph_begin(void) {
+  JH_NEED_INIT();
+  JH_HIP(hipStreamBeginCapture(g_rt.stream, hipStreamCaptureModeThreadLocal));
+  return 0;
+}
+
+int jh_graph_end(jh_graph *out) {
+  JH_NEED_INIT();
+  if (!out) return fail(-5, "null output");
+  hipGraph_t graph = nullptr;
+  JH_HIP(hipStreamEndCapture(g_rt.stream, &graph));
+  hipGraphExec_t exec = nullptr;
+  hipError_t err = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  if (err != hipSuccess) return fail((int)err, "hipGraphInstantiate failed: %s", hipGetErrorString(err));
+  *out = (jh_graph)exec;
+  return 0;
+}
+
+int jh_graph_launch(jh_graph graph) {
+  JH_NEED_INIT();
+  if (!graph) return fail(-5, "null graph");
+  JH_HIP(hipGraphLaunch((hipGraphExec_t)graph, g_rt.stream));
+  return 0;
+}
+
+int jh_graph_destroy(jh_graph graph) {
+  JH_NEED_INIT();
+  if (!graph) return 0;
+  JH_HIP(hipGraphExecDestroy((hipGraphExec_t)graph));
+  return 0;
+}
+
 int jh_sync(void) {
   JH_NEED_INIT();
   JH_HIP(hipStreamSynchronize(g_rt.stream));

@@ -1,0 +1,63 @@
+"""A compiled jit program captured into a HIP graph.
+
+`JitProgram.execute` (src/frontend/jit.ts:111-162) is a fixed list of kernel dispatches over buffers whose
+sizes are known at compile time.  `GraphedProgram` allocates every intermediate and output once, records the
+dispatches into one graph (`jh_graph_begin/end`) and replays them with a single `jh_graph_launch`: no host
+work per kernel, no allocator traffic per call.  Inputs are bound at capture time: write new data into the
+same input slots (or capture again) to run on other values.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, List, Sequence
+
+from .jit import JitProgram
+
+
+class GraphedProgram:
+    def __init__(self, backend, prog: JitProgram, inputs: Sequence[int]):
+        if len(inputs) != prog.nargs:
+            raise ValueError(f"jit program takes {prog.nargs} inputs, got {len(inputs)}")
+        self.backend, self.prog = backend, prog
+        self._slots: Dict[int, int] = {i: s for i, s in enumerate(inputs)}
+        self._owned: List[int] = []
+        for s in inputs:
+            backend.incRef(s)
+            self._owned.append(s)
+        steps = [s for s in prog.steps if s.kind == "execute"]
+        exes = [backend.prepareKernelSync(s.kernel) for s in steps]  # compile + load before any capture
+        for s in steps:
+            slot = backend.malloc(s.kernel.bytes)
+            self._slots[s.output] = slot
+            self._owned.append(slot)
+
+        def issue():
+            for s, exe in zip(steps, exes):
+                backend.dispatch(exe, [self._slots[i] for i in s.inputs], [self._slots[s.output]])
+
+        issue()  # one eager pass: every code object is resident before the capture starts
+        backend.dev.sync()
+        trace, backend.trace = backend.trace, None  # event records are not part of the graph
+        try:
+            backend.dev.graph_begin()
+            try:
+                issue()
+            finally:
+                self._graph = backend.dev.graph_end()
+        finally:
+            backend.trace = trace
+        self.outputs = [self._slots[o] for o in prog.outputs]
+        self.kernels = len(steps)
+
+    def launch(self) -> None:
+        """Queue one replay of the whole program (asynchronous, in order with everything else)."""
+        self.backend.dev.graph_launch(self._graph)
+
+    def close(self) -> None:
+        if self._graph is not None:
+            self.backend.dev.sync()
+            self.backend.dev.graph_destroy(self._graph)
+            self._graph = None
+            for s in self._owned:
+                self.backend.decRef(s)
+            self._owned = []

@@ -69,6 +69,10 @@ _SIGNATURES = {
     "jh_launch_repeat": (ctypes.c_int, [ctypes.c_void_p] + [ctypes.c_uint32] * 7 +
                          [ctypes.POINTER(ctypes.c_void_p), ctypes.c_int]),
     "jh_sync": (ctypes.c_int, []),
+    "jh_graph_begin": (ctypes.c_int, []),
+    "jh_graph_end": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p)]),
+    "jh_graph_launch": (ctypes.c_int, [ctypes.c_void_p]),
+    "jh_graph_destroy": (ctypes.c_int, [ctypes.c_void_p]),
     "jh_event_create": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p)]),
     "jh_event_record": (ctypes.c_int, [ctypes.c_void_p]),
     "jh_event_query": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]),
@@ -220,6 +224,21 @@ class Device:
 
     def sync(self) -> None:
         check(self.lib.jh_sync(), "jh_sync")
+
+    # -- graphs ---------------------------------------------------------------------------------
+    def graph_begin(self) -> None:
+        check(self.lib.jh_graph_begin(), "jh_graph_begin")
+
+    def graph_end(self) -> int:
+        g = ctypes.c_void_p()
+        check(self.lib.jh_graph_end(ctypes.byref(g)), "jh_graph_end")
+        return g.value
+
+    def graph_launch(self, graph: int) -> None:
+        check(self.lib.jh_graph_launch(ctypes.c_void_p(graph)), "jh_graph_launch")
+
+    def graph_destroy(self, graph: int) -> None:
+        check(self.lib.jh_graph_destroy(ctypes.c_void_p(graph)), "jh_graph_destroy")
 
     # -- events ---------------------------------------------------------------------------------
     def event(self) -> int:

@@ -23,7 +23,7 @@ def _check(got, A, B, K, out_f16=True):
 
 
 SHAPES = [(128, 128, 64), (256, 256, 128), (200, 264, 136), (32, 32, 32), (512, 384, 1000 // 8 * 8), (96, 1024, 72),
-          (1024, 1024, 1024)]
+          (1024, 1024, 1024), (128, 128, 32), (256, 512, 96), (2048, 256, 160), (1024, 64, 1024), (512, 768, 768)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES, ids=lambda v: str(v))

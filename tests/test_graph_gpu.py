@@ -1,0 +1,68 @@
+"""A jit program replayed as one HIP graph: every replay must equal the eager run of the same program, also
+with unrelated eager work and synchronisation between replays and after the inputs were overwritten in place."""
+import numpy as np
+import pytest
+
+from gpu_util import WARM_ONLY, backend
+from jaxjs_hip import workloads as W
+from jaxjs_hip.alu import numpyDtype
+from jaxjs_hip.graph import GraphedProgram
+from jit_util import run_program
+from test_jit import block_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def _eager(be, prog, arrays):
+    return run_program(be, prog, arrays)
+
+
+def _check_program(prog, make_arrays, rounds=3):
+    be = backend()
+    const_slots = []
+    for c in prog.consts:
+        k = c.kernel()
+        s = be.malloc(k.bytes)
+        be.dispatch(be.prepareKernelSync(k), [], [s])
+        const_slots.append(s)
+    arrays = make_arrays(0)
+    in_slots = [be.malloc(a.nbytes, a.tobytes()) for a in arrays]
+    g = GraphedProgram(be, prog, const_slots + in_slots)
+    out_dtypes = {s.output: s.kernel.dtype for s in prog.steps if s.kind == "execute"}
+    try:
+        for r in range(rounds):
+            if r > 0:  # new input values, written into the slots the graph was captured with
+                arrays = make_arrays(r)
+                for slot, a in zip(in_slots, arrays):
+                    be.dev.h2d(be.slotPointer(slot), a.tobytes())
+            want = _eager(be, prog, arrays)  # eager work (allocations, launches, reads) between replays
+            g.launch()
+            g.launch()  # back-to-back replays are fine too: same inputs, same outputs
+            for slot, oid, w in zip(g.outputs, prog.outputs, want):
+                got = np.frombuffer(be.readSync(slot), dtype=numpyDtype(out_dtypes[oid]))
+                np.testing.assert_array_equal(got.view(np.uint8), w.view(np.uint8), err_msg=f"replay {r}")
+    finally:
+        g.close()
+        for s in const_slots + in_slots:
+            be.decRef(s)
+
+
+def test_row_softmax_argmax_graph():
+    prog = W.rowSoftmaxArgmaxProgram(128, 777)
+    if WARM_ONLY:
+        pytest.skip("kernels are compiled by the program tests")
+    _check_program(prog, lambda r: [np.random.default_rng(r).standard_normal((128, 777)).astype(np.float32)])
+    assert len([s for s in prog.steps if s.kind == "execute"]) == 4
+
+
+def test_gpt2_block_graph():
+    batch, seq, d, heads, d_ff = 2, 64, 128, 2, 512
+    prog = W.gpt2BlockProgram(batch, seq, d, heads, d_ff)
+    if WARM_ONLY:
+        pytest.skip("kernels are compiled by the program tests")
+    order = ["x"] + list(W.GPT2_BLOCK_PARAMS)
+
+    def arrays(r):
+        a = block_inputs(batch, seq, d, d_ff, np.float16, seed=100 + r)
+        return [a[n] for n in order]
+    _check_program(prog, arrays)
