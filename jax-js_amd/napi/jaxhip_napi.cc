@@ -305,6 +305,33 @@ napi_value EventDestroy(napi_env env, napi_callback_info info) {
   return nullptr;
 }
 
+napi_value GraphBegin(napi_env env, napi_callback_info) {  // launches queued until graphEnd() are recorded, not run
+  JH_OK(jh_graph_begin());
+  return nullptr;
+}
+
+napi_value GraphEnd(napi_env env, napi_callback_info) {  // -> BigInt graph handle
+  jh_graph g = nullptr;
+  JH_OK(jh_graph_end(&g));
+  return make_u64(env, (uint64_t)(uintptr_t)g);
+}
+
+napi_value GraphLaunch(napi_env env, napi_callback_info info) {
+  Args a(env, info);
+  uint64_t g;
+  if (a.argc < 1 || !get_u64(env, a.argv[0], &g)) { napi_throw_type_error(env, nullptr, "graphLaunch(graph)"); return nullptr; }
+  JH_OK(jh_graph_launch((jh_graph)(uintptr_t)g));
+  return nullptr;
+}
+
+napi_value GraphDestroy(napi_env env, napi_callback_info info) {
+  Args a(env, info);
+  uint64_t g;
+  if (a.argc < 1 || !get_u64(env, a.argv[0], &g)) { napi_throw_type_error(env, nullptr, "graphDestroy(graph)"); return nullptr; }
+  JH_OK(jh_graph_destroy((jh_graph)(uintptr_t)g));
+  return nullptr;
+}
+
 napi_value AbiVersion(napi_env env, napi_callback_info) {
   napi_value out;
   napi_create_int32(env, jh_abi_version(), &out);
@@ -319,7 +346,8 @@ NAPI_MODULE_INIT() {
       {"h2d", H2D}, {"d2h", D2H}, {"compile", Compile}, {"moduleLoad", ModuleLoad}, {"moduleUnload", ModuleUnload},
       {"moduleFunction", ModuleFunction}, {"launch", Launch}, {"sync", Sync}, {"eventCreate", EventCreate},
       {"eventRecord", EventRecord}, {"eventQuery", EventQuery}, {"eventElapsedMs", EventElapsed},
-      {"eventDestroy", EventDestroy}, {"abiVersion", AbiVersion},
+      {"eventDestroy", EventDestroy}, {"graphBegin", GraphBegin}, {"graphEnd", GraphEnd}, {"graphLaunch", GraphLaunch},
+      {"graphDestroy", GraphDestroy}, {"abiVersion", AbiVersion},
   };
   for (const auto& e : table) {
     napi_value fn;
