@@ -87,6 +87,47 @@ def cpu_baseline_matmul(n, seconds=12.0):
                        f"{spent:.1f} s on one host core; {os.cpu_count()} cores present")
 
 
+def cpu_baseline_secondary():
+    """CPU figures beside the secondary workloads (one host core, reported only): the Wasm K-SIMD matvec loop
+    restated in C on the full f32 stand-in of W[11008,4096], and the Wasm-mode evaluation of the fused
+    sum(exp(x-m)*sigmoid(x)) row kernel on 64 of the 8192 rows."""
+    from oracle import oracle
+    from jaxjs_hip import AluExp, AluOp, DType, ShapeTracker, hostrand
+    from jaxjs_hip.lowering import reduceKernel
+
+    L = oracle.lib()
+    M, K = 11008, 4096
+    W = hostrand.normal(1003, (M, K), 0.02, np.float32)
+    x = hostrand.normal(1003, (K,), 1.0, np.float32, stream=1)
+    y = np.empty(M, np.float32)
+    best = 1e9
+    for _ in range(5):
+        t0 = time.perf_counter()
+        rc = L.jo_wasm_matvec_f32(W.ctypes.data_as(ctypes.c_void_p), x.ctypes.data_as(ctypes.c_void_p),
+                                  y.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(M), ctypes.c_int64(K))
+        best = min(best, time.perf_counter() - t0)
+        assert rc == 0
+    out = {"matvec_f32_W[11008,4096]": {"ms": round(best * 1e3, 3), "GB/s": round((M * K * 4 + K * 4 + M * 4) / best / 1e9, 2),
+                                          "kind": "port", "cores": 1}}
+    rows, Lc = 64, 4096
+    X = hostrand.normal(1002, (rows, Lc), 1.0, np.float32)
+    f = DType.Float32
+    st = ShapeTracker.fromShape([rows, Lc])
+    stm = ShapeTracker.fromShape([rows]).reshape([rows, 1]).expand([rows, Lc])
+
+    def body(v, mm):
+        sig = AluExp.reciprocal(AluExp.add(AluExp.exp(AluExp.sub(AluExp.f32(0), v)), AluExp.f32(1)))
+        return AluExp.mul(AluExp.exp(AluExp.add(v, AluExp.sub(AluExp.f32(0), mm))), sig)
+    k = reduceKernel([rows, Lc], [(f, st), (f, stm)], body, AluOp.Add)
+    m = X.max(axis=1)
+    t0 = time.perf_counter()
+    oracle.run_kernel(k, [X, m], oracle.MODE_WASM)
+    dt = time.perf_counter() - t0
+    out["c2_sum_exp_sigmoid"] = {"ms_for_64_of_8192_rows": round(dt * 1e3, 2), "GB/s": round(rows * Lc * 4 / dt / 1e9, 3),
+                                 "kind": "port (interpreter of the kernel, Wasm numerics)", "cores": 1}
+    return out
+
+
 def bench_program_gpt2(be, hostrand, timed):
     """GPT-2-small block forward (batch 8, seq 1024, d 768, 12 heads, d_ff 3072, f16) as the traced jit program:
     every Kernel timed alone on the program's own buffers, and the whole program timed back to back."""
@@ -338,6 +379,8 @@ def main():
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline_matmul(n)
+        if not args.no_extra:
+            result["extra"]["cpu_secondary"] = cpu_baseline_secondary()
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result))
