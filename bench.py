@@ -350,6 +350,17 @@ def main():
 
         extra["c5_gpt2_block_b8_l1024_f16"] = bench_program_gpt2(be, hostrand, timed)
 
+        # Convolution through the view algebra (no implicit-GEMM class yet: the kernel takes a generic reduce class).
+        from jaxjs_hip import jit as J, library as Lb
+        from jaxjs_hip.jit import ShapedArray
+        for cdt, npdt, tag in ((DType.Float16, np.float16, "f16"), (DType.Float32, np.float32, "f32")):
+            cx, cw = (32, 64, 56, 56), (64, 64, 3, 3)
+            cprog = J.jit(lambda a, b: Lb.convGeneralDilated(a, b, [1, 1], "SAME"), [ShapedArray(cx, cdt), ShapedArray(cw, cdt)])
+            ck = cprog.kernels[0]
+            run(f"conv3x3_same_{tag}[32,64,56,56]x[64,64,3,3]", ck,
+                [hostrand.normal(1007, cx, 1.0, npdt), hostrand.normal(1007, cw, 0.05, npdt, stream=1)],
+                2.0 * 32 * 64 * 56 * 56 * 64 * 9, "TFLOP/s", PEAK_F16_TFLOPS if cdt == DType.Float16 else PEAK_F32_MATRIX_TFLOPS)
+
         # Routines: sort / argsort of f32 [8192, 4096] rows (native bitonic network in LDS).
         from jaxjs_hip.routine import Routine, Routines, RoutineType
         rows, L = 8192, 4096

@@ -37,6 +37,9 @@ def choose_tile(g: dict) -> Dict[str, int]:
     # 128x256 0.84, 256x128 0.79, 128x128 0.72 with two workgroups resident per CU (0.64 alone).  The fixed
     # overhead (pipeline fill + epilogue) is about 100 k-steps.  This picks big tiles for big problems and
     # smaller ones when 256x256 would leave the last round of CUs nearly empty (e.g. 288 tiles on 256 CUs).
+    if g["M"] <= 64 and g["N"] >= 256:
+        # Few rows (e.g. 64 output channels of a convolution against thousands of positions): a 64-row tile.
+        return dict(BM=64, BN=256, WM=1, WN=4)
     if g["N"] <= 64 and g["M"] >= 128:
         # A 128-wide tile would compute and store a half-empty block (attention's probabilities x V, N = head
         # size 64): measured 30 % faster with 128x64 tiles, which is then bound by reading A.
@@ -53,6 +56,14 @@ def choose_tile(g: dict) -> Dict[str, int]:
         if best is None or cost < best[0]:
             best = (cost, dict(BM=bm, BN=bn, **extra))
     return best[1]
+
+
+def _strip_casts(e: AluExp) -> AluExp:
+    """Drop float<->float casts around an operand (the MFMA consumes the storage type)."""
+    while e.op == AluOp.Cast and e.dtype in (DType.Float16, DType.Float32, DType.Float64) and \
+            e.src[0].dtype in (DType.Float16, DType.Float32):
+        e = e.src[0]
+    return e
 
 
 def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelSource:
@@ -106,6 +117,43 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
               + "\n".join(cg.take_lines()) + f"\n  return ({out_t})({value});\n}}")
     epi_args = "".join(f", {n}" for n in names)
 
+    # Element loaders for gather operands: the operand's lowered expression (masked load through its view
+    # chain) with the flat output index rebuilt from (tile row, batch coordinates) and ridx = k.
+    gather_fns, gather_calls, gather_flags = [], {}, {}
+    lowered = _strip_casts(t.exp)
+    operand_exps = {g["gid_a"]: None, g["gid_b"]: None}
+    if g.get("a_gather") or g.get("b_gather"):
+        assert lowered.op == AluOp.Mul
+        for side in lowered.src:
+            gids = {n.arg[0] for n in side.collect(lambda x: x.op == AluOp.GlobalIndex)}
+            if len(gids) != 1:
+                raise ValueError("gather operand must read exactly one buffer")
+            operand_exps[gids.pop()] = _strip_casts(side)
+    for tag, gid, is_gather, extent, c_stride in (("a", g["gid_a"], g.get("a_gather"), g["M"], g["c_sm"]),
+                                                  ("b", g["gid_b"], g.get("b_gather"), g["N"], g["c_sn"])):
+        gather_flags[tag] = 1 if is_gather else 0
+        if not is_gather:
+            gather_calls[tag] = f"({in_t})0"
+            continue
+        flat = AluExp.mul(AluExp.special(I32, "row", max(extent, 1)), AluExp.i32(c_stride))
+        for k, (size, _sa, _sb, sc) in enumerate(g["batch"]):
+            flat = AluExp.add(AluExp.mul(AluExp.special(I32, f"b{k}", size), AluExp.i32(sc)), flat)
+        kvar = AluExp.special(I32, "k", max(g["K"], 1))
+
+        def _retarget_operand(node, flat=flat, kvar=kvar):
+            if node.op == AluOp.Special and node.arg[0] == "gidx":
+                return flat
+            if node.op == AluOp.Special and node.arg[0] == "ridx":
+                return kvar
+            return None
+        oexp = operand_exps[gid].rewrite(_retarget_operand).simplify()
+        gcg = HipExpCodegen(names, {"row": "row", "k": "k", "b0": "b0", "b1": "b1", "b2": "b2"}, "  ", prefix=f"g{tag}", numerics=numerics)
+        gcg.countReferences(oexp)
+        gval = strip_parens(gcg.run(oexp))
+        gather_fns.append(f"static __device__ __forceinline__ {in_t} jh_gather_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
+                          + "\n".join(gcg.take_lines()) + f"\n  return ({in_t})({gval});\n}}")
+        gather_calls[tag] = f"jh_gather_{tag}(row, k, jh_b0, jh_b1, jh_b2{epi_args})"
+
     # Batch index decode, innermost batch axis last in g["batch"].
     lines = ["  {", "    int rem = batch;"]
     for k, (size, sa, sb, sc) in reversed(list(enumerate(g["batch"]))):
@@ -119,7 +167,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     tmpl = "gemm_f16.hip.inc" if g["dtype"] == DType.Float16 else "gemm_f32.hip.inc"
     # Fast path: direct global->LDS loads need whole tiles (no bounds predicates) and 32-deep slabs.
     full = g["M"] % BM == 0 and g["N"] % BN == 0 and g["K"] % 32 == 0 and BM >= 128 and BN >= 128
-    dlds = g["dtype"] == DType.Float16 and full and tile.get("DLDS", 1)
+    any_gather = bool(g.get("a_gather") or g.get("b_gather"))
+    dlds = g["dtype"] == DType.Float16 and full and tile.get("DLDS", 1) and not any_gather
     if dlds:
         tmpl = "gemm_f16_dlds.hip.inc"
     if dlds:
@@ -143,9 +192,13 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                      FETCH_B=tile.get("FB", 1), IGLP=tile.get("IGLP", -1), SCHED_FENCE=tile.get("FENCE", 0))
     else:
         sched = {}
+    if not dlds:
+        sched.update(GATHER_FNS="\n".join(gather_fns), A_GATHER=gather_flags["a"], B_GATHER=gather_flags["b"],
+                     GATHER_A_CALL=gather_calls["a"], GATHER_B_CALL=gather_calls["b"])
     src = _prelude(numerics) + fill(template(tmpl), dict(sched, 
         M=g["M"], N=g["N"], K=g["K"], BM=BM, BN=BN, WM=WM, WN=WN,
-        A_KCONTIG=1 if g["a_sk"] == 1 or g["K"] == 1 else 0, B_KCONTIG=1 if g["b_sk"] == 1 or g["K"] == 1 else 0,
+        A_KCONTIG=1 if g["a_sk"] == 1 or g["K"] == 1 or g.get("a_gather") else 0,
+        B_KCONTIG=1 if g["b_sk"] == 1 or g["K"] == 1 or g.get("b_gather") else 0,
         NBATCH=nbatch, EPILOGUE_FN=epi_fn, NAME=name, PARAMS=params,
         A_OFF=g["a_off"], B_OFF=g["b_off"], BATCH_DECODE="\n".join(lines),
         A_PTR=names[g["gid_a"]], B_PTR=names[g["gid_b"]],
@@ -155,6 +208,9 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     tiles = -(-g["M"] // BM) * -(-g["N"] // BN) * nbatch
     step = LaunchStep(name, (tiles, 1, 1), (nthreads, 1, 1), 0, [("in", i) for i in range(kernel.nargs)] + [("out", 0)])
     need = _min_bytes(t.epilogue)
+    if any_gather:
+        for gid_, b_ in _min_bytes(t.exp).items():
+            need[gid_] = max(need.get(gid_, 0), b_)
     eb = byteWidth(g["dtype"])
     need[g["gid_a"]] = max(need.get(g["gid_a"], 0), g["a_len"] * eb)
     need[g["gid_b"]] = max(need.get(g["gid_b"], 0), g["b_len"] * eb)

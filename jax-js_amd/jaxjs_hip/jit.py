@@ -12,8 +12,8 @@ Kernel sequence to the `hip` backend that `jit()` would:
   JitProgram.execute                      src/frontend/jit.ts:111-162
 
 Only the primitives whose lowering is a fused Kernel are covered (elementwise, Compare, Where,
-Reduce, Dot, Transpose/Reshape/Broadcast/Flip/Shrink/Pad); routines, Gather, RandomBits, Conv and
-Concatenate/Split are not traced here.
+Reduce, Dot, Conv, Pool, Transpose/Reshape/Broadcast/Flip/Shrink/Pad); routines, Gather, RandomBits,
+PoolTranspose and Concatenate/Split are not traced here.
 """
 
 from __future__ import annotations
@@ -23,6 +23,7 @@ from dataclasses import dataclass, field
 from typing import Any, Callable, Dict, List, Optional, Sequence, Set, Tuple, Union
 
 from .alu import AluExp, AluOp, AluVar, DType, Kernel, Reduction, byteWidth, isFloatDtype
+from .convolution import ConvParams, checkConvShape, checkPoolShape, pool, prepareConv
 from .shape import ShapeTracker, prod, unravelAlu
 
 # ---- abstract values ------------------------------------------------------------------------------
@@ -113,8 +114,8 @@ class JaxprEqn:
     outBinders: List[Var]
 
 
-VIEW_PRIMITIVES = ("Transpose", "Broadcast", "Reshape", "Flip", "Shrink", "Pad")
-REDUCE_PRIMITIVES = ("Reduce", "Dot")
+VIEW_PRIMITIVES = ("Transpose", "Broadcast", "Reshape", "Flip", "Shrink", "Pad")  # src/frontend/jit.ts:905-912
+REDUCE_PRIMITIVES = ("Reduce", "Dot", "Conv")
 UNARY_FUSABLE = ("Neg", "Reciprocal", "Floor", "Ceil", "StopGradient", "Cast", "Bitcast", "Sin", "Cos", "Asin", "Atan",
                  "Exp", "Log", "Erf", "Erfc", "Sqrt")
 BINARY_FUSABLE = ("Add", "Mul", "Idiv", "Mod", "Min", "Max", "BitCombine", "BitShift")
@@ -338,6 +339,11 @@ def _out_aval(prim: str, avals: List[ShapedArray], params: Dict[str, Any]) -> Sh
     if prim == "Dot":
         c = promoteAvals(avals[0], avals[1])
         return ShapedArray(c.shape[:-1], c.dtype, c.weak)
+    if prim == "Conv":
+        c = promoteAvals(ShapedArray((), avals[0].dtype, avals[0].weak), ShapedArray((), avals[1].dtype, avals[1].weak))
+        return ShapedArray(tuple(checkConvShape(avals[0].shape, avals[1].shape, params["conv"])), c.dtype, c.weak)
+    if prim == "Pool":
+        return ShapedArray(tuple(checkPoolShape(avals[0].shape, params["window"], params["strides"])), avals[0].dtype, avals[0].weak)
     if prim == "Transpose":
         return ShapedArray(tuple(avals[0].shape[p] for p in params["perm"]), avals[0].dtype, avals[0].weak)
     if prim in ("Reshape", "Broadcast"):
@@ -383,6 +389,16 @@ def greaterEqual(x, y): return bind1("Compare", [y, x], dict(op="LessEqual"))  #
 
 def dot(x, y):
     return bind1("Dot", [x, y])
+
+
+def conv(x, y, params: ConvParams):
+    """The Conv primitive (src/frontend/core.ts:295-312): shapes are checked when the output aval is formed."""
+    return bind1("Conv", [x, y], dict(conv=params))
+
+
+def poolWindows(x, window, strides):
+    """The Pool primitive: `[..., *spatial] -> [..., *out, *window]` (a view; reduce the trailing axes)."""
+    return bind1("Pool", [x], dict(window=tuple(window), strides=tuple(strides)))
 
 
 def transpose(x, perm=None):
@@ -524,6 +540,16 @@ def _dot_rule(exps, avals, params):
     return _reduce_rule([c], [cs], dict(op=AluOp.Add, axis=[cs.ndim - 1]))
 
 
+def _conv_rule(exps, avals, params):
+    """src/frontend/jit.ts:622-635: re-view both operands, then it is a Dot."""
+    stX, stY = prepareConv(ShapeTracker.fromShape(list(avals[0].shape)), ShapeTracker.fromShape(list(avals[1].shape)), params["conv"])
+    a = reshapeViews(exps[0], lambda st: st.compose(stX))
+    b = reshapeViews(exps[1], lambda st: st.compose(stY))
+    as_ = ShapedArray(tuple(stX.shape), avals[0].dtype, avals[0].weak)
+    bs_ = ShapedArray(tuple(stY.shape), avals[1].dtype, avals[1].weak)
+    return _dot_rule([a, b], [as_, bs_], {})
+
+
 def _flip_rule(st, params):
     arg = [False] * len(st.shape)
     for ax in params["axis"]:
@@ -556,6 +582,8 @@ JIT_RULES: Dict[str, Callable] = {
     "Sqrt": _unop(lambda a, p: AluExp.sqrt(a)),
     "Reduce": _reduce_rule,
     "Dot": _dot_rule,
+    "Conv": _conv_rule,
+    "Pool": _reshape_rule(lambda st, p: pool(st, list(p["window"]), list(p["strides"]))),
     "Compare": _broadcasted(lambda e, p: aluCompare(e[0], e[1], p["op"])),
     "Where": _broadcasted(lambda e, p: AluExp.where(e[0], e[1], e[2]), skipCastIdx=(0,)),
     "Transpose": _reshape_rule(lambda st, p: st.permute(p["perm"])),
@@ -634,9 +662,14 @@ def splitGraphDataflow(jaxpr: Jaxpr, maxArgs: int) -> Set[Var]:
         materialized.add(cur)
 
     for eqn in jaxpr.eqns:
-        if eqn.primitive != "Dot":
+        if eqn.primitive == "Dot":
+            shapes = [eqn.inputs[0].aval.shape, eqn.inputs[1].aval.shape]
+        elif eqn.primitive == "Conv":
+            lhs, rhs = prepareConv(ShapeTracker.fromShape(list(eqn.inputs[0].aval.shape)),
+                                   ShapeTracker.fromShape(list(eqn.inputs[1].aval.shape)), eqn.params["conv"])
+            shapes = [tuple(lhs.shape), tuple(rhs.shape)]
+        else:
             continue
-        shapes = [eqn.inputs[0].aval.shape, eqn.inputs[1].aval.shape]
         promoted = generalBroadcast(shapes[0], shapes[1])
         for i, x in enumerate(eqn.inputs):
             if isinstance(x, Var) and hasReuse(shapes[i], promoted):

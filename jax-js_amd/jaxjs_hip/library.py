@@ -103,6 +103,40 @@ def einsum(subscripts: str, a: Tracer, b: Tracer):
     return res.transpose([order.index(c) for c in out])
 
 
+def padtypeToPads(inShape, filterShape, strides, dilation, padding: str):
+    """"VALID" / "SAME" / "SAME_LOWER" to explicit pads (src/library/lax.ts:133-165)."""
+    kind = padding.upper()
+    if kind == "VALID":
+        return [(0, 0)] * len(inShape)
+    if kind not in ("SAME", "SAME_LOWER"):
+        raise ValueError(f"Unknown padding type: {kind}")
+    out = [-(-size // s) for size, s in zip(inShape, strides)]
+    sizes = [max(0, (o - 1) * s + 1 + (k - 1) * d - i) for o, s, k, d, i in zip(out, strides, filterShape, dilation, inShape)]
+    if kind == "SAME":
+        return [(sz >> 1, sz - (sz >> 1)) for sz in sizes]
+    return [(sz - (sz >> 1), sz >> 1) for sz in sizes]
+
+
+def convGeneralDilated(lhs: Tracer, rhs: Tracer, windowStrides: Sequence[int], padding, lhsDilation=None, rhsDilation=None):
+    """`lax.conv_general_dilated` with one feature group: lhs `[N, C, *xs]`, rhs `[O, C, *ks]` (lax.ts:268-343)."""
+    n = lhs.ndim - 2
+    rd = list(rhsDilation) if rhsDilation is not None else [1] * n
+    ld = list(lhsDilation) if lhsDilation is not None else [1] * n
+    if isinstance(padding, str):
+        if any(d != 1 for d in ld):
+            raise ValueError("String padding is not supported for transposed convolutions")
+        padding = padtypeToPads(lhs.shape[2:], rhs.shape[2:], windowStrides, rd, padding)
+    from .convolution import ConvParams
+    return J.conv(lhs, rhs, ConvParams(0, list(windowStrides), [tuple(p) for p in padding], ld, rd))
+
+
+def reduceWindow(x: Tracer, op: AluOp, window: Sequence[int], strides: Optional[Sequence[int]] = None):
+    """`lax.reduceWindow` for a plain reduction: Pool view, then reduce the window axes (lax.ts:479-502)."""
+    strides = list(strides) if strides is not None else [1] * len(window)
+    p = J.poolWindows(x, window, strides)
+    return J.reduce(p, op, list(range(p.ndim - len(window), p.ndim)))
+
+
 def arange_const(start: int, stop: int, step: int = 1, dtype: DType = DType.Int32, shape: Optional[Sequence[int]] = None) -> ConstArray:
     """`arange(...)` (optionally reshaped): start + cast(idx)*step, realised by a nullary kernel."""
     size = max(0, -(-(stop - start) // step)) if step > 0 else max(0, -((start - stop) // step))

@@ -274,11 +274,26 @@ def match_gemm(kernel: Kernel) -> Optional[dict]:
         return None
     if a.dtype not in (DType.Float16, DType.Float32):
         return None
-    fa, fb = _flatten_k_split(a.arg[1]), _flatten_k_split(b.arg[1])
-    if fa is None or fb is None:
+    # An operand that is not one plain strided view (masked, or several views: the patches of a convolution,
+    # a padded or dilated activation) is a *gather* operand: its tile is loaded element by element through
+    # its own index expression.  Only its outermost view is looked at here, and only to see which output
+    # axes it depends on (stride 0 = independent).
+    def describe(gv):
+        f = _flatten_k_split(gv.arg[1])
+        if f is not None and f[0].mask is None:
+            return f[0], f[1], f[2], False
+        outer = gv.arg[1].views[-1]
+        if outer.mask is not None:
+            return None
+        return outer, 0, 0, True
+
+    da, db = describe(a), describe(b)
+    if da is None or db is None:
         return None
-    (va, ka0, ka1), (vb, kb0, kb1) = fa, fb
-    if va.mask is not None or vb.mask is not None or va.shape != vb.shape or len(va.shape) < 1:
+    (va, ka0, ka1, ga), (vb, kb0, kb1, gb) = da, db
+    if ga and gb:
+        return None  # at least one operand streams through vector loads
+    if va.shape != vb.shape or len(va.shape) < 1:
         return None
     shape = list(va.shape)
     if shape[-1] != re.size or math.prod(shape[:-1]) != kernel.size or kernel.size == 0 or re.size == 0:
@@ -288,7 +303,7 @@ def match_gemm(kernel: Kernel) -> Optional[dict]:
         if len(gv.src) != len(expected) or any(x.simplify() is not y for x, y in zip(gv.src, expected)):
             return None
     ska, skb = va.strides[-1], vb.strides[-1]
-    if shape[-1] > 1 and (ska == 0 or skb == 0):
+    if shape[-1] > 1 and ((ska == 0 and not ga) or (skb == 0 and not gb)):
         return None
     # Output strides: row-major over shape[:-1].
     outs = [1] * (len(shape) - 1)
@@ -307,7 +322,8 @@ def match_gemm(kernel: Kernel) -> Optional[dict]:
     for ax in axes:
         if merged and merged[-1][0] == ax[0]:
             p = merged[-1]
-            if all(p[k] == ax[k] * ax[1] for k in (2, 3, 4)):
+            nest = [4] + ([] if ga else [2]) + ([] if gb else [3])  # a gather operand's own strides do not matter
+            if all(p[k] == ax[k] * ax[1] for k in nest):
                 merged[-1] = [p[0], p[1] * ax[1], ax[2], ax[3], ax[4]]
                 continue
         merged.append(ax)
@@ -332,12 +348,33 @@ def match_gemm(kernel: Kernel) -> Optional[dict]:
         c_sm=m[4], c_sn=n[4],
         batch=[(x[1], x[2], x[3], x[4]) for x in bs],
         a_len=_span(va, ka0, ka1), b_len=_span(vb, kb0, kb1),
+        a_gather=ga, b_gather=gb, a_node=a, b_node=b,
     )
+    if ga:
+        info.update(a_off=0, a_sm=0, a_sk=1, a_k0=shape[-1], a_sk1=0, a_len=0)
+    if gb:
+        info.update(b_off=0, b_sn=0, b_sk=1, b_k0=shape[-1], b_sk1=0, b_len=0)
+    # The tile writes C with its lanes along n: when the output is contiguous along m instead (the first
+    # operand indexes the fastest output axis), exchange the operands' roles -- A.B^T and B.A^T are the same sums.
+    if info["c_sm"] == 1 and info["c_sn"] != 1 and info["N"] > 1:
+        sw = dict(info)
+        for x, y in (("gid_a", "gid_b"), ("a_off", "b_off"), ("a_sm", "b_sn"), ("a_sk", "b_sk"), ("a_k0", "b_k0"),
+                     ("a_sk1", "b_sk1"), ("a_len", "b_len"), ("a_gather", "b_gather"), ("a_node", "b_node"), ("M", "N"),
+                     ("c_sm", "c_sn")):
+            sw[x], sw[y] = info[y], info[x]
+        sw["batch"] = [(n, sb, sa, sc) for n, sa, sb, sc in info["batch"]]
+        info = sw
     # Negative strides (flipped views) are left to the generic path.
     if min(info["a_sm"], info["a_sk"], info["b_sn"], info["b_sk"], info["a_off"], info["b_off"]) < 0:
         return None
-    if any(min(x[1:]) < 0 for x in info["batch"]):
+    ga, gb = info["a_gather"], info["b_gather"]
+    if any(min(x[1:]) < 0 for x in info["batch"]) and not (ga or gb):
         return None
+    if ga or gb:
+        # batch strides of the gather operand are never used; keep the plain operand's and the output's
+        info["batch"] = [(n, 0 if ga else sa, 0 if gb else sb, sc) for n, sa, sb, sc in info["batch"]]
+        if any(min(x[1:]) < 0 for x in info["batch"]):
+            return None
     return info
 
 
@@ -477,6 +514,10 @@ def _gemm_worthwhile(g: dict) -> bool:
         # A two-level k axis is only loaded along unit-stride runs, and no k-slab may straddle two runs.
         return k0 == g["K"] or (sk == 1 and k0 % 64 == 0 and sk1 % vec == 0 and sk1 > 0)
 
-    return (operand_ok(g["a_sk"], g["a_sm"], g["M"], g["a_off"], bstr_a)
-            and operand_ok(g["b_sk"], g["b_sn"], g["N"], g["b_off"], bstr_b)
+    if g.get("a_gather") or g.get("b_gather"):
+        # The gather loader packs 8 (f16) / 4 (f32) consecutive k per store and has no ragged-k path.
+        if g["K"] % vec != 0:
+            return False
+    return ((g.get("a_gather") or operand_ok(g["a_sk"], g["a_sm"], g["M"], g["a_off"], bstr_a))
+            and (g.get("b_gather") or operand_ok(g["b_sk"], g["b_sn"], g["N"], g["b_off"], bstr_b))
             and split_ok(g["a_k0"], g["a_sk"], g["a_sk1"]) and split_ok(g["b_k0"], g["b_sk"], g["b_sk1"]))

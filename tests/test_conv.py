@@ -1,0 +1,214 @@
+"""Convolution and pooling through the restated view algebra (src/frontend/convolution.ts) and jit rule
+(src/frontend/jit.ts:622-635): the reference's tables (test/conv.test.ts:24-58, 71-80), brute-force window
+extraction, and random convolutions against a direct numpy loop -- replayed on the CPU oracle here, and on the GPU
+in the `gpu`-marked tests."""
+import itertools
+
+import numpy as np
+import pytest
+
+from jaxjs_hip import jit as J
+from jaxjs_hip import library as L
+from jaxjs_hip.alu import AluExp, AluOp, DType
+from jaxjs_hip.convolution import ConvParams, checkConvShape, pool, prepareConv
+from jaxjs_hip.jit import ShapedArray
+from jaxjs_hip.shape import ShapeTracker
+from jit_util import run_program
+from oracle.backend import OracleBackend
+
+F32 = DType.Float32
+
+
+def f32(x):
+    return np.asarray(x, dtype=np.float32)
+
+
+def run_on(backend, fn, *arrays, dtype=F32):
+    prog = J.jit(fn, [ShapedArray(tuple(a.shape), dtype) for a in arrays])
+    return prog, run_program(backend, prog, arrays)
+
+
+def run(fn, *arrays):
+    return run_on(OracleBackend(), fn, *arrays)
+
+
+def conv_reference(x, w, strides, padding, lhs_dilation=None, rhs_dilation=None):
+    """Direct loops in float64: x [N,C,*xs], w [O,C,*ks]."""
+    n = x.ndim - 2
+    ld = lhs_dilation or [1] * n
+    rd = rhs_dilation or [1] * n
+    xs = x.shape[2:]
+    dil = np.zeros(x.shape[:2] + tuple((s - 1) * d + 1 for s, d in zip(xs, ld)), np.float64)
+    dil[(slice(None), slice(None)) + tuple(slice(None, None, d) for d in ld)] = x
+    pads = [(max(p0, 0), max(p1, 0)) for p0, p1 in padding]
+    dil = np.pad(dil, [(0, 0), (0, 0)] + pads)
+    crop = tuple(slice(max(-p0, 0), dil.shape[2 + i] - max(-p1, 0)) for i, (p0, p1) in enumerate(padding))
+    dil = dil[(slice(None), slice(None)) + crop]
+    ks = w.shape[2:]
+    out_sp = [-(-(dil.shape[2 + i] - ((ks[i] - 1) * rd[i] + 1) + 1) // strides[i]) for i in range(n)]
+    out = np.zeros((x.shape[0], w.shape[0]) + tuple(out_sp), np.float64)
+    for o in itertools.product(*[range(s) for s in out_sp]):
+        for k in itertools.product(*[range(s) for s in ks]):
+            pos = tuple(o[i] * strides[i] + k[i] * rd[i] for i in range(n))
+            patch = dil[(slice(None), slice(None)) + pos]          # [N, C]
+            out[(slice(None), slice(None)) + o] += patch @ w[(slice(None), slice(None)) + k].astype(np.float64).T
+    return out
+
+
+# ---- the reference's tables ------------------------------------------------------------------------------
+
+def test_1d_convolution_tables():
+    x, y = f32([[[1, 2, 3, 4, 5]]]), f32([[[2, 0.5, -1]]])
+    _, (r,) = run(lambda a, b: L.convGeneralDilated(a, b, [1], "VALID"), x, y)
+    np.testing.assert_array_equal(r, [0, 1.5, 3])
+    prog, (r,) = run(lambda a, b: L.convGeneralDilated(a, b, [1], "SAME"), x, y)
+    np.testing.assert_array_equal(r, [-1.5, 0, 1.5, 3, 10.5])
+    assert len(prog.kernels) == 1 and prog.kernels[0].reduction.size == 3
+
+
+def test_same_and_same_lower_padding():
+    x, y = np.ones((1, 1, 5), np.float32), np.ones((1, 1, 4), np.float32)
+    _, (r,) = run(lambda a, b: L.convGeneralDilated(a, b, [1], "SAME"), x, y)
+    np.testing.assert_array_equal(r, [3, 4, 4, 3, 2])
+    _, (r,) = run(lambda a, b: L.convGeneralDilated(a, b, [1], "SAME_LOWER"), x, y)
+    np.testing.assert_array_equal(r, [2, 3, 4, 4, 3])
+
+
+def test_2d_convolution_table():
+    x = f32([[3, 1, 5], [2, 2, 9]]).reshape(1, 1, 2, 3)
+    y = f32([[1, 2], [3, 4]]).reshape(1, 1, 2, 2)
+    _, (r,) = run(lambda a, b: L.convGeneralDilated(a, b, [1, 1], "VALID"), x, y)
+    np.testing.assert_array_equal(r, [19, 53])
+
+
+def test_transposed_convolution_table():
+    """lhsDilation 2 with padding [2,2] (test/conv.test.ts:71-80); here through the generic Conv view algebra."""
+    x, k = f32([[[1, 2, 3]]]), f32([[[1, 10, 100]]])
+    _, (r,) = run(lambda a, b: L.convGeneralDilated(a, b, [1], [(2, 2)], lhsDilation=[2]), x, k)
+    np.testing.assert_array_equal(r, [100, 10, 201, 20, 302, 30, 3])
+
+
+# ---- brute force --------------------------------------------------------------------------------------------
+
+CONV_CASES = [
+    dict(x=(2, 3, 9), w=(4, 3, 3), strides=[1], padding=[(0, 0)]),
+    dict(x=(2, 3, 9), w=(4, 3, 3), strides=[2], padding=[(1, 2)]),
+    dict(x=(1, 2, 10), w=(3, 2, 3), strides=[1], padding=[(2, 2)], rd=[2]),
+    dict(x=(1, 2, 5), w=(3, 2, 3), strides=[1], padding=[(2, 1)], ld=[2]),
+    dict(x=(1, 2, 6), w=(2, 2, 3), strides=[1], padding=[(-1, 2)], ld=[2]),
+    dict(x=(2, 3, 8, 7), w=(5, 3, 3, 3), strides=[1, 1], padding=[(1, 1), (1, 1)]),
+    dict(x=(2, 3, 8, 7), w=(5, 3, 3, 2), strides=[2, 1], padding=[(0, 1), (1, 0)]),
+    dict(x=(1, 4, 9, 9), w=(2, 4, 3, 3), strides=[2, 2], padding=[(1, 1), (1, 1)], rd=[2, 1]),
+    dict(x=(1, 2, 5, 4, 3), w=(2, 2, 2, 2, 2), strides=[1, 1, 1], padding=[(0, 0), (1, 0), (0, 1)]),
+    dict(x=(3, 8, 6, 6), w=(16, 8, 1, 1), strides=[1, 1], padding=[(0, 0), (0, 0)]),
+]
+
+
+def _conv_case(c, backend):
+    rng = np.random.default_rng(3)
+    x = rng.integers(-4, 5, c["x"]).astype(np.float32)
+    w = rng.integers(-3, 4, c["w"]).astype(np.float32)
+    prog, (r,) = run_on(backend, lambda a, b: L.convGeneralDilated(a, b, c["strides"], c["padding"], lhsDilation=c.get("ld"),
+                                                                  rhsDilation=c.get("rd")), x, w)
+    want = conv_reference(x, w, c["strides"], c["padding"], c.get("ld"), c.get("rd"))
+    np.testing.assert_array_equal(r.reshape(want.shape), want)  # small integers: exact in f32
+    return prog
+
+
+@pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "x".join(map(str, c["x"])) + "*" + "x".join(map(str, c["w"])))
+def test_convolution_matches_direct_loops(case):
+    prog = _conv_case(case, OracleBackend())
+    assert len(prog.kernels) == 1  # one reduce kernel over C * prod(ks)
+
+
+def test_pooling_and_window_reductions():
+    x = np.random.default_rng(4).integers(-9, 10, (2, 3, 8, 9)).astype(np.float32)
+    _, (r,) = run(lambda a: L.reduceWindow(a, AluOp.Max, [2, 2], [2, 2]), x)
+    want = x[:, :, :8, :8].reshape(2, 3, 4, 2, 4, 2).max(axis=(3, 5))
+    np.testing.assert_array_equal(r.reshape(want.shape), want)
+    _, (r,) = run(lambda a: L.reduceWindow(a, AluOp.Add, [3, 3], [1, 1]).mul(1 / 9), x)
+    want = sum(x[:, :, dy:dy + 6, dx:dx + 7] for dy in range(3) for dx in range(3)) / 9
+    np.testing.assert_allclose(r.reshape(want.shape), want, rtol=1e-6)
+    _, (r,) = run(lambda a: L.reduceWindow(a, AluOp.Min, [3], [2]), x)  # window on the last axis only
+    want = np.stack([x[..., 2 * o:2 * o + 3].min(-1) for o in range(4)], -1)
+    np.testing.assert_array_equal(r.reshape(want.shape), want)
+
+
+def test_conv_consumer_materialises_a_computed_operand():
+    """An activation feeding a convolution is computed once, not once per output channel (jit.ts:891-950)."""
+    x = f32(np.arange(2 * 3 * 6).reshape(2, 3, 6) / 10)
+    w = f32(np.ones((4, 3, 3)))
+    prog, (r,) = run(lambda a, b: L.convGeneralDilated(J.exp(a), b, [1], "VALID"), x, w)
+    assert len(prog.kernels) == 2 and prog.kernels[0].reduction is None
+    np.testing.assert_allclose(r.reshape(2, 4, 4), conv_reference(np.exp(x), w, [1], [(0, 0)]), rtol=1e-5)
+
+
+def test_shape_errors():
+    p = ConvParams(0, [1], [(0, 0)], [1], [1])
+    with pytest.raises(ValueError):
+        checkConvShape([1, 2, 5], [3, 4, 3], p)  # channel mismatch
+    with pytest.raises(ValueError):
+        checkConvShape([1, 2, 2], [3, 2, 3], p)  # kernel larger than input
+
+
+# ---- GPU --------------------------------------------------------------------------------------------------
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "x".join(map(str, c["x"])) + "*" + "x".join(map(str, c["w"])))
+def test_convolution_on_gpu(case):
+    from gpu_util import WARM_ONLY, backend
+    if WARM_ONLY:
+        from jaxjs_hip.kernelgen import generate
+        from jaxjs_hip.runtime import compile_source
+        prog = J.jit(lambda a, b: L.convGeneralDilated(a, b, case["strides"], case["padding"], lhsDilation=case.get("ld"),
+                                                       rhsDilation=case.get("rd")), [ShapedArray(case["x"], F32), ShapedArray(case["w"], F32)])
+        for k in prog.kernels:
+            for src in generate(k).sources:
+                compile_source(src)
+        pytest.skip("warm-up run: compiled only")
+    _conv_case(case, backend())
+
+
+@pytest.mark.gpu
+def test_resnet_shaped_convolution_and_pooling_on_gpu():
+    """3x3 stride-1 'SAME' convolution [8,64,28,28] * [64,64,3,3] in f32 against float64 loops on a sample of the
+    outputs (K-scaled bound), and a 2x2 max pool, both on the GPU."""
+    from gpu_util import WARM_ONLY, backend
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((8, 64, 28, 28)).astype(np.float32)
+    w = (rng.standard_normal((64, 64, 3, 3)) * 0.05).astype(np.float32)
+    conv_prog = J.jit(lambda a, b: L.convGeneralDilated(a, b, [1, 1], "SAME"), [ShapedArray(x.shape, F32), ShapedArray(w.shape, F32)])
+    pool_prog = J.jit(lambda a: L.reduceWindow(a, AluOp.Max, [2, 2], [2, 2]), [ShapedArray(x.shape, F32)])
+    if WARM_ONLY:
+        from jaxjs_hip.kernelgen import generate
+        from jaxjs_hip.runtime import compile_source
+        conv16 = J.jit(lambda a, b: L.convGeneralDilated(a, b, [1, 1], "SAME"),
+                       [ShapedArray(x.shape, DType.Float16), ShapedArray(w.shape, DType.Float16)])
+        for k in conv_prog.kernels + pool_prog.kernels + conv16.kernels:
+            for src in generate(k).sources:
+                compile_source(src)
+        pytest.skip("warm-up run: compiled only")
+    be = backend()
+    # The patches operand is a masked three-view tracker: the kernel must take the MFMA class through its
+    # element-gather loader, not the generic row reduction.
+    assert be.prepareKernelSync(conv_prog.kernels[0]).data.ks.klass == "gemm"
+    conv16 = J.jit(lambda a, b: L.convGeneralDilated(a, b, [1, 1], "SAME"),
+                   [ShapedArray(x.shape, DType.Float16), ShapedArray(w.shape, DType.Float16)])
+    assert be.prepareKernelSync(conv16.kernels[0]).data.ks.klass == "gemm"
+    x16, w16 = x.astype(np.float16), w.astype(np.float16)
+    (r16,) = run_program(be, conv16, [x16, w16])
+    r16 = r16.reshape(8, 64, 28, 28).astype(np.float64)
+    xp16 = np.pad(x16.astype(np.float64), [(0, 0), (0, 0), (1, 1), (1, 1)])
+    for (n, o, i, j) in rng.integers(0, [8, 64, 28, 28], (200, 4)):
+        want = float((xp16[n, :, i:i + 3, j:j + 3] * w16[o].astype(np.float64)).sum())
+        assert abs(r16[n, o, i, j] - want) <= 1e-2 * abs(want) + 2e-2
+    (r,) = run_program(be, conv_prog, [x, w])
+    r = r.reshape(8, 64, 28, 28)
+    xp = np.pad(x.astype(np.float64), [(0, 0), (0, 0), (1, 1), (1, 1)])
+    for (n, o, i, j) in rng.integers(0, [8, 64, 28, 28], (200, 4)):
+        patch = xp[n, :, i:i + 3, j:j + 3]
+        want = float((patch * w[o].astype(np.float64)).sum())
+        mag = float((np.abs(patch) * np.abs(w[o])).sum())
+        assert abs(r[n, o, i, j] - want) <= 2 * 576 * np.finfo(np.float32).eps * mag + 1e-6
+    (p,) = run_program(be, pool_prog, [x])
+    np.testing.assert_array_equal(p.reshape(8, 64, 14, 14), x.reshape(8, 64, 14, 2, 14, 2).max(axis=(3, 5)))
