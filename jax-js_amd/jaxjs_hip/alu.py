@@ -754,8 +754,16 @@ class AluExp:
             lo, hi = unbounded
         if self.dtype == DType.Bool:
             lo, hi = _clamp(lo, 0, 1), _clamp(hi, 0, 1)
+        # Integer arithmetic is exact modulo 2^32: a bound outside the type's range means the value may have
+        # wrapped, so nothing is known.  (The reference only clamps the lower bound of uint32 to 0,
+        # src/alu.ts:570-572, which folds `0 - x` on uint32 to the constant 0; that is not followed here.)
         if self.dtype == DType.Uint32:
+            if op in (AluOp.Add, AluOp.Sub, AluOp.Mul, AluOp.Idiv, AluOp.Mod) and (lo < 0 or hi > 4294967295):
+                lo, hi = 0, INF
             lo = max(0, lo)
+        if self.dtype == DType.Int32 and op in (AluOp.Add, AluOp.Sub, AluOp.Mul):
+            if lo < -2147483648 or hi > 2147483647:
+                lo, hi = -INF, INF
         self._range = (lo, hi)
         return self._range
 

@@ -224,3 +224,17 @@ def test_simplify_unravel_roundtrip():  # src/shape.test.ts:401-417
         iexpr, vexpr = st.toAluExp(unravelAlu(st.shape, idx))
         assert vexpr.resolve() == 1
         assert iexpr is idx
+
+
+def test_unsigned_and_signed_wraparound_is_not_folded_away():
+    """`0 - x` on uint32 wraps to 2^32 - x: its range is unknown, not [0, 0]; same for int32 products that overflow.
+    (Found by differential fuzzing: min(c, (0 - u) * (u * u) / 7) had been folded to the constant 0.)"""
+    u = AluExp.special(DType.Uint32, "u", 1 << 20)
+    neg = AluExp.sub(AluExp.u32(0), u)
+    assert neg.max > 0 and neg.simplify().op != AluOp.Const
+    e = AluExp.min(AluExp.u32(12345), AluExp.idiv(AluExp.mul(neg, AluExp.mul(u, u)), AluExp.u32(7))).simplify()
+    assert e.op != AluOp.Const
+    assert e.evaluate({"u": 3}) == min(12345, (((0 - 3) % 2**32) * 9 % 2**32) // 7)
+    i = AluExp.special(DType.Int32, "i", 1 << 20)
+    sq = AluExp.mul(AluExp.mul(i, i), AluExp.i32(4096))  # up to 2^52 mathematically: wraps in int32
+    assert AluExp.cmplt(sq, AluExp.i32(0)).simplify().op != AluOp.Const

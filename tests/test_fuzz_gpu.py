@@ -1,0 +1,137 @@
+"""Differential fuzzing of the kernel path: random typed expression trees over a few input buffers, lowered as map
+kernels and as reductions in both memory orientations, GPU against the CPU oracle (Wasm mode).  Integer, unsigned and
+bool results must be bit-exact; f32 results within the map tolerance (rel 1e-5 + atol 1e-6; reductions K-scaled)."""
+import math
+import random
+
+import numpy as np
+import pytest
+
+from gpu_util import WARM_ONLY, assert_parity
+from jaxjs_hip import AluExp, AluOp, DType, ShapeTracker
+from jaxjs_hip.lowering import mapKernel, reduceKernel
+
+pytestmark = pytest.mark.gpu
+F32, I32, U32, BOOL = DType.Float32, DType.Int32, DType.Uint32, DType.Bool
+
+
+def rand_exp(rng, leaves, dtype, depth):
+    """A random expression of `dtype` over typed leaves {dtype: [AluExp]}; float subtrees stay well conditioned
+    (bounded magnitudes, no cancellation-prone transcendentals of large arguments)."""
+    if depth == 0 or rng.random() < 0.15:
+        if rng.random() < 0.75 and leaves.get(dtype):
+            return rng.choice(leaves[dtype])
+        if dtype == F32:
+            return AluExp.f32(rng.choice([0.0, 1.0, -1.0, 0.5, 2.0, 3.25, -0.75]))
+        if dtype == I32:
+            return AluExp.i32(rng.choice([0, 1, -1, 2, 3, 7, -5, 100, 65537]))
+        if dtype == U32:
+            return AluExp.u32(rng.choice([0, 1, 2, 3, 7, 255, 65537, 0x80000001]))
+        return AluExp.bool(rng.random() < 0.5)
+    sub = lambda dt: rand_exp(rng, leaves, dt, depth - 1)  # noqa: E731
+    r = rng.random()
+    if dtype == BOOL:
+        if r < 0.45:
+            dt = rng.choice([F32, I32, U32])
+            return (AluExp.cmplt if rng.random() < 0.6 else AluExp.cmpne)(sub(dt), sub(dt))
+        if r < 0.6:
+            return sub(BOOL).not_()
+        if r < 0.8:
+            return AluExp.cast(BOOL, sub(rng.choice([I32, U32, F32])))
+        return (AluExp.add if rng.random() < 0.5 else AluExp.mul)(sub(BOOL), sub(BOOL))  # or / and
+    if r < 0.12:
+        return AluExp.where(sub(BOOL), sub(dtype), sub(dtype))
+    if r < 0.22:
+        src = rng.choice([d for d in (F32, I32, U32, BOOL) if d != dtype])
+        inner = sub(src)
+        if src == F32 and dtype != F32:
+            inner = AluExp.mul(inner, AluExp.f32(rng.choice([1.0, 1000.0, 3e9])))  # exercise saturation too
+        return AluExp.cast(dtype, inner)
+    if dtype == F32:
+        if r < 0.5:
+            return rng.choice([AluExp.add, AluExp.sub, AluExp.mul])(sub(F32), sub(F32))
+        if r < 0.6:
+            return (AluExp.min if rng.random() < 0.5 else AluExp.max)(sub(F32), sub(F32))
+        if r < 0.68:
+            return AluExp.mul(sub(F32), AluExp.reciprocal(AluExp.add(AluExp.mul(sub(F32), sub(F32)), AluExp.f32(1.0))))
+        if r < 0.76:
+            return AluExp.sqrt(AluExp.add(AluExp.mul(sub(F32), sub(F32)), AluExp.f32(0.25)))
+        if r < 0.84:
+            return rng.choice([AluExp.floor, AluExp.ceil])(sub(F32))
+        if r < 0.92:  # transcendentals of a bounded argument
+            bounded = AluExp.min(AluExp.max(sub(F32), AluExp.f32(-4.0)), AluExp.f32(4.0))
+            return rng.choice([AluExp.exp, AluExp.sin, AluExp.cos, AluExp.atan, AluExp.erf])(bounded)
+        return AluExp.bitcast(F32, AluExp.bitCombine(AluExp.bitcast(U32, sub(F32)), AluExp.u32(0x7fffffff), "and"))  # |x|
+    # integer kinds
+    k = AluExp.i32 if dtype == I32 else AluExp.u32
+    if r < 0.5:
+        return rng.choice([AluExp.add, AluExp.sub, AluExp.mul])(sub(dtype), sub(dtype))
+    if r < 0.62:
+        return (AluExp.min if rng.random() < 0.5 else AluExp.max)(sub(dtype), sub(dtype))
+    if r < 0.74:  # division by a non-zero constant or by (x | 1)
+        den = k(rng.choice([1, 2, 3, 7, 10, 255])) if rng.random() < 0.6 else AluExp.bitCombine(sub(dtype), k(1), "or")
+        if dtype == I32 and den.op != AluOp.Const:
+            den = AluExp.max(den, k(1))  # avoid INT_MIN / -1
+        return (AluExp.idiv if rng.random() < 0.5 else AluExp.mod)(sub(dtype), den)
+    if r < 0.86:
+        return AluExp.bitCombine(sub(dtype), sub(dtype), rng.choice(["and", "or", "xor"]))
+    return AluExp.bitShift(sub(dtype), k(rng.choice([0, 1, 5, 13, 31])), rng.choice(["shl", "shr"]))
+
+
+def make_inputs(rng, n):
+    npr = np.random.default_rng(rng.randrange(1 << 30))
+    f = npr.normal(0, 2, n).astype(np.float32)
+    f[npr.integers(0, n, max(n // 40, 1))] = 0.0
+    i = npr.integers(-1000, 1000, n).astype(np.int32)
+    i[npr.integers(0, n, 4)] = [0x7fffffff, -0x80000000, -1, 0]
+    u = npr.integers(0, 1 << 32, n, dtype=np.uint64).astype(np.uint32)
+    b = npr.integers(0, 2, n).astype(np.int32)
+    return [(F32, f), (I32, i), (U32, u), (BOOL, b)]
+
+
+def leaves_for(views):
+    out = {}
+    for v in views:
+        out.setdefault(v.dtype, []).append(v)
+    return out
+
+
+@pytest.mark.parametrize("seed", range(150))
+def test_random_map_kernels(seed):
+    rng = random.Random(1000 + seed)
+    n = rng.choice([1, 5, 64, 1000, 4099, 65536 + 3])
+    inputs = make_inputs(rng, n)
+    out_dt = rng.choice([F32, F32, I32, U32, BOOL])
+    st = ShapeTracker.fromShape([n])
+    if rng.random() < 0.3 and n > 1:
+        st = st.flip([True])
+    k = mapKernel([n], [(dt, st) for dt, _ in inputs], lambda *vs: rand_exp(rng, leaves_for(vs), out_dt, rng.choice([3, 4, 5])))
+    arrays = [a for _, a in inputs]
+    if out_dt == F32:
+        assert_parity(k, arrays, rtol=1e-5, atol=1e-6)
+    else:
+        assert_parity(k, arrays, exact=True)
+
+
+@pytest.mark.parametrize("seed", range(100))
+def test_random_reductions(seed):
+    rng = random.Random(5000 + seed)
+    rows, L = rng.choice([(1, 1000), (7, 129), (64, 64), (300, 33), (5, 4097), (1000, 8)])
+    inputs = make_inputs(rng, rows * L)
+    out_dt = rng.choice([F32, I32, U32, BOOL])
+    op = rng.choice([AluOp.Add, AluOp.Max, AluOp.Min] + ([AluOp.Mul] if out_dt in (I32, U32, BOOL) else []))
+    if rng.random() < 0.5:
+        st = ShapeTracker.fromShape([rows, L])
+    else:
+        st = ShapeTracker.fromShape([L, rows]).permute([1, 0])  # reduce axis strided in memory
+    depth = rng.choice([2, 3])
+    k = reduceKernel([rows, L], [(dt, st) for dt, _ in inputs], lambda *vs: rand_exp(rng, leaves_for(vs), out_dt, depth), op,
+                     epilogue=(lambda acc: AluExp.add(acc, AluExp.const(out_dt, 1))) if out_dt in (I32, U32, F32) and rng.random() < 0.5 else None)
+    arrays = [a for _, a in inputs]
+    if out_dt == F32:
+        if op == AluOp.Add:
+            assert_parity(k, arrays, rtol=2e-5 * max(1.0, math.sqrt(L)), atol=1e-4 * L)
+        else:
+            assert_parity(k, arrays, rtol=1e-5, atol=1e-6)
+    else:
+        assert_parity(k, arrays, exact=True)
