@@ -135,3 +135,61 @@ def test_random_reductions(seed):
             assert_parity(k, arrays, rtol=1e-5, atol=1e-6)
     else:
         assert_parity(k, arrays, exact=True)
+
+
+def _random_view(rng):
+    """A random chain of movement ops on an int32 base array; returns (tracker, base, numpy view)."""
+    shape = [rng.choice([1, 2, 3, 8, 17, 40]) for _ in range(rng.choice([1, 2, 3]))]
+    base = np.arange(1, int(np.prod(shape)) + 1, dtype=np.int32)
+    ref = base.reshape(shape)
+    st = ShapeTracker.fromShape(shape)
+    for _ in range(rng.choice([1, 2, 3, 4, 5])):
+        op = rng.choice(["permute", "flip", "pad", "shrink", "reshape", "expand"])
+        nd = ref.ndim
+        if op == "permute":
+            perm = list(range(nd))
+            rng.shuffle(perm)
+            st, ref = st.permute(perm), ref.transpose(perm)
+        elif op == "flip":
+            fl = [rng.random() < 0.5 for _ in range(nd)]
+            st = st.flip(fl)
+            ref = ref[tuple(slice(None, None, -1) if f else slice(None) for f in fl)]
+        elif op == "pad":
+            pads = [(rng.choice([0, 1, 3]), rng.choice([0, 2])) for _ in range(nd)]
+            st, ref = st.pad(pads), np.pad(ref, pads)
+        elif op == "shrink":
+            arg = []
+            for s in ref.shape:
+                b = rng.randrange(0, s)
+                arg.append((b, rng.randrange(b + 1, s + 1)))
+            st = st.shrink(arg)
+            ref = ref[tuple(slice(b, e) for b, e in arg)]
+        elif op == "reshape":
+            n = ref.size
+            divs = [d for d in range(1, n + 1) if n % d == 0]
+            a = rng.choice(divs)
+            new = [a, n // a] if rng.random() < 0.7 else [n]
+            st, ref = st.reshape(new), ref.reshape(new)
+        elif op == "expand" and ref.size < 20000:
+            k = rng.choice([1, 2, 5])
+            st = st.reshape([1] + list(ref.shape)).expand([k] + list(ref.shape))
+            ref = np.broadcast_to(ref.reshape((1,) + ref.shape), (k,) + ref.shape)
+    return st, base, np.ascontiguousarray(ref)
+
+
+@pytest.mark.parametrize("seed", range(80))
+def test_random_view_chains_in_maps_and_reductions(seed):
+    """Movement ops are pure index arithmetic (multi-view trackers, masks, negative strides): the GPU result must
+    equal numpy's on the same chain, bit for bit, as an elementwise kernel and under a row reduction."""
+    rng = random.Random(9000 + seed)
+    st, base, ref = _random_view(rng)
+    shape = list(st.shape)
+    k = mapKernel(shape, [(I32, st)], lambda v: AluExp.add(AluExp.mul(v, AluExp.i32(3)), AluExp.i32(1)))
+    got, _, _ = assert_parity(k, [base], exact=True)
+    np.testing.assert_array_equal(got.reshape(ref.shape), ref * 3 + 1)
+    if len(shape) >= 1 and shape[-1] >= 1:
+        op = rng.choice([AluOp.Add, AluOp.Max, AluOp.Min])
+        kr = reduceKernel(shape, [(I32, st)], lambda v: v, op)
+        got, _, _ = assert_parity(kr, [base], exact=True)
+        want = {AluOp.Add: ref.sum(-1, dtype=np.int64).astype(np.int32), AluOp.Max: ref.max(-1), AluOp.Min: ref.min(-1)}[op]
+        np.testing.assert_array_equal(got.reshape(want.shape), want)
