@@ -34,7 +34,7 @@ def reduceKernel(shape: Sequence[int], inputs: Sequence[tuple], fn: Callable[...
     exp = fn(*src)
     re = Reduction(exp.dtype, op, shape[-1])
     if epilogue is not None:
-        re = Reduction(exp.dtype, op, shape[-1], epilogue(AluVar.acc(re.dtype)))
+        re = Reduction(exp.dtype, op, shape[-1], epilogue(AluVar.acc(exp.dtype)))
     return Kernel(len(inputs), prod(shape[:-1]), exp, re)
 
 

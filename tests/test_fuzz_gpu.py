@@ -193,3 +193,58 @@ def test_random_view_chains_in_maps_and_reductions(seed):
         got, _, _ = assert_parity(kr, [base], exact=True)
         want = {AluOp.Add: ref.sum(-1, dtype=np.int64).astype(np.int32), AluOp.Max: ref.max(-1), AluOp.Min: ref.min(-1)}[op]
         np.testing.assert_array_equal(got.reshape(want.shape), want)
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_contractions(seed):
+    """Random contraction shapes and operand layouts (either operand stored k-major or row-major, optional batch
+    axis shared or broadcast, optional fused bias/cast epilogue) with small integer data: every class the tuner may
+    pick (direct-LDS / general / f32 GEMM, swapped roles, or a plain reduction for thin shapes) must be exact."""
+    from jaxjs_hip.lowering import reduceKernel as rk
+    rng = random.Random(7000 + seed)
+    dim = lambda: rng.choice([1, 8, 31] if rng.random() < 0.15 else [64, 100, 128, 160, 256, 300, 512])  # noqa: E731
+    M, N = dim(), dim()
+    K = rng.choice([8, 32, 40, 64, 96, 128, 136, 512])
+    batch = rng.choice([[], [], [3], [2, 2]])
+    dt, npdt = rng.choice([(DType.Float16, np.float16), (DType.Float32, np.float32)])
+    npr = np.random.default_rng(seed)
+    full = batch + [M, N, K]
+    nb = len(batch)
+    a_t, b_t = rng.random() < 0.3, rng.random() < 0.5
+    b_shared = bool(batch) and rng.random() < 0.4
+    lim = 2 if dt == DType.Float16 else 3  # |sum| <= lim^2 * K stays exactly representable in the output type
+    A = npr.integers(-lim, lim + 1, batch + ([K, M] if a_t else [M, K])).astype(npdt)
+    B = npr.integers(-lim, lim + 1, ([] if b_shared else batch) + ([N, K] if b_t else [K, N])).astype(npdt)
+    stA = ShapeTracker.fromShape(list(A.shape))
+    if a_t:
+        stA = stA.permute(list(range(nb)) + [nb + 1, nb])
+    stA = stA.reshape(batch + [M, 1, K]).expand(full)
+    stB = ShapeTracker.fromShape(list(B.shape))
+    if not b_t:
+        off = 0 if b_shared else nb
+        stB = stB.permute(list(range(off)) + [off + 1, off])
+    stB = stB.reshape(([1] * nb if b_shared else batch) + [1, N, K]).expand(full)
+    with_bias = rng.random() < 0.4
+    bias = npr.integers(-5, 6, [N]).astype(npdt)
+    inputs = [(dt, stA), (dt, stB)]
+    epilogue = None
+    if with_bias:
+        from jaxjs_hip import AluVar
+        from jaxjs_hip.shape import unravelAlu
+        def epilogue(acc):
+            n_idx = unravelAlu(batch + [M, N], AluVar.gidx)[-1]
+            return AluExp.add(acc, AluExp.globalIndex(dt, 2, N, n_idx))
+    k = rk(full, inputs, lambda a, b: AluExp.mul(a, b), AluOp.Add, epilogue=epilogue)
+    arrays = [A, B] + ([bias] if with_bias else [])
+    if with_bias:
+        from jaxjs_hip import Kernel
+        k = Kernel(3, k.size, k.exp_raw, k.reduction)
+    got, want, ks = assert_parity(k, arrays, exact=True)
+    Am = A.astype(np.float64)
+    Bm = B.astype(np.float64)
+    if a_t:
+        Am = np.swapaxes(Am, -1, -2)
+    if b_t:
+        Bm = np.swapaxes(Bm, -1, -2)
+    ref = Am @ Bm + (bias.astype(np.float64) if with_bias else 0)
+    np.testing.assert_array_equal(got.astype(np.float64).reshape(ref.shape), ref.astype(npdt).astype(np.float64), err_msg=str(ks.info))
