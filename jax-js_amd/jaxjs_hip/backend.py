@@ -29,7 +29,7 @@ from typing import Dict, List, Optional, Sequence
 from .alu import Kernel, byteWidth
 from .errors import HipRuntimeError, SlotError, UnsupportedRoutineError
 from .kernelgen import KernelSource, generate
-from .routine import Routine, runCpuRoutine
+from .routine import Routine
 from .runtime import Device, compile_source, pack_args
 
 
@@ -183,9 +183,7 @@ class HipBackend:
 
         if routine.name not in SUPPORTED_ROUTINES:
             raise UnsupportedRoutineError(routine.name, "hip")
-        ks = generateRoutine(routine, self.numerics)
-        if ks is None:
-            return Executable(routine, None)  # host path, as the reference's Wasm backend runs every routine
+        ks = generateRoutine(routine, self.numerics)  # raises UnsupportedRoutineError when there is no GPU plan
         modules = [self.dev.load_module(compile_source(src, f"{ks.klass}.hip")) for src in ks.sources]
         functions = [self.dev.function(modules[s.module], s.name) for s in ks.steps]
         scratch = [self.dev.malloc(self._rounded(b)) for b in ks.scratch_bytes]
@@ -226,16 +224,8 @@ class HipBackend:
     def dispatch(self, exe: Executable, inputs: Sequence[int], outputs: Sequence[int], repeat: int = 1) -> None:
         ins = [self._get(s) for s in inputs]
         outs = [self._get(s) for s in outputs]
-        if isinstance(exe.source, Routine) and exe.data is not None:
-            self._dispatch_routine(exe, ins, outs)
-            return
         if isinstance(exe.source, Routine):
-            host_in = [self.dev.d2h(s["ptr"], 0, s["size"]) for s in ins]
-            host_out = [bytearray(s["size"]) for s in outs]
-            runCpuRoutine(exe.source, host_in, host_out)
-            for s, data in zip(outs, host_out):
-                if s["size"]:
-                    self.dev.h2d(s["ptr"], data)
+            self._dispatch_routine(exe, ins, outs)
             return
 
         kernel: Kernel = exe.source

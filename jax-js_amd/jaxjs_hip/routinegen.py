@@ -1,8 +1,13 @@
 """Native launch plans for routines (the non-fusable operations, src/routine.ts:20-102).
 
-Sort and Argsort along the last axis run on the GPU (template `sort.hip.inc`: keyed 64-bit words, bitonic
-network, LDS tiles + global passes).  Routines without a native plan return None here and take the host path
-the reference's Wasm backend takes for every routine (src/backend/wasm.ts:158-165, 216-220).
+Every routine runs on the GPU; there is no host path.  A combination without a plan (an element type the
+kernels do not cover, an extent beyond a kernel's stated limit) raises `UnsupportedRoutineError` at prepare
+time, which is what the Backend interface prescribes for a routine a backend lacks (src/backend.ts:236-240).
+
+  Sort, Argsort                               `sort.hip.inc`     32-bit and float16 keys
+  Scatter                                     `scatter.hip.inc`  float32/float16/int32/uint32/bool updates
+  TriangularSolve, Cholesky, LU, JacobiEigh   `linalg.hip.inc`   float32
+  Fft                                         `fft.hip.inc`      float32
 """
 
 from __future__ import annotations
@@ -11,7 +16,8 @@ from typing import Optional
 
 from .alu import DType, byteWidth
 from .kernelgen import KernelSource, LaunchStep, _prelude, fill, template
-from .routine import Routine, Routines
+from .errors import UnsupportedRoutineError
+from .routine import Routine, Routines, ScatterOp
 from .shape import prod
 
 _SORT_KINDS = {DType.Float32: (0, "float"), DType.Float16: (1, "jh_f16"), DType.Int32: (2, "int"),
@@ -26,10 +32,221 @@ def _next_pow2(n: int) -> int:
     return p
 
 
-def generateRoutine(routine: Routine, numerics: str = "wasm") -> Optional[KernelSource]:
-    if routine.name in (Routines.Sort, Routines.Argsort):
-        return _gen_sort(routine, numerics)
-    return None
+def generateRoutine(routine: Routine, numerics: str = "wasm") -> KernelSource:
+    gen = {Routines.Sort: _gen_sort, Routines.Argsort: _gen_sort, Routines.Scatter: _gen_scatter,
+           Routines.TriangularSolve: _gen_trisolve, Routines.Cholesky: _gen_cholesky, Routines.LU: _gen_lu,
+           Routines.JacobiEigh: _gen_jacobi, Routines.Fft: _gen_fft}.get(routine.name)
+    ks = gen(routine, numerics) if gen is not None else None
+    if ks is None:
+        raise UnsupportedRoutineError(routine.name, "hip")
+    return ks
+
+
+def _empty(klass: str, **info) -> KernelSource:
+    return KernelSource([], [], [], klass, {}, dict(info))
+
+
+def _round64(n: int, cap: int = 1024) -> int:
+    return max(64, min(cap, (n + 63) // 64 * 64))
+
+
+_LINALG_DEFAULTS = dict(ROUTINE=0, N=1, M=1, THREADS=64, UNIT=0, IN_LDS=0, MAX_SWEEPS=0, TOL="0.0")
+
+
+def _linalg_source(numerics: str, **params) -> str:
+    return _prelude(numerics) + fill(template("linalg.hip.inc"), {**_LINALG_DEFAULTS, **params})
+
+
+def _all_f32(t) -> bool:
+    return all(d == DType.Float32 for d in t.inputDtypes)
+
+
+def _gen_cholesky(routine: Routine, numerics: str) -> Optional[KernelSource]:
+    t = routine.type
+    shape = list(t.inputShapes[0])
+    if len(shape) < 2:
+        raise ValueError("cholesky: input must be at least 2D")
+    n, m = shape[-2], shape[-1]
+    if n != m:
+        raise ValueError(f"cholesky: input must be square, got [{n}, {m}]")
+    if not _all_f32(t) or n > 8192:
+        return None
+    batch = prod(shape[:-2])
+    if batch == 0 or n == 0:
+        return _empty("cholesky", n=n, batch=batch)
+    threads = _round64(n)
+    src = _linalg_source(numerics, ROUTINE=0, N=n, THREADS=threads)
+    steps = [LaunchStep("jh_cholesky", (batch, 1, 1), (threads, 1, 1), 0, [("in", 0), ("out", 0), ("scratch", 0)])]
+    return KernelSource([src], steps, [batch * n * n * 4], "cholesky", {0: batch * n * n * 4}, dict(n=n, batch=batch, threads=threads))
+
+
+def _gen_trisolve(routine: Routine, numerics: str) -> Optional[KernelSource]:
+    t = routine.type
+    a_shape, b_shape = list(t.inputShapes[0]), list(t.inputShapes[1])
+    if len(a_shape) < 2:
+        raise ValueError(f"triangular_solve: a must be at least 2D, got {a_shape}")
+    if len(b_shape) < 2:
+        raise ValueError(f"triangular_solve: b must be at least 2D, got {b_shape}")
+    n = a_shape[-2]
+    if n != a_shape[-1] or n != b_shape[-1]:
+        raise ValueError(f"triangular_solve: incompatible shapes a={a_shape}, b={b_shape}")
+    if not _all_f32(t):
+        return None
+    mats, m = prod(a_shape[:-2]), b_shape[-2]
+    if prod(b_shape[:-2]) != mats:
+        raise ValueError(f"triangular_solve: incompatible shapes a={a_shape}, b={b_shape}")
+    if mats == 0 or m == 0 or n == 0:
+        return _empty("trisolve", n=n, m=m, batch=mats)
+    threads = 64 if m <= 64 else 256
+    unit = 1 if (routine.params or {}).get("unitDiagonal", False) else 0
+    src = _linalg_source(numerics, ROUTINE=1, N=n, M=m, THREADS=threads, UNIT=unit)
+    blocks = mats * ((m + threads - 1) // threads)
+    steps = [LaunchStep("jh_trisolve", (blocks, 1, 1), (threads, 1, 1), 0, [("in", 0), ("in", 1), ("out", 0), ("scratch", 0)])]
+    need = {0: mats * n * n * 4, 1: mats * m * n * 4}
+    return KernelSource([src], steps, [mats * m * n * 4], "trisolve", need, dict(n=n, m=m, batch=mats, threads=threads))
+
+
+def _gen_lu(routine: Routine, numerics: str) -> Optional[KernelSource]:
+    t = routine.type
+    shape = list(t.inputShapes[0])
+    if len(shape) < 2:
+        raise ValueError("lu: input must be at least 2D")
+    m, n = shape[-2], shape[-1]
+    if not _all_f32(t) or m > 4096:  # the multipliers of one column live in LDS as doubles
+        return None
+    batch = prod(shape[:-2])
+    if batch == 0 or m == 0:
+        return _empty("lu", m=m, n=n, batch=batch)
+    threads = _round64(max(m, n))
+    src = _linalg_source(numerics, ROUTINE=2, N=n, M=m, THREADS=threads)
+    steps = [LaunchStep("jh_lu", (batch, 1, 1), (threads, 1, 1), 0, [("in", 0), ("out", 0), ("out", 1), ("out", 2)])]
+    return KernelSource([src], steps, [], "lu", {0: batch * m * n * 4}, dict(m=m, n=n, batch=batch, threads=threads))
+
+
+def _gen_jacobi(routine: Routine, numerics: str) -> Optional[KernelSource]:
+    t = routine.type
+    shape = list(t.inputShapes[0])
+    if len(shape) < 2:
+        raise ValueError("jacobi_eigh: input must be at least 2D")
+    n = shape[-1]
+    if n != shape[-2]:
+        raise ValueError(f"jacobi_eigh: input must be square, got {shape}")
+    if t.inputDtypes[0] not in (DType.Float32, DType.Float16, DType.Float64):
+        raise TypeError("jacobi_eigh: input must be floating-point")
+    if not _all_f32(t) or n > 16384:
+        return None
+    batch = prod(shape[:-2])
+    if batch == 0 or n == 0:
+        return _empty("jacobi", n=n, batch=batch)
+    params = routine.params or {}
+    threads = _round64(n)
+    in_lds = 1 if 2 * n * n * 4 <= 60 * 1024 else 0
+    src = _linalg_source(numerics, ROUTINE=3, N=n, THREADS=threads, IN_LDS=in_lds, MAX_SWEEPS=int(params["maxSweeps"]),
+                         TOL=repr(float(params["tolerance"])))
+    steps = [LaunchStep("jh_jacobi", (batch, 1, 1), (threads, 1, 1), 0, [("in", 0), ("out", 0), ("out", 1)])]
+    return KernelSource([src], steps, [], "jacobi", {0: batch * n * n * 4}, dict(n=n, batch=batch, threads=threads, in_lds=bool(in_lds)))
+
+
+def _gen_fft(routine: Routine, numerics: str) -> Optional[KernelSource]:
+    t = routine.type
+    shape = list(t.inputShapes[0])
+    if len(shape) < 1:
+        raise ValueError("fft: input must be at least 1D")
+    n = shape[-1]
+    if n < 1:
+        raise ValueError(f"fft: final axis must be non-empty, got {n}")
+    if t.inputDtypes[0] != t.inputDtypes[1] or t.inputDtypes[0] not in (DType.Float32, DType.Float16, DType.Float64):
+        raise ValueError("fft: expected matching floating-point real/imag arrays")
+    params = routine.params or {}
+    factors = [int(f) for f in params["factors"]]
+    if prod(factors) != n or any(f < 1 for f in factors):
+        raise ValueError(f"fft: factors {factors} do not multiply to the axis length {n}")
+    if not _all_f32(t) or n >= (1 << 30):
+        return None
+    rows = prod(shape[:-1])
+    if rows == 0:
+        return _empty("fft", n=n, rows=rows)
+    src = _prelude(numerics) + fill(template("fft.hip.inc"), dict(N=n, ROWS=rows, INVERSE=1 if params.get("inverse") else 0,
+                                                                  NF=len(factors), FACTORS=", ".join(map(str, factors)) or "1"))
+    blocks = max(1, min((rows * n + 255) // 256, 1 << 20))
+    S = len(factors)
+    out_pair, tmp_pair = [("out", 0), ("out", 1)], [("scratch", 0), ("scratch", 1)]
+    target = lambda s: out_pair if (S - 1 - s) % 2 == 0 else tmp_pair  # noqa: E731  (stage -1 is the permutation)
+    steps = [LaunchStep("jh_fft_permute", (blocks, 1, 1), (256, 1, 1), 0, [("in", 0), ("in", 1)] + target(-1))]
+    prev = 1
+    for s, radix in enumerate(factors):
+        steps.append(LaunchStep("jh_fft_stage", (blocks, 1, 1), (256, 1, 1), 0,
+                                target(s - 1) + target(s) + [("const", prev), ("const", radix), ("const", 1 if s == S - 1 else 0)]))
+        prev *= radix
+    scratch = [rows * n * 4, rows * n * 4] if S >= 1 else [8, 8]
+    need = {0: rows * n * 4, 1: rows * n * 4}
+    return KernelSource([src], steps, scratch, "fft", need, dict(n=n, rows=rows, factors=factors, launches=len(steps)))
+
+
+_SCATTER_KINDS = {DType.Float32: (0, "float"), DType.Float16: (1, "jh_f16"), DType.Int32: (2, "int"), DType.Uint32: (3, "jh_u32"),
+                  DType.Bool: (4, "int")}
+
+
+def _gen_scatter(routine: Routine, numerics: str) -> Optional[KernelSource]:
+    """Index arithmetic of src/routine.ts:226-296, unrolled over the output axes at generation time."""
+    t = routine.type
+    params = routine.params or {}
+    op = ScatterOp(getattr(params["op"], "value", params["op"]))
+    out_shape, axes, out_dim = [int(x) for x in params["shape"]], [int(x) for x in params["axis"]], int(params["outDim"])
+    unique = bool(params.get("uniqueIndices", False))
+    ushape = list(t.inputShapes[0])
+    index_shapes = [list(s) for s in t.inputShapes[1:]]
+    dtype = t.inputDtypes[0]
+    if dtype not in _SCATTER_KINDS or any(d not in (DType.Int32, DType.Uint32) for d in t.inputDtypes[1:]):
+        return None
+    if len(axes) != len(index_shapes):
+        raise ValueError(f"scatter: {len(axes)} indexed axes but {len(index_shapes)} index arrays")
+    U, OUT = prod(ushape), prod(out_shape)
+    if U >= (1 << 31) or OUT >= (1 << 31):
+        return None
+    if OUT == 0:
+        return _empty("scatter", updates=U, out=OUT)
+    index_rank = max((len(s) for s in index_shapes), default=0)
+    ustrides = [prod(ushape[d + 1:]) for d in range(len(ushape))]
+    ostrides = [prod(out_shape[d + 1:]) for d in range(len(out_shape))]
+    free_dims = [d for d in range(len(ushape)) if d < out_dim or d >= out_dim + index_rank]
+    if len(free_dims) != len(out_shape) - len(axes):
+        raise ValueError(f"scatter: updates of shape {ushape} do not match output {out_shape} indexed on {axes}")
+    coord = lambda d: f"((i / {ustrides[d]}ll) % {ushape[d]}ll)"  # noqa: E731
+    lines, free_i = [], 0
+    for axis, extent in enumerate(out_shape):
+        if axis in axes:
+            k = axes.index(axis)
+            ishape = index_shapes[k]
+            istrides = [prod(ishape[j + 1:]) for j in range(len(ishape))]
+            first = out_dim + index_rank - len(ishape)
+            terms = [f"{coord(first + j)} * {istrides[j]}ll" for j in range(len(ishape)) if ishape[j] != 1]
+            cast = "(jh_i64)" if t.inputDtypes[1 + k] == DType.Int32 else "(jh_i64)(jh_u32)"
+            lines.append(f"  c = {cast}idx{k}[{' + '.join(terms) or '0'}];")
+        else:
+            lines.append(f"  c = {coord(free_dims[free_i])};")
+            free_i += 1
+        lines.append(f"  if (c < 0 || c >= {extent}ll) return -1;")
+        lines.append(f"  o += c * {ostrides[axis]}ll;")
+    accumulate = op != ScatterOp.Update and not unique
+    mode = 2 if accumulate else (0 if unique else 1)
+    kind, ctype = _SCATTER_KINDS[dtype]
+    nidx = len(index_shapes)
+    src = _prelude(numerics) + fill(template("scatter.hip.inc"), dict(
+        U=U, OUT=OUT, MODE=mode, KIND=kind, T=ctype, DEST_CODE="\n".join(lines),
+        INDEX_PARAMS="".join(f", const int* __restrict__ idx{k}" for k in range(nidx)),
+        INDEX_ARGS="".join(f", idx{k}" for k in range(nidx))))
+    idx_args = [("in", 1 + k) for k in range(nidx)]
+    grid = lambda count: (max(1, min((count + 255) // 256, 1 << 20)), 1, 1)  # noqa: E731
+    steps = [LaunchStep("jh_scatter_fill", grid(OUT), (256, 1, 1), 0, [("out", 0), ("scratch", 0)])]
+    if U > 0:
+        if mode == 1:
+            steps.append(LaunchStep("jh_scatter_claim", grid(U), (256, 1, 1), 0, [("scratch", 0)] + idx_args))
+        steps.append(LaunchStep("jh_scatter_apply", grid(U), (256, 1, 1), 0, [("in", 0), ("out", 0), ("scratch", 0)] + idx_args))
+    need = {0: U * byteWidth(dtype)}
+    for k, ishape in enumerate(index_shapes):
+        need[1 + k] = prod(ishape) * 4
+    return KernelSource([src], steps, [OUT * 4 if mode == 1 else 8], "scatter", need, dict(updates=U, out=OUT, mode=mode, launches=len(steps)))
 
 
 def _gen_sort(routine: Routine, numerics: str) -> Optional[KernelSource]:
@@ -38,7 +255,7 @@ def _gen_sort(routine: Routine, numerics: str) -> Optional[KernelSource]:
     if len(shape) == 0:
         raise ValueError(f"{routine.name.value.lower()}: cannot sort a scalar")
     if dtype not in _SORT_KINDS:
-        return None  # float64 keys do not fit the 32-bit key: host path
+        return None  # float64 keys do not fit the 32-bit key
     n = shape[-1]
     rows = prod(shape[:-1])
     argsort = routine.name == Routines.Argsort

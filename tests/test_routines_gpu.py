@@ -1,12 +1,14 @@
 """Native Sort / Argsort routines on the GPU against the reference's tables (test/numpy.test.ts:4631-4800) and
-against the host restatement of src/routine.ts:185-213 (`runCpuRoutine`) on random data."""
+against the CPU checker's restatement of src/routine.ts:185-213 on random data."""
 import numpy as np
 import pytest
 
 from gpu_util import WARM_ONLY, backend
 from jaxjs_hip import DType
 from jaxjs_hip.alu import numpyDtype
-from jaxjs_hip.routine import Routine, Routines, RoutineType, runCpuRoutine
+from jaxjs_hip.errors import UnsupportedRoutineError
+from jaxjs_hip.routine import Routine, Routines, RoutineType
+from oracle.routines import runCpuRoutine
 
 pytestmark = pytest.mark.gpu
 RNG = np.random.default_rng(21)
@@ -30,7 +32,6 @@ def run(name, x, dtype):
         pytest.skip("warm-up run: compiled only")
     be = backend()
     exe = be.prepareRoutineSync(routine)
-    assert exe.data is not None, "expected the native plan, not the host path"
     src = be.malloc(x.nbytes, x.tobytes())
     outs = [be.malloc(x.size * 4 if i == 1 else x.nbytes) for i in range(len(routine.type.outputShapes))]
     be.dispatch(exe, [src], outs)
@@ -130,13 +131,6 @@ def test_zero_sized_rows_and_unsupported_dtype_path():
     assert be.readSync(b) == b""
     be.decRef(a)
     be.decRef(b)
-    # float64 keeps the host path (64-bit keys): same results, different route.
-    x = RNG.normal(0, 1, (4, 50))
-    routine = make(Routines.Sort, x.shape, DType.Float64)
-    exe = be.prepareRoutineSync(routine)
-    assert exe.data is None
-    s, o = be.malloc(x.nbytes, x.tobytes()), be.malloc(x.nbytes)
-    be.dispatch(exe, [s], [o])
-    np.testing.assert_array_equal(np.frombuffer(be.readSync(o), np.float64).reshape(x.shape), np.sort(x, -1))
-    be.decRef(s)
-    be.decRef(o)
+    # float64 keys do not fit the 64-bit key|position words: refused at prepare time, never run on the host.
+    with pytest.raises(UnsupportedRoutineError):
+        be.prepareRoutineSync(make(Routines.Sort, (4, 50), DType.Float64))
