@@ -119,6 +119,8 @@ REDUCE_PRIMITIVES = ("Reduce", "Dot", "Conv")
 UNARY_FUSABLE = ("Neg", "Reciprocal", "Floor", "Ceil", "StopGradient", "Cast", "Bitcast", "Sin", "Cos", "Asin", "Atan",
                  "Exp", "Log", "Erf", "Erfc", "Sqrt")
 BINARY_FUSABLE = ("Add", "Mul", "Idiv", "Mod", "Min", "Max", "BitCombine", "BitShift")
+# Primitives handed to the backend as a unit (src/frontend/core.ts:154-163): primitive name == routine name.
+ROUTINE_PRIMITIVES = ("Sort", "Argsort", "Scatter", "TriangularSolve", "Cholesky", "LU", "JacobiEigh", "Fft")
 
 
 @dataclass
@@ -357,6 +359,60 @@ def _out_aval(prim: str, avals: List[ShapedArray], params: Dict[str, Any]) -> Sh
     raise NotImplementedError(f"jit: primitive {prim}")
 
 
+def _routine_out_avals(prim: str, avals: List[ShapedArray], params: Dict[str, Any]) -> List[ShapedArray]:
+    """Output types of the routine primitives (src/frontend/jaxpr.ts:976-1062)."""
+    a = avals[0]
+    same = ShapedArray(tuple(a.shape), a.dtype, a.weak)
+    if prim in ("Sort", "Argsort"):
+        if a.ndim == 0:
+            raise TypeError(f"{prim.lower()}: requires at least 1D input")
+        return [same] if prim == "Sort" else [same, ShapedArray(tuple(a.shape), DType.Int32, False)]
+    if prim == "Scatter":
+        return [ShapedArray(tuple(params["shape"]), a.dtype, a.weak)]
+    if prim == "TriangularSolve":
+        b = avals[1]
+        if a.ndim < 2 or b.ndim < 2:
+            raise TypeError("triangular_solve: operands must be at least 2D")
+        if (tuple(a.shape[:-2]) != tuple(b.shape[:-2]) or a.dtype != b.dtype or a.shape[-2] != a.shape[-1]
+                or a.shape[-1] != b.shape[-1]):
+            raise TypeError(f"triangular_solve: mismatch {a.shape} vs {b.shape}")
+        return [ShapedArray(tuple(b.shape), b.dtype, a.weak and b.weak)]
+    if prim in ("Cholesky", "JacobiEigh"):
+        if a.ndim < 2 or a.shape[-2] != a.shape[-1]:
+            raise TypeError(f"{prim.lower()}: requires a batch of square matrices, got {a.shape}")
+        if prim == "Cholesky":
+            return [same]
+        if a.dtype not in (DType.Float16, DType.Float32, DType.Float64):
+            raise TypeError("jacobi_eigh: requires floating-point input")
+        return [same, same]
+    if prim == "LU":
+        if a.ndim < 2:
+            raise TypeError("lu: requires at least 2D input")
+        batch, (m, n) = tuple(a.shape[:-2]), a.shape[-2:]
+        return [same, ShapedArray(batch + (min(m, n),), DType.Int32, False), ShapedArray(batch + (m,), DType.Int32, False)]
+    if prim == "Fft":
+        b = avals[1]
+        if tuple(a.shape) != tuple(b.shape) or a.dtype != b.dtype:
+            raise TypeError("fft: real and imag arrays must match")
+        if a.ndim < 1 or a.dtype not in (DType.Float16, DType.Float32, DType.Float64):
+            raise TypeError("fft: requires floating-point input of at least 1D")
+        if prod(list(params["factors"])) != a.shape[-1]:
+            raise TypeError(f"fft: factorization {params['factors']} does not match size {a.shape[-1]}")
+        return [same, same]
+    raise NotImplementedError(prim)
+
+
+def bind(prim: str, args: Sequence[TracerValue], params: Optional[Dict[str, Any]] = None) -> List[Tracer]:
+    """Multi-output primitive application; the routine primitives go through here."""
+    if not _builders:
+        raise RuntimeError("bind outside of a trace")
+    ts = [_raise(a) for a in args]
+    params = dict(params or {})
+    outs = [Var(av) for av in _routine_out_avals(prim, [t.aval for t in ts], params)]
+    _builders[-1].eqns.append(JaxprEqn(prim, [t.atom for t in ts], params, outs))
+    return [Tracer(o) for o in outs]
+
+
 def bind1(prim: str, args: Sequence[TracerValue], params: Optional[Dict[str, Any]] = None) -> Tracer:
     if not _builders:
         raise RuntimeError("bind1 outside of a trace")
@@ -425,6 +481,49 @@ def broadcast(x, shape, axis):
 def shrink(x, slices):
     """`x.slice(...)`: keep `[start, end)` per axis."""
     return bind1("Shrink", [x], dict(slice=[tuple(s) for s in slices]))
+
+
+def flip(x, axis):
+    x = _raise(x)
+    return bind1("Flip", [x], dict(axis=_normalize_axis(axis, x.ndim)))
+
+
+def sort(x):
+    return bind("Sort", [x])[0]
+
+
+def argsort(x):
+    """Returns (sorted values, int32 indices) along the last axis (src/frontend/core.ts:600-605)."""
+    return tuple(bind("Argsort", [x]))
+
+
+def scatter(updates, indices, params):
+    return bind("Scatter", [updates] + list(indices), params)[0]
+
+
+def triangularSolve(a, b, lower: bool = False, unitDiagonal: bool = False):
+    """Solves `a @ x.T = b.T`; a lower-triangular system is flipped into the upper-triangular form the routine
+    takes (src/frontend/core.ts:530-555)."""
+    if lower:
+        a, b = flip(a, [-2, -1]), flip(b, [-1])
+    x = bind("TriangularSolve", [a, b], dict(unitDiagonal=bool(unitDiagonal)))[0]
+    return flip(x, [-1]) if lower else x
+
+
+def cholesky(x):
+    return bind("Cholesky", [x])[0]
+
+
+def lu(x):
+    return tuple(bind("LU", [x]))
+
+
+def jacobiEigh(x, maxSweeps: int, tolerance: float):
+    return tuple(bind("JacobiEigh", [x], dict(maxSweeps=int(maxSweeps), tolerance=float(tolerance))))
+
+
+def fft(real, imag, factors, inverse: bool):
+    return tuple(bind("Fft", [real, imag], dict(factors=[int(f) for f in factors], inverse=bool(inverse))))
 
 
 def reduce(x, op: AluOp, axis=None, keepdims=False):
@@ -680,6 +779,16 @@ def splitGraphDataflow(jaxpr: Jaxpr, maxArgs: int) -> Set[Var]:
                 if isinstance(x, Var):
                     markNonViewProducer(x)
 
+    # A routine reads whole buffers: each operand must be dispatched before it.  The reference marks the operand's
+    # non-view producer (src/frontend/jit.ts:990-999) and then refuses an operand that is still a view of it
+    # ("routine primitive input is not imm", jit.ts:307-311, e.g. the flips of a lower-triangular solve); here the
+    # operand itself is materialised, so such a view is realised by a copy kernel instead of failing.
+    for eqn in jaxpr.eqns:
+        if eqn.primitive in ROUTINE_PRIMITIVES:
+            for x in eqn.inputs:
+                if isinstance(x, Var) and x in varToDefn:
+                    materialized.add(x)
+
     # Backwards: a node is black when it is an output, a reduction endpoint, materialised, or when two
     # different black nodes are reachable from it through non-black nodes.
     black: Set[Var] = set()
@@ -690,7 +799,7 @@ def splitGraphDataflow(jaxpr: Jaxpr, maxArgs: int) -> Set[Var]:
             nextBlack[v] = v
     for i in range(len(jaxpr.eqns) - 1, -1, -1):
         eqn = jaxpr.eqns[i]
-        if (i in endpointEqns or any(v in materialized for v in eqn.outBinders)
+        if (i in endpointEqns or eqn.primitive in ROUTINE_PRIMITIVES or any(v in materialized for v in eqn.outBinders)
                 or any(v in black for v in eqn.outBinders)):
             for v in eqn.outBinders:
                 black.add(v)
@@ -752,10 +861,12 @@ def splitGraphDataflow(jaxpr: Jaxpr, maxArgs: int) -> Set[Var]:
 @dataclass
 class JitStep:
     kind: str                      # "malloc" | "execute" | "free"
-    kernel: Optional[Kernel] = None
+    kernel: Optional[Kernel] = None    # an "execute" step runs either a Kernel (one output) ...
     inputs: List[int] = field(default_factory=list)
     output: int = -1
     size: int = 0
+    routine: Any = None                # ... or a Routine with `outputs`
+    outputs: List[int] = field(default_factory=list)
 
 
 @dataclass
@@ -767,7 +878,11 @@ class JitProgram:
 
     @property
     def kernels(self) -> List[Kernel]:
-        return [s.kernel for s in self.steps if s.kind == "execute"]
+        return [s.kernel for s in self.steps if s.kind == "execute" and s.kernel is not None]
+
+    @property
+    def routines(self) -> List[Any]:
+        return [s.routine for s in self.steps if s.kind == "execute" and s.routine is not None]
 
     def execute(self, backend, inputs: Sequence[int], prepared: Optional[Dict[int, Any]] = None) -> List[int]:
         """Run on `backend` with input slots (closed-over constants first).  Returns output slots owned
@@ -778,6 +893,9 @@ class JitProgram:
         for k, step in enumerate(self.steps):
             if step.kind == "malloc":
                 scope[step.output] = backend.malloc(step.size)
+            elif step.kind == "execute" and step.routine is not None:
+                exe = prepared[k] if prepared is not None else backend.prepareRoutineSync(step.routine)
+                backend.dispatch(exe, [scope[i] for i in step.inputs], [scope[o] for o in step.outputs])
             elif step.kind == "execute":
                 exe = prepared[k] if prepared is not None else backend.prepareKernelSync(step.kernel)
                 backend.dispatch(exe, [scope[i] for i in step.inputs], [scope[step.output]])
@@ -791,7 +909,8 @@ class JitProgram:
         return outs
 
     def prepare(self, backend) -> Dict[int, Any]:
-        return {k: backend.prepareKernelSync(s.kernel) for k, s in enumerate(self.steps) if s.kind == "execute"}
+        return {k: (backend.prepareRoutineSync(s.routine) if s.routine is not None else backend.prepareKernelSync(s.kernel))
+                for k, s in enumerate(self.steps) if s.kind == "execute"}
 
 
 def jitCompile(jaxpr: Jaxpr, consts: Sequence[ConstArray] = (), maxArgs: int = 64) -> JitProgram:
@@ -803,6 +922,30 @@ def jitCompile(jaxpr: Jaxpr, consts: Sequence[ConstArray] = (), maxArgs: int = 6
     # ctx values: ("imm", id) | ("exp", exp, args) | ("red", exp, reduction, args)
     ctx: Dict[Var, tuple] = {v: ("imm", i) for i, v in enumerate(jaxpr.inBinders)}
     for eqn in jaxpr.eqns:
+        if eqn.primitive in ROUTINE_PRIMITIVES:  # src/frontend/jit.ts:290-327
+            from .alu import byteWidth
+            from .routine import Routine, Routines, RoutineType
+
+            rtype = RoutineType([list(x.aval.shape) for x in eqn.inputs], [x.aval.dtype for x in eqn.inputs],
+                                [list(v.aval.shape) for v in eqn.outBinders], [v.aval.dtype for v in eqn.outBinders])
+            r_inputs: List[int] = []
+            for x in eqn.inputs:
+                if not isinstance(x, Var):
+                    raise NotImplementedError(f"jit: literal operand of routine {eqn.primitive}")
+                jv = ctx[x]
+                if jv[0] != "imm":
+                    raise RuntimeError(f"jit: routine primitive {eqn.primitive} input is not imm")
+                r_inputs.append(jv[1])
+            r_outputs: List[int] = []
+            for v in eqn.outBinders:
+                out_id = next_id[0]
+                next_id[0] += 1
+                steps.append(JitStep("malloc", output=out_id, size=v.aval.size * byteWidth(v.aval.dtype)))
+                r_outputs.append(out_id)
+                ctx[v] = ("imm", out_id)
+            steps.append(JitStep("execute", routine=Routine(Routines(eqn.primitive), rtype, dict(eqn.params) or None),
+                                 inputs=r_inputs, outputs=r_outputs))
+            continue
         rule = JIT_RULES.get(eqn.primitive)
         if rule is None:
             raise NotImplementedError(f"JIT not implemented for primitive {eqn.primitive}")
@@ -870,16 +1013,18 @@ def jitCompile(jaxpr: Jaxpr, consts: Sequence[ConstArray] = (), maxArgs: int = 6
 
     # Free every intermediate after its last use (JitProgramBuilder.insertFreeSteps).
     last_use: Dict[int, int] = {}
+    written = lambda s: s.outputs if s.routine is not None else [s.output]  # noqa: E731
     for k, s in enumerate(steps):
         if s.kind == "execute":
             for i in s.inputs:
                 last_use[i] = k
-            last_use.setdefault(s.output, k)
+            for o in written(s):
+                last_use.setdefault(o, k)
     final: List[JitStep] = []
     for k, s in enumerate(steps):
         final.append(s)
         if s.kind == "execute":
-            for i in dict.fromkeys(s.inputs + [s.output]):
+            for i in dict.fromkeys(s.inputs + written(s)):
                 if i >= nargs and i not in outputs and last_use.get(i) == k:
                     final.append(JitStep("free", output=i))
     return JitProgram(final, nargs, outputs, list(consts))

@@ -8,6 +8,9 @@ the backend is handed, so it is kept literally:
   arange / tri (lazy constants)                       src/frontend/array.ts:1570-1627
   argmax                                              src/library/numpy.ts:533-556
   dotProductAttention                                 src/library/nn.ts:478-583
+  sort / argsort along an axis                        src/frontend/core.ts:1043-1075
+  linalg: cholesky, triangularSolve, solve            src/library/lax-linalg.ts:35-50, 212-244; numpy-linalg.ts:274-318
+  eigh (unsorted), fft along an axis                  src/library/lax-linalg.ts:52-100; numpy-fft.ts:50-66, 126-157
 """
 
 from __future__ import annotations
@@ -176,3 +179,106 @@ def dotProductAttention(query: Tracer, key: Tracer, value: Tracer, isCausal: boo
         scores = J.where(tri_const(L, S, 0), scores, -math.inf)
     attn = softmax(scores, -1)
     return einsum("BNLS,BSNH->BLNH", attn, value)
+
+
+def _axis_to_last(ndim: int, axis: int):
+    axis = axis + ndim if axis < 0 else axis
+    perm = [d for d in range(ndim) if d != axis] + [axis]
+    inv = [perm.index(d) for d in range(ndim)]
+    return axis, perm, inv
+
+
+def sort(a: Tracer, axis: int = -1):
+    """Sort along `axis`: the routine sorts the last axis, other axes are moved there and back."""
+    axis, perm, inv = _axis_to_last(a.ndim, axis)
+    if a.shape[axis] <= 1:
+        return a
+    if axis == a.ndim - 1:
+        return J.sort(a)
+    return J.sort(a.transpose(perm)).transpose(inv)
+
+
+def argsort(a: Tracer, axis: int = -1):
+    axis, perm, inv = _axis_to_last(a.ndim, axis)
+    if axis == a.ndim - 1:
+        return J.argsort(a)[1]
+    return J.argsort(a.transpose(perm))[1].transpose(inv)
+
+
+def _swap_last_two(x: Tracer):
+    return x.transpose(list(range(x.ndim - 2)) + [x.ndim - 1, x.ndim - 2])
+
+
+def cholesky(a: Tracer, upper: bool = False):
+    L = J.cholesky(a)
+    return _swap_last_two(L) if upper else L
+
+
+def triangularSolve(a: Tracer, b: Tracer, leftSide: bool = False, lower: bool = False, transposeA: bool = False,
+                    unitDiagonal: bool = False):
+    """`a @ x = b` (leftSide) or `x @ a = b`: reduced to the primitive's `a @ x.T = b.T` by transposes."""
+    if not leftSide:
+        transposeA = not transposeA
+    else:
+        b = _swap_last_two(b)
+    if transposeA:
+        a = _swap_last_two(a)
+        lower = not lower
+    x = J.triangularSolve(a, b, lower=lower, unitDiagonal=unitDiagonal)
+    return _swap_last_two(x) if leftSide else x
+
+
+def solve(a: Tracer, b: Tracer):
+    """`numpy.linalg.solve` for equal batch dimensions: LU with partial pivoting, the permutation applied as a 0/1
+    matrix product, then a unit-lower and an upper triangular solve."""
+    n = a.shape[-1]
+    if a.ndim < 2 or a.shape[-2] != n:
+        raise ValueError(f"solve: a must be a batch of square matrices, got {a.shape}")
+    b_is_1d = b.ndim == 1
+    if b_is_1d:
+        b = b.reshape(list(b.shape) + [1])
+    if b.shape[-2] != n or tuple(a.shape[:-2]) != tuple(b.shape[:-2]):
+        raise ValueError(f"solve: leading dimension of b must match size of a, got a={a.shape}, b={b.shape}")
+    lu, _pivots, permutation = J.lu(a)
+    P = J.equal(arange_const(0, n), permutation.reshape(list(permutation.shape) + [1])).astype(b.dtype)
+    LPb = triangularSolve(lu, matmul(P, b), leftSide=True, lower=True, unitDiagonal=True)
+    x = triangularSolve(lu, LPb, leftSide=True, lower=False)
+    return x.reshape(list(x.shape[:-1])) if b_is_1d else x
+
+
+def eigh_unsorted(x: Tracer, symmetrizeInput: bool = True):
+    """Eigenvectors (columns) and the diagonalised matrix, without the final sort by eigenvalue (which is a
+    gather in the reference); sweep count and tolerance as in the reference's wrapper."""
+    n = x.shape[-1]
+    if symmetrizeInput:
+        x = x.add(_swap_last_two(x)).mul(0.5)
+    d, v = J.jacobiEigh(x, maxSweeps=max(8, 2 * n), tolerance=1e-6)
+    return v, d
+
+
+def factorFftSize(n: int) -> List[int]:
+    factors: List[int] = []
+    for radix in (4, 2, 3, 5, 7):
+        while n % radix == 0:
+            factors.append(radix)
+            n //= radix
+    radix = 11
+    while radix * radix <= n:
+        while n % radix == 0:
+            factors.append(radix)
+            n //= radix
+        radix += 2
+    if n > 1:
+        factors.append(n)
+    return factors
+
+
+def fft(real: Tracer, imag: Tracer, axis: int = -1, inverse: bool = False):
+    axis, perm, inv = _axis_to_last(real.ndim, axis)
+    n = real.shape[axis]
+    if axis != real.ndim - 1:
+        real, imag = real.transpose(perm), imag.transpose(perm)
+    re, im = J.fft(real, imag, factorFftSize(n), inverse)
+    if axis != real.ndim - 1:
+        re, im = re.transpose(inv), im.transpose(inv)
+    return re, im

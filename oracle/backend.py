@@ -13,6 +13,7 @@ from typing import Dict, List, Optional, Sequence
 import numpy as np
 
 from . import oracle
+from . import routines as routine_oracle
 
 
 class OracleBackend:
@@ -50,7 +51,13 @@ class OracleBackend:
     def prepareKernelSync(self, kernel):
         return kernel
 
+    def prepareRoutineSync(self, routine):
+        return routine
+
     def dispatch(self, exe, inputs: Sequence[int], outputs: Sequence[int]) -> None:
+        if hasattr(exe, "type") and hasattr(exe, "name"):  # a Routine
+            routine_oracle.runCpuRoutine(exe, [bytes(self._slots[s][0]) for s in inputs], [self._slots[s][0] for s in outputs])
+            return
         kernel = exe
         out = oracle.run_kernel(kernel, [bytes(self._slots[s][0]) for s in inputs], self.mode)
         raw = np.ascontiguousarray(out).tobytes()

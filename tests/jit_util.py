@@ -16,10 +16,15 @@ def run_program(backend, prog, arrays, out_dtypes_shapes=None):
     in_slots = [backend.malloc(np.ascontiguousarray(a).nbytes, np.ascontiguousarray(a).tobytes()) for a in arrays]
     outs = prog.execute(backend, const_slots + in_slots)
     results = []
-    out_kernels = {s.output: s.kernel for s in prog.steps if s.kind == "execute"}
+    out_dtypes = {}
+    for s in prog.steps:
+        if s.kind == "execute" and s.routine is not None:
+            out_dtypes.update(zip(s.outputs, s.routine.type.outputDtypes))
+        elif s.kind == "execute":
+            out_dtypes[s.output] = s.kernel.dtype
     for slot, oid in zip(outs, prog.outputs):
         raw = backend.readSync(slot)
-        results.append(np.frombuffer(raw, dtype=numpyDtype(out_kernels[oid].dtype)).copy())
+        results.append(np.frombuffer(raw, dtype=numpyDtype(out_dtypes[oid])).copy())
     for s in const_slots + in_slots + outs:
         backend.decRef(s)
     return results

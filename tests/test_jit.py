@@ -240,3 +240,68 @@ def test_gpt2_block_program_structure_and_values_f32():
     (y,) = run_program(OracleBackend(), prog, [arrs[n] for n in order])
     want = block_reference(arrs["x"].astype(np.float64), {n: arrs[n].astype(np.float64) for n in order[1:]}, heads)
     np.testing.assert_allclose(y.reshape(batch, seq, d), want, rtol=2e-4, atol=2e-5)
+
+
+# ---- routine primitives inside traced programs (src/frontend/jit.ts:290-327, 990-1008) -----------------------------
+
+def steps_of(prog):
+    return [(s.routine.name.value if s.routine is not None else "kernel") for s in prog.steps if s.kind == "execute"]
+
+
+def test_routine_outputs_and_operands_are_dispatch_boundaries():
+    x = np.random.default_rng(0).standard_normal((6, 4)).astype(np.float32)
+    # exp feeds the routine: it must be its own kernel; the routine's output feeds a fused map
+    prog, (y,) = run(lambda a: J.sort(J.exp(a)).mul(2.0), x)
+    assert steps_of(prog) == ["kernel", "Sort", "kernel"]
+    np.testing.assert_allclose(y.reshape(6, 4), np.sort(np.exp(x), -1) * 2, rtol=1e-6)
+    # sort along axis 0: the transposed operand is realised by a copy kernel, the result is transposed back lazily
+    prog, (s0, a0) = run(lambda a: (L.sort(a, 0), L.argsort(a, 0)), x)
+    assert steps_of(prog).count("Sort") == 1 and steps_of(prog).count("Argsort") == 1
+    np.testing.assert_array_equal(s0.reshape(6, 4), np.sort(x, 0))
+    np.testing.assert_array_equal(a0.reshape(6, 4), np.argsort(x, 0, kind="stable"))
+    assert prog.routines[0].type.inputShapes == [[4, 6]]
+
+
+def test_solve_is_lu_plus_two_triangular_solves():
+    rng = np.random.default_rng(1)
+    a = (rng.standard_normal((3, 8, 8)) + 4 * np.eye(8)).astype(np.float32)
+    b = rng.standard_normal((3, 8, 2)).astype(np.float32)
+    prog, (x,) = run(lambda a, b: L.solve(a, b), a, b)
+    assert [n for n in steps_of(prog) if n != "kernel"] == ["LU", "TriangularSolve", "TriangularSolve"]
+    assert [r.params for r in prog.routines] == [None, {"unitDiagonal": True}, {"unitDiagonal": False}]
+    np.testing.assert_allclose(x.reshape(3, 8, 2), np.linalg.solve(a.astype(np.float64), b), rtol=1e-4, atol=1e-5)
+    v = rng.standard_normal((8,)).astype(np.float32)
+    _, (x1,) = run(lambda a, b: L.solve(a, b), a[0], v)
+    np.testing.assert_allclose(x1, np.linalg.solve(a[0].astype(np.float64), v), rtol=1e-4, atol=1e-5)
+
+
+def test_triangular_solve_variants_match_the_reference_tables():  # test/lax-linalg.test.ts:332-436
+    Lm, b = f32([[2, 0], [1, 3]]), f32([[4], [7]])
+    _, (x,) = run(lambda a, b: L.triangularSolve(a, b, leftSide=True, lower=True), Lm, b)
+    np.testing.assert_allclose(x, [2, 5 / 3], rtol=1e-6)
+    _, (x,) = run(lambda a, b: L.triangularSolve(a, b, leftSide=True, lower=True, transposeA=True), f32([[1, 1e6], [1, 1]]), f32([[1], [1]]))
+    np.testing.assert_allclose(x, [0, 1], atol=1e-6)
+    _, (x,) = run(lambda a, b: L.triangularSolve(a, b), f32([[2, 1], [0, 3]]), f32([[4, 7]]))
+    np.testing.assert_allclose(x, [2, 5 / 3], rtol=1e-6)
+
+
+def test_cholesky_upper_eigh_and_fft_along_an_axis():
+    rng = np.random.default_rng(2)
+    x = f32([[2, 1], [1, 2]])
+    _, (lo, up) = run(lambda a: (L.cholesky(a), L.cholesky(a, upper=True)), x)
+    np.testing.assert_allclose(lo.reshape(2, 2), [[1.4142135, 0], [0.70710677, 1.2247449]], rtol=1e-6)  # lax-linalg.ts:27-32
+    np.testing.assert_allclose(up.reshape(2, 2), lo.reshape(2, 2).T)
+    a = rng.standard_normal((2, 6, 6)).astype(np.float32)
+    prog, (v, d) = run(lambda a: L.eigh_unsorted(a), a)
+    assert prog.routines[0].params == {"maxSweeps": 12, "tolerance": 1e-6}
+    sym = (a + a.transpose(0, 2, 1)) * 0.5
+    v, d = v.reshape(2, 6, 6), d.reshape(2, 6, 6)
+    for k in range(2):
+        np.testing.assert_allclose((v[k] * np.diagonal(d[k])) @ v[k].T, sym[k], atol=1e-5)
+    re, im = rng.standard_normal((12, 5)).astype(np.float32), rng.standard_normal((12, 5)).astype(np.float32)
+    prog, (r, i) = run(lambda r, i: L.fft(r, i, 0), re, im)
+    assert prog.routines[0].params == {"factors": [4, 3], "inverse": False} and prog.routines[0].type.inputShapes == [[5, 12]] * 2
+    np.testing.assert_allclose((r + 1j * i).reshape(12, 5), np.fft.fft(re + 1j * im, axis=0), atol=1e-5)
+    _, (r2, i2) = run(lambda r, i: L.fft(*L.fft(r, i, 0), 0, inverse=True), re, im)
+    np.testing.assert_allclose(r2.reshape(12, 5), re, atol=1e-6)
+    np.testing.assert_allclose(i2.reshape(12, 5), im, atol=1e-6)

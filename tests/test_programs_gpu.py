@@ -21,8 +21,12 @@ pytestmark = pytest.mark.gpu
 def warm(prog):
     from jaxjs_hip.kernelgen import generate
     from jaxjs_hip.runtime import compile_source
+    from jaxjs_hip.routinegen import generateRoutine
     for k in prog.kernels + [c.kernel() for c in prog.consts]:
         for src in generate(k).sources:
+            compile_source(src)
+    for r in prog.routines:
+        for src in generateRoutine(r).sources:
             compile_source(src)
     pytest.skip("warm-up run: compiled only")
 
@@ -119,3 +123,50 @@ def test_gpt2_block_full_size_f16_batch0_against_float64():
         want = block_reference(arrs["x"][b:b + 1].astype(np.float64), P, heads)[0]
         err = np.abs(y[b] - want)
         assert err.max() < 6e-2 and err.mean() < 4e-3, (b, err.max(), err.mean())
+
+
+def _routine_program_cases():
+    from jaxjs_hip import jit as J
+    from jaxjs_hip import library as L
+    rng = np.random.default_rng(9)
+    f = np.float32
+    a = (rng.standard_normal((4, 40, 40)) + 6 * np.eye(40)).astype(f)
+    b = rng.standard_normal((4, 40, 3)).astype(f)
+    g = rng.standard_normal((3, 24, 24))
+    spd = (g @ g.transpose(0, 2, 1) + 24 * np.eye(24)).astype(f)
+    x = rng.standard_normal((33, 50)).astype(f)
+    re, im = rng.standard_normal((48, 7)).astype(f), rng.standard_normal((48, 7)).astype(f)
+    return {
+        # name: (function, inputs, exact?)
+        "solve": (lambda a, b: L.solve(a, b), [a, b], True),
+        "cholesky_then_reconstruct": (lambda s: L.matmul(L.cholesky(s), L.cholesky(s, upper=True)), [spd], False),
+        "sort_argsort_axis0": (lambda x: (L.sort(J.exp(x), 0), L.argsort(x, 0)), [x], False),
+        "eigh_unsorted": (lambda s: L.eigh_unsorted(s), [spd], True),
+        "fft_axis0_roundtrip": (lambda r, i: L.fft(*L.fft(r, i, 0), 0, inverse=True), [re, im], False),
+        "lower_triangular_solve": (lambda s, b: L.triangularSolve(L.cholesky(s), b, leftSide=True, lower=True), [spd, rng.standard_normal((3, 24, 5)).astype(f)], True),
+    }
+
+
+@pytest.mark.parametrize("name", ["solve", "cholesky_then_reconstruct", "sort_argsort_axis0", "eigh_unsorted", "fft_axis0_roundtrip",
+                                  "lower_triangular_solve"])
+def test_programs_with_routines(name):
+    """Kernels and routines interleaved in one traced program (LU + triangular solves + the permutation product,
+    Cholesky feeding a GEMM, sort of a computed operand along axis 0 ...): hip backend against the oracle backend.
+    Programs whose kernels are maps, copies and small exact products around bit-exact routines must agree bit for bit;
+    the others within the float32 map tolerance scaled by the contraction length."""
+    from jaxjs_hip import jit as J
+    from jaxjs_hip.jit import ShapedArray
+    fn, arrays, exact = _routine_program_cases()[name]
+    prog = J.jit(fn, [ShapedArray(tuple(a.shape), DType.Float32) for a in arrays])
+    assert prog.routines
+    if WARM_ONLY:
+        warm(prog)
+    want = run_program(OracleBackend(), prog, arrays)
+    got = run_program(backend(), prog, arrays)
+    for g, w in zip(got, want):
+        if g.dtype.kind != "f":
+            np.testing.assert_array_equal(g, w)
+        elif exact and name != "solve":
+            np.testing.assert_array_equal(g, w)
+        else:
+            np.testing.assert_allclose(g, w, rtol=2e-5, atol=2e-5 * np.abs(w).max())
