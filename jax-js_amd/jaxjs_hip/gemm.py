@@ -7,6 +7,8 @@ and fills the template.
 
 from __future__ import annotations
 
+import math
+
 from typing import Dict, List
 
 from .alu import AluExp, AluOp, DType, Kernel, byteWidth
@@ -66,6 +68,126 @@ def _strip_casts(e: AluExp) -> AluExp:
     return e
 
 
+
+# ---- row-vector gather: eight consecutive rows of a gather operand in one 128-bit load ------------------------------
+#
+# For an operand whose memory runs along its tile-row axis (the pixels of a stride-1 convolution's image operand),
+# element (row0 + e, k) for an aligned row0 (row0 % 8 == 0) and e in 0..7 sits at index(row0, k) + e, and its mask is
+# a conjunction of comparisons that are linear in e.  `_lin` proves that shape on the operand's own simplified
+# expression: it splits an expression f(row) evaluated at row0 + e into rest(row0) + coef * e, pushing e out of
+# `% D` and `/ D` when the rest is a multiple of 8 * coef that divides D.
+
+def _has_row(e: AluExp) -> bool:
+    return bool(e.collect(lambda x: x.op == AluOp.Special and x.arg[0] == "row"))
+
+
+def _multiple_of(e: AluExp, m: int, group: int) -> bool:
+    if m == 1:
+        return True
+    if e.op == AluOp.Const:
+        return int(e.arg) % m == 0
+    if e.op == AluOp.Special and e.arg[0] == "row":
+        return group % m == 0
+    if e.op in (AluOp.Add, AluOp.Sub):
+        return _multiple_of(e.src[0], m, group) and _multiple_of(e.src[1], m, group)
+    if e.op == AluOp.Mul:
+        for x, y in ((e.src[0], e.src[1]), (e.src[1], e.src[0])):
+            if y.op == AluOp.Const:
+                c = abs(int(y.arg))
+                if c % m == 0:
+                    return True
+                return c != 0 and _multiple_of(x, m // math.gcd(m, c), group)
+        return False
+    if e.op == AluOp.Mod and e.src[1].op == AluOp.Const and int(e.src[1].arg) % m == 0:
+        return _multiple_of(e.src[0], m, group)
+    return False
+
+
+def _lin(e: AluExp, group: int = 8):
+    """(coef, rest) with e(row0 + t) == rest(row0) + coef * t for every aligned row0 and t in [0, group), or None."""
+    if not _has_row(e):
+        return 0, e
+    if e.dtype != DType.Int32:
+        return None
+    if e.op == AluOp.Special:
+        return 1, e
+    if e.op in (AluOp.Add, AluOp.Sub):
+        a, b = _lin(e.src[0], group), _lin(e.src[1], group)
+        if a is None or b is None:
+            return None
+        if e.op == AluOp.Add:
+            return a[0] + b[0], AluExp.add(a[1], b[1])
+        return a[0] - b[0], AluExp.sub(a[1], b[1])
+    if e.op == AluOp.Mul:
+        for x, y in ((e.src[0], e.src[1]), (e.src[1], e.src[0])):
+            if y.op == AluOp.Const:
+                a = _lin(x, group)
+                if a is None:
+                    return None
+                return a[0] * int(y.arg), AluExp.mul(a[1], y)
+        return None
+    if e.op in (AluOp.Mod, AluOp.Idiv) and e.src[1].op == AluOp.Const:
+        D = int(e.src[1].arg)
+        a = _lin(e.src[0], group)
+        if a is None or D <= 0:
+            return None
+        coef, rest = a
+        if coef == 0:
+            return 0, AluExp(e.op, e.dtype, (rest, e.src[1]))
+        step = coef * group
+        if coef < 0 or rest.min < 0 or D % step != 0 or not _multiple_of(rest, step, group):
+            return None
+        return (coef, AluExp.mod(rest, e.src[1])) if e.op == AluOp.Mod else (0, AluExp.idiv(rest, e.src[1]))
+    return None
+
+
+def rows8_form(oexp: AluExp, extent: int, group: int = 8):
+    """For a gather operand's expression in (row, k, batch coordinates): (index at the group's first row, mask as a
+    function of the extra variable `e` or None when unmasked, the GlobalIndex node) if `group` consecutive rows of
+    every aligned group load `group` consecutive elements; else None."""
+    cond = None
+    node = oexp
+    if node.op == AluOp.Where:
+        zero = node.src[2]
+        if zero.op != AluOp.Const or float(zero.arg) != 0.0:
+            return None
+        cond, node = node.src[0], node.src[1]
+    if node.op != AluOp.GlobalIndex:
+        return None
+    a = _lin(node.src[0], group)
+    if a is None or a[0] != 1:
+        return None
+    idx0 = a[1].simplify()
+    evar = AluExp.special(DType.Int32, "e", group)
+    cond_e = None
+    if cond is not None:
+        atoms = []
+        for atom in cond.splitOp(AluOp.Mul):
+            neg = False
+            inner = atom
+            if inner.op == AluOp.Cmpne and inner.src[1].op == AluOp.Const and inner.src[0].dtype == DType.Bool and bool(inner.src[1].arg) is True:
+                neg, inner = True, inner.src[0]
+            if inner.op != AluOp.Cmplt:
+                if _has_row(inner):
+                    return None
+                atoms.append(atom)
+                continue
+            sides = []
+            for side in inner.src:
+                la = _lin(side, group)
+                if la is None:
+                    return None
+                coef, rest = la
+                sides.append(AluExp.add(rest, AluExp.mul(evar, AluExp.i32(coef))) if coef else rest)
+            lt = AluExp.cmplt(sides[0], sides[1])
+            atoms.append(AluExp.cmpne(lt, AluExp.bool(True)) if neg else lt)
+        cond_e = atoms[0]
+        for x in atoms[1:]:
+            cond_e = AluExp.mul(cond_e, x)
+        cond_e = cond_e.simplify()
+    return idx0, cond_e, node
+
+
 def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelSource:
     g = t.gemm
     re = kernel.reduction
@@ -119,7 +241,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
 
     # Element loaders for gather operands: the operand's lowered expression (masked load through its view
     # chain) with the flat output index rebuilt from (tile row, batch coordinates) and ridx = k.
-    gather_fns, gather_calls, gather_flags = [], {}, {}
+    gather_fns, gather_calls, gather_flags, gather_group = [], {}, {}, {}
     lowered = _strip_casts(t.exp)
     operand_exps = {g["gid_a"]: None, g["gid_b"]: None}
     if g.get("a_gather") or g.get("b_gather"):
@@ -153,6 +275,52 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         gather_fns.append(f"static __device__ __forceinline__ {in_t} jh_gather_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
                           + "\n".join(gcg.take_lines()) + f"\n  return ({in_t})({gval});\n}}")
         gather_calls[tag] = f"jh_gather_{tag}(row, k, jh_b0, jh_b1, jh_b2{epi_args})"
+        # Row-vector loader: when G = 8 or 4 consecutive rows of an aligned group read G consecutive elements, one
+        # unaligned G-element load replaces G element loads and their index arithmetic; masked lanes are zeroed
+        # afterwards (pairs measured slower than the element loader and are not used).  A group whose bytes would leave the buffer (first/last rows of the whole array, where the
+        # out-of-range part is masked anyway) takes the element loader through an out-of-line call.
+        r8, G = None, 0
+        if g["dtype"] == DType.Float16 and tile.get("ROWS8", 1):
+            for G in (8, 4):
+                r8 = rows8_form(oexp, extent, G)
+                if r8 is not None:
+                    break
+        if r8 is not None:
+            idx0, cond_e, gnode = r8
+            vnames = {"row": "row", "e": "e", "k": "k", "b0": "b0", "b1": "b1", "b2": "b2"}
+            icg = HipExpCodegen(names, vnames, "  ", prefix=f"i{tag}", numerics=numerics)
+            icg.countReferences(idx0)
+            ival = strip_parens(icg.run(idx0))
+            ilines = "\n".join(icg.take_lines())
+            gather_fns.append(f"static __device__ __forceinline__ int jh_gindex_{tag}(int row, int k, int b0, int b1, int b2) {{\n"
+                              f"{ilines}\n  return {ival};\n}}")
+            if cond_e is not None:
+                mcg = HipExpCodegen(names, vnames, "  ", prefix=f"m{tag}", numerics=numerics)
+                mcg.countReferences(cond_e)
+                mval = strip_parens(mcg.run(cond_e))
+                gather_fns.append(f"static __device__ __forceinline__ bool jh_gmask_{tag}(int row, int e, int k, int b0, int b1, int b2) {{\n"
+                                  + "\n".join(mcg.take_lines()) + f"\n  return {mval};\n}}")
+                mask = f"if (!jh_gmask_{tag}(r, e, k, b0, b1, b2)) part[e] = (jh_f16)0;"
+            else:
+                mask = ""
+            buf = names[gnode.arg[0]]
+            gather_fns.append(
+                f"typedef jh_f16 jh_part_{tag} __attribute__((ext_vector_type({G})));\n"
+                f"struct __attribute__((packed, aligned(2))) jh_part_u_{tag} {{ jh_part_{tag} v; }};\n"
+                f"static __device__ __attribute__((noinline)) jh_part_{tag} jh_gather_edge_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
+                f"  jh_part_{tag} part;\n#pragma unroll\n  for (int e = 0; e < {G}; ++e) part[e] = jh_gather_{tag}(row + e, k, b0, b1, b2{epi_args});\n  return part;\n}}\n"
+                f"static __device__ __forceinline__ jh_half8 jh_gather8_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
+                f"  jh_half8 v;\n#pragma unroll\n  for (int j = 0; j < {8 // G}; ++j) {{\n"
+                f"    const int r = row + j * {G};\n    const int i0 = jh_gindex_{tag}(r, k, b0, b1, b2);\n    jh_part_{tag} part;\n"
+                f"    if ((unsigned)i0 <= (unsigned)({gnode.arg[1]} - {G})) {{\n"
+                f"      part = reinterpret_cast<const jh_part_u_{tag}*>({buf} + i0)->v;\n"
+                f"#pragma unroll\n      for (int e = 0; e < {G}; ++e) {{ {mask} }}\n"
+                f"    }} else {{\n      part = jh_gather_edge_{tag}(r, k, b0, b1, b2{epi_args});\n    }}\n"
+                f"#pragma unroll\n    for (int e = 0; e < {G}; ++e) v[j * {G} + e] = part[e];\n  }}\n"
+                f"  return v;\n}}")
+            gather_calls[tag] = f"jh_gather8_{tag}(row, k, jh_b0, jh_b1, jh_b2{epi_args})"
+            gather_flags[tag] = 2
+            gather_group[tag] = G
 
     # Batch index decode, innermost batch axis last in g["batch"].
     lines = ["  {", "    int rem = batch;"]
@@ -197,8 +365,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                      GATHER_A_CALL=gather_calls["a"], GATHER_B_CALL=gather_calls["b"])
     src = _prelude(numerics) + fill(template(tmpl), dict(sched, 
         M=g["M"], N=g["N"], K=g["K"], BM=BM, BN=BN, WM=WM, WN=WN,
-        A_KCONTIG=1 if g["a_sk"] == 1 or g["K"] == 1 or g.get("a_gather") else 0,
-        B_KCONTIG=1 if g["b_sk"] == 1 or g["K"] == 1 or g.get("b_gather") else 0,
+        A_KCONTIG=0 if gather_flags["a"] == 2 else (1 if g["a_sk"] == 1 or g["K"] == 1 or g.get("a_gather") else 0),
+        B_KCONTIG=0 if gather_flags["b"] == 2 else (1 if g["b_sk"] == 1 or g["K"] == 1 or g.get("b_gather") else 0),
         NBATCH=nbatch, EPILOGUE_FN=epi_fn, NAME=name, PARAMS=params,
         A_OFF=g["a_off"], B_OFF=g["b_off"], BATCH_DECODE="\n".join(lines),
         A_PTR=names[g["gid_a"]], B_PTR=names[g["gid_b"]],
@@ -216,4 +384,6 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     need[g["gid_b"]] = max(need.get(g["gid_b"], 0), g["b_len"] * eb)
     info = dict(BM=BM, BN=BN, WM=WM, WN=WN, BK=32 if dlds else (64 if g["dtype"] == DType.Float16 else 16), direct_lds=bool(dlds), tiles=tiles, a_kcontig=g["a_sk"] == 1, b_kcontig=g["b_sk"] == 1,
                 M=g["M"], N=g["N"], K=g["K"], nbatch=nbatch)
+    if any_gather:
+        info["gather"] = {tag: {0: "none", 1: "element", 2: f"rows{gather_group.get(tag, 8)}"}[gather_flags[tag]] for tag in ("a", "b")}
     return KernelSource([src], [step], [], "gemm", need, info)

@@ -212,3 +212,60 @@ def test_resnet_shaped_convolution_and_pooling_on_gpu():
         assert abs(r[n, o, i, j] - want) <= 2 * 576 * np.finfo(np.float32).eps * mag + 1e-6
     (p,) = run_program(be, pool_prog, [x])
     np.testing.assert_array_equal(p.reshape(8, 64, 14, 14), x.reshape(8, 64, 14, 2, 14, 2).max(axis=(3, 5)))
+
+
+# f16 convolutions whose image operand is (or is not) eligible for the row-vector gather loader: image widths that are
+# a multiple of 8 or of 4 only (shorter vectors), other widths (element loader), padding on every
+# side, dilation, more than two spatial dims, strides (element loader), ragged pixel counts.
+F16_CONV_CASES = [
+    dict(x=(2, 8, 16, 16), w=(32, 8, 3, 3), strides=[1, 1], padding="SAME", loader="rows8"),
+    dict(x=(3, 16, 8, 24), w=(32, 16, 3, 3), strides=[1, 1], padding="SAME", loader="rows8"),
+    dict(x=(2, 8, 28, 28), w=(32, 8, 3, 3), strides=[1, 1], padding="SAME", loader="rows4"),
+    dict(x=(2, 8, 14, 14), w=(32, 8, 3, 3), strides=[1, 1], padding="SAME", loader="element"),
+    dict(x=(2, 8, 30, 30), w=(32, 8, 3, 3), strides=[1, 1], padding="VALID", loader="rows4"),
+    dict(x=(1, 8, 20, 40), w=(32, 8, 5, 5), strides=[1, 1], padding=[(3, 1), (0, 4)], loader="rows8"),
+    dict(x=(2, 8, 24, 24), w=(32, 8, 3, 3), strides=[1, 1], padding="SAME", rd=[2, 2], loader="rows8"),
+    dict(x=(2, 16, 64), w=(32, 16, 3), strides=[1], padding="SAME", loader="rows8"),
+    dict(x=(1, 8, 6, 8, 16), w=(32, 8, 3, 3, 3), strides=[1, 1, 1], padding="SAME", loader="rows8"),
+    dict(x=(2, 8, 7, 7), w=(32, 8, 3, 3), strides=[1, 1], padding="SAME", loader="element"),
+    dict(x=(2, 8, 32, 32), w=(32, 8, 3, 3), strides=[2, 2], padding="SAME", loader="element"),
+    dict(x=(2, 8, 16, 16), w=(32, 8, 1, 1), strides=[1, 1], padding="VALID", loader=None),
+]
+
+
+def _f16_conv_program(c):
+    return J.jit(lambda a, b: L.convGeneralDilated(a, b, c["strides"], c["padding"], rhsDilation=c.get("rd")),
+                 [ShapedArray(c["x"], DType.Float16), ShapedArray(c["w"], DType.Float16)])
+
+
+@pytest.mark.parametrize("case", F16_CONV_CASES, ids=lambda c: "x".join(map(str, c["x"])) + "*" + "x".join(map(str, c["w"])))
+def test_f16_convolution_loader_choice(case):
+    """Which loader the generator picks is decided on the host: check it without a GPU."""
+    from jaxjs_hip.kernelgen import generate
+    ks = generate(_f16_conv_program(case).kernels[0])
+    if case["loader"] is None:
+        assert "gather" not in ks.info or set(ks.info["gather"].values()) == {"none"}
+    else:
+        assert ks.klass == "gemm" and case["loader"] in ks.info["gather"].values(), ks.info
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", F16_CONV_CASES, ids=lambda c: "x".join(map(str, c["x"])) + "*" + "x".join(map(str, c["w"])))
+def test_f16_convolution_on_gpu_is_exact_on_small_integers(case):
+    from gpu_util import WARM_ONLY, backend
+    prog = _f16_conv_program(case)
+    if WARM_ONLY:
+        from jaxjs_hip.kernelgen import generate
+        from jaxjs_hip.runtime import compile_source
+        for src in generate(prog.kernels[0]).sources:
+            compile_source(src)
+        pytest.skip("warm-up run: compiled only")
+    rng = np.random.default_rng(12)
+    x = rng.integers(-2, 3, case["x"]).astype(np.float16)
+    w = rng.integers(-2, 3, case["w"]).astype(np.float16)
+    (r,) = run_program(backend(), prog, [x, w])
+    pads = case["padding"]
+    if isinstance(pads, str):
+        pads = L.padtypeToPads(case["x"][2:], case["w"][2:], case["strides"], case.get("rd") or [1] * len(case["strides"]), pads)
+    want = conv_reference(x.astype(np.float32), w.astype(np.float32), case["strides"], pads, None, case.get("rd"))
+    np.testing.assert_array_equal(r.reshape(want.shape).astype(np.float64), want)  # |sums| < 2048: exact in f16
