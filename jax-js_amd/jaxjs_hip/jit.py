@@ -120,6 +120,8 @@ UNARY_FUSABLE = ("Neg", "Reciprocal", "Floor", "Ceil", "StopGradient", "Cast", "
                  "Exp", "Log", "Erf", "Erfc", "Sqrt")
 BINARY_FUSABLE = ("Add", "Mul", "Idiv", "Mod", "Min", "Max", "BitCombine", "BitShift")
 # Primitives handed to the backend as a unit (src/frontend/core.ts:154-163): primitive name == routine name.
+# Their outputs index their inputs in several different ways: always dispatched (src/frontend/jit.ts:972-977).
+HETEROGENEOUS_VIEW_PRIMITIVES = ("RandomBits", "Gather")
 ROUTINE_PRIMITIVES = ("Sort", "Argsort", "Scatter", "TriangularSolve", "Cholesky", "LU", "JacobiEigh", "Fft")
 
 
@@ -356,13 +358,64 @@ def _out_aval(prim: str, avals: List[ShapedArray], params: Dict[str, Any]) -> Sh
         return ShapedArray(tuple(e - s for s, e in params["slice"]), avals[0].dtype, avals[0].weak)
     if prim == "Pad":
         return ShapedArray(tuple(d + a + b for d, (a, b) in zip(avals[0].shape, params["width"])), avals[0].dtype, avals[0].weak)
+    if prim == "Concatenate":
+        ax = params["axis"]
+        first = avals[0]
+        for x in avals:
+            if x.ndim != first.ndim or any(i != ax and a != b for i, (a, b) in enumerate(zip(x.shape, first.shape))):
+                raise TypeError(f"Concatenate: inputs {first.shape} and {x.shape} must match shapes except on axis {ax}")
+        shape = list(first.shape)
+        shape[ax] = sum(x.shape[ax] for x in avals)
+        d = ShapedArray((), first.dtype, first.weak)
+        for x in avals[1:]:
+            d = promoteAvals(d, ShapedArray((), x.dtype, x.weak))
+        return ShapedArray(tuple(shape), d.dtype, d.weak)
+    if prim == "RandomBits":
+        k0, k1 = avals
+        shape = tuple(params["shape"])
+        if k0.dtype != DType.Uint32 or k1.dtype != DType.Uint32:
+            raise TypeError(f"RandomBits requires uint32 keys, got {k0.dtype} and {k1.dtype}")
+        if tuple(k0.shape) != tuple(k1.shape) or shape[:k0.ndim] != tuple(k0.shape):
+            raise TypeError(f"RandomBits: generated shape {shape} must match key shape {k0.shape}")
+        return ShapedArray(shape, DType.Uint32, False)
+    if prim == "Gather":
+        x, indices = avals[0], avals[1:]
+        return ShapedArray(tuple(gatherShape(x.shape, indices, params["axis"], params["outDim"])), x.dtype, x.weak)
     raise NotImplementedError(f"jit: primitive {prim}")
+
+
+def gatherShape(operandShape, indices: Sequence[ShapedArray], axis: Sequence[int], outDim: int) -> List[int]:
+    """Result shape of `x[:, ...indices, :]` with the index dimensions placed at `outDim` (src/frontend/jaxpr.ts:774-800)."""
+    for a in indices:
+        if a.dtype not in (DType.Int32, DType.Uint32):
+            raise TypeError(f"indices must be Int32 or Uint32, got {a.dtype}")
+    if len(axis) != len(indices):
+        raise TypeError(f"got {list(axis)} axes but {len(indices)} indices")
+    if not indices:
+        raise TypeError("must have at least one index")
+    if any(a < 0 or a >= len(operandShape) for a in axis):
+        raise TypeError("axis out of bounds")
+    if outDim < 0 or outDim > len(operandShape) - len(axis):
+        raise TypeError("outDim out of bounds")
+    if len(set(axis)) != len(axis):
+        raise TypeError("axes are not unique")
+    indexShape: Tuple[int, ...] = ()
+    for a in indices:
+        indexShape = generalBroadcast(indexShape, a.shape)
+    result = [d for i, d in enumerate(operandShape) if i not in set(axis)]
+    result[outDim:outDim] = list(indexShape)
+    return result
 
 
 def _routine_out_avals(prim: str, avals: List[ShapedArray], params: Dict[str, Any]) -> List[ShapedArray]:
     """Output types of the routine primitives (src/frontend/jaxpr.ts:976-1062)."""
     a = avals[0]
     same = ShapedArray(tuple(a.shape), a.dtype, a.weak)
+    if prim == "Split":  # a fusable multi-output primitive, not a routine (src/frontend/jaxpr.ts:913-927)
+        ax, sizes = params["axis"], list(params["sizes"])
+        if a.shape[ax] != sum(sizes):
+            raise TypeError(f"Split: sizes {sizes} do not sum to dimension {a.shape[ax]} on axis {ax}")
+        return [ShapedArray(tuple(a.shape[:ax]) + (sz,) + tuple(a.shape[ax + 1:]), a.dtype, a.weak) for sz in sizes]
     if prim in ("Sort", "Argsort"):
         if a.ndim == 0:
             raise TypeError(f"{prim.lower()}: requires at least 1D input")
@@ -486,6 +539,34 @@ def shrink(x, slices):
 def flip(x, axis):
     x = _raise(x)
     return bind1("Flip", [x], dict(axis=_normalize_axis(axis, x.ndim)))
+
+
+def concatenate(xs, axis: int):
+    xs = [_raise(x) for x in xs]
+    if not xs:
+        raise ValueError("concatenate requires at least one input")
+    (axis,) = _normalize_axis(axis, xs[0].ndim)
+    return bind1("Concatenate", xs, dict(axis=axis))
+
+
+def split(x, axis: int, sizes):
+    x = _raise(x)
+    (axis,) = _normalize_axis(axis, x.ndim)
+    sizes = [int(sz) for sz in sizes]
+    if any(sz < 0 for sz in sizes) or sum(sizes) != x.shape[axis]:
+        raise ValueError(f"split: sizes must be nonnegative and sum to the size of axis {axis}, got {sizes}")
+    return bind("Split", [x], dict(axis=axis, sizes=sizes))
+
+
+def randomBits(k0, k1, shape, mode="xor"):
+    return bind1("RandomBits", [k0, k1], dict(shape=tuple(shape), mode=mode))
+
+
+def gather(x, indices, axis, outDim: int):
+    """`x[:, ...indices, :]` with the broadcast index dimensions starting at `outDim` (src/frontend/core.ts:414-434)."""
+    x = _raise(x)
+    axis = [a + x.ndim if a < 0 else a for a in axis]
+    return bind1("Gather", [x] + list(indices), dict(axis=axis, outDim=int(outDim)))
 
 
 def sort(x):
@@ -656,7 +737,84 @@ def _flip_rule(st, params):
     return st.flip(arg)
 
 
+def _concatenate_rule(exps, avals, params):
+    """Every input cast to the common type, padded with zeros to the final extent, then summed (jit.ts:666-685)."""
+    axis = params["axis"]
+    ndim = avals[0].ndim
+    sizes = [a.shape[axis] for a in avals]
+    final = sum(sizes)
+    d = ShapedArray((), avals[0].dtype, avals[0].weak)
+    for a in avals[1:]:
+        d = promoteAvals(d, ShapedArray((), a.dtype, a.weak))
+    cum, src = 0, []
+    for e, size in zip(exps, sizes):
+        padding = [(cum, final - cum - size) if i == axis else (0, 0) for i in range(ndim)]
+        src.append(reshapeViews(AluExp.cast(d.dtype, e), lambda st, padding=padding: st.pad(padding)))
+        cum += size
+    out = src[0]
+    for x in src[1:]:
+        out = AluExp.add(out, x)
+    return [out], None
+
+
+def _split_rule(exps, avals, params):
+    a, aval = exps[0], avals[0]
+    out, start = [], 0
+    for size in params["sizes"]:
+        sl = [(start, start + size) if d == params["axis"] else (0, aval.shape[d]) for d in range(aval.ndim)]
+        out.append(reshapeViews(a, lambda st, sl=sl: st.shrink(sl)))
+        start += size
+    return out, None
+
+
+def _random_bits_rule(keys, avals, params):
+    """threefry2x32(k0, k1, 0, position within the key's block) (jit.ts:698-714)."""
+    shape, keyShape = list(params["shape"]), list(avals[0].shape)
+
+    def mapping(st):
+        if list(st.shape) != shape:
+            return st.broadcast(shape, list(range(len(st.shape), len(shape))))
+        return None
+    k0, k1 = reshapeViews(keys[0], mapping), reshapeViews(keys[1], mapping)
+    c1 = AluExp.mod(AluExp.cast(DType.Uint32, AluVar.gidx), AluExp.u32(max(prod(shape[len(keyShape):]), 1)))
+    return [AluExp.threefry2x32(k0, k1, AluExp.u32(0), c1, params.get("mode", "xor"))], None
+
+
+def _gather_rule(exps, avals, params):
+    """The operand's flat index is rebuilt from the output coordinates, with the gathered axes read from the
+    (broadcast) index arrays (jit.ts:715-763)."""
+    x, indices = exps[0], exps[1:]
+    xs, ishapes = avals[0], avals[1:]
+    axis, outDim = list(params["axis"]), params["outDim"]
+    axisSet = set(axis)
+    indexShape: Tuple[int, ...] = ()
+    for a in ishapes:
+        indexShape = generalBroadcast(indexShape, a.shape)
+    finalShape = [d for i, d in enumerate(xs.shape) if i not in axisSet]
+    finalShape[outDim:outDim] = list(indexShape)
+    idxAll = unravelAlu(finalShape, AluVar.gidx)
+    idxNonaxis = list(idxAll)
+    del idxNonaxis[outDim:outDim + len(indexShape)]
+    src: List[Optional[AluExp]] = list(idxNonaxis)
+    for i in range(len(xs.shape)):
+        if i in axisSet:
+            src.insert(i, None)
+    for i, iexp in enumerate(indices):
+        def mapping(st):
+            lead = list(range(outDim + len(indexShape) - len(st.shape)))
+            return st.broadcast(finalShape, lead + list(range(outDim + len(indexShape), len(finalShape))))
+        src[axis[i]] = AluExp.cast(DType.Int32, reshapeViews(iexp, mapping))
+    index, valid = ShapeTracker.fromShape(list(xs.shape)).toAluExp(src)
+    if not valid.resolve():
+        raise RuntimeError("internal: expected full validity mask in Gather")
+    return [x.substitute({"gidx": index})], None
+
+
 JIT_RULES: Dict[str, Callable] = {
+    "Concatenate": _concatenate_rule,
+    "Split": _split_rule,
+    "RandomBits": _random_bits_rule,
+    "Gather": _gather_rule,
     "Add": _broadcasted(lambda e, p: AluExp.add(e[0], e[1])),
     "Mul": _broadcasted(lambda e, p: AluExp.mul(e[0], e[1])),
     "Idiv": _broadcasted(lambda e, p: AluExp.idiv(e[0], e[1])),
@@ -774,7 +932,7 @@ def splitGraphDataflow(jaxpr: Jaxpr, maxArgs: int) -> Set[Var]:
             if isinstance(x, Var) and hasReuse(shapes[i], promoted):
                 markNonViewProducer(x)
     for eqn in jaxpr.eqns:
-        if eqn.primitive == "Pad":  # Pad needs clean inputs
+        if eqn.primitive in ("Pad", "Concatenate"):  # padding an expression would pad its inner views: needs clean inputs
             for x in eqn.inputs:
                 if isinstance(x, Var):
                     markNonViewProducer(x)
@@ -799,7 +957,8 @@ def splitGraphDataflow(jaxpr: Jaxpr, maxArgs: int) -> Set[Var]:
             nextBlack[v] = v
     for i in range(len(jaxpr.eqns) - 1, -1, -1):
         eqn = jaxpr.eqns[i]
-        if (i in endpointEqns or eqn.primitive in ROUTINE_PRIMITIVES or any(v in materialized for v in eqn.outBinders)
+        if (i in endpointEqns or eqn.primitive in ROUTINE_PRIMITIVES or eqn.primitive in HETEROGENEOUS_VIEW_PRIMITIVES
+                or any(v in materialized for v in eqn.outBinders)
                 or any(v in black for v in eqn.outBinders)):
             for v in eqn.outBinders:
                 black.add(v)

@@ -11,6 +11,8 @@ the backend is handed, so it is kept literally:
   sort / argsort along an axis                        src/frontend/core.ts:1043-1075
   linalg: cholesky, triangularSolve, solve            src/library/lax-linalg.ts:35-50, 212-244; numpy-linalg.ts:274-318
   eigh (unsorted), fft along an axis                  src/library/lax-linalg.ts:52-100; numpy-fft.ts:50-66, 126-157
+  stack, take, takeAlongAxis, absolute, clip, log1p   src/library/numpy.ts:971-985, 1493-1567, 2433-2452, 2854-2884
+  random: bits, split, uniform, exponential, normal   src/library/random.ts:53-135, 350-356, 511-525
 """
 
 from __future__ import annotations
@@ -282,3 +284,116 @@ def fft(real: Tracer, imag: Tracer, axis: int = -1, inverse: bool = False):
     if axis != real.ndim - 1:
         re, im = re.transpose(inv), im.transpose(inv)
     return re, im
+
+
+def stack(xs: Sequence[Tracer], axis: int = 0):
+    xs = [J._raise(x) for x in xs]
+    if not xs:
+        raise ValueError("Need at least one array to stack")
+    if any(tuple(x.shape) != tuple(xs[0].shape) for x in xs):
+        raise ValueError(f"Cannot stack arrays with different shapes: {[list(x.shape) for x in xs]}")
+    nd = xs[0].ndim + 1
+    axis = axis + nd if axis < 0 else axis
+    newShape = list(xs[0].shape[:axis]) + [1] + list(xs[0].shape[axis:])
+    return J.concatenate([x.reshape(newShape) for x in xs], axis)
+
+
+def take(a: Tracer, indices: Tracer, axis: Optional[int] = None):
+    if axis is None:
+        a, axis = a.reshape([-1]), 0
+    axis = axis + a.ndim if axis < 0 else axis
+    return J.gather(a, [indices], [axis], axis)
+
+
+def takeAlongAxis(a: Tracer, indices: Tracer, axis: int = -1):
+    """One index array per axis: the given one on `axis`, aranges elsewhere, all broadcast to the output shape."""
+    if a.ndim != indices.ndim:
+        raise ValueError(f"takeAlongAxis: input and indices must have the same rank, got {list(a.shape)} and {list(indices.shape)}")
+    axis = axis + a.ndim if axis < 0 else axis
+    outShape = list(indices.shape)
+    for i in range(a.ndim):
+        if i == axis:
+            continue
+        if a.shape[i] != indices.shape[i] and a.shape[i] != 1 and indices.shape[i] != 1:
+            raise ValueError(f"takeAlongAxis: non-axis dimensions must broadcast, got {list(a.shape)} and {list(indices.shape)}")
+        outShape[i] = max(a.shape[i], indices.shape[i])
+    coords = []
+    for i in range(a.ndim):
+        if i == axis:
+            c = indices
+        else:
+            shape = [1] * a.ndim
+            shape[i] = a.shape[i]
+            c = J._raise(arange_const(0, a.shape[i], 1, DType.Int32, shape=shape))
+        coords.append(J.broadcast(c, outShape, []) if list(c.shape) != outShape else c)
+    return J.gather(a, coords, list(range(a.ndim)), 0)
+
+
+def absolute(x: Tracer):
+    return J.where(J.less(x, 0), x.mul(-1), x)
+
+
+def clip(a: Tracer, lo=None, hi=None):
+    if hi is not None:
+        a = J.minimum(a, hi)
+    if lo is not None:
+        a = J.maximum(a, lo)
+    return a
+
+
+def log1p(x: Tracer):
+    """Series through x^10 (Horner) for |x| <= 0.2, log(1 + x) elsewhere."""
+    cutoff = 0.2
+    useSeries = J.lessEqual(absolute(x), cutoff)
+    sx = clip(x, -cutoff, cutoff)
+    series = (sx.mul(-1 / 10).add(1 / 9).mul(sx).sub(1 / 8).mul(sx).add(1 / 7).mul(sx).sub(1 / 6).mul(sx).add(1 / 5).mul(sx)
+              .sub(1 / 4).mul(sx).add(1 / 3).mul(sx).sub(1 / 2).mul(sx).add(1).mul(sx))
+    return J.where(useSeries, series, J.log(x.add(1)))
+
+
+def _key_halves(key: Tracer):
+    if key.dtype != DType.Uint32 or key.ndim < 1 or key.shape[-1] != 2:
+        raise ValueError(f"Invalid key shape: {list(key.shape)}. Expected last dimension to be 2 with uint32 type.")
+    keyShape = list(key.shape[:-1])
+    k0, k1 = J.split(key, -1, [1, 1])
+    return k0.reshape(keyShape), k1.reshape(keyShape)
+
+
+def random_bits(key: Tracer, shape: Sequence[int] = ()):
+    k0, k1 = _key_halves(key)
+    return J.randomBits(k0, k1, list(shape))
+
+
+def random_split(key: Tracer, num=2):
+    shape = [num] if isinstance(num, int) else list(num)
+    if any(n <= 0 for n in shape):
+        raise ValueError(f"Invalid split length: {shape}. Must be positive integers.")
+    k0, k1 = _key_halves(key)
+    return stack([J.randomBits(k0, k1, shape, 0), J.randomBits(k0, k1, shape, 1)], -1)
+
+
+def random_uniform(key: Tracer, shape: Sequence[int] = (), minval: float = 0.0, maxval: float = 1.0):
+    """23 random mantissa bits under the exponent of 1.0, minus 1: uniform in [0, 1)."""
+    if minval >= maxval:
+        raise ValueError(f"Invalid range: [{minval}, {maxval}).")
+    mantissa = random_bits(key, shape).div(J.scalar(1 << 9, DType.Uint32))
+    float12 = mantissa.add(J.scalar(0x3F800000, DType.Uint32))
+    rand = J.bind1("Bitcast", [float12], dict(dtype=DType.Float32)).sub(1)
+    if minval == 0 and maxval == 1:
+        return rand
+    return rand.mul(maxval - minval).add(minval)
+
+
+def random_exponential(key: Tracer, shape: Sequence[int] = ()):
+    return J.neg(log1p(J.neg(random_uniform(key, shape))))
+
+
+def random_normal(key: Tracer, shape: Sequence[int] = ()):
+    """Box-Muller, first variate only."""
+    keys = random_split(key, 2)
+    ka, kb = J.split(keys, 0, [1, 1])
+    u1 = random_uniform(ka.reshape([2]), shape)
+    u2 = random_uniform(kb.reshape([2]), shape)
+    radius = J.sqrt(log1p(J.neg(u1)).mul(-2))
+    theta = u2.mul(2 * math.pi)
+    return radius.mul(J.bind1("Cos", [theta]))

@@ -305,3 +305,86 @@ def test_cholesky_upper_eigh_and_fft_along_an_axis():
     _, (r2, i2) = run(lambda r, i: L.fft(*L.fft(r, i, 0), 0, inverse=True), re, im)
     np.testing.assert_allclose(r2.reshape(12, 5), re, atol=1e-6)
     np.testing.assert_allclose(i2.reshape(12, 5), im, atol=1e-6)
+
+
+# ---- Concatenate / Split / Gather / RandomBits (src/frontend/jit.ts:666-763) -------------------------------------------
+
+U32, I32 = DType.Uint32, DType.Int32
+
+
+def run_typed(fn, arrays, dtypes):
+    prog = J.jit(fn, [ShapedArray(tuple(a.shape), d) for a, d in zip(arrays, dtypes)])
+    be = OracleBackend()
+    outs = run_program(be, prog, arrays)
+    assert be.live_slots() == 0
+    return prog, outs
+
+
+def prng_key(seed):
+    return np.array([0, seed], np.uint32)  # random.key(seed) = [0, seed] (src/library/random.ts:62-76)
+
+
+def test_random_bits_and_split_match_jax():  # test/random.test.ts:21-48
+    _, (b,) = run_typed(lambda k: L.random_bits(k), [prng_key(0)], [U32])
+    assert b.tolist() == [4070199207]
+    _, (b,) = run_typed(lambda k: L.random_bits(k, [4]), [prng_key(10)], [U32])
+    assert b.tolist() == [169096361, 1572511259, 2689743692, 2228103506]
+    prog, (s,) = run_typed(lambda k: L.random_split(k, 3), [prng_key(1)], [U32])
+    assert s.reshape(3, 2).tolist() == [[507451445, 1853169794], [1948878966, 4237131848], [2441914641, 3819641963]]
+    # RandomBits results are always dispatched (their views are heterogeneous), and Concatenate reads clean inputs
+    assert sum(1 for k in prog.kernels if k.exp.collect(lambda n: n.op.name == "Threefry2x32")) == 2
+
+
+def test_uniform_and_normal_distributions():  # test/random.test.ts:50-120 (ranges and moments)
+    _, (z,) = run_typed(lambda k: L.random_uniform(k, [2, 3], 10, 15), [prng_key(42)], [U32])
+    assert z.dtype == np.float32 and np.all((z >= 10) & (z < 15))
+    _, (u,) = run_typed(lambda k: L.random_uniform(k, [50000]), [prng_key(5)], [U32])
+    assert 0 <= u.min() and u.max() < 1 and abs(u.mean() - 0.5) < 0.01 and abs(u.var() * 12 - 1) < 0.03
+    _, (n,) = run_typed(lambda k: L.random_normal(k, [50000]), [prng_key(3)], [U32])
+    assert abs(n.mean()) < 0.02 and abs(n.std() - 1) < 0.02 and abs(np.mean(np.abs(n) < 1) - 0.6827) < 0.01
+    _, (e,) = run_typed(lambda k: L.random_exponential(k, [50000]), [prng_key(4)], [U32])
+    assert e.min() >= 0 and abs(e.mean() - 1) < 0.03
+
+
+def test_gather_take_and_take_along_axis():
+    x = np.arange(24, dtype=np.float32).reshape(4, 6)
+    idx = np.array([[3, 0], [1, 1]], np.int32)
+    prog, (t,) = run_typed(lambda a, i: L.take(a, i, 1), [x, idx], [F32, I32])
+    np.testing.assert_array_equal(t.reshape(4, 2, 2), np.take(x, idx, 1))
+    assert len(prog.kernels) == 1
+    _, (t,) = run_typed(lambda a, i: L.take(a, i), [x, idx], [F32, I32])
+    np.testing.assert_array_equal(t.reshape(2, 2), np.take(x, idx))
+    order = np.argsort(-x, axis=1).astype(np.int32)
+    _, (t,) = run_typed(lambda a, i: L.takeAlongAxis(a, i, 1), [x, order], [F32, I32])
+    np.testing.assert_array_equal(t.reshape(4, 6), np.take_along_axis(x, order, 1))
+    # two index arrays on non-adjacent axes, index dims placed at outDim=0; a computed operand is gathered in-kernel
+    y = np.arange(2 * 3 * 4, dtype=np.float32).reshape(2, 3, 4)
+    i0, i2 = np.array([1, 0, 1], np.int32), np.array([3, 2, 0], np.int32)
+    prog, (g,) = run_typed(lambda a, p, q: J.gather(a.mul(2.0), [p, q], [0, 2], 0), [y, i0, i2], [F32, I32, I32])
+    np.testing.assert_array_equal(g.reshape(3, 3), (y * 2)[i0, :, i2])
+    assert len(prog.kernels) == 1
+    # eigh's final step: sort eigenvalues, reorder the vectors' columns by the same permutation
+    vals = np.array([[3.0, 1.0, 2.0]], np.float32)
+    vecs = np.arange(9, dtype=np.float32).reshape(1, 3, 3)
+    _, (w, v) = run_typed(lambda d, m: (L.takeAlongAxis(d, L.argsort(d), -1), L.takeAlongAxis(m, L.argsort(d).reshape([1, 1, 3]), -1)),
+                          [vals, vecs], [F32, F32])
+    assert w.tolist() == [1, 2, 3] and v.reshape(3, 3).tolist() == [[1, 2, 0], [4, 5, 3], [7, 8, 6]]
+
+
+def test_concatenate_stack_and_split():
+    x = np.arange(24, dtype=np.float32).reshape(4, 6)
+    prog, (c,) = run_typed(lambda a, b: J.concatenate([a.mul(2.0), b], 0), [x, x[:2]], [F32, F32])
+    np.testing.assert_array_equal(c.reshape(6, 6), np.concatenate([x * 2, x[:2]], 0))
+    assert len(prog.kernels) == 2  # the scaled operand is dispatched first: padding an expression would pad its views
+    _, (c,) = run_typed(lambda a, b: J.concatenate([a, b.astype(F32)], 1), [x, np.ones((4, 1), np.int32)], [F32, I32])
+    np.testing.assert_array_equal(c.reshape(4, 7), np.concatenate([x, np.ones((4, 1), np.float32)], 1))
+    _, (s,) = run_typed(lambda a, b: L.stack([a, b], 1), [x, -x], [F32, F32])
+    np.testing.assert_array_equal(s.reshape(4, 2, 6), np.stack([x, -x], 1))
+    prog, (a, b, c) = run_typed(lambda a: J.split(a, 1, [2, 3, 1]), [x], [F32])
+    np.testing.assert_array_equal(a.reshape(4, 2), x[:, :2])
+    np.testing.assert_array_equal(b.reshape(4, 3), x[:, 2:5])
+    np.testing.assert_array_equal(c.reshape(4, 1), x[:, 5:])
+    with pytest.raises(ValueError):
+        run_typed(lambda a: J.split(a, 1, [2, 3]), [x], [F32])
+    with pytest.raises(TypeError):
+        run_typed(lambda a, b: J.concatenate([a, b], 0), [x, x[:, :2]], [F32, F32])
