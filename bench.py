@@ -282,6 +282,11 @@ def main():
             n_warm = int(min(max(30.0 / max(est, 1e-4), warm), 20000))
             n_steps = int(min(max(5.0 / max(est, 1e-4), steps), 5000))
             w_ms, e_ms = timed(be, ex, slots, o, n_steps, n_warm)
+            # Memory clocks can take longer than the warm-up to come back after a long host-side pause (input
+            # generation): measure a second block and keep the faster one.
+            w2, e2 = timed(be, ex, slots, o, n_steps, 0)
+            if e2 < e_ms:
+                w_ms, e_ms = w2, e2
             for s in slots + [o]:
                 be.decRef(s)
             rate = work / (e_ms * 1e-3) / (1e9 if unit == "GB/s" else 1e12)
