@@ -118,10 +118,44 @@ class HipBackend {
     return Promise.resolve().then(() => this.prepareKernelSync(plan));
   }
 
+  // A routine plan (`routine`, `inputBytes[]`, `outputBytes[]` beside the common fields) prepares exactly like a
+  // kernel plan: compile, load, look the entry points up, allocate scratch (src/backend.ts:197-203).
+  prepareRoutineSync(plan) {
+    if (plan.routine === undefined) throw new Error('prepareRoutineSync expects a routine plan');
+    return this.prepareKernelSync(plan);
+  }
+
+  prepareRoutine(plan) {
+    return Promise.resolve().then(() => this.prepareRoutineSync(plan));
+  }
+
+  _dispatchRoutine(exe, ins, outs) {
+    const plan = exe.source;
+    if (ins.length !== plan.inputBytes.length || outs.length !== plan.outputBytes.length) {
+      throw new Error(plan.routine + ' takes ' + plan.inputBytes.length + ' inputs and ' + plan.outputBytes.length + ' outputs');
+    }
+    plan.inputBytes.forEach((b, i) => {
+      if (ins[i].size < b) throw new Error('input ' + i + ' holds ' + ins[i].size + ' bytes, the routine addresses ' + b);
+    });
+    plan.outputBytes.forEach((b, i) => {
+      if (outs[i].size < b) throw new Error('output ' + i + ' holds ' + outs[i].size + ' bytes, the routine addresses ' + b);
+    });
+    plan.steps.forEach((st, i) => {
+      const args = st.args.map((a) => {
+        if (a[0] === 'in') return ins[a[1]].ptr;
+        if (a[0] === 'out') return outs[a[1]].ptr;
+        if (a[0] === 'scratch') return exe.data.scratch[a[1]];
+        return BigInt(a[1]);  // by-value 64-bit integer: same 8-byte argument cell as a pointer
+      });
+      addon.launch(exe.data.functions[i], st.grid, st.block, st.shared, args);
+    });
+  }
+
   dispatch(exe, inputs, outputs) {
     const plan = exe.source;
     const ins = inputs.map((s) => this._get(s));
     const outs = outputs.map((s) => this._get(s));
+    if (plan.routine !== undefined) return this._dispatchRoutine(exe, ins, outs);
     if (outs.length !== 1) throw new Error('a Kernel has exactly one output');
     if (outs[0].size < plan.outputBytes) {
       throw new Error('output slot holds ' + outs[0].size + ' bytes, kernel writes ' + plan.outputBytes);

@@ -2,7 +2,8 @@
 //
 //   node run_plan.js cases.json results.json
 //
-// cases.json: [{name, plan, inputs: [base64...]}]; results.json: [{name, output: base64}] plus the outcome of
+// cases.json: [{name, plan, inputs: [base64...]}]; results.json: [{name, output: base64}] (routine plans:
+// [{name, outputs: [base64...]}]) plus the outcome of
 // the Backend-protocol checks below (slot errors, refcounts, zero-size buffers, ranged reads), which restate
 // src/backend.test.ts:88-135 for this device.
 'use strict';
@@ -42,8 +43,18 @@ function main() {
   const be = new HipBackend(0);
   const results = { device: be.info, protocol: protocolChecks(be), cases: [] };
   cases.forEach((c) => {
-    const exe = be.prepareKernelSync(c.plan);
     const ins = c.inputs.map((b64) => { const buf = Buffer.from(b64, 'base64'); return be.malloc(buf.length, buf); });
+    if (c.plan.routine !== undefined) {
+      const exe = be.prepareRoutineSync(c.plan);
+      const outs = c.plan.outputBytes.map((b) => be.malloc(b));
+      be.dispatch(exe, ins, outs);
+      be.dispatch(exe, ins, outs);
+      const raws = outs.map((o) => Buffer.from(be.readSync(o)).toString('base64'));
+      ins.concat(outs).forEach((s) => be.decRef(s));
+      results.cases.push({ name: c.name, outputs: raws });
+      return;
+    }
+    const exe = be.prepareKernelSync(c.plan);
     const out = be.malloc(c.plan.outputBytes);
     be.dispatch(exe, ins, [out]);
     be.dispatch(exe, ins, [out]);  // a second dispatch of the same executable must give the same bytes

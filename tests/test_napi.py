@@ -13,7 +13,7 @@ import pytest
 from jaxjs_hip import AluExp, AluOp, DType, ShapeTracker
 from jaxjs_hip.alu import numpyDtype
 from jaxjs_hip.lowering import mapKernel, matmulKernel, matvecKernel, reduceKernel
-from jaxjs_hip.plan import exportPlan
+from jaxjs_hip.plan import exportPlan, exportRoutinePlan
 from oracle import oracle
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -105,3 +105,60 @@ def test_javascript_backend_replays_plans(tmp_path):
         else:
             np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4, err_msg=name)
     np.testing.assert_array_equal(np.frombuffer(base64.b64decode(res["cases"][0]["output"]), np.float32), [6, 10, 12])
+
+
+def _routine_cases():
+    import routine_util as R
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((3, 20000)).astype(np.float32)          # sort: LDS tiles + global passes (by-value stride arguments)
+    a = rng.standard_normal((2, 24, 24))
+    spd = (a @ a.transpose(0, 2, 1) + 24 * np.eye(24)).astype(np.float32)
+    re, im = rng.standard_normal((4, 60)).astype(np.float32), rng.standard_normal((4, 60)).astype(np.float32)
+    upd, idx = rng.integers(-9, 10, (500, 3)).astype(np.float32), rng.integers(-1, 41, (500,)).astype(np.int32)
+    from jaxjs_hip.routine import Routine, Routines, RoutineType
+    F, I = DType.Float32, DType.Int32
+    return [
+        ("sort", Routine(Routines.Sort, RoutineType([[3, 20000]], [F], [[3, 20000]], [F])), [x]),
+        ("argsort", Routine(Routines.Argsort, RoutineType([[3, 20000]], [F], [[3, 20000]] * 2, [F, I])), [x]),
+        ("cholesky", R.cholesky(spd), [spd]),
+        ("lu", R.lu(spd), [spd]),
+        ("fft", R.fft(re, im), [re, im]),
+        ("scatter_update", R.scatter(upd, [idx], "update", [40, 3], [0], 0), [upd, idx]),
+    ]
+
+
+def test_routine_plan_is_plain_data():
+    name, routine, xs = _routine_cases()[0]
+    plan = exportRoutinePlan(routine)
+    assert json.loads(json.dumps(plan)) == plan and plan["routine"] == "Sort" and plan["outputBytes"] == [240000]
+    assert any(kind == "const" for st in plan["steps"] for kind, _ in st["args"])  # the global passes take (k, j) by value
+
+
+@pytest.mark.gpu
+@needs_node
+def test_javascript_backend_replays_routine_plans(tmp_path):
+    """prepareRoutine/dispatch of the JavaScript backend: several launches per routine, several outputs, by-value
+    integer arguments; outputs compared with the CPU checker (bit-exact except Fft, see the routine tests)."""
+    import routine_util as R
+    cases = _routine_cases()
+    if os.environ.get("JAXHIP_WARM") == "1":
+        for _, r, _ in cases:
+            exportRoutinePlan(r)
+        pytest.skip("warm-up run: nothing to execute")
+    payload = [dict(name=n, plan=exportRoutinePlan(r), inputs=[base64.b64encode(np.ascontiguousarray(x).tobytes()).decode() for x in xs])
+               for n, r, xs in cases]
+    src, dst = tmp_path / "cases.json", tmp_path / "results.json"
+    src.write_text(json.dumps(payload))
+    out = subprocess.run([NODE, os.path.join(NAPI, "run_plan.js"), str(src), str(dst)], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stdout + out.stderr
+    res = json.loads(dst.read_text())
+    for (name, routine, xs), r in zip(cases, res["cases"]):
+        assert r["name"] == name
+        want = R.run_oracle(routine, xs)
+        t = routine.type
+        for raw, w, dt, shape in zip(r["outputs"], want, t.outputDtypes, t.outputShapes):
+            got = np.frombuffer(base64.b64decode(raw), dtype=numpyDtype(dt)).reshape(shape)
+            if name == "fft":
+                np.testing.assert_allclose(got, w, rtol=0, atol=1e-5 * np.abs(w).max(), err_msg=name)
+            else:
+                assert R.bits_equal(got, w), name
