@@ -155,7 +155,7 @@ def rows8_form(oexp: AluExp, extent: int, group: int = 8):
     if node.op != AluOp.GlobalIndex:
         return None
     a = _lin(node.src[0], group)
-    if a is None or a[0] != 1:
+    if a is None or (group > 1 and a[0] != 1):
         return None
     idx0 = a[1].simplify()
     evar = AluExp.special(DType.Int32, "e", group)
@@ -186,6 +186,69 @@ def rows8_form(oexp: AluExp, extent: int, group: int = 8):
             cond_e = AluExp.mul(cond_e, x)
         cond_e = cond_e.simplify()
     return idx0, cond_e, node
+
+
+
+# ---- tap-major k order for convolution-like gather operands -----------------------------------------------------------
+#
+# The patch operand of a convolution reads element k = c * T + tap (T filter taps, tap fastest) of channel plane c:
+# its index is `plane(c) + window(row, tap)` and its padding mask does not depend on c at all.  Walking k in the order
+# k' = tap * C + c instead (a permutation of the reduction, applied to both operands alike) makes a slab of consecutive
+# k' one tap over consecutive channels: the index/mask arithmetic is done once per (rows, tap) and each further channel
+# costs one add and one load.
+
+def _has_special(e: AluExp, name: str) -> bool:
+    return bool(e.collect(lambda x: x.op == AluOp.Special and x.arg[0] == name))
+
+
+def _affine_in(e: AluExp, name: str):
+    """(coef, rest) with e == rest + coef * name, `name` reached only through +, - and * const; else None."""
+    if not _has_special(e, name):
+        return 0, e
+    if e.op == AluOp.Special:
+        return 1, AluExp.i32(0)
+    if e.dtype != DType.Int32:
+        return None
+    if e.op in (AluOp.Add, AluOp.Sub):
+        a, b = _affine_in(e.src[0], name), _affine_in(e.src[1], name)
+        if a is None or b is None:
+            return None
+        return (a[0] + b[0], AluExp.add(a[1], b[1])) if e.op == AluOp.Add else (a[0] - b[0], AluExp.sub(a[1], b[1]))
+    if e.op == AluOp.Mul:
+        for x, y in ((e.src[0], e.src[1]), (e.src[1], e.src[0])):
+            if y.op == AluOp.Const:
+                a = _affine_in(x, name)
+                return None if a is None else (a[0] * int(y.arg), AluExp.mul(a[1], y))
+    return None
+
+
+def tap_major_form(oexp: AluExp, K: int):
+    """For a gather operand's expression in (row, k, batch coordinates): try k = c * T + tap for every T that the
+    expression divides k by.  Returns dict(T, C, cs, exp) where `exp` is the operand re-expressed in (row, tap, batch
+    coordinates) at c = 0, the element of channel c sitting `c * cs` further on and the mask not involving c; or None."""
+    kvars = oexp.collect(lambda x: x.op == AluOp.Idiv and x.src[0].op == AluOp.Special and x.src[0].arg[0] == "k" and x.src[1].op == AluOp.Const)
+    cands = sorted({int(x.src[1].arg) for x in kvars}, reverse=True)
+    for T in cands:
+        if T <= 1 or K % T != 0 or (K // T) % 8 != 0:
+            continue
+        C = K // T
+        cvar, tvar = AluExp.special(DType.Int32, "c", C), AluExp.special(DType.Int32, "tap", T)
+        kexp = AluExp.add(AluExp.mul(cvar, AluExp.i32(T)), tvar)
+        e = oexp.rewrite(lambda n: kexp if (n.op == AluOp.Special and n.arg[0] == "k") else None).simplify()
+        node, cond = e, None
+        if node.op == AluOp.Where:
+            if node.src[2].op != AluOp.Const or float(node.src[2].arg) != 0.0:
+                continue
+            cond, node = node.src[0], node.src[1]
+        if node.op != AluOp.GlobalIndex or (cond is not None and _has_special(cond, "c")):
+            continue
+        a = _affine_in(node.src[0], "c")
+        if a is None or a[0] <= 0:
+            continue
+        base = AluExp.globalIndex(node.dtype, node.arg[0], node.arg[1], a[1].simplify())
+        exp0 = base if cond is None else AluExp.where(cond, base, e.src[2])
+        return dict(T=T, C=C, cs=a[0], exp=exp0)
+    return None
 
 
 def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelSource:
@@ -241,7 +304,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
 
     # Element loaders for gather operands: the operand's lowered expression (masked load through its view
     # chain) with the flat output index rebuilt from (tile row, batch coordinates) and ridx = k.
-    gather_fns, gather_calls, gather_flags, gather_group = [], {}, {}, {}
+    gather_fns, gather_calls, gather_flags, gather_group, gather_oexp, gather_slow = [], {}, {}, {}, {}, {}
     lowered = _strip_casts(t.exp)
     operand_exps = {g["gid_a"]: None, g["gid_b"]: None}
     if g.get("a_gather") or g.get("b_gather"):
@@ -269,6 +332,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                 return kvar
             return None
         oexp = operand_exps[gid].rewrite(_retarget_operand).simplify()
+        gather_oexp[tag] = oexp
         gcg = HipExpCodegen(names, {"row": "row", "k": "k", "b0": "b0", "b1": "b1", "b2": "b2"}, "  ", prefix=f"g{tag}", numerics=numerics)
         gcg.countReferences(oexp)
         gval = strip_parens(gcg.run(oexp))
@@ -300,27 +364,97 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                 mval = strip_parens(mcg.run(cond_e))
                 gather_fns.append(f"static __device__ __forceinline__ bool jh_gmask_{tag}(int row, int e, int k, int b0, int b1, int b2) {{\n"
                                   + "\n".join(mcg.take_lines()) + f"\n  return {mval};\n}}")
-                mask = f"if (!jh_gmask_{tag}(r, e, k, b0, b1, b2)) part[e] = (jh_f16)0;"
-            else:
-                mask = ""
             buf = names[gnode.arg[0]]
+            maskbit = f"jh_gmask_{tag}(r, e, k, b0, b1, b2)" if cond_e is not None else "true"
+            # The loader only forms addresses and mask bits and issues the loads (no use of the loaded data, no
+            # branches): the stager applies the mask when it writes the slab to LDS, one slab later, so the eight
+            # loads of a block are in flight together.  A group that would leave the buffer loads from a clamped
+            # address and is flagged; the stager replaces it through the out-of-line element loader afterwards.
             gather_fns.append(
                 f"typedef jh_f16 jh_part_{tag} __attribute__((ext_vector_type({G})));\n"
                 f"struct __attribute__((packed, aligned(2))) jh_part_u_{tag} {{ jh_part_{tag} v; }};\n"
-                f"static __device__ __attribute__((noinline)) jh_part_{tag} jh_gather_edge_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
-                f"  jh_part_{tag} part;\n#pragma unroll\n  for (int e = 0; e < {G}; ++e) part[e] = jh_gather_{tag}(row + e, k, b0, b1, b2{epi_args});\n  return part;\n}}\n"
-                f"static __device__ __forceinline__ jh_half8 jh_gather8_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
-                f"  jh_half8 v;\n#pragma unroll\n  for (int j = 0; j < {8 // G}; ++j) {{\n"
-                f"    const int r = row + j * {G};\n    const int i0 = jh_gindex_{tag}(r, k, b0, b1, b2);\n    jh_part_{tag} part;\n"
-                f"    if ((unsigned)i0 <= (unsigned)({gnode.arg[1]} - {G})) {{\n"
-                f"      part = reinterpret_cast<const jh_part_u_{tag}*>({buf} + i0)->v;\n"
-                f"#pragma unroll\n      for (int e = 0; e < {G}; ++e) {{ {mask} }}\n"
-                f"    }} else {{\n      part = jh_gather_edge_{tag}(r, k, b0, b1, b2{epi_args});\n    }}\n"
-                f"#pragma unroll\n    for (int e = 0; e < {G}; ++e) v[j * {G} + e] = part[e];\n  }}\n"
-                f"  return v;\n}}")
+                f"static __device__ __attribute__((noinline)) jh_half8 jh_gather8_slow_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
+                f"  jh_half8 v;\n#pragma unroll\n  for (int e = 0; e < 8; ++e) v[e] = jh_gather_{tag}(row + e, k, b0, b1, b2{epi_args});\n  return v;\n}}\n"
+                f"static __device__ __forceinline__ jh_g8 jh_gather8_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
+                f"  jh_g8 out;\n  out.keep = 0u;\n#pragma unroll\n  for (int j = 0; j < {8 // G}; ++j) {{\n"
+                f"    const int r = row + j * {G};\n    const int i0 = jh_gindex_{tag}(r, k, b0, b1, b2);\n"
+                f"    const bool inside = (unsigned)i0 <= (unsigned)({gnode.arg[1]} - {G});\n"
+                f"    if (!inside) out.keep |= 0x100u;\n"
+                f"    const jh_part_{tag} part = reinterpret_cast<const jh_part_u_{tag}*>({buf} + (inside ? i0 : 0))->v;\n"
+                f"#pragma unroll\n    for (int e = 0; e < {G}; ++e) {{ out.v[j * {G} + e] = part[e]; if ({maskbit}) out.keep |= 1u << (j * {G} + e); }}\n  }}\n"
+                f"  return out;\n}}")
+            gather_slow[tag] = f"jh_gather8_slow_{tag}(row, k, jh_b0, jh_b1, jh_b2{epi_args})"
             gather_calls[tag] = f"jh_gather8_{tag}(row, k, jh_b0, jh_b1, jh_b2{epi_args})"
             gather_flags[tag] = 2
             gather_group[tag] = G
+
+    # Tap-major k order (see `tap_major_form`): one gather operand whose k splits into (channel, tap), the other a plain
+    # strided operand.  Both are then loaded through block/chunk loaders that take the first k' of eight consecutive
+    # ones: k' = tap * C + c, original k = c * T + tap.
+    tap_major = None
+    gtags = [tg for tg in ("a", "b") if gather_flags[tg]]
+    if g["dtype"] == DType.Float16 and tile.get("TAPMAJOR", 0) and len(gtags) == 1 and g["K"] % 8 == 0:
+        gt = gtags[0]
+        pt = "b" if gt == "a" else "a"
+        tm = tap_major_form(gather_oexp[gt], g["K"])
+        plain_ok = g[f"{pt}_k0"] == g["K"] and not g.get(f"{pt}_gather")
+        if tm is not None and plain_ok:
+            form, G = None, 0
+            for G in (8, 4, 1):
+                form = rows8_form(tm["exp"], 0, G)
+                if form is not None:
+                    break
+            if form is not None:
+                idx0, cond_e, gnode = form
+                T, C, CS = tm["T"], tm["C"], tm["cs"]
+                vnames = {"row": "row", "e": "e", "tap": "tap", "b0": "b0", "b1": "b1", "b2": "b2"}
+                icg = HipExpCodegen(names, vnames, "  ", prefix=f"ti{gt}", numerics=numerics)
+                icg.countReferences(idx0)
+                ival = strip_parens(icg.run(idx0))
+                gather_fns.append(f"static __device__ __forceinline__ int jh_tindex_{gt}(int row, int tap, int b0, int b1, int b2) {{\n"
+                                  + "\n".join(icg.take_lines()) + f"\n  return {ival};\n}}")
+                if cond_e is not None:
+                    mcg = HipExpCodegen(names, vnames, "  ", prefix=f"tm{gt}", numerics=numerics)
+                    mcg.countReferences(cond_e)
+                    mval = strip_parens(mcg.run(cond_e))
+                    gather_fns.append(f"static __device__ __forceinline__ bool jh_tmask_{gt}(int row, int e, int tap, int b0, int b1, int b2) {{\n"
+                                      + "\n".join(mcg.take_lines()) + f"\n  return {mval};\n}}")
+                    mask_bits = f"jh_tmask_{gt}(r, e, tap, b0, b1, b2)"
+                else:
+                    mask_bits = "true"
+                buf, LEN, NG = names[gnode.arg[0]], gnode.arg[1], 8 // G
+                gather_fns.append(
+                    f"typedef jh_f16 jh_tpart_{gt} __attribute__((ext_vector_type({G})));\n"
+                    f"struct __attribute__((packed, aligned(2))) jh_tpart_u_{gt} {{ jh_tpart_{gt} v; }};\n"
+                    f"static __device__ __attribute__((noinline)) jh_half8 jh_gather8_tslow_{gt}(int row, int kp, int b0, int b1, int b2{epi_params}) {{\n"
+                    f"  const int tap = kp / {C};\n  const int k = (kp - tap * {C}) * {T} + tap;\n"
+                    f"  jh_half8 v;\n#pragma unroll\n  for (int e = 0; e < 8; ++e) v[e] = jh_gather_{gt}(row + e, k, b0, b1, b2{epi_args});\n  return v;\n}}\n"
+                    f"// Eight consecutive k' (one tap, channels c0 .. c0+7) of eight consecutive rows: loads only; the mask (one\n"
+                    f"// per block, it does not depend on the channel) is applied when the block is written to LDS.\n"
+                    f"static __device__ __forceinline__ jh_gblock jh_gather_block_{gt}(int row, int kbase, int b0, int b1, int b2{epi_params}) {{\n"
+                    f"  jh_gblock out;\n  out.keep = 0u;\n  const int tap = kbase / {C};\n  const int c0 = kbase - tap * {C};\n"
+                    f"#pragma unroll\n  for (int j = 0; j < {NG}; ++j) {{\n    const int r = row + j * {G};\n"
+                    f"    const int i0 = jh_tindex_{gt}(r, tap, b0, b1, b2) + c0 * {CS};\n"
+                    f"    const bool inside = i0 >= 0 && (long long)i0 + 7ll * {CS} <= {LEN}ll - {G};\n"
+                    f"    if (!inside) out.keep |= 0x100u;\n"
+                    f"#pragma unroll\n    for (int e = 0; e < {G}; ++e) if ({mask_bits}) out.keep |= 1u << (j * {G} + e);\n"
+                    f"    const jh_f16* const src = {buf} + (inside ? i0 : 0);\n"
+                    f"#pragma unroll\n    for (int i = 0; i < 8; ++i) {{\n"
+                    f"      const jh_tpart_{gt} part = reinterpret_cast<const jh_tpart_u_{gt}*>(src + (inside ? i * {CS} : 0))->v;\n"
+                    f"#pragma unroll\n      for (int e = 0; e < {G}; ++e) out.v[i][j * {G} + e] = part[e];\n    }}\n  }}\n  return out;\n}}")
+                gather_slow[gt] = f"jh_gather8_tslow_{gt}(row, k, jh_b0, jh_b1, jh_b2{epi_args})"
+                gather_calls[gt] = f"jh_gather_block_{gt}(row, k, jh_b0, jh_b1, jh_b2{epi_args})"
+                gather_flags[gt], gather_group[gt] = 3, G
+                # the plain operand, eight consecutive k' at a time: elements T * stride apart
+                srow, sk = (g["a_sm"], g["a_sk"]) if pt == "a" else (g["b_sn"], g["b_sk"])
+                gather_fns.append(
+                    f"static __device__ __forceinline__ jh_half8 jh_gather_chunk_{pt}(const jh_f16* __restrict__ base, int row, int kbase) {{\n"
+                    f"  const int tap = kbase / {C};\n  const int c0 = kbase - tap * {C};\n"
+                    f"  const jh_f16* p = base + (long long)row * {srow}ll + ((long long)c0 * {T} + tap) * {sk}ll;\n  jh_half8 v;\n"
+                    f"#pragma unroll\n  for (int e = 0; e < 8; ++e) v[e] = p[(long long)e * {T * sk}ll];\n  return v;\n}}")
+                gather_calls[pt] = f"jh_gather_chunk_{pt}({'Ap' if pt == 'a' else 'Bp'}, row, k)"
+                gather_flags[pt] = 4
+                tap_major = dict(T=T, C=C, group=G)
 
     # Batch index decode, innermost batch axis last in g["batch"].
     lines = ["  {", "    int rem = batch;"]
@@ -362,11 +496,12 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         sched = {}
     if not dlds:
         sched.update(GATHER_FNS="\n".join(gather_fns), A_GATHER=gather_flags["a"], B_GATHER=gather_flags["b"],
-                     GATHER_A_CALL=gather_calls["a"], GATHER_B_CALL=gather_calls["b"])
+                     GATHER_A_CALL=gather_calls["a"], GATHER_B_CALL=gather_calls["b"],
+                     GATHER_A_SLOW=gather_slow.get("a", "jh_half8{0, 0, 0, 0, 0, 0, 0, 0}"), GATHER_B_SLOW=gather_slow.get("b", "jh_half8{0, 0, 0, 0, 0, 0, 0, 0}"))
     src = _prelude(numerics) + fill(template(tmpl), dict(sched, 
         M=g["M"], N=g["N"], K=g["K"], BM=BM, BN=BN, WM=WM, WN=WN,
-        A_KCONTIG=0 if gather_flags["a"] == 2 else (1 if g["a_sk"] == 1 or g["K"] == 1 or g.get("a_gather") else 0),
-        B_KCONTIG=0 if gather_flags["b"] == 2 else (1 if g["b_sk"] == 1 or g["K"] == 1 or g.get("b_gather") else 0),
+        A_KCONTIG=0 if gather_flags["a"] in (2, 3) else (1 if g["a_sk"] == 1 or g["K"] == 1 or gather_flags["a"] in (1, 4) else 0),
+        B_KCONTIG=0 if gather_flags["b"] in (2, 3) else (1 if g["b_sk"] == 1 or g["K"] == 1 or gather_flags["b"] in (1, 4) else 0),
         NBATCH=nbatch, EPILOGUE_FN=epi_fn, NAME=name, PARAMS=params,
         A_OFF=g["a_off"], B_OFF=g["b_off"], BATCH_DECODE="\n".join(lines),
         A_PTR=names[g["gid_a"]], B_PTR=names[g["gid_b"]],
@@ -385,5 +520,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     info = dict(BM=BM, BN=BN, WM=WM, WN=WN, BK=32 if dlds else (64 if g["dtype"] == DType.Float16 else 16), direct_lds=bool(dlds), tiles=tiles, a_kcontig=g["a_sk"] == 1, b_kcontig=g["b_sk"] == 1,
                 M=g["M"], N=g["N"], K=g["K"], nbatch=nbatch)
     if any_gather:
-        info["gather"] = {tag: {0: "none", 1: "element", 2: f"rows{gather_group.get(tag, 8)}"}[gather_flags[tag]] for tag in ("a", "b")}
+        info["gather"] = {tag: {0: "none", 1: "element", 2: f"rows{gather_group.get(tag, 8)}", 3: f"tap-major rows{gather_group.get(tag, 8)}",
+                                4: "tap-major strided"}[gather_flags[tag]] for tag in ("a", "b")}
+        if tap_major is not None:
+            info["tap_major"] = tap_major
     return KernelSource([src], [step], [], "gemm", need, info)

@@ -215,8 +215,8 @@ def test_resnet_shaped_convolution_and_pooling_on_gpu():
 
 
 # f16 convolutions whose image operand is (or is not) eligible for the row-vector gather loader: image widths that are
-# a multiple of 8 or of 4 only (shorter vectors), other widths (element loader), padding on every
-# side, dilation, more than two spatial dims, strides (element loader), ragged pixel counts.
+# a multiple of 8 or of 4 only (shorter vectors), other widths and strides (element loader), padding on every
+# side, dilation, one to three spatial dims, ragged pixel counts.
 F16_CONV_CASES = [
     dict(x=(2, 8, 16, 16), w=(32, 8, 3, 3), strides=[1, 1], padding="SAME", loader="rows8"),
     dict(x=(3, 16, 8, 24), w=(32, 16, 3, 3), strides=[1, 1], padding="SAME", loader="rows8"),
@@ -247,23 +247,34 @@ def test_f16_convolution_loader_choice(case):
         assert "gather" not in ks.info or set(ks.info["gather"].values()) == {"none"}
     else:
         assert ks.klass == "gemm" and case["loader"] in ks.info["gather"].values(), ks.info
+        # the optional tap-major k order (k' = tap * C + c) applies to every one of them
+        tm = generate(_f16_conv_program(case).kernels[0], gemm_tile=(("TAPMAJOR", 1),))
+        assert tm.info["tap_major"]["T"] == int(np.prod(case["w"][2:])) and any(v.startswith("tap-major rows") for v in tm.info["gather"].values())
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("tap_major", [0, 1], ids=["k-order", "tap-major"])
 @pytest.mark.parametrize("case", F16_CONV_CASES, ids=lambda c: "x".join(map(str, c["x"])) + "*" + "x".join(map(str, c["w"])))
-def test_f16_convolution_on_gpu_is_exact_on_small_integers(case):
+def test_f16_convolution_on_gpu_is_exact_on_small_integers(case, tap_major):
     from gpu_util import WARM_ONLY, backend
     prog = _f16_conv_program(case)
+    opts = dict(gemm_tile=(("TAPMAJOR", 1),)) if tap_major else {}
     if WARM_ONLY:
         from jaxjs_hip.kernelgen import generate
         from jaxjs_hip.runtime import compile_source
-        for src in generate(prog.kernels[0]).sources:
+        for src in generate(prog.kernels[0], **opts).sources:
             compile_source(src)
         pytest.skip("warm-up run: compiled only")
     rng = np.random.default_rng(12)
     x = rng.integers(-2, 3, case["x"]).astype(np.float16)
     w = rng.integers(-2, 3, case["w"]).astype(np.float16)
-    (r,) = run_program(backend(), prog, [x, w])
+    be = backend()
+    exe = be.prepareKernelSync(prog.kernels[0], **opts)
+    sx, sw, so = be.malloc(x.nbytes, x.tobytes()), be.malloc(w.nbytes, w.tobytes()), be.malloc(prog.kernels[0].bytes)
+    be.dispatch(exe, [sx, sw], [so])
+    r = np.frombuffer(be.readSync(so), np.float16).copy()
+    for s_ in (sx, sw, so):
+        be.decRef(s_)
     pads = case["padding"]
     if isinstance(pads, str):
         pads = L.padtypeToPads(case["x"][2:], case["w"][2:], case["strides"], case.get("rd") or [1] * len(case["strides"]), pads)
