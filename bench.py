@@ -208,6 +208,69 @@ def bench_program_gpt2(be, hostrand, timed):
             "model_flops": flops, "TFLOP/s": round(flops / (total_ms * 1e-3) / 1e12, 1), "per_kernel": kernels}
 
 
+def bench_program_gpt2_fused(be, hostrand, timed):
+    """The same block traced with the backend's fused `Attention` routine in place of the reference's seven attention
+    kernels (a front-end switch, not the reference's composition): whole program eager and as a HIP graph, and the
+    attention launch alone (causal: FLOP counted for the visible half of the score matrix plus the diagonal blocks)."""
+    from jaxjs_hip import workloads as W
+    from jaxjs_hip.graph import GraphedProgram
+
+    batch, seq, d, heads, d_ff = 8, 1024, 768, 12, 3072
+    prog = W.gpt2BlockProgram(batch, seq, d, heads, d_ff, fusedAttention=True)
+    shapes = W.gpt2BlockShapes(batch, seq, d, d_ff)
+    order = ["x"] + list(W.GPT2_BLOCK_PARAMS)
+    ins = []
+    for j, name in enumerate(order):
+        if name in ("ln1_g", "ln2_g"):
+            arr = np.ones(shapes[name], np.float16)
+        elif name in ("ln1_b", "ln2_b"):
+            arr = np.zeros(shapes[name], np.float16)
+        else:
+            arr = hostrand.normal(1005, shapes[name], 0.02, np.float16, stream=j)
+        ins.append(upload(be, arr))
+    assert not prog.consts
+    prepared = prog.prepare(be)
+    dev = be.dev
+
+    def measure(fn, reps=10):
+        for _ in range(5):
+            fn()
+        dev.sync()
+        e0, e1 = dev.event(), dev.event()
+        dev.record(e0)
+        for _ in range(reps):
+            fn()
+        dev.record(e1)
+        dev.sync()
+        ms = dev.elapsed_ms(e0, e1) / reps
+        dev.destroy_event(e0)
+        dev.destroy_event(e1)
+        return ms
+
+    def eager():
+        for o in prog.execute(be, ins, prepared):
+            be.decRef(o)
+
+    eager_ms = measure(eager)
+    gp = GraphedProgram(be, prog, ins)
+    graph_ms = measure(gp.launch)
+    gp.close()
+    # the attention launch alone, on operands of the block's shape
+    step = next(s for s in prog.steps if s.kind == "execute" and s.routine is not None)
+    qkv = [upload(be, hostrand.normal(1006, (batch, seq, heads, d // heads), 1.0, np.float16, stream=j)) for j in range(3)]
+    out = be.malloc(batch * seq * d * 2)
+    exe = be.prepareRoutineSync(step.routine)
+    attn_ms = measure(lambda: be.dispatch(exe, qkv, [out]), reps=50)
+    for sl in ins + qkv + [out]:
+        be.decRef(sl)
+    H = d // heads
+    full = 4.0 * batch * heads * seq * seq * H
+    return {"steps_in_program": sum(1 for s in prog.steps if s.kind == "execute"), "ms": round(eager_ms, 4), "ms_as_hip_graph": round(graph_ms, 4),
+            "TFLOP/s": round(1.417e11 / (eager_ms * 1e-3) / 1e12, 1),
+            "attention_alone": {"ms": round(attn_ms, 5), "TFLOP/s_full_matrix_convention": round(full / (attn_ms * 1e-3) / 1e12, 1),
+                                "TFLOP/s_causal_half": round(full / 2 / (attn_ms * 1e-3) / 1e12, 1)}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -354,6 +417,7 @@ def main():
         del Am, Bm
 
         extra["c5_gpt2_block_b8_l1024_f16"] = bench_program_gpt2(be, hostrand, timed)
+        extra["c5_gpt2_block_b8_l1024_f16_fused_attention"] = bench_program_gpt2_fused(be, hostrand, timed)
 
         # Convolution through the view algebra (no implicit-GEMM class yet: the kernel takes a generic reduce class).
         from jaxjs_hip import jit as J, library as Lb

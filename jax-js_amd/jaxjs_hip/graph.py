@@ -25,15 +25,19 @@ class GraphedProgram:
             backend.incRef(s)
             self._owned.append(s)
         steps = [s for s in prog.steps if s.kind == "execute"]
-        exes = [backend.prepareKernelSync(s.kernel) for s in steps]  # compile + load before any capture
+        # compile + load before any capture; a routine step is several launches and outputs, recorded the same way
+        exes = [backend.prepareRoutineSync(s.routine) if s.routine is not None else backend.prepareKernelSync(s.kernel) for s in steps]
+        sizes = {s.output: s.size for s in prog.steps if s.kind == "malloc"}
         for s in steps:
-            slot = backend.malloc(s.kernel.bytes)
-            self._slots[s.output] = slot
-            self._owned.append(slot)
+            for o in (s.outputs if s.routine is not None else [s.output]):
+                slot = backend.malloc(sizes[o])
+                self._slots[o] = slot
+                self._owned.append(slot)
 
         def issue():
             for s, exe in zip(steps, exes):
-                backend.dispatch(exe, [self._slots[i] for i in s.inputs], [self._slots[s.output]])
+                outs = s.outputs if s.routine is not None else [s.output]
+                backend.dispatch(exe, [self._slots[i] for i in s.inputs], [self._slots[o] for o in outs])
 
         issue()  # one eager pass: every code object is resident before the capture starts
         backend.dev.sync()

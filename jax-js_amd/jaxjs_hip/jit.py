@@ -122,7 +122,8 @@ BINARY_FUSABLE = ("Add", "Mul", "Idiv", "Mod", "Min", "Max", "BitCombine", "BitS
 # Primitives handed to the backend as a unit (src/frontend/core.ts:154-163): primitive name == routine name.
 # Their outputs index their inputs in several different ways: always dispatched (src/frontend/jit.ts:972-977).
 HETEROGENEOUS_VIEW_PRIMITIVES = ("RandomBits", "Gather")
-ROUTINE_PRIMITIVES = ("Sort", "Argsort", "Scatter", "TriangularSolve", "Cholesky", "LU", "JacobiEigh", "Fft")
+ROUTINE_PRIMITIVES = ("Sort", "Argsort", "Scatter", "TriangularSolve", "Cholesky", "LU", "JacobiEigh", "Fft",
+                      "Attention")  # the last one is this backend's extension (fused attention), see routine.py
 
 
 @dataclass
@@ -443,6 +444,11 @@ def _routine_out_avals(prim: str, avals: List[ShapedArray], params: Dict[str, An
             raise TypeError("lu: requires at least 2D input")
         batch, (m, n) = tuple(a.shape[:-2]), a.shape[-2:]
         return [same, ShapedArray(batch + (min(m, n),), DType.Int32, False), ShapedArray(batch + (m,), DType.Int32, False)]
+    if prim == "Attention":
+        k, v = avals[1], avals[2]
+        if a.ndim != 4 or tuple(k.shape) != tuple(v.shape) or k.ndim != 4 or (k.shape[0], k.shape[2], k.shape[3]) != (a.shape[0], a.shape[2], a.shape[3]):
+            raise TypeError(f"attention: shape mismatch q={a.shape} k={k.shape} v={v.shape}")
+        return [same]
     if prim == "Fft":
         b = avals[1]
         if tuple(a.shape) != tuple(b.shape) or a.dtype != b.dtype:
@@ -601,6 +607,11 @@ def lu(x):
 
 def jacobiEigh(x, maxSweeps: int, tolerance: float):
     return tuple(bind("JacobiEigh", [x], dict(maxSweeps=int(maxSweeps), tolerance=float(tolerance))))
+
+
+def attention(q, k, v, scale: float, isCausal: bool):
+    """Fused scaled-dot-product attention as one backend routine (an extension; the reference composes it)."""
+    return bind("Attention", [q, k, v], dict(scale=float(scale), isCausal=bool(isCausal)))[0]
 
 
 def fft(real, imag, factors, inverse: bool):

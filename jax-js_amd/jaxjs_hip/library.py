@@ -169,13 +169,20 @@ def argmax(a: Tracer, axis: int):
     return length.sub(idx.max(axis))
 
 
-def dotProductAttention(query: Tracer, key: Tracer, value: Tracer, isCausal: bool = False, scale: Optional[float] = None):
-    """[B,L,N,H] attention with equal query and key/value head counts (nn.ts:478-583)."""
+def dotProductAttention(query: Tracer, key: Tracer, value: Tracer, isCausal: bool = False, scale: Optional[float] = None,
+                        fused: bool = False):
+    """[B,L,N,H] attention with equal query and key/value head counts (nn.ts:478-583).  `fused=True` hands the whole
+    chain to the backend as one `Attention` routine when the shapes fit its kernel (float16, head size 64, L a multiple
+    of 128, S of 64) -- a front-end switch the reference does not have; otherwise the reference's composition is
+    traced."""
     B, L, N, H = query.shape
     S = key.shape[1]
     if key.shape != value.shape or key.shape[0] != B or key.shape[3] != H or key.shape[2] != N:
         raise ValueError("dotProductAttention: shape mismatch")
     scale = 1 / math.sqrt(H) if scale is None else scale
+    if (fused and H == 64 and L % 128 == 0 and S % 64 == 0
+            and all(t.dtype == DType.Float16 for t in (query, key, value))):
+        return J.attention(query, key, value, scale, isCausal)
     scores = einsum("BLNH,BSNH->BNLS", query, key).mul(scale)
     if isCausal:
         scores = J.where(tri_const(L, S, 0), scores, -math.inf)

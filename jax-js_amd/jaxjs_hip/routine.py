@@ -24,6 +24,10 @@ class Routines(str, Enum):
     LU = "LU"
     JacobiEigh = "JacobiEigh"
     Fft = "Fft"
+    # Not in the reference's enum: fused scaled-dot-product attention (the front-end change src/library/nn.ts:478-583
+    # would need in order to hand the whole QK^T -> mask -> softmax -> PV chain to a backend as one unit).
+    # Inputs q [B,L,N,H], k and v [B,S,N,H]; output [B,L,N,H]; params {scale, isCausal}.
+    Attention = "Attention"
 
     def __str__(self):
         return self.value

@@ -8,6 +8,7 @@ time, which is what the Backend interface prescribes for a routine a backend lac
   Scatter                                     `scatter.hip.inc`  float32/float16/int32/uint32/bool updates
   TriangularSolve, Cholesky, LU, JacobiEigh   `linalg.hip.inc`   float32
   Fft                                         `fft.hip.inc`      float32
+  Attention (extension, not in the reference) `attention.hip.inc` float16, head size 64
 """
 
 from __future__ import annotations
@@ -35,7 +36,7 @@ def _next_pow2(n: int) -> int:
 def generateRoutine(routine: Routine, numerics: str = "wasm") -> KernelSource:
     gen = {Routines.Sort: _gen_sort, Routines.Argsort: _gen_sort, Routines.Scatter: _gen_scatter,
            Routines.TriangularSolve: _gen_trisolve, Routines.Cholesky: _gen_cholesky, Routines.LU: _gen_lu,
-           Routines.JacobiEigh: _gen_jacobi, Routines.Fft: _gen_fft}.get(routine.name)
+           Routines.JacobiEigh: _gen_jacobi, Routines.Fft: _gen_fft, Routines.Attention: _gen_attention}.get(routine.name)
     ks = gen(routine, numerics) if gen is not None else None
     if ks is None:
         raise UnsupportedRoutineError(routine.name, "hip")
@@ -284,3 +285,34 @@ def _gen_sort(routine: Routine, numerics: str) -> Optional[KernelSource]:
     scratch = [rows * P * 8] if P > tile else [8]
     need = {0: rows * n * byteWidth(dtype)}
     return KernelSource([src], steps, scratch, "sort", need, dict(n=n, rows=rows, P=P, tile=tile, argsort=argsort, launches=len(steps)))
+
+
+def _gen_attention(routine: Routine, numerics: str) -> Optional[KernelSource]:
+    """Fused attention over contiguous [B, L, N, 64] / [B, S, N, 64] float16 operands."""
+    import math
+
+    t = routine.type
+    params = routine.params or {}
+    if len(t.inputShapes) != 3 or any(len(s) != 4 for s in t.inputShapes):
+        raise ValueError("attention: expected q [B,L,N,H], k [B,S,N,H], v [B,S,N,H]")
+    (B, L, N, H), ks, vs = t.inputShapes
+    if list(ks) != list(vs) or ks[0] != B or ks[2] != N or ks[3] != H:
+        raise ValueError(f"attention: shape mismatch q={t.inputShapes[0]} k={ks} v={vs}")
+    S = ks[1]
+    if any(d != DType.Float16 for d in t.inputDtypes) or H != 64 or L % 128 != 0 or S % 64 != 0:
+        return None
+    if B * N * L == 0:
+        return _empty("attention", B=B, L=L, S=S, N=N)
+    if B * N * (L // 128) >= (1 << 31) or max(B * L * N * H, B * S * N * H) >= (1 << 31):
+        return None
+    scale = float(params.get("scale", 1 / math.sqrt(H)))
+    strides = lambda T: dict(B=T * N * H, P=N * H, N=H)  # noqa: E731  contiguous [B, T, N, H]
+    sq, sk = strides(L), strides(S)
+    src = _prelude(numerics) + fill(template("attention.hip.inc"), dict(
+        B=B, NH=N, L=L, S=S, CAUSAL=1 if params.get("isCausal") else 0, SCALE_LOG2E=repr(scale * math.log2(math.e)),
+        QB=sq["B"], QL=sq["P"], QN=sq["N"], KB=sk["B"], KS=sk["P"], KN=sk["N"], VB=sk["B"], VS=sk["P"], VN=sk["N"],
+        OB=sq["B"], OL=sq["P"], ON=sq["N"]))
+    blocks = B * N * (L // 128)
+    steps = [LaunchStep("jh_attention", (blocks, 1, 1), (256, 1, 1), 0, [("in", 0), ("in", 1), ("in", 2), ("out", 0)])]
+    need = {0: B * L * N * H * 2, 1: B * S * N * H * 2, 2: B * S * N * H * 2}
+    return KernelSource([src], steps, [], "attention", need, dict(B=B, L=L, S=S, N=N, H=H, causal=bool(params.get("isCausal")), blocks=blocks))

@@ -31,10 +31,12 @@ def gpt2BlockShapes(batch: int, seq: int, d_model: int, d_ff: int) -> Dict[str, 
                 w_fc1=(d_model, d_ff), b_fc1=(d_ff,), w_fc2=(d_ff, d_model), b_fc2=(d_model,))
 
 
-def gpt2BlockProgram(batch: int, seq: int, d_model: int, heads: int, d_ff: int, dtype: DType = DType.Float16) -> JitProgram:
+def gpt2BlockProgram(batch: int, seq: int, d_model: int, heads: int, d_ff: int, dtype: DType = DType.Float16,
+                     fusedAttention: bool = False) -> JitProgram:
     """Pre-LayerNorm transformer block forward under one jit: LayerNorm (standardize * g + b), fused QKV
     projection with bias, causal softmax attention, output projection + residual, LayerNorm, tanh-GELU MLP +
-    residual.  Inputs in order: x, then GPT2_BLOCK_PARAMS (weights stored [in, out])."""
+    residual.  Inputs in order: x, then GPT2_BLOCK_PARAMS (weights stored [in, out]).  `fusedAttention` traces
+    the attention chain as the backend's `Attention` routine instead of the reference's seven kernels."""
     H = d_model // heads
     shapes = gpt2BlockShapes(batch, seq, d_model, d_ff)
 
@@ -43,7 +45,7 @@ def gpt2BlockProgram(batch: int, seq: int, d_model: int, heads: int, d_ff: int, 
         qkv = L.matmul(h, w_qkv).add(b_qkv)
         full = [(0, batch), (0, seq)]
         q, k, v = (J.shrink(qkv, full + [(i * d_model, (i + 1) * d_model)]).reshape([batch, seq, heads, H]) for i in range(3))
-        a = L.dotProductAttention(q, k, v, isCausal=True).reshape([batch, seq, d_model])
+        a = L.dotProductAttention(q, k, v, isCausal=True, fused=fusedAttention).reshape([batch, seq, d_model])
         x = x.add(L.matmul(a, w_o).add(b_o))
         h = L.standardize(x).mul(ln2_g).add(ln2_b)
         m = L.gelu(L.matmul(h, w_fc1).add(b_fc1))

@@ -5,6 +5,7 @@ run as GPU kernels or raise.
   Sort / Argsort      numpy (TypedArray.prototype.sort order: NaNs last; Argsort stable)   src/routine.ts:185-213
   Scatter             numpy, sequential semantics (later updates win, adds in order)        src/routine.ts:226-296
   TriangularSolve, Cholesky, LU, JacobiEigh, Fft   C (`routines_oracle.c`), float32 only    src/routine.ts:298-640
+  Attention           numpy float64 (the fused-attention extension)                        src/library/nn.ts:478-583
 
 Parity pinning: the linear-algebra and FFT functions are checked in `tests/test_routines_oracle.py` against what
 the mathematics fixes (reconstruction identities, numpy.linalg / numpy.fft / scipy on well-conditioned inputs)
@@ -149,8 +150,26 @@ def runCpuRoutine(routine, inputs: Sequence, outputs: Sequence) -> None:
         if lib().ro_fft(_ptr(re), _ptr(im), _ptr(o_re), _ptr(o_im), re.size // n, n, _ptr(factors), len(factors), int(bool(params["inverse"]))):
             raise MemoryError("fft oracle: allocation failed")
         outs[0][...], outs[1][...] = o_re, o_im
+    elif name == "Attention":
+        outs[0][...] = attention(ins[0], ins[1], ins[2], float(params["scale"]), bool(params.get("isCausal", False))).astype(outs[0].dtype)
     else:
         raise NotImplementedError(name)
+
+
+def attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float, causal: bool) -> np.ndarray:
+    """softmax_s(scale * q.k (+ mask s <= l)) @ v over [B,L,N,H] / [B,S,N,H] operands, in float64: the function the
+    reference's dotProductAttention composes from einsum, where(tri) and softmax (src/library/nn.ts:478-583).  Not a
+    reference routine; it checks the fused GPU kernel, and is itself checked against the unfused composition replayed
+    kernel by kernel on the CPU checker."""
+    q64, k64, v64 = q.astype(np.float64), k.astype(np.float64), v.astype(np.float64)
+    scores = np.einsum("blnh,bsnh->bnls", q64, k64) * scale
+    if causal:
+        L, S = scores.shape[-2:]
+        scores = np.where(np.arange(S)[None, :] <= np.arange(L)[:, None], scores, -np.inf)
+    scores = scores - scores.max(axis=-1, keepdims=True)
+    p = np.exp(scores)
+    p /= p.sum(axis=-1, keepdims=True)
+    return np.einsum("bnls,bsnh->blnh", p, v64)
 
 
 def scatter(t, ins: List[np.ndarray], out: np.ndarray, params: dict) -> None:

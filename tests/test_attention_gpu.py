@@ -1,0 +1,83 @@
+"""The fused attention kernel (an extension routine, `Routines.Attention`) on the GPU against the float64 checker, and
+the GPT-2 block traced with it against the block traced the reference's way.  Float16 in, float16 out, f32 softmax
+statistics: bound = 1e-2 relative + a few f16 ulps of values of order 1 (the stated f16 tolerance)."""
+import math
+
+import numpy as np
+import pytest
+
+import routine_util as R
+from gpu_util import WARM_ONLY, backend
+from jaxjs_hip import DType
+from jaxjs_hip import workloads as W
+from jaxjs_hip.errors import UnsupportedRoutineError
+from jaxjs_hip.routine import Routine, Routines, RoutineType
+from jit_util import run_program
+from test_jit import block_inputs, block_reference
+
+pytestmark = pytest.mark.gpu
+F16 = DType.Float16
+
+
+def attention_routine(B, L, S, N, causal, scale=None, H=64):
+    t = RoutineType([[B, L, N, H], [B, S, N, H], [B, S, N, H]], [F16] * 3, [[B, L, N, H]], [F16])
+    return Routine(Routines.Attention, t, dict(scale=1 / math.sqrt(H) if scale is None else scale, isCausal=causal))
+
+
+CASES = [(1, 128, 64, 1), (1, 128, 128, 1), (2, 256, 256, 3), (1, 384, 192, 2), (1, 128, 320, 2), (2, 1024, 1024, 4)]
+
+
+@pytest.mark.parametrize("causal", [False, True], ids=["full", "causal"])
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "B%d_L%d_S%d_N%d" % c)
+def test_attention_matches_float64(case, causal):
+    B, L, S, N = case
+    rng = np.random.default_rng(B * 1000 + L + S + N)
+    q, k, v = [rng.standard_normal((B, T, N, 64)).astype(np.float16) for T in (L, S, S)]
+    routine = attention_routine(B, L, S, N, causal)
+    got, ks = R.run_gpu(routine, [q, k, v])
+    want = R.run_oracle(routine, [q, k, v])
+    np.testing.assert_allclose(got[0].astype(np.float64), want[0].astype(np.float64), rtol=1e-2, atol=3e-3, err_msg=str(ks.info))
+
+
+def test_attention_is_stable_for_large_scores_and_peaked_rows():
+    rng = np.random.default_rng(4)
+    q, k, v = [rng.standard_normal((1, 256, 2, 64)).astype(np.float16) for _ in range(3)]
+    q *= np.float16(6.0)   # scores of order +-50: exp would overflow f16/f32 without the running maximum
+    k[:, 17] *= np.float16(4.0)  # one dominant key
+    for causal in (False, True):
+        routine = attention_routine(1, 256, 256, 2, causal, scale=1.0)
+        got, _ = R.run_gpu(routine, [q, k, v])
+        want = R.run_oracle(routine, [q, k, v])
+        assert np.isfinite(got[0]).all()
+        np.testing.assert_allclose(got[0].astype(np.float64), want[0].astype(np.float64), rtol=1e-2, atol=4e-3)
+
+
+def test_shapes_outside_the_kernel_are_refused_not_faked():
+    if WARM_ONLY:
+        pytest.skip("nothing to compile")
+    be = backend()
+    for routine in (attention_routine(1, 100, 128, 1, False), attention_routine(1, 128, 100, 1, False), attention_routine(1, 128, 128, 1, False, H=32)):
+        with pytest.raises(UnsupportedRoutineError):
+            be.prepareRoutineSync(routine)
+
+
+def test_gpt2_block_with_fused_attention():
+    """Small block (d=128, 2 heads of 64): fused against the float64 block restatement and against the unfused program
+    on the same GPU.  The front-end switch falls back to the reference's composition when the shapes do not fit."""
+    batch, seq, d, heads, d_ff = 2, 128, 128, 2, 512
+    fused = W.gpt2BlockProgram(batch, seq, d, heads, d_ff, fusedAttention=True)
+    plain = W.gpt2BlockProgram(batch, seq, d, heads, d_ff)
+    assert [r.name for r in fused.routines] == [Routines.Attention] and not plain.routines
+    assert len(fused.kernels) == len(plain.kernels) - 7 + 3  # seven attention kernels out, three operand copies in
+    assert not W.gpt2BlockProgram(batch, 64, d, heads, d_ff, fusedAttention=True).routines  # L = 64: composition kept
+    if WARM_ONLY:
+        from test_programs_gpu import warm
+        warm(fused)
+    arrs = block_inputs(batch, seq, d, d_ff, np.float16)
+    order = ["x"] + list(W.GPT2_BLOCK_PARAMS)
+    arrays = [arrs[n] for n in order]
+    (y,) = run_program(backend(), fused, arrays)
+    (y0,) = run_program(backend(), plain, arrays)
+    want = block_reference(arrs["x"].astype(np.float64), {n: arrs[n].astype(np.float64) for n in order[1:]}, heads)
+    np.testing.assert_allclose(y.astype(np.float64).reshape(batch, seq, d), want, rtol=3e-2, atol=3e-2)
+    np.testing.assert_allclose(y.astype(np.float64), y0.astype(np.float64), rtol=2e-2, atol=2e-2)

@@ -28,7 +28,12 @@ def _check_program(prog, make_arrays, rounds=3):
     arrays = make_arrays(0)
     in_slots = [be.malloc(a.nbytes, a.tobytes()) for a in arrays]
     g = GraphedProgram(be, prog, const_slots + in_slots)
-    out_dtypes = {s.output: s.kernel.dtype for s in prog.steps if s.kind == "execute"}
+    out_dtypes = {}
+    for s in prog.steps:
+        if s.kind == "execute" and s.routine is not None:
+            out_dtypes.update(zip(s.outputs, s.routine.type.outputDtypes))
+        elif s.kind == "execute":
+            out_dtypes[s.output] = s.kernel.dtype
     try:
         for r in range(rounds):
             if r > 0:  # new input values, written into the slots the graph was captured with
@@ -66,3 +71,29 @@ def test_gpt2_block_graph():
         a = block_inputs(batch, seq, d, d_ff, np.float16, seed=100 + r)
         return [a[n] for n in order]
     _check_program(prog, arrays)
+
+
+def test_graph_replay_of_programs_with_routine_steps():
+    """Routine steps (several launches, several outputs) are captured like kernels: LU + triangular solves (`solve`) and
+    the block with the fused-attention routine replay bit for bit what the eager path gives."""
+    from jaxjs_hip import jit as J
+    from jaxjs_hip import library as L
+    from jaxjs_hip.alu import DType
+    from jaxjs_hip.jit import ShapedArray
+    solve = J.jit(lambda x, y: L.solve(x, y), [ShapedArray((4, 40, 40), DType.Float32), ShapedArray((4, 40, 3), DType.Float32)])
+    batch, seq, d, heads, d_ff = 2, 128, 128, 2, 512
+    block = W.gpt2BlockProgram(batch, seq, d, heads, d_ff, fusedAttention=True)
+    assert solve.routines and block.routines
+    if WARM_ONLY:
+        pytest.skip("kernels are compiled by the program tests")
+
+    def systems(r):
+        rng = np.random.default_rng(r)
+        return [(rng.standard_normal((4, 40, 40)) + 6 * np.eye(40)).astype(np.float32), rng.standard_normal((4, 40, 3)).astype(np.float32)]
+    _check_program(solve, systems)
+    order = ["x"] + list(W.GPT2_BLOCK_PARAMS)
+
+    def arrays(r):
+        a = block_inputs(batch, seq, d, d_ff, np.float16, seed=200 + r)
+        return [a[n] for n in order]
+    _check_program(block, arrays)

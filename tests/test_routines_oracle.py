@@ -207,3 +207,36 @@ def test_fft_reference_tables_and_any_factor_order():
     for factors in ([4, 3, 5], [5, 3, 4], [2, 2, 15], [60]):
         re, im = R.run_oracle(R.fft(xr, xi, False, factors), [xr, xi])
         np.testing.assert_allclose(re + 1j * im, want, atol=2e-5)
+
+
+def test_attention_checker_against_reference_tables_and_composition():
+    """The fused-attention checker (not a reference routine): the reference's dotProductAttention tables
+    (test/nn.test.ts:274-390) and, on random float16 operands, the unfused composition replayed kernel by kernel."""
+    import math
+    from oracle.routines import attention
+    q = np.array([[[[1, 0, 0, 0]], [[0, 1, 0, 0]]]], F32)
+    v = np.array([[[[1, 2, 3, 4]], [[5, 6, 7, 8]]]], F32)
+    a, b = 0.62245935, 0.37754068
+    np.testing.assert_allclose(attention(q, q, v, 0.5, False)[0, 0, 0], [a * 1 + b * 5, a * 2 + b * 6, a * 3 + b * 7, a * 4 + b * 8], atol=1e-6)
+    e = np.array([[[[1, 0]], [[0, 1]]]], F32)
+    np.testing.assert_allclose(attention(e, e, e, 1.0, False)[0, 0, 0], [0.7310586, 0.26894143], atol=1e-6)
+    qc = np.array([[[[1, 0]], [[0.2, 0.2]], [[1, 1]]]], F32)
+    kc = np.array([[[[1, 0]], [[0, 1]], [[1, 1]]]], F32)
+    vc = np.array([[[[1, 0]], [[0, 1]], [[0, 0]]]], F32)
+    y = attention(qc, kc, vc, 1 / math.sqrt(2), True)
+    c = 1 / (2 + math.exp(math.sqrt(0.5)))
+    np.testing.assert_allclose(y[0, :, 0], [[1, 0], [0.5, 0.5], [c, c]], atol=1e-7)
+    from jaxjs_hip import jit as J
+    from jaxjs_hip import library as L
+    from jaxjs_hip.jit import ShapedArray
+    from jit_util import run_program
+    from oracle.backend import OracleBackend
+    ops = [RNG.standard_normal((2, 128, 2, 64)).astype(np.float16) for _ in range(3)]
+    for causal in (False, True):
+        outs = []
+        for fused in (False, True):
+            prog = J.jit(lambda x, y_, z: L.dotProductAttention(x, y_, z, isCausal=causal, fused=fused), [ShapedArray((2, 128, 2, 64), DType.Float16)] * 3)
+            assert len(prog.routines) == (1 if fused else 0)
+            (o,) = run_program(OracleBackend(), prog, ops)
+            outs.append(o.astype(np.float64))
+        np.testing.assert_allclose(outs[1], outs[0], rtol=1e-2, atol=4e-3)  # the unfused chain rounds to f16 seven times
