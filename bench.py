@@ -271,6 +271,51 @@ def bench_program_gpt2_fused(be, hostrand, timed):
                                 "TFLOP/s_causal_half": round(full / 2 / (attn_ms * 1e-3) / 1e12, 1)}}
 
 
+def bench_reference_routine_cases(be):
+    """The cases of the reference's own routine benches on this backend (bench/fft.bench.ts:6-13, sort.bench.ts:15-16,
+    cholesky-webgpu.bench.ts:16): one dispatch + fence per iteration as there, best of 5; operands resident."""
+    from jaxjs_hip import DType
+    from jaxjs_hip.library import factorFftSize
+    from jaxjs_hip.routine import Routine, Routines, RoutineType
+
+    F = DType.Float32
+    out = {}
+
+    def best_ms(routine, arrays, out_bytes, reps=5):
+        exe = be.prepareRoutineSync(routine)
+        ins = [upload(be, a) for a in arrays]
+        outs = [be.malloc(b) for b in out_bytes]
+        be.dispatch(exe, ins, outs)
+        be.dev.sync()
+        best = float("inf")
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            be.dispatch(exe, ins, outs)
+            be.dev.sync()
+            best = min(best, (time.perf_counter() - t0) * 1e3)
+        for s in ins + outs:
+            be.decRef(s)
+        return round(best, 4)
+
+    for name, shape, phase in (("256", (256,), 0.0), ("1024", (1024,), 0.01), ("1000", (1000,), 0.02), ("64x256", (64, 256), 0.03),
+                               ("100k", (100_000,), 0.04), ("1m", (1_000_000,), 0.05)):
+        i = np.arange(int(np.prod(shape)), dtype=np.float64)
+        mk = lambda ph: (np.sin((i + 1) * (0.013 + ph)) + 0.25 * np.cos((i + 3) * (0.037 + ph))).astype(np.float32).reshape(shape)  # noqa: E731
+        rt = Routine(Routines.Fft, RoutineType([list(shape)] * 2, [F, F], [list(shape)] * 2, [F, F]),
+                     dict(factors=factorFftSize(shape[-1]), inverse=False))
+        out[f"fft {name}"] = {"ms": best_ms(rt, [mk(phase), mk(phase + 0.01)], [i.size * 4] * 2)}
+    rng = np.random.default_rng(0)
+    x = rng.random((32768, 1024), dtype=np.float32)
+    out["sort 32768x1024"] = {"ms": best_ms(Routine(Routines.Sort, RoutineType([[32768, 1024]], [F], [[32768, 1024]], [F])), [x], [x.nbytes])}
+    out["argsort 32768x1024"] = {"ms": best_ms(Routine(Routines.Argsort, RoutineType([[32768, 1024]], [F], [[32768, 1024]] * 2, [F, DType.Int32])),
+                                               [x], [x.nbytes] * 2)}
+    for n in (128, 256, 512, 1024, 2048):
+        a = rng.standard_normal((n, n)).astype(np.float32)
+        spd = (a.T @ a + n * np.eye(n, dtype=np.float32)).astype(np.float32)
+        out[f"cholesky {n}x{n}"] = {"ms": best_ms(Routine(Routines.Cholesky, RoutineType([[n, n]], [F], [[n, n]], [F])), [spd], [spd.nbytes])}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -455,6 +500,7 @@ def main():
                 be.decRef(o)
         be.decRef(xs)
         del X
+        extra["reference_routine_benches"] = bench_reference_routine_cases(be)
         result["extra"] = extra
 
     if not args.no_cpu:

@@ -24,6 +24,7 @@ from .shape import prod
 _SORT_KINDS = {DType.Float32: (0, "float"), DType.Float16: (1, "jh_f16"), DType.Int32: (2, "int"),
                DType.Uint32: (3, "jh_u32"), DType.Bool: (2, "int")}
 SORT_TILE = 8192  # 64 KB of LDS: rows up to 8192 elements never leave the CU
+CHOLESKY_PANEL_FROM = 192  # matrix order from which Cholesky runs panel by panel over the whole chip
 
 
 def _next_pow2(n: int) -> int:
@@ -75,6 +76,20 @@ def _gen_cholesky(routine: Routine, numerics: str) -> Optional[KernelSource]:
     batch = prod(shape[:-2])
     if batch == 0 or n == 0:
         return _empty("cholesky", n=n, batch=batch)
+    if n >= CHOLESKY_PANEL_FROM and batch * n * n < (1 << 31):
+        # Large matrices: 32-column panels, two launches each, every launch spread over the chip; the same sums in the
+        # same order as the single-workgroup kernel (bit-identical results).
+        src = _linalg_source(numerics, ROUTINE=4, N=n, M=batch)
+        grid1 = lambda count: (max(1, min((count + 255) // 256, 1 << 16)), 1, 1)  # noqa: E731
+        steps = [LaunchStep("jh_chol_zero", grid1(batch * n * n), (256, 1, 1), 0, [("out", 0)])]
+        for j0 in range(0, n, 32):
+            steps.append(LaunchStep("jh_chol_bulk", (batch * ((n - j0 + 63) // 64), 1, 1), (256, 1, 1), 0,
+                                    [("in", 0), ("out", 0), ("scratch", 0), ("const", j0)]))
+            after = max(0, n - j0 - 32)
+            steps.append(LaunchStep("jh_chol_panel", (batch * max(1, (after + 63) // 64), 1, 1), (64, 1, 1), 0,
+                                    [("scratch", 0), ("out", 0), ("const", j0)]))
+        return KernelSource([src], steps, [batch * n * 32 * 8], "cholesky", {0: batch * n * n * 4},
+                            dict(n=n, batch=batch, panels=(n + 31) // 32, launches=len(steps)))
     threads = _round64(n)
     src = _linalg_source(numerics, ROUTINE=0, N=n, THREADS=threads)
     steps = [LaunchStep("jh_cholesky", (batch, 1, 1), (threads, 1, 1), 0, [("in", 0), ("out", 0), ("scratch", 0)])]

@@ -36,11 +36,13 @@ def spd(batch, n):
     return (a @ np.swapaxes(a, -1, -2) + n * np.eye(n)).astype(F32)
 
 
-@pytest.mark.parametrize("shape", [(1, 1), (2, 2), (3, 3), (5, 17, 17), (2, 3, 64, 64), (200, 200), (1100, 1100)], ids=str)
+@pytest.mark.parametrize("shape", [(1, 1), (2, 2), (3, 3), (5, 17, 17), (2, 3, 64, 64), (191, 191), (192, 192), (200, 200), (2, 333, 333),
+                                   (1100, 1100), (2048, 2048)], ids=str)
 def test_cholesky(shape):
     x = spd(tuple(shape[:-2]), shape[-1])
     x = x + np.triu(RNG.standard_normal(x.shape), 1).astype(F32)  # the upper triangle must not matter
     got, want, ks = both(R.cholesky(x), [x])
+    assert ("panels" in ks.info) == (shape[-1] >= 192)  # large matrices run panel by panel over the whole chip
     assert_bits(got, want, f"cholesky {shape} {ks.info}")
 
 
@@ -49,6 +51,11 @@ def test_cholesky_not_positive_definite_and_empty():
     got, want, _ = both(R.cholesky(x), [x])
     assert np.isnan(got[0][0, 1, 1]) and got[0][1, 1, 1] == np.float32(np.sqrt(2.0))
     assert_bits(got, want)
+    big = spd((), 256)
+    big[100, 100] = -5.0  # pivot 100 goes negative: NaNs from there on, in the same places, also panel by panel
+    got, want, ks = both(R.cholesky(big), [big])
+    assert "panels" in ks.info and np.isnan(got[0][100, 100]) and np.isfinite(got[0][:100, :100]).all()
+    assert_bits(got, want, "non-PD through panels")
     e = np.zeros((0, 4, 4), F32)
     got, _ = R.run_gpu(R.cholesky(e), [e])
     assert got[0].shape == (0, 4, 4)
