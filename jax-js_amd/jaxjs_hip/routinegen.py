@@ -156,7 +156,7 @@ def _gen_jacobi(routine: Routine, numerics: str) -> Optional[KernelSource]:
         return _empty("jacobi", n=n, batch=batch)
     params = routine.params or {}
     threads = _round64(n)
-    in_lds = 1 if 2 * n * n * 4 <= 60 * 1024 else 0
+    in_lds = 1 if 2 * n * n * 4 <= 150 * 1024 else 0  # both matrices in the CU's 160 KB of LDS: n <= 138
     src = _linalg_source(numerics, ROUTINE=3, N=n, THREADS=threads, IN_LDS=in_lds, MAX_SWEEPS=int(params["maxSweeps"]),
                          TOL=repr(float(params["tolerance"])))
     steps = [LaunchStep("jh_jacobi", (batch, 1, 1), (threads, 1, 1), 0, [("in", 0), ("out", 0), ("out", 1)])]

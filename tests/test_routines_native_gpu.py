@@ -94,11 +94,12 @@ def test_lu_ties_zero_pivots_and_nans():
     assert_bits(got, want)
 
 
-@pytest.mark.parametrize("shape", [(1, 1), (2, 2), (3, 3), (4, 20, 20), (2, 64, 64), (100, 100)], ids=str)
+@pytest.mark.parametrize("shape", [(1, 1), (2, 2), (3, 3), (4, 20, 20), (2, 64, 64), (100, 100), (2, 128, 128), (150, 150)], ids=str)
 def test_jacobi_eigh(shape):
     a = RNG.standard_normal(shape)
     sym = (a + np.swapaxes(a, -1, -2)).astype(F32) + np.triu(RNG.standard_normal(shape), 1).astype(F32)
     got, want, ks = both(R.jacobi_eigh(sym), [sym])
+    assert ks.info["in_lds"] == (shape[-1] <= 138)
     assert_bits(got, want, f"jacobi_eigh {shape} {ks.info}")
 
 
