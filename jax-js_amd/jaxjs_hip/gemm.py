@@ -468,13 +468,21 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
 
     tmpl = "gemm_f16.hip.inc" if g["dtype"] == DType.Float16 else "gemm_f32.hip.inc"
     # Fast path: direct global->LDS loads need whole tiles (no bounds predicates) and 32-deep slabs.
-    full = g["M"] % BM == 0 and g["N"] % BN == 0 and g["K"] % 32 == 0 and BM >= 128 and BN >= 128
+    dBK = tile.get("BK", 32)
+    if dBK not in (32, 64):
+        raise ValueError(f"direct-to-LDS slab depth must be 32 or 64, got {dBK}")
+    full = g["M"] % BM == 0 and g["N"] % BN == 0 and g["K"] % dBK == 0 and BM >= 128 and BN >= 128
     any_gather = bool(g.get("a_gather") or g.get("b_gather"))
     dlds = g["dtype"] == DType.Float16 and full and tile.get("DLDS", 1) and not any_gather
     if dlds:
         tmpl = "gemm_f16_dlds.hip.inc"
     if dlds:
-        sched = dict(STAGES=tile.get("STAGES", 4), PIPE=tile.get("PIPE", 1), SGB=tile.get("SGB", 1), ASM_LOAD=tile.get("ASM", 1))
+        sched = dict(BK=dBK, STAGES=tile.get("STAGES", 4 if dBK == 32 else 2), PIPE=tile.get("PIPE", 1), SGB=tile.get("SGB", 1), ASM_LOAD=tile.get("ASM", 1))
+        sched["RING"] = ring = tile.get("RING", 0)
+        if ring and (ring != 5 or BM != BN or not sched["PIPE"]):
+            raise ValueError("the unit ring is five units of a square block tile under the phase-pipelined loop")
+        if (ring * BM * dBK * 2 if ring else sched["STAGES"] * (BM + BN) * dBK * 2) > 160 * 1024:
+            raise ValueError(f"{ring or sched['STAGES']} {'units' if ring else 'stages'} of a {BM}x{BN}x{dBK} slab do not fit the 160 KiB of LDS")
         # Vector epilogue: needs unit column stride and 8-element alignment of every row / batch start of C.
         # It pays when the epilogue itself reads buffers (bias, residual): those become 128-bit loads.  A plain
         # cast-and-store epilogue measures the same either way and keeps the simpler path.
@@ -517,7 +525,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     eb = byteWidth(g["dtype"])
     need[g["gid_a"]] = max(need.get(g["gid_a"], 0), g["a_len"] * eb)
     need[g["gid_b"]] = max(need.get(g["gid_b"], 0), g["b_len"] * eb)
-    info = dict(BM=BM, BN=BN, WM=WM, WN=WN, BK=32 if dlds else (64 if g["dtype"] == DType.Float16 else 16), direct_lds=bool(dlds), tiles=tiles, a_kcontig=g["a_sk"] == 1, b_kcontig=g["b_sk"] == 1,
+    info = dict(BM=BM, BN=BN, WM=WM, WN=WN, BK=dBK if dlds else (64 if g["dtype"] == DType.Float16 else 16), direct_lds=bool(dlds), tiles=tiles, a_kcontig=g["a_sk"] == 1, b_kcontig=g["b_sk"] == 1,
                 M=g["M"], N=g["N"], K=g["K"], nbatch=nbatch)
     if any_gather:
         info["gather"] = {tag: {0: "none", 1: "element", 2: f"rows{gather_group.get(tag, 8)}", 3: f"tap-major rows{gather_group.get(tag, 8)}",
