@@ -468,7 +468,12 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
 
     tmpl = "gemm_f16.hip.inc" if g["dtype"] == DType.Float16 else "gemm_f32.hip.inc"
     # Fast path: direct global->LDS loads need whole tiles (no bounds predicates) and 32-deep slabs.
-    dBK = tile.get("BK", 32)
+    # Slab depth.  When both operands run along k in memory, 64-deep slabs make every row of a slab one whole
+    # 128-byte line (a 32-deep slab asks for the two halves of each line about a microsecond apart, as two requests):
+    # measured +7..21 % on every tile shape.  An operand that runs along m or n is fetched in whole lines either way,
+    # and the shorter pipeline that 64-deep slabs leave room for then costs more than it gains.
+    both_k = g["a_sk"] == 1 and g["b_sk"] == 1 and g["K"] % 64 == 0 and g["K"] >= 128
+    dBK = tile.get("BK", 64 if both_k and tile.get("PIPE", 1) else 32)
     if dBK not in (32, 64):
         raise ValueError(f"direct-to-LDS slab depth must be 32 or 64, got {dBK}")
     full = g["M"] % BM == 0 and g["N"] % BN == 0 and g["K"] % dBK == 0 and BM >= 128 and BN >= 128
@@ -477,8 +482,16 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     if dlds:
         tmpl = "gemm_f16_dlds.hip.inc"
     if dlds:
-        sched = dict(BK=dBK, STAGES=tile.get("STAGES", 4 if dBK == 32 else 2), PIPE=tile.get("PIPE", 1), SGB=tile.get("SGB", 1), ASM_LOAD=tile.get("ASM", 1))
-        sched["RING"] = ring = tile.get("RING", 0)
+        # Stages that fit the 160 KiB of LDS: four of a 32-deep slab; of a 64-deep slab four (128x128), three
+        # (128x256, 256x128), or the five-unit ring (256x256: 2.5 slabs).
+        ring_default = 5 if dBK == 64 and (BM, BN) == (256, 256) and "STAGES" not in tile and tile.get("PIPE", 1) else 0
+        stages_default = 4 if dBK == 32 else min(4, (160 * 1024) // ((BM + BN) * dBK * 2))
+        sched = dict(BK=dBK, STAGES=tile.get("STAGES", stages_default), PIPE=tile.get("PIPE", 1), SGB=tile.get("SGB", 1), ASM_LOAD=tile.get("ASM", 1))
+        # Scalar-base addressing needs every lane offset inside one slab of a tile to fit 32 bits.
+        span = 2 * max((BM - 1) * abs(g["a_sm"]) + dBK * abs(g["a_sk"]), (BN - 1) * abs(g["b_sn"]) + dBK * abs(g["b_sk"]))
+        sched["SADDR"] = 1 if tile.get("SADDR", 1) and span < 2 ** 31 and g["a_sm"] >= 0 and g["a_sk"] >= 0 and g["b_sn"] >= 0 and g["b_sk"] >= 0 else 0
+        sched.update(PIN=tile.get("PIN", 1), BAR_AT=tile.get("BAR_AT", 2), READ_AHEAD=tile.get("RA", 1), LOADS_LATE=tile.get("LATE", 1))
+        sched["RING"] = ring = tile.get("RING", ring_default)
         if ring and (ring != 5 or BM != BN or not sched["PIPE"]):
             raise ValueError("the unit ring is five units of a square block tile under the phase-pipelined loop")
         if (ring * BM * dBK * 2 if ring else sched["STAGES"] * (BM + BN) * dBK * 2) > 160 * 1024:
@@ -527,6 +540,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     need[g["gid_b"]] = max(need.get(g["gid_b"], 0), g["b_len"] * eb)
     info = dict(BM=BM, BN=BN, WM=WM, WN=WN, BK=dBK if dlds else (64 if g["dtype"] == DType.Float16 else 16), direct_lds=bool(dlds), tiles=tiles, a_kcontig=g["a_sk"] == 1, b_kcontig=g["b_sk"] == 1,
                 M=g["M"], N=g["N"], K=g["K"], nbatch=nbatch)
+    if dlds:
+        info.update(stages=sched["STAGES"], ring=sched["RING"])
     if any_gather:
         info["gather"] = {tag: {0: "none", 1: "element", 2: f"rows{gather_group.get(tag, 8)}", 3: f"tap-major rows{gather_group.get(tag, 8)}",
                                 4: "tap-major strided"}[gather_flags[tag]] for tag in ("a", "b")}

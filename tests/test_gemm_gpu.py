@@ -118,6 +118,46 @@ def test_gemm_8192_cubed_sampled():
     _check(got.reshape(n, n)[rows], A[rows], B, n)
 
 
+def test_gemm_8192_cubed_nt_sampled():
+    """The same shape with B stored [N, K]: both operands run along k, which takes the 64-deep slabs and the
+    five-unit LDS ring."""
+    n = 8192
+    A = RNG.uniform(-1, 1, (n, n)).astype(np.float16)
+    Bt = RNG.uniform(-1, 1, (n, n)).astype(np.float16)
+    got, ks = device_run(matmulKernel(n, n, n, DType.Float16, b_transposed=True), [A, Bt])
+    assert ks.klass == "gemm" and ks.info["BK"] == 64 and ks.info["ring"] == 5, ks.info
+    rows = sorted(set(list(range(0, n, 353)) + [255, 256, n - 1]))
+    _check(got.reshape(n, n)[rows], A[rows], Bt.T, n)
+
+
+# Direct-to-LDS pipeline variants: (M, N, K, B stored [N, K], tile options).  K values give 1, 2, 3, 5, 6 and 17
+# slabs (the ring's period is five slabs); every schedule option is exercised on both slab depths.
+DLDS_VARIANTS = [
+    (256, 256, 64, True, dict(BK=64, RING=5)), (256, 256, 128, True, dict()), (256, 512, 192, True, dict()),
+    (512, 256, 320, True, dict()), (256, 256, 384, False, dict(BK=64, RING=5)), (512, 768, 1088, True, dict()),
+    (512, 768, 1088, False, dict(BK=64, RING=5)), (512, 768, 1088, True, dict(RA=2)), (512, 768, 1088, True, dict(LATE=0)),
+    (512, 768, 1088, True, dict(PIN=0)), (512, 768, 1088, True, dict(SADDR=0)), (512, 768, 1088, True, dict(BAR_AT=0)),
+    (512, 768, 1056, False, dict()), (512, 768, 1056, False, dict(PIN=0, SADDR=0)), (512, 768, 1056, True, dict(BK=32)),
+    (512, 768, 1056, False, dict(LATE=0, BAR_AT=4)), (256, 256, 32, False, dict()),
+    (512, 512, 1088, True, dict(BM=128, BN=128)), (512, 512, 1088, True, dict(BM=128, BN=128, RA=2)),
+    (512, 512, 1088, True, dict(BM=256, BN=128)), (512, 512, 1088, True, dict(BM=128, BN=256, WM=1, WN=4)),
+    (512, 512, 192, False, dict(BM=256, BN=128, BK=64, STAGES=3)), (512, 512, 1056, False, dict(BM=128, BN=128)),
+    (512, 512, 1024, True, dict(BM=256, BN=128, BK=64, STAGES=2)),
+]
+
+
+@pytest.mark.parametrize("M,N,K,bt,tile", DLDS_VARIANTS, ids=lambda v: "-".join(f"{k}{x}" for k, x in v.items()) or "default" if isinstance(v, dict) else str(v))
+def test_gemm_f16_direct_lds_variants(M, N, K, bt, tile):
+    A = RNG.uniform(-1, 1, (M, K)).astype(np.float16)
+    B = RNG.uniform(-1, 1, (K, N)).astype(np.float16)
+    k = matmulKernel(M, N, K, DType.Float16, b_transposed=bt)
+    got, ks = device_run(k, [A, np.ascontiguousarray(B.T) if bt else B], gemm_tile=tuple(sorted(tile.items())))
+    assert ks.klass == "gemm" and ks.info["direct_lds"], ks.info
+    if bt and "BK" not in tile and K % 64 == 0 and K >= 128:
+        assert ks.info["BK"] == 64, ks.info
+    _check(got, A, B, K)
+
+
 F32_SHAPES = [(64, 64, 64), (128, 128, 64), (200, 264, 136), (1024, 1024, 1024), (96, 1028, 72), (512, 384, 100)]
 
 
