@@ -65,3 +65,27 @@ def test_every_class_compiles_for_gfx950(name, kernel, klass):
     assert ks.klass == klass
     for src in ks.sources:
         assert len(compile_source(src, f"{name}.hip", use_cache=False)) > 1000
+
+
+def test_direct_lds_gemm_pipeline_choice_and_limits():
+    """Slab depth and LDS pipeline of the f16 fast path: 64-deep slabs only when both operands run along k, the
+    five-unit ring for the 256x256 tile, classical stages otherwise; configurations that exceed the 160 KiB of LDS are
+    refused when the source is generated, not at launch."""
+    def info(M, N, K, bt, **tile):
+        return generate(matmulKernel(M, N, K, DType.Float16, b_transposed=bt), gemm_tile=tuple(sorted(tile.items())) if tile else None).info
+
+    nn = info(8192, 8192, 8192, False)
+    assert (nn["BM"], nn["BN"], nn["BK"], nn["stages"], nn["ring"]) == (256, 256, 32, 4, 0)
+    nt = info(8192, 8192, 8192, True)
+    assert (nt["BM"], nt["BN"], nt["BK"], nt["ring"]) == (256, 256, 64, 5)
+    assert info(512, 512, 1024, True, BM=128, BN=128)["stages"] == 4
+    assert info(512, 512, 1024, True, BM=256, BN=128)["stages"] == 3
+    assert info(512, 512, 96, True, BM=128, BN=128)["BK"] == 32      # K is no multiple of 64
+    assert info(512, 512, 64, True, BM=128, BN=128)["BK"] == 32      # a single 64-deep slab: nothing to pipeline
+    for bad in (dict(BK=64, STAGES=3), dict(BK=64, RING=4), dict(BK=48)):
+        with pytest.raises(ValueError):
+            info(8192, 8192, 8192, True, **bad)
+    with pytest.raises(ValueError):
+        info(512, 512, 1024, True, BM=256, BN=128, BK=64, RING=5)    # the ring needs a square block tile
+    ks = generate(matmulKernel(512, 512, 1024, DType.Float16, b_transposed=True))
+    assert len(compile_source(ks.sources[0], "gemm_nt64.hip", use_cache=False)) > 1000
