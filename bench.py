@@ -257,11 +257,13 @@ def bench_program_gpt2_fused(be, hostrand, timed):
     gp.close()
     # the attention launch alone, on operands of the block's shape
     step = next(s for s in prog.steps if s.kind == "execute" and s.routine is not None)
-    qkv = [upload(be, hostrand.normal(1006, (batch, seq, heads, d // heads), 1.0, np.float16, stream=j)) for j in range(3)]
+    # (q, k and v reach the routine as three strided windows of the QKV projection's [batch, seq, 3d] output)
+    assert all(v is not None for v in step.routine.params["views"]) and len(set(step.inputs)) == 1
+    qkv = upload(be, hostrand.normal(1006, (batch, seq, 3 * d), 1.0, np.float16))
     out = be.malloc(batch * seq * d * 2)
     exe = be.prepareRoutineSync(step.routine)
-    attn_ms = measure(lambda: be.dispatch(exe, qkv, [out]), reps=50)
-    for sl in ins + qkv + [out]:
+    attn_ms = measure(lambda: be.dispatch(exe, [qkv, qkv, qkv], [out]), reps=50)
+    for sl in ins + [qkv, out]:
         be.decRef(sl)
     H = d // heads
     full = 4.0 * batch * heads * seq * seq * H

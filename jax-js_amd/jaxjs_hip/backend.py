@@ -205,6 +205,8 @@ class HipBackend:
         for what, slots, shapes, dtypes in (("input", ins, t.inputShapes, t.inputDtypes), ("output", outs, t.outputShapes, t.outputDtypes)):
             for i, (s, shape, dt) in enumerate(zip(slots, shapes, dtypes)):
                 need = prod(shape) * byteWidth(dt)
+                if what == "input" and i in prep.ks.min_input_bytes:  # an operand passed as a view of a larger buffer
+                    need = prep.ks.min_input_bytes[i]
                 if s["size"] < need:
                     raise ValueError(f"{what} {i} holds {s['size']} bytes, the routine addresses {need}")
         for step, fn in zip(prep.ks.steps, prep.functions):

@@ -122,6 +122,9 @@ BINARY_FUSABLE = ("Add", "Mul", "Idiv", "Mod", "Min", "Max", "BitCombine", "BitS
 # Primitives handed to the backend as a unit (src/frontend/core.ts:154-163): primitive name == routine name.
 # Their outputs index their inputs in several different ways: always dispatched (src/frontend/jit.ts:972-977).
 HETEROGENEOUS_VIEW_PRIMITIVES = ("RandomBits", "Gather")
+# Routines that take an operand as base buffer + strides + offset, with the views each one accepts (fused attention:
+# 128-bit loads along the head dimension, so unit stride there and everything else a multiple of 8 elements).
+STRIDED_OPERAND_ROUTINES = {"Attention": lambda strides, offset: strides[-1] == 1 and offset % 8 == 0 and all(s % 8 == 0 for s in strides[:-1])}
 ROUTINE_PRIMITIVES = ("Sort", "Argsort", "Scatter", "TriangularSolve", "Cholesky", "LU", "JacobiEigh", "Fft",
                       "Attention")  # the last one is this backend's extension (fused attention), see routine.py
 
@@ -952,11 +955,16 @@ def splitGraphDataflow(jaxpr: Jaxpr, maxArgs: int) -> Set[Var]:
     # non-view producer (src/frontend/jit.ts:990-999) and then refuses an operand that is still a view of it
     # ("routine primitive input is not imm", jit.ts:307-311, e.g. the flips of a lower-triangular solve); here the
     # operand itself is materialised, so such a view is realised by a copy kernel instead of failing.
+    # The fused-attention routine addresses its operands through strides, so a plain strided view of a buffer (the
+    # q/k/v slices of one QKV projection) is passed as it is: only the view's producer is materialised.
     for eqn in jaxpr.eqns:
         if eqn.primitive in ROUTINE_PRIMITIVES:
             for x in eqn.inputs:
                 if isinstance(x, Var) and x in varToDefn:
-                    materialized.add(x)
+                    if eqn.primitive in STRIDED_OPERAND_ROUTINES:
+                        markNonViewProducer(x)
+                    else:
+                        materialized.add(x)
 
     # Backwards: a node is black when it is an output, a reduction endpoint, materialised, or when two
     # different black nodes are reachable from it through non-black nodes.
@@ -1083,6 +1091,28 @@ class JitProgram:
                 for k, s in enumerate(self.steps) if s.kind == "execute"}
 
 
+def _plain_strided_view(jv: tuple, aval: ShapedArray):
+    """(buffer id, strides, offset, elements addressed) when the pending value `jv` is nothing but one unmasked strided
+    view of one buffer, read at the identity index; else None."""
+    if jv[0] != "exp" or len(jv[2]) != 1:
+        return None
+    e = jv[1]
+    if e.op != AluOp.GlobalView or e.dtype != aval.dtype:
+        return None
+    gid, st = e.arg
+    if len(st.views) != 1 or list(st.shape) != list(aval.shape):
+        return None
+    v = st.views[0]
+    if v.mask is not None or any(s < 0 for s in v.strides):
+        return None
+    want = unravelAlu(list(st.shape), AluVar.gidx)
+    if len(want) != len(e.src) or any(a.simplify().getHash() != b.simplify().getHash() for a, b in zip(want, e.src)):
+        return None
+    strides = [0 if d == 1 else int(sd) for d, sd in zip(st.shape, v.strides)]
+    elements = int(v.offset) + sum((d - 1) * sd for d, sd in zip(st.shape, strides)) + 1
+    return jv[2][gid], strides, int(v.offset), elements
+
+
 def jitCompile(jaxpr: Jaxpr, consts: Sequence[ConstArray] = (), maxArgs: int = 64) -> JitProgram:
     nargs = len(jaxpr.inBinders)
     black = splitGraphDataflow(jaxpr, maxArgs)
@@ -1099,13 +1129,31 @@ def jitCompile(jaxpr: Jaxpr, consts: Sequence[ConstArray] = (), maxArgs: int = 6
             rtype = RoutineType([list(x.aval.shape) for x in eqn.inputs], [x.aval.dtype for x in eqn.inputs],
                                 [list(v.aval.shape) for v in eqn.outBinders], [v.aval.dtype for v in eqn.outBinders])
             r_inputs: List[int] = []
+            r_views: List[Any] = []
             for x in eqn.inputs:
                 if not isinstance(x, Var):
                     raise NotImplementedError(f"jit: literal operand of routine {eqn.primitive}")
                 jv = ctx[x]
+                view = None
+                if jv[0] != "imm" and eqn.primitive in STRIDED_OPERAND_ROUTINES:
+                    view = _plain_strided_view(jv, x.aval)
+                    if view is not None and not STRIDED_OPERAND_ROUTINES[eqn.primitive](view[1], view[2]):
+                        view = None
+                    if view is None:  # anything else (masked, computed, a reduction): realised by a copy kernel first
+                        kernel = Kernel(len(jv[-1]), x.aval.size, jv[1], jv[2] if jv[0] == "red" else None)
+                        out_id = next_id[0]
+                        next_id[0] += 1
+                        steps.append(JitStep("malloc", output=out_id, size=kernel.bytes))
+                        steps.append(JitStep("execute", kernel=kernel, inputs=list(jv[-1]), output=out_id))
+                        jv = ctx[x] = ("imm", out_id)
+                if view is not None:
+                    r_inputs.append(view[0])
+                    r_views.append(dict(strides=view[1], offset=view[2], elements=view[3]))
+                    continue
                 if jv[0] != "imm":
                     raise RuntimeError(f"jit: routine primitive {eqn.primitive} input is not imm")
                 r_inputs.append(jv[1])
+                r_views.append(None)
             r_outputs: List[int] = []
             for v in eqn.outBinders:
                 out_id = next_id[0]
@@ -1113,7 +1161,10 @@ def jitCompile(jaxpr: Jaxpr, consts: Sequence[ConstArray] = (), maxArgs: int = 6
                 steps.append(JitStep("malloc", output=out_id, size=v.aval.size * byteWidth(v.aval.dtype)))
                 r_outputs.append(out_id)
                 ctx[v] = ("imm", out_id)
-            steps.append(JitStep("execute", routine=Routine(Routines(eqn.primitive), rtype, dict(eqn.params) or None),
+            r_params = dict(eqn.params)
+            if any(v is not None for v in r_views):
+                r_params["views"] = r_views
+            steps.append(JitStep("execute", routine=Routine(Routines(eqn.primitive), rtype, r_params or None),
                                  inputs=r_inputs, outputs=r_outputs))
             continue
         rule = JIT_RULES.get(eqn.primitive)

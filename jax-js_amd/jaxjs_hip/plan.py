@@ -46,5 +46,5 @@ def exportRoutinePlan(routine: Routine, numerics: str = "wasm") -> Dict[str, Any
     ks = generateRoutine(routine, numerics)
     t = routine.type
     return dict(_common(ks), routine=routine.name.value,
-                inputBytes=[prod(s) * byteWidth(d) for s, d in zip(t.inputShapes, t.inputDtypes)],
+                inputBytes=[ks.min_input_bytes.get(i, prod(s) * byteWidth(d)) for i, (s, d) in enumerate(zip(t.inputShapes, t.inputDtypes))],
                 outputBytes=[prod(s) * byteWidth(d) for s, d in zip(t.outputShapes, t.outputDtypes)])

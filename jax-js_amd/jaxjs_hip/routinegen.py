@@ -303,7 +303,8 @@ def _gen_sort(routine: Routine, numerics: str) -> Optional[KernelSource]:
 
 
 def _gen_attention(routine: Routine, numerics: str) -> Optional[KernelSource]:
-    """Fused attention over contiguous [B, L, N, 64] / [B, S, N, 64] float16 operands."""
+    """Fused attention over [B, L, N, 64] / [B, S, N, 64] float16 operands (contiguous, or strided views with unit
+    stride along the head dimension)."""
     import math
 
     t = routine.type
@@ -321,13 +322,26 @@ def _gen_attention(routine: Routine, numerics: str) -> Optional[KernelSource]:
     if B * N * (L // 128) >= (1 << 31) or max(B * L * N * H, B * S * N * H) >= (1 << 31):
         return None
     scale = float(params.get("scale", 1 / math.sqrt(H)))
-    strides = lambda T: dict(B=T * N * H, P=N * H, N=H)  # noqa: E731  contiguous [B, T, N, H]
-    sq, sk = strides(L), strides(S)
+    # Each operand is a base buffer read through (batch, position, head) strides and an offset: contiguous
+    # [B, T, N, H] unless the caller passes a view (`params["views"]`, e.g. the q/k/v slices of one QKV projection).
+    views = list(params.get("views") or [None, None, None])
+    lay, need = [], {}
+    for i, T in enumerate((L, S, S)):
+        v = views[i]
+        if v is None:
+            lay.append((T * N * H, N * H, H, 0))
+            need[i] = B * T * N * H * 2
+        else:
+            sb, sp, sn, sh = v["strides"]
+            if (sh != 1 and H > 1) or v["offset"] % 8 or sb % 8 or sp % 8 or sn % 8 or min(sb, sp, sn) < 0 or v["elements"] >= (1 << 31):
+                return None
+            lay.append((sb, sp, sn, v["offset"]))
+            need[i] = v["elements"] * 2
+    (qb, ql, qn, qo), (kb, ksp, kn, ko), (vb, vsp, vn, vo) = lay
     src = _prelude(numerics) + fill(template("attention.hip.inc"), dict(
         B=B, NH=N, L=L, S=S, CAUSAL=1 if params.get("isCausal") else 0, SCALE_LOG2E=repr(scale * math.log2(math.e)),
-        QB=sq["B"], QL=sq["P"], QN=sq["N"], KB=sk["B"], KS=sk["P"], KN=sk["N"], VB=sk["B"], VS=sk["P"], VN=sk["N"],
-        OB=sq["B"], OL=sq["P"], ON=sq["N"]))
+        QB=qb, QL=ql, QN=qn, QOFF=qo, KB=kb, KS=ksp, KN=kn, KOFF=ko, VB=vb, VS=vsp, VN=vn, VOFF=vo,
+        OB=L * N * H, OL=N * H, ON=H))
     blocks = B * N * (L // 128)
     steps = [LaunchStep("jh_attention", (blocks, 1, 1), (256, 1, 1), 0, [("in", 0), ("in", 1), ("in", 2), ("out", 0)])]
-    need = {0: B * L * N * H * 2, 1: B * S * N * H * 2, 2: B * S * N * H * 2}
     return KernelSource([src], steps, [], "attention", need, dict(B=B, L=L, S=S, N=N, H=H, causal=bool(params.get("isCausal")), blocks=blocks))

@@ -55,13 +55,21 @@ def _ptr(a: np.ndarray):
     return a.ctypes.data_as(ctypes.c_void_p)
 
 
-def _typed(bufs: Sequence, dtypes, shapes, writable: bool) -> List[np.ndarray]:
+def _typed(bufs: Sequence, dtypes, shapes, writable: bool, views=None) -> List[np.ndarray]:
+    """Host buffers as arrays of the routine's operand types.  `views[i]`, when given, says operand i is a strided
+    window (element strides, offset) onto a larger buffer instead of the whole of a contiguous one."""
     out = []
-    for buf, dt, shape in zip(bufs, dtypes, shapes):
+    for i, (buf, dt, shape) in enumerate(zip(bufs, dtypes, shapes)):
         a = np.frombuffer(buf, dtype=_NP[str(dt)])
         if writable and not a.flags.writeable:
             raise ValueError("routine outputs must be writable buffers")
-        out.append(a.reshape(shape))
+        v = views[i] if views else None
+        if v is None:
+            out.append(a.reshape(shape))
+        else:
+            if v["elements"] > a.size:
+                raise ValueError(f"operand {i}: the view addresses {v['elements']} elements of a buffer of {a.size}")
+            out.append(np.lib.stride_tricks.as_strided(a[v["offset"]:], shape=tuple(shape), strides=tuple(sd * a.itemsize for sd in v["strides"]), writeable=False))
     return out
 
 
@@ -76,7 +84,7 @@ def runCpuRoutine(routine, inputs: Sequence, outputs: Sequence) -> None:
     t = routine.type
     name = str(routine.name)
     params = routine.params or {}
-    ins = _typed(inputs, t.inputDtypes, t.inputShapes, False)
+    ins = _typed(inputs, t.inputDtypes, t.inputShapes, False, params.get("views"))
     outs = _typed(outputs, t.outputDtypes, t.outputShapes, True)
     if name == "Sort":
         if ins[0].ndim == 0:

@@ -52,6 +52,45 @@ def test_attention_is_stable_for_large_scores_and_peaked_rows():
         np.testing.assert_allclose(got[0].astype(np.float64), want[0].astype(np.float64), rtol=1e-2, atol=4e-3)
 
 
+def _view(strides, offset, shape):
+    return dict(strides=list(strides), offset=offset, elements=offset + sum((d - 1) * s for d, s in zip(shape, strides)) + 1)
+
+
+@pytest.mark.parametrize("causal", [False, True], ids=["full", "causal"])
+def test_attention_reads_operands_through_strides(causal):
+    """q, k and v as three windows of one [B, L, 3*N*64] buffer (the output of a fused QKV projection), and k/v stored
+    head-major ([B, N, S, 64]): the routine takes the base buffers with strides and offsets, no copies."""
+    B, L, N, H = 2, 256, 3, 64
+    rng = np.random.default_rng(11)
+    qkv = rng.standard_normal((B, L, 3 * N * H)).astype(np.float16)
+    t = RoutineType([[B, L, N, H]] * 3, [F16] * 3, [[B, L, N, H]], [F16])
+    st = (L * 3 * N * H, 3 * N * H, H, 1)
+    views = [_view(st, i * N * H, (B, L, N, H)) for i in range(3)]
+    routine = Routine(Routines.Attention, t, dict(scale=0.125, isCausal=causal, views=views))
+    got, ks = R.run_gpu(routine, [qkv, qkv, qkv])
+    q, k, v = [qkv[..., i * N * H:(i + 1) * N * H].reshape(B, L, N, H) for i in range(3)]
+    want = R.run_oracle(attention_routine(B, L, L, N, causal), [q, k, v])
+    np.testing.assert_allclose(got[0].astype(np.float64), want[0].astype(np.float64), rtol=1e-2, atol=3e-3)
+    np.testing.assert_array_equal(R.run_oracle(routine, [qkv, qkv, qkv])[0], want[0])  # the checker reads views too
+    # head-major keys and values, contiguous queries
+    kh, vh = [np.ascontiguousarray(np.transpose(a, (0, 2, 1, 3))) for a in (k, v)]
+    hm = _view((N * L * H, H, L * H, 1), 0, (B, L, N, H))
+    routine = Routine(Routines.Attention, t, dict(scale=0.125, isCausal=causal, views=[None, hm, hm]))
+    got2, _ = R.run_gpu(routine, [np.ascontiguousarray(q), kh, vh])
+    np.testing.assert_array_equal(got2[0], got[0])
+
+
+def test_strided_operands_the_kernel_cannot_load_are_refused():
+    if WARM_ONLY:
+        pytest.skip("nothing to compile")
+    B, L, N, H = 1, 128, 1, 64
+    t = RoutineType([[B, L, N, H]] * 3, [F16] * 3, [[B, L, N, H]], [F16])
+    for bad in (_view((L * N * H, N * H, H, 1), 4, (B, L, N, H)), _view((L * N * H * 2, N * H * 2, H * 2, 2), 0, (B, L, N, H)),
+                _view((L * 68, 68, 68, 1), 0, (B, L, N, H))):
+        with pytest.raises(UnsupportedRoutineError):
+            backend().prepareRoutineSync(Routine(Routines.Attention, t, dict(scale=0.125, isCausal=False, views=[bad, None, None])))
+
+
 def test_shapes_outside_the_kernel_are_refused_not_faked():
     if WARM_ONLY:
         pytest.skip("nothing to compile")
@@ -68,7 +107,8 @@ def test_gpt2_block_with_fused_attention():
     fused = W.gpt2BlockProgram(batch, seq, d, heads, d_ff, fusedAttention=True)
     plain = W.gpt2BlockProgram(batch, seq, d, heads, d_ff)
     assert [r.name for r in fused.routines] == [Routines.Attention] and not plain.routines
-    assert len(fused.kernels) == len(plain.kernels) - 7 + 3  # seven attention kernels out, three operand copies in
+    assert len(fused.kernels) == len(plain.kernels) - 7  # seven attention kernels out; q, k, v are views of the QKV output
+    assert all(v is not None for v in fused.routines[0].params["views"])
     assert not W.gpt2BlockProgram(batch, 64, d, heads, d_ff, fusedAttention=True).routines  # L = 64: composition kept
     if WARM_ONLY:
         from test_programs_gpu import warm

@@ -262,6 +262,35 @@ def test_routine_outputs_and_operands_are_dispatch_boundaries():
     assert prog.routines[0].type.inputShapes == [[4, 6]]
 
 
+def test_attention_routine_takes_plain_strided_views_and_copies_the_rest():
+    """The fused-attention routine reads its operands through strides: slices of one buffer reach it as (buffer,
+    strides, offset) with no copy; a view its 128-bit loads cannot take (offset 4) and a computed operand are realised
+    by a kernel first.  Values are checked through the CPU checker, which reads the same views."""
+    from oracle.routines import attention as attention64
+    B, T, N, H = 1, 128, 2, 64
+    rng = np.random.default_rng(5)
+    qkv = rng.standard_normal((B, T, 3 * N * H)).astype(np.float16)
+
+    def slices(a):
+        parts = [J.reshape(J.shrink(a, [(0, B), (0, T), (i * N * H, (i + 1) * N * H)]), (B, T, N, H)) for i in range(3)]
+        return J.attention(parts[0], parts[1], parts[2], 0.125, True)
+    prog, (y,) = run_typed(slices, [qkv], [DType.Float16])
+    assert steps_of(prog) == ["Attention"]
+    views = prog.routines[0].params["views"]
+    assert [v["offset"] for v in views] == [0, N * H, 2 * N * H] and views[0]["strides"] == [0, 3 * N * H, H, 1]  # batch of one: stride 0
+    q, k, v = [qkv[..., i * N * H:(i + 1) * N * H].reshape(B, T, N, H) for i in range(3)]
+    want = attention64(q, k, v, 0.125, True)
+    np.testing.assert_allclose(y.reshape(B, T, N, H).astype(np.float64), want, rtol=2e-3, atol=2e-3)
+
+    wide = rng.standard_normal((B, T, N, H + 4)).astype(np.float16)
+    prog, (y2,) = run_typed(lambda a, b: J.attention(J.shrink(a, [(0, B), (0, T), (0, N), (4, H + 4)]), b.mul(2.0), b, 0.125, False),
+                            [wide, np.ascontiguousarray(q)], [DType.Float16] * 2)
+    assert steps_of(prog) == ["kernel", "kernel", "Attention"]  # the misaligned slice and the computed operand
+    assert prog.routines[0].params.get("views") in (None, [None, None, None])
+    want2 = attention64(wide[..., 4:], (q * np.float16(2)).astype(np.float16), q, 0.125, False)
+    np.testing.assert_allclose(y2.reshape(B, T, N, H).astype(np.float64), want2, rtol=2e-3, atol=2e-3)
+
+
 def test_solve_is_lu_plus_two_triangular_solves():
     rng = np.random.default_rng(1)
     a = (rng.standard_normal((3, 8, 8)) + 4 * np.eye(8)).astype(np.float32)
