@@ -163,6 +163,9 @@ def _gen_jacobi(routine: Routine, numerics: str) -> Optional[KernelSource]:
     return KernelSource([src], steps, [], "jacobi", {0: batch * n * n * 4}, dict(n=n, batch=batch, threads=threads, in_lds=bool(in_lds)))
 
 
+FFT_FUSED_MAX_N = 8192  # 16 bytes of LDS per point: 128 KiB
+
+
 def _gen_fft(routine: Routine, numerics: str) -> Optional[KernelSource]:
     t = routine.type
     shape = list(t.inputShapes[0])
@@ -182,10 +185,21 @@ def _gen_fft(routine: Routine, numerics: str) -> Optional[KernelSource]:
     rows = prod(shape[:-1])
     if rows == 0:
         return _empty("fft", n=n, rows=rows)
-    src = _prelude(numerics) + fill(template("fft.hip.inc"), dict(N=n, ROWS=rows, INVERSE=1 if params.get("inverse") else 0,
-                                                                  NF=len(factors), FACTORS=", ".join(map(str, factors)) or "1"))
-    blocks = max(1, min((rows * n + 255) // 256, 1 << 20))
+    # Rows that fit the LDS twice over (16 bytes per point) run in one launch, one workgroup per row, unless there are
+    # too few rows for that to use the chip (a single long row is quicker spread over many workgroups per stage).
     S = len(factors)
+    fused = S >= 1 and n <= FFT_FUSED_MAX_N and (n <= 2048 or rows >= 64)
+    if "singleLaunch" in params:  # tests pin either path
+        fused = bool(params["singleLaunch"]) and S >= 1 and n <= FFT_FUSED_MAX_N
+    threads = min(1024, max(64, _round64(n)))
+    src = _prelude(numerics) + fill(template("fft.hip.inc"), dict(N=n, ROWS=rows, INVERSE=1 if params.get("inverse") else 0,
+                                                                  NF=len(factors), FACTORS=", ".join(map(str, factors)) or "1",
+                                                                  FUSED=1 if fused else 0, FUSED_THREADS=threads))
+    need = {0: rows * n * 4, 1: rows * n * 4}
+    if fused:
+        steps = [LaunchStep("jh_fft_rows", (min(rows, 1 << 16), 1, 1), (threads, 1, 1), 0, [("in", 0), ("in", 1), ("out", 0), ("out", 1)])]
+        return KernelSource([src], steps, [], "fft", need, dict(n=n, rows=rows, factors=factors, launches=1, fused=True))
+    blocks = max(1, min((rows * n + 255) // 256, 1 << 20))
     out_pair, tmp_pair = [("out", 0), ("out", 1)], [("scratch", 0), ("scratch", 1)]
     target = lambda s: out_pair if (S - 1 - s) % 2 == 0 else tmp_pair  # noqa: E731  (stage -1 is the permutation)
     steps = [LaunchStep("jh_fft_permute", (blocks, 1, 1), (256, 1, 1), 0, [("in", 0), ("in", 1)] + target(-1))]
@@ -195,8 +209,7 @@ def _gen_fft(routine: Routine, numerics: str) -> Optional[KernelSource]:
                                 target(s - 1) + target(s) + [("const", prev), ("const", radix), ("const", 1 if s == S - 1 else 0)]))
         prev *= radix
     scratch = [rows * n * 4, rows * n * 4] if S >= 1 else [8, 8]
-    need = {0: rows * n * 4, 1: rows * n * 4}
-    return KernelSource([src], steps, scratch, "fft", need, dict(n=n, rows=rows, factors=factors, launches=len(steps)))
+    return KernelSource([src], steps, scratch, "fft", need, dict(n=n, rows=rows, factors=factors, launches=len(steps), fused=False))
 
 
 _SCATTER_KINDS = {DType.Float32: (0, "float"), DType.Float16: (1, "jh_f16"), DType.Int32: (2, "int"), DType.Uint32: (3, "jh_u32"),

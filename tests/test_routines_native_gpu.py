@@ -130,6 +130,22 @@ def test_fft(n, inverse):
         np.testing.assert_allclose(g, w, rtol=0, atol=1e-5 * scale, err_msg=str(ks.info))
 
 
+@pytest.mark.parametrize("shape", [(3, 8), (2, 60), (1, 1000), (5, 1024), (70, 4096), (2, 8192)], ids=str)
+def test_fft_single_launch_and_staged_paths_give_the_same_bits(shape):
+    """Short rows run in one launch with the stages in LDS, long or few rows one launch per stage through HBM: the
+    same operations per element in the same order, so not a bit may differ (forward and inverse)."""
+    from jaxjs_hip.routine import Routine
+    re, im = RNG.standard_normal(shape).astype(F32), RNG.standard_normal(shape).astype(F32)
+    for inverse in (False, True):
+        base = R.fft(re, im, inverse)
+        one = Routine(base.name, base.type, dict(base.params, singleLaunch=True))
+        many = Routine(base.name, base.type, dict(base.params, singleLaunch=False))
+        a, ka = R.run_gpu(one, [re, im])
+        b, kb = R.run_gpu(many, [re, im])
+        assert ka.info["launches"] == 1 and kb.info["launches"] == 1 + len(base.params["factors"])
+        assert_bits(a, b, f"{shape} inverse={inverse}")
+
+
 def test_fft_factor_orders_and_validation():
     re, im = RNG.standard_normal((2, 60)).astype(F32), RNG.standard_normal((2, 60)).astype(F32)
     for factors in ([4, 3, 5], [5, 3, 4], [2, 2, 15], [60]):
