@@ -212,6 +212,8 @@ class HipExpCodegen:
                    AluOp.Log: "log", AluOp.Erf: "erf", AluOp.Erfc: "erfc"}
             if op in fns:
                 call = f"jh_{fns[op]}_f32((float)({a}))" if dtype != DType.Float32 else f"jh_{fns[op]}_f32({a})"
+                if dtype == DType.Float16 and op in (AluOp.Exp, AluOp.Log):
+                    call = f"jh_{fns[op]}_f16((float)({a}))"  # hardware exp2/log2: float16 has no Wasm polynomial to follow
                 if dtype == DType.Float64 and self.numerics != "wasm" and op not in (AluOp.Erf, AluOp.Erfc):
                     return f"__ocml_{fns[op]}_f64({a})", False
                 return (call if dtype == DType.Float32 else f"({ct})({call})"), False
