@@ -248,3 +248,68 @@ def test_random_contractions(seed):
         Bm = np.swapaxes(Bm, -1, -2)
     ref = Am @ Bm + (bias.astype(np.float64) if with_bias else 0)
     np.testing.assert_array_equal(got.astype(np.float64).reshape(ref.shape), ref.astype(npdt).astype(np.float64), err_msg=str(ks.info))
+
+
+# ---- float16 -----------------------------------------------------------------------------------------------------
+F16 = DType.Float16
+
+
+def rand_f16_exp(rng, leaves, depth):
+    """A random float16 expression: every operation rounds to float16 (as the reference's float16 arrays do), so the
+    GPU's native half arithmetic and the checker agree bit for bit except where a transcendental or a division is
+    involved (one float16 ulp); magnitudes stay small enough that nothing overflows."""
+    if depth == 0 or rng.random() < 0.2:
+        if rng.random() < 0.8:
+            return rng.choice(leaves[F16])
+        return AluExp.const(F16, rng.choice([0.0, 1.0, -1.0, 0.5, 2.0, -0.75]))
+    sub = lambda: rand_f16_exp(rng, leaves, depth - 1)  # noqa: E731
+    r = rng.random()
+    if r < 0.4:
+        return rng.choice([AluExp.add, AluExp.sub, AluExp.mul])(sub(), sub())
+    if r < 0.5:
+        return (AluExp.min if rng.random() < 0.5 else AluExp.max)(sub(), sub())
+    if r < 0.6:
+        return AluExp.where(AluExp.cmplt(sub(), sub()), sub(), sub())
+    bounded = AluExp.min(AluExp.max(sub(), AluExp.const(F16, -3.0)), AluExp.const(F16, 3.0))
+    if r < 0.7:
+        return AluExp.exp(bounded)
+    if r < 0.78:
+        return AluExp.log(AluExp.add(AluExp.mul(bounded, bounded), AluExp.const(F16, 0.5)))
+    if r < 0.86:
+        return AluExp.sqrt(AluExp.add(AluExp.mul(bounded, bounded), AluExp.const(F16, 0.25)))
+    if r < 0.93:
+        return AluExp.reciprocal(AluExp.add(AluExp.mul(bounded, bounded), AluExp.const(F16, 1.0)))
+    if r < 0.97:
+        return AluExp.cast(F16, AluExp.mul(AluExp.cast(F32, bounded), rng.choice(leaves[F32])))
+    return AluExp.cast(F16, AluExp.cast(I32, AluExp.mul(bounded, AluExp.const(F16, 4.0))))
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_f16_kernels(seed):
+    """Maps and reductions over float16 buffers (packs of 8 halves, f32 accumulation of f16 sums, native half
+    arithmetic) against the checker, within the float16 tolerance (rel 1e-2)."""
+    rng = random.Random(9000 + seed)
+    npr = np.random.default_rng(seed)
+    reduce_ = seed % 3 == 2
+    if reduce_:
+        rows, L = rng.choice([(1, 1000), (7, 129), (64, 64), (300, 33), (5, 2049)])
+        n = rows * L
+        st = ShapeTracker.fromShape([rows, L]) if rng.random() < 0.5 else ShapeTracker.fromShape([L, rows]).permute([1, 0])
+    else:
+        n = rng.choice([1, 7, 64, 1000, 4099, 65536 + 5])
+        st = ShapeTracker.fromShape([n])
+        if rng.random() < 0.3 and n > 1:
+            st = st.flip([True])
+    h1, h2 = (npr.normal(0, 1.5, n).astype(np.float16) for _ in range(2))
+    f = npr.uniform(-2, 2, n).astype(np.float32)
+    ins = [(F16, st), (F16, st), (F32, st)]
+    body = lambda *vs: rand_f16_exp(rng, {F16: list(vs[:2]), F32: [vs[2]]}, rng.choice([2, 3, 4]))  # noqa: E731
+    if reduce_:
+        op = rng.choice([AluOp.Add, AluOp.Max, AluOp.Min])
+        k = reduceKernel([rows, L], ins, body, op)
+        tol = dict(rtol=1e-2, atol=1e-2 * (math.sqrt(L) if op == AluOp.Add else 1.0))
+    else:
+        k = mapKernel([n], ins, body)
+        tol = dict(rtol=1e-2, atol=1e-2)
+    assert k.dtype == F16
+    assert_parity(k, [h1, h2, f], **tol)
