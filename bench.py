@@ -315,6 +315,43 @@ def bench_reference_routine_cases(be):
         a = rng.standard_normal((n, n)).astype(np.float32)
         spd = (a.T @ a + n * np.eye(n, dtype=np.float32)).astype(np.float32)
         out[f"cholesky {n}x{n}"] = {"ms": best_ms(Routine(Routines.Cholesky, RoutineType([[n, n]], [F], [[n, n]], [F])), [spd], [spd.nbytes])}
+
+    # Traced programs (bench/svd.bench.ts:11-15, bench/argreduce.bench.ts:16-48): one eager execution + fence per
+    # iteration, best of 3; constants and inputs resident.
+    from jaxjs_hip import jit as J
+    from jaxjs_hip import library as L
+    from jaxjs_hip.jit import ShapedArray
+
+    def best_prog_ms(fn, arrays, reps=3):
+        prog = J.jit(fn, [ShapedArray(tuple(a.shape), F) for a in arrays])
+        const_slots = []
+        for c in prog.consts:
+            k = c.kernel()
+            slot = be.malloc(k.bytes)
+            be.dispatch(be.prepareKernelSync(k), [], [slot])
+            const_slots.append(slot)
+        ins = const_slots + [upload(be, a) for a in arrays]
+        prepared = prog.prepare(be)
+        best = float("inf")
+        for it in range(reps + 1):
+            t0 = time.perf_counter()
+            outs = prog.execute(be, ins, prepared)
+            be.dev.sync()
+            if it:
+                best = min(best, (time.perf_counter() - t0) * 1e3)
+            for o in outs:
+                be.decRef(o)
+        for sl in ins:
+            be.decRef(sl)
+        return round(best, 4)
+
+    for name, shape in (("128x128", (128, 128)), ("1024x128", (1024, 128)), ("32768x256", (32768, 256))):
+        a = rng.standard_normal(shape).astype(np.float32)
+        out[f"svdvals {name}"] = {"ms": best_prog_ms(lambda x: L.svdvals(x), [a])}
+        out[f"thin svd {name}"] = {"ms": best_prog_ms(lambda x: L.svd(x), [a])}
+    v10k, m2d = rng.random(10000, dtype=np.float32), rng.random((100, 1000), dtype=np.float32)
+    out["argmax 10k elements"] = {"ms": best_prog_ms(lambda x: L.argmax(x, 0), [v10k])}
+    out["argmax along axis (100x1000)"] = {"ms": best_prog_ms(lambda x: L.argmax(x, 1), [m2d])}
     return out
 
 

@@ -545,6 +545,11 @@ def shrink(x, slices):
     return bind1("Shrink", [x], dict(slice=[tuple(s) for s in slices]))
 
 
+def pad(x, width):
+    """Zero padding `[(before, after), ...]` per axis (the Pad primitive, src/frontend/core.ts:253-262)."""
+    return bind1("Pad", [x], dict(width=[tuple(w) for w in width]))
+
+
 def flip(x, axis):
     x = _raise(x)
     return bind1("Flip", [x], dict(axis=_normalize_axis(axis, x.ndim)))

@@ -265,6 +265,82 @@ def eigh_unsorted(x: Tracer, symmetrizeInput: bool = True):
     return v, d
 
 
+def diagonal(x: Tracer, offset: int = 0, axis1: int = 0, axis2: int = 1):
+    """The diagonal as a view, appended as the last axis: move the two axes last, flatten them, pad or shrink to
+    `diag * (m + 1)` elements, reshape to `[diag, m + 1]` and keep column `offset` (src/frontend/core.ts:958-1000)."""
+    if offset < 0:
+        return diagonal(x, -offset, axis2, axis1)
+    axis1, axis2 = (a + x.ndim if a < 0 else a for a in (axis1, axis2))
+    if axis1 == axis2:
+        raise ValueError("axis1 and axis2 must not be equal")
+    if offset >= x.shape[axis2]:
+        raise ValueError("offset exceeds axis size")
+    if (axis1, axis2) != (x.ndim - 2, x.ndim - 1):
+        x = x.transpose([i for i in range(x.ndim) if i not in (axis1, axis2)] + [axis1, axis2])
+    batch = list(x.shape[:-2])
+    n, m = x.shape[-2:]
+    diag = min(n, m - offset)
+    x = x.reshape(batch + [n * m])
+    npad = diag * (m + 1) - n * m
+    if npad > 0:
+        x = J.pad(x, [(0, 0)] * len(batch) + [(0, npad)])
+    elif npad < 0:
+        x = J.shrink(x, [(0, d) for d in batch] + [(0, n * m + npad)])
+    x = x.reshape(batch + [diag, m + 1])
+    return J.shrink(x, [(0, d) for d in batch + [diag]] + [(offset, offset + 1)]).reshape(batch + [diag])
+
+
+def eigh(x: Tracer, lower: bool = True, sortEigenvalues: bool = True, symmetrizeInput: bool = True):
+    """`(eigenvectors, eigenvalues)` of a batch of symmetric matrices, eigenvalues ascending: the Jacobi routine, then
+    argsort of the diagonal and two gathers (src/library/lax-linalg.ts:52-89)."""
+    n = x.shape[-1]
+    if x.ndim < 2 or x.shape[-2] != n:
+        raise ValueError(f"eigh: expected a batch of square matrices, got {list(x.shape)}")
+    if symmetrizeInput:
+        x = x.add(_swap_last_two(x)).mul(0.5)
+    elif not lower:
+        x = _swap_last_two(x)
+    d, v = J.jacobiEigh(x, maxSweeps=max(8, 2 * n), tolerance=1e-6)
+    values = diagonal(d, 0, -2, -1)
+    if not sortEigenvalues:
+        return v, values
+    order = argsort(values)
+    return takeAlongAxis(v, order.reshape(list(x.shape[:-2]) + [1, n]), -1), takeAlongAxis(values, order, -1)
+
+
+def svd(a: Tracer, computeUv: bool = True, fullMatrices: bool = False):
+    """Thin singular value decomposition through the symmetric eigendecomposition of the smaller Gram matrix
+    (src/library/lax-linalg.ts:102-163): `s = sqrt(max(flip(eigenvalues), 0))`, the other factor from one more product
+    scaled by `1/s` (0 where s is 0)."""
+    if a.ndim < 2:
+        raise ValueError(f"svd: input must be at least 2D, got {list(a.shape)}")
+    m, n = a.shape[-2:]
+    if fullMatrices and m != n:
+        raise ValueError("svd: fullMatrices=true is only supported for square input")
+    batch, k = list(a.shape[:-2]), min(m, n)
+    singular = lambda values: J.sqrt(J.maximum(J.flip(values, -1), 0.0))  # noqa: E731
+    inverse = lambda s: J.where(J.greater(s, 0.0), J.reciprocal(s), 0.0)  # noqa: E731
+    if m >= n:
+        v, values = eigh(matmul(_swap_last_two(a), a), symmetrizeInput=False)
+        s = singular(values)
+        if not computeUv:
+            return s
+        vDesc = J.flip(v, -1)
+        u = matmul(a, vDesc).mul(inverse(s).reshape(batch + [1, k]))
+        return u, s, _swap_last_two(vDesc)
+    u, values = eigh(matmul(a, _swap_last_two(a)), symmetrizeInput=False)
+    s = singular(values)
+    if not computeUv:
+        return s
+    uDesc = J.flip(u, -1)
+    vh = matmul(_swap_last_two(uDesc), a).mul(inverse(s).reshape(batch + [k, 1]))
+    return uDesc, s, vh
+
+
+def svdvals(a: Tracer):
+    return svd(a, computeUv=False)
+
+
 def factorFftSize(n: int) -> List[int]:
     factors: List[int] = []
     for radix in (4, 2, 3, 5, 7):

@@ -336,6 +336,60 @@ def test_cholesky_upper_eigh_and_fft_along_an_axis():
     np.testing.assert_allclose(i2.reshape(12, 5), im, atol=1e-6)
 
 
+def test_eigh_svd_and_diagonal_reference_tables():
+    """test/lax-linalg.test.ts:138-275 and test/numpy-linalg.test.ts:128-225: sorted eigenpairs, the selected triangle,
+    thin SVD of tall, wide and batched matrices, singular values alone; `diagonal` for every offset and axis order."""
+    d3 = f32([[3, 0, 0], [0, 1, 0], [0, 0, 2]])
+    _, (vec, val) = run(lambda a: L.eigh(a), d3)
+    np.testing.assert_allclose(val, [1, 2, 3], atol=1e-6)
+    np.testing.assert_allclose(vec.reshape(3, 3), [[0, 0, 1], [1, 0, 0], [0, 1, 0]], atol=1e-6)
+    _, (vec, val) = run(lambda a: L.eigh(a, sortEigenvalues=False), d3)
+    np.testing.assert_allclose(val, [3, 1, 2], atol=1e-6)
+    np.testing.assert_allclose(vec.reshape(3, 3), np.eye(3), atol=1e-6)
+    x = f32([[4, 1, 2], [1, 3, 0.5], [2, 0.5, 5]])
+    _, (vec, val) = run(lambda a: L.eigh(a), x)
+    vec = vec.reshape(3, 3)
+    np.testing.assert_allclose((vec * val) @ vec.T, x, atol=1e-3)
+    np.testing.assert_allclose(vec.T @ vec, np.eye(3), atol=1e-3)
+    xb = f32([[[2, 1], [1, 2]], [[3, 1], [1, 3]]])
+    _, (vec, val) = run(lambda a: L.eigh(a), xb)
+    np.testing.assert_allclose(val.reshape(2, 2), [[1, 3], [2, 4]], atol=1e-4)
+    tri = f32([[2, 100], [1, 2]])
+    _, (_, lo) = run(lambda a: L.eigh(a, symmetrizeInput=False, lower=True), tri)
+    _, (_, up) = run(lambda a: L.eigh(a, symmetrizeInput=False, lower=False), tri)
+    np.testing.assert_allclose(lo, [1, 3], atol=1e-4)
+    np.testing.assert_allclose(up, [-98, 102], rtol=1e-4, atol=1e-4)
+
+    tall = f32([[1, 2], [3, 4], [5, 6]])
+    prog, (u, sv, vh) = run(lambda a: L.svd(a), tall)
+    assert steps_of(prog).count("JacobiEigh") == 1 and steps_of(prog).count("Argsort") == 1
+    u, vh = u.reshape(3, 2), vh.reshape(2, 2)
+    np.testing.assert_allclose((u * sv) @ vh, tall, atol=1e-3)
+    np.testing.assert_allclose(u.T @ u, np.eye(2), atol=1e-3)
+    np.testing.assert_allclose(vh @ vh.T, np.eye(2), atol=1e-3)
+    np.testing.assert_allclose(sv, [9.525518, 0.514301], rtol=1e-4, atol=1e-4)
+    wide = f32([[1, 2, 3], [4, 5, 6]])
+    _, (u, sv, vh) = run(lambda a: L.svd(a), wide)
+    u, vh = u.reshape(2, 2), vh.reshape(2, 3)
+    np.testing.assert_allclose((u * sv) @ vh, wide, atol=1e-3)
+    np.testing.assert_allclose(vh @ vh.T, np.eye(2), atol=1e-3)
+    batched = f32([[[1, 2], [3, 4], [5, 6]], [[2, 0], [0, 3], [4, 0]]])
+    _, (u, sv, vh) = run(lambda a: L.svd(a), batched)
+    u, sv, vh = u.reshape(2, 3, 2), sv.reshape(2, 2), vh.reshape(2, 2, 2)
+    np.testing.assert_allclose((u * sv[:, None, :]) @ vh, batched, atol=1e-3)
+    _, (sv,) = run(lambda a: L.svdvals(a), f32([[3, 0], [0, 4]]))
+    np.testing.assert_allclose(sv, [4, 3], atol=1e-4)
+    with pytest.raises(ValueError):
+        run(lambda a: L.svd(a, fullMatrices=True), tall)
+
+    m = np.arange(2 * 4 * 6, dtype=np.float32).reshape(2, 4, 6)
+    for offset, a1, a2 in ((0, 1, 2), (1, 1, 2), (-2, 1, 2), (3, 2, 1), (0, 0, 2), (1, 2, 0), (5, -2, -1)):
+        prog, (d,) = run(lambda t: L.diagonal(t, offset, a1, a2), m)
+        want = np.diagonal(m, offset, a1, a2)
+        np.testing.assert_array_equal(d.reshape(want.shape), want)
+        assert steps_of(prog) == ["kernel"]  # a view: one copy kernel
+
+
 # ---- Concatenate / Split / Gather / RandomBits (src/frontend/jit.ts:666-763) -------------------------------------------
 
 U32, I32 = DType.Uint32, DType.Int32

@@ -172,6 +172,33 @@ def test_programs_with_routines(name):
             np.testing.assert_allclose(g, w, rtol=2e-5, atol=2e-5 * np.abs(w).max())
 
 
+@pytest.mark.parametrize("shape", [(3, 200, 24), (2, 16, 130), (1, 512, 64)], ids=str)
+def test_svd_program(shape):
+    """`svd` as the reference composes it (Gram product, Jacobi eigendecomposition routine, argsort + gathers, one more
+    product scaled by 1/s; src/library/lax-linalg.ts:102-163) traced and run on the GPU: singular values against
+    numpy's float64 SVD, reconstruction and orthogonality of the factors.  (The factors themselves are not compared
+    with the CPU run element by element: the Gram matrices of the two differ in the last place and near-degenerate
+    eigenvectors may rotate.)"""
+    from jaxjs_hip import jit as J
+    from jaxjs_hip import library as L
+    from jaxjs_hip.jit import ShapedArray
+    a = np.random.default_rng(21).standard_normal(shape).astype(np.float32)
+    prog = J.jit(lambda x: L.svd(x), [ShapedArray(shape, DType.Float32)])
+    assert [r.name.value for r in prog.routines] == ["JacobiEigh", "Argsort"]
+    if WARM_ONLY:
+        warm(prog)
+    u, sv, vh = run_program(backend(), prog, [a])
+    m, n = shape[-2:]
+    k = min(m, n)
+    u, sv, vh = u.reshape(shape[0], m, k).astype(np.float64), sv.reshape(shape[0], k).astype(np.float64), vh.reshape(shape[0], k, n).astype(np.float64)
+    want = np.linalg.svd(a.astype(np.float64), compute_uv=False)
+    # the Gram matrix squares the condition number: singular values are good to ~eps * s_max^2 / s
+    np.testing.assert_allclose(sv, want, rtol=2e-3, atol=2e-4 * want.max())
+    np.testing.assert_allclose((u * sv[:, None, :]) @ vh, a, atol=2e-3 * np.abs(a).max())
+    eye = np.broadcast_to(np.eye(k), (shape[0], k, k))
+    np.testing.assert_allclose(vh @ vh.transpose(0, 2, 1) if m >= n else u.transpose(0, 2, 1) @ u, eye, atol=2e-4)
+
+
 def _indexing_and_random_cases():
     from jaxjs_hip import jit as J
     from jaxjs_hip import library as L
