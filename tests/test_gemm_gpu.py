@@ -196,3 +196,21 @@ def test_gemm_f32_integer_exact_and_checker():
     got, _ = device_run(k, [A, B])
     want = oracle.run_kernel(k, [A, B], oracle.MODE_WASM)
     np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("H,D", [(4, 64), (3, 128), (2, 192)], ids=str)
+def test_gemm_f16_two_level_k_with_deep_slabs(H, D):
+    """A stored [H, M, D] and contracted over (h, d) against B stored [N, H*D]: both operands run along k, A in runs of
+    D with a jump between heads (the attention output feeding an out-projection whose weights are stored [out, in]).
+    D is a multiple of 64, so the 64-deep slabs never straddle two runs."""
+    M, N, K = 512, 512, H * D
+    A3 = RNG.uniform(-1, 1, (H, M, D)).astype(np.float16)
+    Bt = RNG.uniform(-1, 1, (N, K)).astype(np.float16)
+    full = [M, N, K]
+    stA = ShapeTracker.fromShape([H, M, D]).permute([1, 0, 2]).reshape([M, 1, K]).expand(full)
+    stB = ShapeTracker.fromShape([N, K]).reshape([1, N, K]).expand(full)
+    k = reduceKernel(full, [(DType.Float16, stA), (DType.Float16, stB)], lambda a, b: AluExp.mul(a, b), AluOp.Add)
+    got, ks = device_run(k, [A3, Bt])
+    assert ks.klass == "gemm" and ks.info["direct_lds"] and ks.info["BK"] == 64, ks.info
+    A = np.ascontiguousarray(A3.transpose(1, 0, 2)).reshape(M, K)
+    _check(got, A, Bt.T, K)
