@@ -24,6 +24,7 @@ from .shape import prod
 _SORT_KINDS = {DType.Float32: (0, "float"), DType.Float16: (1, "jh_f16"), DType.Int32: (2, "int"),
                DType.Uint32: (3, "jh_u32"), DType.Bool: (2, "int")}
 SORT_TILE = 8192  # 64 KB of LDS: rows up to 8192 elements never leave the CU
+SORT_GROUP = 8    # elements a thread sorts in registers at the end of every stage (4 for rows of <= 256: more threads stay busy)
 CHOLESKY_PANEL_FROM = 192  # matrix order from which Cholesky runs panel by panel over the whole chip
 
 
@@ -297,7 +298,7 @@ def _gen_sort(routine: Routine, numerics: str) -> Optional[KernelSource]:
     kind, ctype = _SORT_KINDS[dtype]
     threads = max(1, min(tile // 2, 1024))
     src = _prelude(numerics) + fill(template("sort.hip.inc"), dict(N=n, P=P, ROWS=rows, TILE=tile, ARGSORT=1 if argsort else 0,
-                                                                   KIND=kind, T=ctype, THREADS=threads))
+                                                                   KIND=kind, T=ctype, THREADS=threads, GROUP=SORT_GROUP if P > 256 else 4))
     tiles = rows * (P // tile)
     outs = [("out", 0), ("out", 1)] if argsort else [("out", 0), ("out", 0)]
     steps = [LaunchStep("jh_sort_local", (tiles, 1, 1), (threads, 1, 1), 0, [("in", 0), ("scratch", 0)] + outs)]
