@@ -193,23 +193,33 @@ def _gen_fft(routine: Routine, numerics: str) -> Optional[KernelSource]:
     if "singleLaunch" in params:  # tests pin either path
         fused = bool(params["singleLaunch"]) and S >= 1 and n <= FFT_FUSED_MAX_N
     threads = min(1024, max(64, _round64(n)))
+    # Twiddle tables: stage s has span_s entries for (q, j) and radix_s^2 for (q, p), 16 bytes each.
+    offsets, spans, prev = [0], [], 1
+    for radix in factors:
+        spans.append(prev * radix + radix * radix)
+        offsets.append(offsets[-1] + spans[-1])
+        prev *= radix
+    lds_entries = max(spans) if spans and 16 * n + 16 * max(spans) <= 150 * 1024 else 0
     src = _prelude(numerics) + fill(template("fft.hip.inc"), dict(N=n, ROWS=rows, INVERSE=1 if params.get("inverse") else 0,
                                                                   NF=len(factors), FACTORS=", ".join(map(str, factors)) or "1",
-                                                                  FUSED=1 if fused else 0, FUSED_THREADS=threads))
+                                                                  TW_OFFSETS=", ".join(map(str, offsets if S else [0, 0])),
+                                                                  FUSED=1 if fused else 0, FUSED_THREADS=threads,
+                                                                  FUSED_TABLE_ENTRIES=lds_entries))
     need = {0: rows * n * 4, 1: rows * n * 4}
     if fused:
         steps = [LaunchStep("jh_fft_rows", (min(rows, 1 << 16), 1, 1), (threads, 1, 1), 0, [("in", 0), ("in", 1), ("out", 0), ("out", 1)])]
-        return KernelSource([src], steps, [], "fft", need, dict(n=n, rows=rows, factors=factors, launches=1, fused=True))
+        return KernelSource([src], steps, [], "fft", need, dict(n=n, rows=rows, factors=factors, launches=1, fused=True, lds_tables=bool(lds_entries)))
     blocks = max(1, min((rows * n + 255) // 256, 1 << 20))
     out_pair, tmp_pair = [("out", 0), ("out", 1)], [("scratch", 0), ("scratch", 1)]
     target = lambda s: out_pair if (S - 1 - s) % 2 == 0 else tmp_pair  # noqa: E731  (stage -1 is the permutation)
-    steps = [LaunchStep("jh_fft_permute", (blocks, 1, 1), (256, 1, 1), 0, [("in", 0), ("in", 1)] + target(-1))]
+    steps = [LaunchStep("jh_fft_permute", (blocks, 1, 1), (256, 1, 1), 0, [("in", 0), ("in", 1)] + target(-1) + [("scratch", 2)])]
     prev = 1
-    for s, radix in enumerate(factors):
+    for s_, radix in enumerate(factors):
         steps.append(LaunchStep("jh_fft_stage", (blocks, 1, 1), (256, 1, 1), 0,
-                                target(s - 1) + target(s) + [("const", prev), ("const", radix), ("const", 1 if s == S - 1 else 0)]))
+                                target(s_ - 1) + target(s_) + [("scratch", 2), ("const", prev), ("const", radix),
+                                                               ("const", 1 if s_ == S - 1 else 0), ("const", s_)]))
         prev *= radix
-    scratch = [rows * n * 4, rows * n * 4] if S >= 1 else [8, 8]
+    scratch = [rows * n * 4, rows * n * 4, max(offsets[-1], 1) * 16] if S >= 1 else [8, 8, 16]
     return KernelSource([src], steps, scratch, "fft", need, dict(n=n, rows=rows, factors=factors, launches=len(steps), fused=False))
 
 
