@@ -77,6 +77,21 @@ def _gen_cholesky(routine: Routine, numerics: str) -> Optional[KernelSource]:
     batch = prod(shape[:-2])
     if batch == 0 or n == 0:
         return _empty("cholesky", n=n, batch=batch)
+    if n >= CHOLESKY_PANEL_FROM and batch * n * n * 8 <= CHOLESKY_RIGHT_LOOKING_MAX_BYTES:
+        # Large matrices, right-looking: the running sums of the whole triangle in a double-precision scratch copy; per
+        # 32-column panel one launch that finishes the panel and one that updates the trailing triangle (bit-identical).
+        src = _linalg_source(numerics, ROUTINE=5, N=n, M=batch)
+        grid1 = lambda count: (max(1, min((count + 255) // 256, 1 << 16)), 1, 1)  # noqa: E731
+        steps = [LaunchStep("jh_chol_init", grid1(batch * n * n), (256, 1, 1), 0, [("in", 0), ("out", 0), ("scratch", 0)])]
+        for j0 in range(0, n, 32):
+            after = max(0, n - j0 - 32)
+            steps.append(LaunchStep("jh_chol_panel", (batch * max(1, (after + 63) // 64), 1, 1), (64, 1, 1), 0,
+                                    [("scratch", 0), ("out", 0), ("const", j0)]))
+            if after > 0:
+                T = (after + 63) // 64
+                steps.append(LaunchStep("jh_chol_update", (batch * T * T, 1, 1), (256, 1, 1), 0, [("out", 0), ("scratch", 0), ("const", j0)]))
+        return KernelSource([src], steps, [batch * n * n * 8], "cholesky", {0: batch * n * n * 4},
+                            dict(n=n, batch=batch, panels=(n + 31) // 32, launches=len(steps), variant="right-looking"))
     if n >= CHOLESKY_PANEL_FROM and batch * n * n < (1 << 31):
         # Large matrices: 32-column panels, two launches each, every launch spread over the chip; the same sums in the
         # same order as the single-workgroup kernel (bit-identical results).
@@ -164,6 +179,7 @@ def _gen_jacobi(routine: Routine, numerics: str) -> Optional[KernelSource]:
     return KernelSource([src], steps, [], "jacobi", {0: batch * n * n * 4}, dict(n=n, batch=batch, threads=threads, in_lds=bool(in_lds)))
 
 
+CHOLESKY_RIGHT_LOOKING_MAX_BYTES = 1 << 30  # the double-precision working copy of all matrices
 FFT_FUSED_MAX_N = 8192  # 16 bytes of LDS per point: 128 KiB
 
 

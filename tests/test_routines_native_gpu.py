@@ -46,6 +46,19 @@ def test_cholesky(shape):
     assert_bits(got, want, f"cholesky {shape} {ks.info}")
 
 
+@pytest.mark.parametrize("shape", [(200, 200), (2, 333, 333), (1100, 1100)], ids=str)
+def test_cholesky_left_looking_panels_when_the_double_copy_is_too_large(shape, monkeypatch):
+    """The right-looking variant keeps a double-precision copy of every matrix; beyond its size limit the left-looking
+    panels run instead.  Same sums in the same order: identical bits."""
+    from jaxjs_hip import routinegen
+    x = spd(tuple(shape[:-2]), shape[-1])
+    right, k1 = R.run_gpu(R.cholesky(x), [x])
+    monkeypatch.setattr(routinegen, "CHOLESKY_RIGHT_LOOKING_MAX_BYTES", 0)
+    left, k2 = R.run_gpu(R.cholesky(x), [x])
+    assert k1.info.get("variant") == "right-looking" and "variant" not in k2.info and "panels" in k2.info
+    assert_bits(left, right, f"cholesky variants {shape}")
+
+
 def test_cholesky_not_positive_definite_and_empty():
     x = np.array([[[1, 2], [2, 1]], [[4, 2], [2, 3]]], F32)
     got, want, _ = both(R.cholesky(x), [x])
