@@ -95,6 +95,27 @@ def test_binary_int_bit_exact(dtype, name):
     assert_parity(mapKernel([n], [(dtype, st), (dtype, st)], fn), [a, b], exact=True)
 
 
+@pytest.mark.parametrize("dtype", [DType.Int32, DType.Uint32])
+def test_constant_multiply_divide_is_folded_as_the_reference_folds_it(dtype):
+    """`(x * A) / B` with B | A is rewritten to `x * (A / B)` by the reference's simplifier with no regard to wrap-around
+    (src/alu.ts:795-806), and every reference backend runs that simplifier (tuneNullopt, src/tuner.ts:219-240).  So for
+    operands whose product overflows, the reference's answer is the folded one, `x * (A / B)` — not `trunc(wrap(x * A) /
+    B)`, which is what evaluating the unsimplified expression gives.  The backend follows the reference; the checker, which
+    by design evaluates unsimplified expressions, is the one that differs here, and only here."""
+    from gpu_util import device_run
+    from oracle import oracle
+    nd = np.int32 if dtype == DType.Int32 else np.uint32
+    x = np.concatenate([INT_SPECIAL, [400000000, -400000000, 1000000007, -1999999973]]).astype(nd)
+    n = len(x)
+    k = mapKernel([n], [(dtype, ShapeTracker.fromShape([n]))], lambda v: AluExp.idiv(AluExp.mul(v, AluExp.const(dtype, 14)), AluExp.const(dtype, 7)))
+    got, _ = device_run(k, [x])
+    np.testing.assert_array_equal(got, (x.astype(np.int64) * 2).astype(nd))  # x * 2, wrapped
+    unsimplified = oracle.run_kernel(k, [x], oracle.MODE_WASM)
+    small = np.abs(x.astype(np.int64)) < (1 << 27)
+    np.testing.assert_array_equal(got[small], unsimplified[small])  # no overflow: the two readings agree
+    assert (got != unsimplified).any()                               # overflow: they do not
+
+
 def test_bool_ops_bit_exact():
     a = np.array([0, 0, 1, 1] * 5, dtype=np.int32)
     b = np.array([0, 1, 0, 1] * 5, dtype=np.int32)
