@@ -53,7 +53,7 @@ def _round64(n: int, cap: int = 1024) -> int:
     return max(64, min(cap, (n + 63) // 64 * 64))
 
 
-_LINALG_DEFAULTS = dict(ROUTINE=0, N=1, M=1, THREADS=64, UNIT=0, IN_LDS=0, MAX_SWEEPS=0, TOL="0.0")
+_LINALG_DEFAULTS = dict(ROUTINE=0, N=1, M=1, THREADS=64, UNIT=0, IN_LDS=0, MAX_SWEEPS=0, TOL="0.0", BATCH=1)
 
 
 def _linalg_source(numerics: str, **params) -> str:
@@ -144,11 +144,28 @@ def _gen_lu(routine: Routine, numerics: str) -> Optional[KernelSource]:
     if len(shape) < 2:
         raise ValueError("lu: input must be at least 2D")
     m, n = shape[-2], shape[-1]
-    if not _all_f32(t) or m > 4096:  # the multipliers of one column live in LDS as doubles
+    if not _all_f32(t):
         return None
     batch = prod(shape[:-2])
     if batch == 0 or m == 0:
         return _empty("lu", m=m, n=n, batch=batch)
+    if min(m, n) >= LU_BY_COLUMNS_FROM and batch * m * n < (1 << 31):
+        # Large matrices: two launches per column, the rank-1 update of the trailing block over the whole chip; the same
+        # operations per element as the single-workgroup kernel (bit-identical).
+        src = _linalg_source(numerics, ROUTINE=6, N=n, M=m, THREADS=1024, BATCH=batch)
+        grid1 = lambda count: (max(1, min((count + 255) // 256, 1 << 16)), 1, 1)  # noqa: E731
+        steps = [LaunchStep("jh_lu_init", grid1(batch * m * n), (256, 1, 1), 0, [("in", 0), ("out", 0), ("out", 2)])]
+        for j in range(min(m, n)):
+            steps.append(LaunchStep("jh_lu_col", (batch, 1, 1), (1024, 1, 1), 0,
+                                    [("out", 0), ("out", 1), ("out", 2), ("scratch", 0), ("scratch", 1), ("const", j)]))
+            rows, cols = m - j - 1, n - j - 1
+            if rows > 0 and cols > 0:
+                steps.append(LaunchStep("jh_lu_update", (batch * ((cols + 63) // 64) * ((rows + 31) // 32), 1, 1), (256, 1, 1), 0,
+                                        [("out", 0), ("scratch", 0), ("scratch", 1), ("const", j)]))
+        return KernelSource([src], steps, [batch * m * 8, max(batch * 4, 16)], "lu", {0: batch * m * n * 4},
+                            dict(m=m, n=n, batch=batch, launches=len(steps), variant="by columns"))
+    if m > 4096:  # single workgroup: the multipliers of one column live in LDS as doubles
+        return None
     threads = _round64(max(m, n))
     src = _linalg_source(numerics, ROUTINE=2, N=n, M=m, THREADS=threads)
     steps = [LaunchStep("jh_lu", (batch, 1, 1), (threads, 1, 1), 0, [("in", 0), ("out", 0), ("out", 1), ("out", 2)])]
@@ -179,6 +196,7 @@ def _gen_jacobi(routine: Routine, numerics: str) -> Optional[KernelSource]:
     return KernelSource([src], steps, [], "jacobi", {0: batch * n * n * 4}, dict(n=n, batch=batch, threads=threads, in_lds=bool(in_lds)))
 
 
+LU_BY_COLUMNS_FROM = 256  # smaller dimension from which LU runs two launches per column over the whole chip
 CHOLESKY_RIGHT_LOOKING_MAX_BYTES = 1 << 30  # the double-precision working copy of all matrices
 FFT_FUSED_MAX_N = 8192  # 16 bytes of LDS per point: 128 KiB
 

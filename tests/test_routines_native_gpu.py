@@ -88,11 +88,26 @@ def test_triangular_solve(case, unit):
     assert_bits(got, want, f"triangular_solve {case} {ks.info}")
 
 
-@pytest.mark.parametrize("shape", [(2, 2), (1, 5), (5, 1), (2, 7, 5), (3, 12, 20), (2, 2, 30, 30), (150, 97), (260, 300)], ids=str)
+@pytest.mark.parametrize("shape", [(2, 2), (1, 5), (5, 1), (2, 7, 5), (3, 12, 20), (2, 2, 30, 30), (150, 97), (260, 300), (255, 400),
+                                   (2, 300, 256), (513, 300), (1024, 1024)], ids=str)
 def test_lu(shape):
     a = RNG.uniform(-1, 1, shape).astype(F32)
     got, want, ks = both(R.lu(a), [a])
+    # from 256 rows and columns on: two launches per column, the trailing update over the whole chip
+    assert (ks.info.get("variant") == "by columns") == (min(shape[-2:]) >= 256)
     assert_bits(got, want, f"lu {shape} {ks.info}")
+
+
+def test_lu_by_columns_zero_pivot_and_nan_columns():
+    """The special cases of the small kernel's test, embedded in matrices large enough for the by-columns variant: a zero
+    pivot column (that step eliminates nothing), equal magnitudes (the first row wins), a NaN that must not win."""
+    a = RNG.uniform(-1, 1, (2, 260, 260)).astype(F32)
+    a[0, :, 3] = 0.0   # stays zero through every update: step 3 meets a zero pivot
+    a[1, 10, 5] = np.nan
+    a[1, 20:23, 7] = [0.75, -0.75, 0.75]
+    got, want, ks = both(R.lu(a), [a])
+    assert ks.info["variant"] == "by columns"
+    assert_bits(got, want, "lu by columns, special columns")
 
 
 def test_lu_ties_zero_pivots_and_nans():
