@@ -53,7 +53,7 @@ def _round64(n: int, cap: int = 1024) -> int:
     return max(64, min(cap, (n + 63) // 64 * 64))
 
 
-_LINALG_DEFAULTS = dict(ROUTINE=0, N=1, M=1, THREADS=64, UNIT=0, IN_LDS=0, MAX_SWEEPS=0, TOL="0.0", BATCH=1)
+_LINALG_DEFAULTS = dict(ROUTINE=0, N=1, M=1, THREADS=64, UNIT=0, IN_LDS=0, MAX_SWEEPS=0, TOL="0.0", BATCH=1, AHEAD=16, STAGED=0, RB=1)
 
 
 def _linalg_source(numerics: str, **params) -> str:
@@ -129,13 +129,21 @@ def _gen_trisolve(routine: Routine, numerics: str) -> Optional[KernelSource]:
         raise ValueError(f"triangular_solve: incompatible shapes a={a_shape}, b={b_shape}")
     if mats == 0 or m == 0 or n == 0:
         return _empty("trisolve", n=n, m=m, batch=mats)
-    threads = 64 if m <= 64 else 256
     unit = 1 if (routine.params or {}).get("unitDiagonal", False) else 0
-    src = _linalg_source(numerics, ROUTINE=1, N=n, M=m, THREADS=threads, UNIT=unit)
+    need = {0: mats * n * n * 4, 1: mats * m * n * 4}
+    if TRISOLVE_STAGED_FROM <= n <= TRISOLVE_STAGED_MAX_N:
+        # one wave of 64 right-hand sides + three waves staging blocks of rows in LDS as doubles (two buffers <= 128 KB)
+        rb = max(1, min(8, TRISOLVE_STAGED_MAX_N // n))
+        src = _linalg_source(numerics, ROUTINE=1, N=n, M=m, THREADS=256, UNIT=unit, AHEAD=TRISOLVE_AHEAD, STAGED=1, RB=rb)
+        steps = [LaunchStep("jh_trisolve_staged", (mats * ((m + 63) // 64), 1, 1), (256, 1, 1), 0,
+                            [("in", 0), ("in", 1), ("out", 0), ("scratch", 0)])]
+        return KernelSource([src], steps, [mats * m * n * 8], "trisolve", need,
+                            dict(n=n, m=m, batch=mats, threads=256, staged=True, rows_per_block=rb))
+    threads = 64 if m <= 64 else 256
+    src = _linalg_source(numerics, ROUTINE=1, N=n, M=m, THREADS=threads, UNIT=unit, AHEAD=TRISOLVE_AHEAD)
     blocks = mats * ((m + threads - 1) // threads)
     steps = [LaunchStep("jh_trisolve", (blocks, 1, 1), (threads, 1, 1), 0, [("in", 0), ("in", 1), ("out", 0), ("scratch", 0)])]
-    need = {0: mats * n * n * 4, 1: mats * m * n * 4}
-    return KernelSource([src], steps, [mats * m * n * 4], "trisolve", need, dict(n=n, m=m, batch=mats, threads=threads))
+    return KernelSource([src], steps, [mats * m * n * 4], "trisolve", need, dict(n=n, m=m, batch=mats, threads=threads, staged=False))
 
 
 def _gen_lu(routine: Routine, numerics: str) -> Optional[KernelSource]:
@@ -196,6 +204,9 @@ def _gen_jacobi(routine: Routine, numerics: str) -> Optional[KernelSource]:
     return KernelSource([src], steps, [], "jacobi", {0: batch * n * n * 4}, dict(n=n, batch=batch, threads=threads, in_lds=bool(in_lds)))
 
 
+TRISOLVE_STAGED_FROM = 128    # matrix size from which TriangularSolve stages the matrix in LDS with helper waves
+TRISOLVE_STAGED_MAX_N = 8192   # two one-row buffers of doubles still fit in LDS
+TRISOLVE_AHEAD = 8       # entries of a row that a right-hand side's thread fetches ahead of its subtraction chain
 LU_BY_COLUMNS_FROM = 256  # smaller dimension from which LU runs two launches per column over the whole chip
 CHOLESKY_RIGHT_LOOKING_MAX_BYTES = 1 << 30  # the double-precision working copy of all matrices
 FFT_FUSED_MAX_N = 8192  # 16 bytes of LDS per point: 128 KiB

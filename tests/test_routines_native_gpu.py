@@ -76,7 +76,8 @@ def test_cholesky_not_positive_definite_and_empty():
         R.run_gpu(R.cholesky(np.zeros((2, 3), F32)), [np.zeros((2, 3), F32)])
 
 
-@pytest.mark.parametrize("case", [((2, 2), 1), ((9, 9), 4), ((3, 30, 30), 7), ((2, 2, 16, 16), 100), ((300, 300), 300), ((64, 64), 1000)], ids=str)
+@pytest.mark.parametrize("case", [((2, 2), 1), ((9, 9), 4), ((3, 30, 30), 7), ((2, 2, 16, 16), 100), ((300, 300), 300), ((64, 64), 1000),
+                                  ((2, 131, 131), 70), ((128, 128), 3), ((1024, 1024), 64)], ids=str)
 @pytest.mark.parametrize("unit", [False, True])
 def test_triangular_solve(case, unit):
     ashape, m = case
@@ -85,6 +86,7 @@ def test_triangular_solve(case, unit):
          + np.tril(RNG.standard_normal(ashape), -1)).astype(F32)  # the strictly lower part must not matter
     b = RNG.standard_normal(ashape[:-2] + (m, n)).astype(F32)
     got, want, ks = both(R.triangular_solve(a, b, unit), [a, b])
+    assert ks.info["staged"] == (n >= 128)  # from 128 on helper waves stage the matrix in LDS as doubles
     assert_bits(got, want, f"triangular_solve {case} {ks.info}")
 
 
