@@ -5,7 +5,7 @@ heuristics (upcast/unroll/group sizes for 32-wide SIMD groups and a 65535-group 
 over; `tuneHip` instead classifies the lowered expression's memory accesses and picks one of the
 hand-written CDNA4 templates:
 
-  map         no reduction: grid-stride, V consecutive outputs per lane, 128-bit loads/stores
+  map         no reduction: V consecutive outputs per lane, 128-bit loads/stores, blocks in buffer order
   reduce_row  reduce axis contiguous in memory: T lanes walk one output's reduce axis with vector
               loads, wave64 shuffle tree (+ LDS across waves) to combine; matvec W[M,K].x is this
               class with one wave per row
