@@ -49,6 +49,19 @@ class _Prepared:
         self.functions = functions  # one per launch step
         self.scratch = scratch      # device pointers owned by this executable
         self.modules = modules
+        # Per launch step: (argument cells, kernelParams array, [(cell, "in"|"out", index)] to fill per dispatch).
+        # Scratch pointers and integer arguments are written once; a dispatch only stores the slot pointers, so a
+        # plan of hundreds of small launches is not bound by building ctypes objects.
+        self.bound = []
+        for step in ks.steps:
+            argv, cells = pack_args([0] * len(step.args))
+            patch = []
+            for c, (kind, i) in enumerate(step.args):
+                if kind in ("in", "out"):
+                    patch.append((c, kind, i))
+                else:
+                    cells[c] = scratch[i] if kind == "scratch" else int(i)
+            self.bound.append((cells, argv, patch))
 
 
 _ALIGN = 256  # allocation granularity; also keeps every slot 128-bit-load aligned
@@ -209,19 +222,11 @@ class HipBackend:
                     need = prep.ks.min_input_bytes[i]
                 if s["size"] < need:
                     raise ValueError(f"{what} {i} holds {s['size']} bytes, the routine addresses {need}")
-        for step, fn in zip(prep.ks.steps, prep.functions):
-            values = []
-            for kind, i in step.args:
-                if kind == "in":
-                    values.append(ins[i]["ptr"])
-                elif kind == "out":
-                    values.append(outs[i]["ptr"])
-                elif kind == "scratch":
-                    values.append(prep.scratch[i])
-                else:
-                    values.append(int(i))
-            argv, keep = pack_args(values)
-            self.dev.launch(fn, step.grid, step.block, step.shared, argv, 1)
+        launch = self.dev.launch
+        for step, fn, (cells, argv, patch) in zip(prep.ks.steps, prep.functions, prep.bound):
+            for c, kind, i in patch:
+                cells[c] = (ins if kind == "in" else outs)[i]["ptr"]
+            launch(fn, step.grid, step.block, step.shared, argv, 1)
 
     def dispatch(self, exe: Executable, inputs: Sequence[int], outputs: Sequence[int], repeat: int = 1) -> None:
         ins = [self._get(s) for s in inputs]
@@ -245,16 +250,9 @@ class HipBackend:
                 raise ValueError(f"input {gid} holds {ins[gid]['size']} bytes, kernel addresses {need}")
         if kernel.size == 0:
             return
-        for step, fn in zip(prep.ks.steps, prep.functions):
-            values = []
-            for kind, i in step.args:
-                if kind == "in":
-                    values.append(ins[i]["ptr"])
-                elif kind == "out":
-                    values.append(outs[0]["ptr"])
-                else:
-                    values.append(prep.scratch[i])
-            argv, keep = pack_args(values)
+        for step, fn, (cells, argv, patch) in zip(prep.ks.steps, prep.functions, prep.bound):
+            for c, kind, i in patch:
+                cells[c] = ins[i]["ptr"] if kind == "in" else outs[0]["ptr"]
             if self.trace is not None:
                 e0, e1 = self.dev.event(), self.dev.event()
                 self.dev.record(e0)
@@ -263,7 +261,6 @@ class HipBackend:
                 self.trace.append((f"{prep.ks.klass}:{step.name}", e0, e1))
             else:
                 self.dev.launch(fn, step.grid, step.block, step.shared, argv, repeat)
-            del keep
 
     def sync(self) -> None:
         """Completion fence (what `read(slot, 0, 0)` stands for in src/frontend/array.ts:827)."""

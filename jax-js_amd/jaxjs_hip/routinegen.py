@@ -207,7 +207,7 @@ def _gen_jacobi(routine: Routine, numerics: str) -> Optional[KernelSource]:
 TRISOLVE_STAGED_FROM = 128    # matrix size from which TriangularSolve stages the matrix in LDS with helper waves
 TRISOLVE_STAGED_MAX_N = 8192   # two one-row buffers of doubles still fit in LDS
 TRISOLVE_AHEAD = 8       # entries of a row that a right-hand side's thread fetches ahead of its subtraction chain
-LU_BY_COLUMNS_FROM = 256  # smaller dimension from which LU runs two launches per column over the whole chip
+LU_BY_COLUMNS_FROM = 192  # smaller dimension from which LU runs two launches per column over the whole chip
 CHOLESKY_RIGHT_LOOKING_MAX_BYTES = 1 << 30  # the double-precision working copy of all matrices
 FFT_FUSED_MAX_N = 8192  # 16 bytes of LDS per point: 128 KiB
 

@@ -261,7 +261,11 @@ class Device:
 
 
 def pack_args(values: Sequence[int]):
-    """kernelParams array for device-pointer arguments: returns (argv, keepalive)."""
-    cells = [ctypes.c_void_p(v) for v in values]
-    argv = (ctypes.c_void_p * len(cells))(*[ctypes.cast(ctypes.pointer(c), ctypes.c_void_p) for c in cells])
+    """kernelParams array for 8-byte arguments (device pointers, integers): returns (argv, keepalive).
+    One array holds the values and one the addresses of its cells; a plan of hundreds of small launches
+    (LU by columns, staged FFT) is bound by this host work, so no per-argument ctypes object is made."""
+    n = len(values)
+    cells = (ctypes.c_uint64 * n)(*values)
+    base = ctypes.addressof(cells)
+    argv = (ctypes.c_void_p * n)(*[base + 8 * i for i in range(n)])
     return argv, cells

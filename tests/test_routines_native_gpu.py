@@ -95,8 +95,8 @@ def test_triangular_solve(case, unit):
 def test_lu(shape):
     a = RNG.uniform(-1, 1, shape).astype(F32)
     got, want, ks = both(R.lu(a), [a])
-    # from 256 rows and columns on: two launches per column, the trailing update over the whole chip
-    assert (ks.info.get("variant") == "by columns") == (min(shape[-2:]) >= 256)
+    # from 192 rows and columns on: two launches per column, the trailing update over the whole chip
+    assert (ks.info.get("variant") == "by columns") == (min(shape[-2:]) >= 192)
     assert_bits(got, want, f"lu {shape} {ks.info}")
 
 
