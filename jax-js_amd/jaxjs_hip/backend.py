@@ -30,7 +30,7 @@ from .alu import Kernel, byteWidth
 from .errors import HipRuntimeError, SlotError, UnsupportedRoutineError
 from .kernelgen import KernelSource, generate
 from .routine import Routine
-from .runtime import Device, compile_source, pack_args
+from .runtime import Device, check, compile_source, pack_args
 
 
 class Executable:
@@ -62,6 +62,8 @@ class _Prepared:
                 else:
                     cells[c] = scratch[i] if kind == "scratch" else int(i)
             self.bound.append((cells, argv, patch))
+        # jh_launch's leading arguments per step, converted once
+        self.launch_head = [(ctypes.c_void_p(fn), *step.grid, *step.block, step.shared) for step, fn in zip(ks.steps, functions)]
 
 
 _ALIGN = 256  # allocation granularity; also keeps every slot 128-bit-load aligned
@@ -222,11 +224,13 @@ class HipBackend:
                     need = prep.ks.min_input_bytes[i]
                 if s["size"] < need:
                     raise ValueError(f"{what} {i} holds {s['size']} bytes, the routine addresses {need}")
-        launch = self.dev.launch
-        for step, fn, (cells, argv, patch) in zip(prep.ks.steps, prep.functions, prep.bound):
+        jh_launch = self.dev.lib.jh_launch
+        for head, (cells, argv, patch) in zip(prep.launch_head, prep.bound):
             for c, kind, i in patch:
                 cells[c] = (ins if kind == "in" else outs)[i]["ptr"]
-            launch(fn, step.grid, step.block, step.shared, argv, 1)
+            rc = jh_launch(*head, argv)
+            if rc:
+                check(rc, "jh_launch")
 
     def dispatch(self, exe: Executable, inputs: Sequence[int], outputs: Sequence[int], repeat: int = 1) -> None:
         ins = [self._get(s) for s in inputs]
@@ -250,10 +254,14 @@ class HipBackend:
                 raise ValueError(f"input {gid} holds {ins[gid]['size']} bytes, kernel addresses {need}")
         if kernel.size == 0:
             return
-        for step, fn, (cells, argv, patch) in zip(prep.ks.steps, prep.functions, prep.bound):
+        for step, fn, head, (cells, argv, patch) in zip(prep.ks.steps, prep.functions, prep.launch_head, prep.bound):
             for c, kind, i in patch:
                 cells[c] = ins[i]["ptr"] if kind == "in" else outs[0]["ptr"]
-            if self.trace is not None:
+            if self.trace is None and repeat == 1:
+                rc = self.dev.lib.jh_launch(*head, argv)
+                if rc:
+                    check(rc, "jh_launch")
+            elif self.trace is not None:
                 e0, e1 = self.dev.event(), self.dev.event()
                 self.dev.record(e0)
                 self.dev.launch(fn, step.grid, step.block, step.shared, argv, repeat)
