@@ -104,6 +104,11 @@ int jh_compile(const char *source, const char *name, const char *const *options,
                void **code, size_t *code_size, char *log, size_t log_size);
 void jh_code_free(void *code);
 
+/* Version of the run-time compiler behind `jh_compile` (hiprtcVersion).  The host side mixes it into the key of its
+ * on-disk code-object cache, so that a toolchain change never reuses stale code objects (the WebGPU backend's
+ * pipeline cache is keyed by shader text alone because the browser owns the compiler, src/backend/webgpu.ts:705-744). */
+int jh_compiler_version(int *major, int *minor);
+
 /* Load a code object on the device and look up a kernel in it. */
 int jh_module_load(const void *code, size_t code_size, jh_module *out);
 int jh_module_unload(jh_module module);

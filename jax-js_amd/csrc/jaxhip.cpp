@@ -51,7 +51,7 @@ int fail(int code, const char *fmt, ...) {
 
 extern "C" {
 
-int jh_abi_version(void) { return 1; }
+int jh_abi_version(void) { return 2; }
 
 const char *jh_last_error(void) { return g_last_error.c_str(); }
 
@@ -224,6 +224,13 @@ int jh_compile(const char *source, const char *name, const char *const *options,
 }
 
 void jh_code_free(void *code) { free(code); }
+
+int jh_compiler_version(int *major, int *minor) {
+  if (!major || !minor) return fail(-5, "null output");
+  hiprtcResult r = hiprtcVersion(major, minor);
+  if (r != HIPRTC_SUCCESS) return fail((int)r, "hiprtcVersion: %s", hiprtcGetErrorString(r));
+  return 0;
+}
 
 int jh_module_load(const void *code, size_t code_size, jh_module *out) {
   JH_NEED_INIT();

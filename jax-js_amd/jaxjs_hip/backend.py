@@ -16,19 +16,21 @@ Mirrors `interface Backend` (reference: src/backend.ts:158-211) member for membe
   observes every earlier dispatch (src/backend.ts:203-210).
 
 Device memory, compilation and launches go through the C ABI of `include/jaxhip.h`; there is no
-host fallback for kernels.  Routines run on the host exactly as the reference's Wasm backend does
-(src/backend/wasm.ts:158-165, 216-220), through device->host->device copies.
+host fallback, neither for kernels nor for routines (the reference's Wasm backend runs routines on
+the host, src/backend/wasm.ts:158-165, 216-220; here every routine is a plan of GPU launches and a
+routine without one raises `UnsupportedRoutineError` at prepare time).
 """
 
 from __future__ import annotations
 
 import asyncio
 import ctypes
+from collections import OrderedDict
 from typing import Dict, List, Optional, Sequence
 
 from .alu import Kernel, byteWidth
 from .errors import HipRuntimeError, SlotError, UnsupportedRoutineError
-from .kernelgen import KernelSource, generate
+from .kernelgen import NUMERICS, KernelSource, generate
 from .routine import Routine
 from .runtime import Device, check, compile_source, pack_args
 
@@ -64,29 +66,68 @@ class _Prepared:
             self.bound.append((cells, argv, patch))
         # jh_launch's leading arguments per step, converted once
         self.launch_head = [(ctypes.c_void_p(fn), *step.grid, *step.block, step.shared) for step, fn in zip(ks.steps, functions)]
+        self.released = False
+
+    def release(self, dev) -> None:
+        """Give back what the executable owns on the device: its scratch buffers and its loaded code objects.  Waits for
+        the stream first, so launches of it that are still queued finish on live code and memory."""
+        if self.released:
+            return
+        self.released = True
+        dev.sync()
+        for ptr in self.scratch:
+            dev.free(ptr)
+        for m in self.modules:
+            dev.unload_module(m)
+        self.scratch, self.modules, self.functions, self.bound, self.launch_head = [], [], [], [], []
 
 
 _ALIGN = 256  # allocation granularity; also keeps every slot 128-bit-load aligned
 
 
+def _freeze(v):
+    if isinstance(v, dict):
+        return tuple(sorted((str(k), _freeze(x)) for k, x in v.items()))
+    if isinstance(v, (list, tuple)):
+        return tuple(_freeze(x) for x in v)
+    if isinstance(v, (int, float, str, bool, type(None))):
+        return (type(v).__name__, v)
+    return ("repr", repr(v))
+
+
+def routineKey(routine: Routine) -> tuple:
+    """Structural identity of a routine: name, operand shapes and dtypes, parameters."""
+    t = routine.type
+    return (str(routine.name), _freeze(t.inputShapes), tuple(str(d) for d in t.inputDtypes), _freeze(t.outputShapes),
+            tuple(str(d) for d in t.outputDtypes), _freeze(routine.params))
+
+
 class HipBackend:
-    """MI355X backend.  `numerics="wasm"` evaluates transcendentals with the reference Wasm
-    backend's polynomials (bit-faithful to the parity oracle); `"native"` uses the device libm."""
+    """MI355X backend.  `numerics="wasm"` evaluates transcendentals with the reference Wasm backend's polynomials,
+    operation for operation (f32 maps within 2 ulp of the parity oracle); the default `"fast"` is the same except that
+    `exp` and `reciprocal` run on the hardware's exp2 / rcp instructions (within rel 1e-5 of the oracle, the bar for f32
+    maps), which is what keeps fused softmax-style rows bound by HBM instead of the VALU; `"native"` uses the device
+    libm."""
 
     type = "hip"
     maxArgs = 64  # kernel parameters are plain pointers; same bound as the Wasm backend (src/backend/wasm.ts:38)
 
-    def __init__(self, device: int = 0, numerics: str = "wasm"):
-        if numerics not in ("wasm", "native"):
-            raise ValueError("numerics must be 'wasm' or 'native'")
+    def __init__(self, device: int = 0, numerics: str = "fast"):
+        if numerics not in NUMERICS:
+            raise ValueError(f"numerics must be one of {NUMERICS}")
         self.numerics = numerics
         self.dev = Device.get(device)
+        from . import tuner
+
+        tuner.set_compute_units(self.dev.info.compute_units)
         self._slots: Dict[int, dict] = {}
         self._next_slot = 1
         self._pool: Dict[int, List[int]] = {}   # rounded size -> free device pointers
         self._pool_bytes = 0
         self._pool_limit = 8 << 30
-        self._exes: Dict[tuple, Executable] = {}
+        self._exes: "OrderedDict[tuple, Executable]" = OrderedDict()
+        self.cacheLimit = 4096
+        self._staging: Dict[int, List[int]] = {}  # capacity -> free pinned host buffers for asynchronous reads
         self.trace: Optional[list] = None       # when a list: (label, start_event, stop_event) per dispatch
 
     # -- memory -----------------------------------------------------------------------------------
@@ -167,27 +208,83 @@ class HipBackend:
         return self.dev.d2h(s["ptr"], start, count)
 
     async def read(self, slot: int, start: Optional[int] = None, count: Optional[int] = None) -> bytearray:
-        # Single-threaded host like the reference; yield once so callers can overlap preparation.
-        await asyncio.sleep(0)
-        return self.readSync(slot, start, count)
+        """Asynchronous read (src/backend.ts:182-186; the staging-buffer map of src/backend/webgpu/reader.ts): the copy
+        into pinned host memory is queued behind every earlier dispatch and the coroutine yields to the event loop until
+        its completion event has passed, so a caller that awaits a result keeps preparing and dispatching other work
+        meanwhile.  The slot may be released while the copy is in flight: a later owner of the memory can only write it
+        through work queued on the same in-order stream, after the copy."""
+        s = self._get(slot)
+        start = 0 if start is None else int(start)
+        count = s["size"] - start if count is None else int(count)
+        if start < 0 or count < 0 or start + count > s["size"]:
+            raise ValueError(f"read range [{start}, {start + count}) outside buffer of {s['size']} bytes")
+        cap, host = self._staging_take(count)
+        ev = self.dev.d2h_async(host, s["ptr"], start, count)
+        try:
+            while not self.dev.event_done(ev):
+                await asyncio.sleep(0)
+            return bytearray(ctypes.string_at(host, count)) if count else bytearray()
+        finally:
+            # leaving early (cancellation) must not hand the buffer on while the copy may still land in it
+            self.dev.lib.jh_event_sync(ctypes.c_void_p(ev))
+            self.dev.destroy_event(ev)
+            self._staging_give(cap, host)
+
+    def _staging_take(self, nbytes: int):
+        """A pinned staging buffer of at least `nbytes` (power-of-two classes from 4 KiB, a few kept per class)."""
+        if nbytes == 0:
+            return 0, 0
+        cap = max(4096, 1 << (nbytes - 1).bit_length())
+        free = self._staging.get(cap)
+        return cap, (free.pop() if free else self.dev.host_alloc(cap))
+
+    def _staging_give(self, cap: int, host: int) -> None:
+        if not host:
+            return
+        free = self._staging.setdefault(cap, [])
+        if len(free) < 4 and cap <= (64 << 20):
+            free.append(host)
+        else:
+            self.dev.host_free(host)
 
     def slotPointer(self, slot: int) -> int:
         """Device address of a slot (for the benchmark harness)."""
         return self._get(slot)["ptr"]
 
     # -- kernels ----------------------------------------------------------------------------------
-    def prepareKernelSync(self, kernel: Kernel, **tune_opts) -> Executable:
-        key = (kernel.key(), self.numerics, tuple(sorted(tune_opts.items())))
-        exe = self._exes.get(key)
-        if exe is not None:
-            return exe
-        ks = generate(kernel, self.numerics, **tune_opts)
+    def _build(self, source, ks: KernelSource) -> Executable:
         modules = [self.dev.load_module(compile_source(src, f"{ks.klass}.hip")) for src in ks.sources]
         functions = [self.dev.function(modules[s.module], s.name) for s in ks.steps]
         scratch = [self.dev.malloc(self._rounded(b)) for b in ks.scratch_bytes]
-        exe = Executable(kernel, _Prepared(ks, functions, scratch, modules))
-        self._exes[key] = exe
+        return Executable(source, _Prepared(ks, functions, scratch, modules))
+
+    def _cached(self, key: tuple):
+        exe = self._exes.get(key)
+        if exe is not None:
+            self._exes.move_to_end(key)
         return exe
+
+    def _remember(self, key: tuple, exe: Executable) -> Executable:
+        """Keep at most `cacheLimit` prepared executables; the least recently prepared one is released (scratch freed,
+        code objects unloaded) when the limit is passed.  Dispatching a released executable raises."""
+        self._exes[key] = exe
+        while len(self._exes) > self.cacheLimit:
+            _, old = self._exes.popitem(last=False)
+            old.data.release(self.dev)
+        return exe
+
+    def clearCache(self) -> None:
+        """Release every prepared executable (device scratch and loaded code objects)."""
+        while self._exes:
+            _, old = self._exes.popitem(last=False)
+            old.data.release(self.dev)
+
+    def prepareKernelSync(self, kernel: Kernel, **tune_opts) -> Executable:
+        key = (kernel.key(), self.numerics, tuple(sorted(tune_opts.items())))
+        exe = self._cached(key)
+        if exe is not None:
+            return exe
+        return self._remember(key, self._build(kernel, generate(kernel, self.numerics, **tune_opts)))
 
     async def prepareKernel(self, kernel: Kernel) -> Executable:
         return self.prepareKernelSync(kernel)
@@ -198,11 +295,14 @@ class HipBackend:
 
         if routine.name not in SUPPORTED_ROUTINES:
             raise UnsupportedRoutineError(routine.name, "hip")
+        # Cached like kernels (the role FpHash plays in src/backend/wasm.ts:125-147): one executable, one set of
+        # scratch buffers and loaded code objects per distinct routine, however often a program prepares it.
+        key = ("routine", routineKey(routine), self.numerics)
+        exe = self._cached(key)
+        if exe is not None:
+            return exe
         ks = generateRoutine(routine, self.numerics)  # raises UnsupportedRoutineError when there is no GPU plan
-        modules = [self.dev.load_module(compile_source(src, f"{ks.klass}.hip")) for src in ks.sources]
-        functions = [self.dev.function(modules[s.module], s.name) for s in ks.steps]
-        scratch = [self.dev.malloc(self._rounded(b)) for b in ks.scratch_bytes]
-        return Executable(routine, _Prepared(ks, functions, scratch, modules))
+        return self._remember(key, self._build(routine, ks))
 
     async def prepareRoutine(self, routine: Routine) -> Executable:
         return self.prepareRoutineSync(routine)
@@ -212,6 +312,8 @@ class HipBackend:
         routine: Routine = exe.source
         prep: _Prepared = exe.data
         t = routine.type
+        if prep.released:
+            raise ValueError("executable was released (evicted from the backend's cache): prepare it again")
         from .alu import byteWidth
         from .shape import prod
 
@@ -241,6 +343,8 @@ class HipBackend:
 
         kernel: Kernel = exe.source
         prep: _Prepared = exe.data
+        if prep.released:
+            raise ValueError("executable was released (evicted from the backend's cache): prepare it again")
         if len(outs) != 1:
             raise ValueError("a Kernel has exactly one output")
         if len(ins) < kernel.nargs:

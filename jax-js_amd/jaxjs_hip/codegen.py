@@ -214,7 +214,7 @@ class HipExpCodegen:
                 call = f"jh_{fns[op]}_f32((float)({a}))" if dtype != DType.Float32 else f"jh_{fns[op]}_f32({a})"
                 if dtype == DType.Float16 and op in (AluOp.Exp, AluOp.Log):
                     call = f"jh_{fns[op]}_f16((float)({a}))"  # hardware exp2/log2: float16 has no Wasm polynomial to follow
-                if dtype == DType.Float64 and self.numerics != "wasm" and op not in (AluOp.Erf, AluOp.Erfc):
+                if dtype == DType.Float64 and self.numerics == "native" and op not in (AluOp.Erf, AluOp.Erfc):
                     return f"__ocml_{fns[op]}_f64({a})", False
                 return (call if dtype == DType.Float32 else f"({ct})({call})"), False
             if op == AluOp.Sqrt:
@@ -231,7 +231,9 @@ class HipExpCodegen:
                     return f"(jh_f16)__builtin_{nm}f((float)({a}))", False
                 return f"__builtin_{nm}f({a})", False
             if op == AluOp.Reciprocal:
-                one = {DType.Float32: "1.0f", DType.Float64: "1.0", DType.Float16: "(jh_f16)1.0f"}[dtype]
+                if dtype == DType.Float32:
+                    return f"jh_rcp_f32({a})", False  # IEEE division, or v_rcp_f32 under the fast numerics
+                one = {DType.Float64: "1.0", DType.Float16: "(jh_f16)1.0f"}[dtype]
                 return f"({ct})({one} / {a})", False
             if op == AluOp.Cast:
                 if dtype == sdt:

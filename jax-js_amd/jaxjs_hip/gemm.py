@@ -14,7 +14,8 @@ from typing import Dict, List
 from .alu import AluExp, AluOp, DType, Kernel, byteWidth
 from .codegen import CTYPE, STORAGE_CTYPE, HipExpCodegen, strip_parens
 from .kernelgen import KernelSource, LaunchStep, _Body, _min_bytes, _prelude, _used_args, fill, template
-from .tuner import CU_COUNT, TuneResult, classify_loads
+from . import tuner
+from .tuner import TuneResult, classify_loads
 
 
 def choose_tile(g: dict) -> Dict[str, int]:
@@ -31,7 +32,7 @@ def choose_tile(g: dict) -> Dict[str, int]:
         # every CU matters most: take the largest tile that still yields two workgroups per CU (the
         # second one hides the first one's staging latency).
         for bm, bn in ((128, 128), (128, 64), (64, 64)):
-            if g["M"] >= bm and g["N"] >= bn and tiles(bm, bn) >= 2 * CU_COUNT:
+            if g["M"] >= bm and g["N"] >= bn and tiles(bm, bn) >= 2 * tuner.CU_COUNT:
                 return dict(BM=bm, BN=bn)
         return dict(BM=64, BN=64)
     # f16: estimated time = (tiles the busiest CU runs) x (tile area) x (K + fixed per-tile overhead) / efficiency.
@@ -51,7 +52,7 @@ def choose_tile(g: dict) -> Dict[str, int]:
                                 (128, 128, 0.72, dict())):
         if (bm > 128 and g["M"] < bm) or (bn > 128 and g["N"] < bn):
             continue
-        per_cu = -(-tiles(bm, bn) // CU_COUNT)
+        per_cu = -(-tiles(bm, bn) // tuner.CU_COUNT)
         if (bm, bn) == (128, 128) and per_cu < 2:
             eff = 0.64
         cost = per_cu * bm * bn * (g["K"] + 100) / eff
@@ -268,6 +269,21 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     out_t = STORAGE_CTYPE[kernel.dtype]
     in_t = STORAGE_CTYPE[g["dtype"]]
 
+    # Split of the k axis over blockIdx.y: every slice is the same kernel on K / split, its f32 accumulators go to a
+    # scratch buffer [slice][output] and a generated fold Kernel adds the slices in order and applies the epilogue
+    # (deterministic: no float atomics).  For launches that would otherwise leave most CUs without a workgroup.
+    split = int(tile.get("SPLITK", 1))
+    K_full = g["K"]
+    if split > 1:
+        vec_k = 8 if g["dtype"] == DType.Float16 else 4
+        if (g.get("a_gather") or g.get("b_gather") or g["a_k0"] != K_full or g["b_k0"] != K_full
+                or K_full % split or (K_full // split) % vec_k):
+            split = 1
+    if split > 1:
+        KS = K_full // split
+        g = dict(g, K=KS, a_k0=KS, b_k0=KS)
+        out_t = "float"
+
     used = _used_args(kernel.nargs, t.epilogue)
     used[g["gid_a"]] = g["dtype"]
     used[g["gid_b"]] = g["dtype"]
@@ -300,6 +316,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     epi_params = "".join(f", const {STORAGE_CTYPE[d or DType.Float32]}* __restrict__ {n}" for d, n in zip(used, names))
     epi_fn = (f"static __device__ __forceinline__ {out_t} jh_epilogue(float acc, int row, int col, int b0, int b1, int b2{epi_params}) {{\n"
               + "\n".join(cg.take_lines()) + f"\n  return ({out_t})({value});\n}}")
+    if split > 1:  # the fold kernel applies the epilogue; a slice stores its raw accumulator
+        epi_fn = f"static __device__ __forceinline__ float jh_epilogue(float acc, int row, int col, int b0, int b1, int b2{epi_params}) {{\n  return acc;\n}}"
     epi_args = "".join(f", {n}" for n in names)
 
     # Element loaders for gather operands: the operand's lowered expression (masked load through its view
@@ -465,8 +483,15 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     nbatch = 1
     for b in g["batch"]:
         nbatch *= b[0]
+    pitch = -(-kernel.size // 8) * 8  # elements between two slices' partial outputs
+    if split > 1:
+        lines.append(f"  a_base += (long long)blockIdx.y * {g['K'] * g['a_sk']}ll; b_base += (long long)blockIdx.y * {g['K'] * g['b_sk']}ll; "
+                     f"c_base += (long long)blockIdx.y * {pitch}ll;")
 
     tmpl = "gemm_f16.hip.inc" if g["dtype"] == DType.Float16 else "gemm_f32.hip.inc"
+    fBK = int(tile.get("BK", 16)) if g["dtype"] == DType.Float32 else 0  # slab depth of the f32 template
+    if g["dtype"] == DType.Float32 and (fBK not in (16, 32, 64) or 2 * (BM + BN) * (fBK + 4) * 4 > 160 * 1024):
+        raise ValueError(f"f32 slab depth {fBK} is not 16, 32 or 64, or two {BM}+{BN}-row slabs of it do not fit the LDS")
     # Fast path: direct global->LDS loads need whole tiles (no bounds predicates) and 32-deep slabs.
     # Slab depth.  When both operands run along k in memory, 64-deep slabs make every row of a slab one whole
     # 128-byte line (a 32-deep slab asks for the two halves of each line about a microsecond apart, as two requests):
@@ -499,8 +524,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         # Vector epilogue: needs unit column stride and 8-element alignment of every row / batch start of C.
         # It pays when the epilogue itself reads buffers (bias, residual): those become 128-bit loads.  A plain
         # cast-and-store epilogue measures the same either way and keeps the simpler path.
-        has_loads = bool(epilogue.collect(lambda x: x.op == AluOp.GlobalIndex))
-        vec = (tile.get("VEPI", 1 if has_loads else 0) and g["c_sn"] == 1 and g["c_sm"] % 8 == 0 and all(b[3] % 8 == 0 for b in g["batch"])
+        has_loads = bool(epilogue.collect(lambda x: x.op == AluOp.GlobalIndex)) and split == 1
+        vec = (split == 1 and tile.get("VEPI", 1 if has_loads else 0) and g["c_sn"] == 1 and g["c_sm"] % 8 == 0 and all(b[3] % 8 == 0 for b in g["batch"])
                and kernel.dtype != DType.Bool)
         if vec:
             vnames = {"acc": "acc", "row": "row", "col": "col", "b0": "b0", "b1": "b1", "b2": "b2"}
@@ -514,7 +539,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         sched = dict(COMMIT_A=tile.get("CA", 2), COMMIT_B=tile.get("CB", 3), FETCH_A=tile.get("FA", 0),
                      FETCH_B=tile.get("FB", 1), IGLP=tile.get("IGLP", -1), SCHED_FENCE=tile.get("FENCE", 0))
     else:
-        sched = {}
+        sched = dict(BK=fBK)
     if not dlds:
         sched.update(GATHER_FNS="\n".join(gather_fns), A_GATHER=gather_flags["a"], B_GATHER=gather_flags["b"],
                      GATHER_A_CALL=gather_calls["a"], GATHER_B_CALL=gather_calls["b"],
@@ -530,7 +555,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         A_K0=g["a_k0"], A_SK1=g["a_sk1"], B_K0=g["b_k0"], B_SK1=g["b_sk1"],
         C_SM=g["c_sm"], C_SN=g["c_sn"], EPILOGUE_ARGS=epi_args))
     tiles = -(-g["M"] // BM) * -(-g["N"] // BN) * nbatch
-    step = LaunchStep(name, (tiles, 1, 1), (nthreads, 1, 1), 0, [("in", i) for i in range(kernel.nargs)] + [("out", 0)])
+    out_arg = ("scratch", 0) if split > 1 else ("out", 0)
+    step = LaunchStep(name, (tiles, split, 1), (nthreads, 1, 1), 0, [("in", i) for i in range(kernel.nargs)] + [out_arg])
     need = _min_bytes(t.epilogue)
     if any_gather:
         for gid_, b_ in _min_bytes(t.exp).items():
@@ -538,8 +564,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     eb = byteWidth(g["dtype"])
     need[g["gid_a"]] = max(need.get(g["gid_a"], 0), g["a_len"] * eb)
     need[g["gid_b"]] = max(need.get(g["gid_b"], 0), g["b_len"] * eb)
-    info = dict(BM=BM, BN=BN, WM=WM, WN=WN, BK=dBK if dlds else (64 if g["dtype"] == DType.Float16 else 16), direct_lds=bool(dlds), tiles=tiles, a_kcontig=g["a_sk"] == 1, b_kcontig=g["b_sk"] == 1,
-                M=g["M"], N=g["N"], K=g["K"], nbatch=nbatch)
+    info = dict(BM=BM, BN=BN, WM=WM, WN=WN, BK=dBK if dlds else (64 if g["dtype"] == DType.Float16 else fBK), direct_lds=bool(dlds), tiles=tiles, a_kcontig=g["a_sk"] == 1, b_kcontig=g["b_sk"] == 1,
+                M=g["M"], N=g["N"], K=K_full, nbatch=nbatch, splitk=split)
     if dlds:
         info.update(stages=sched["STAGES"], ring=sched["RING"])
     if any_gather:
@@ -547,4 +573,11 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                                 4: "tap-major strided"}[gather_flags[tag]] for tag in ("a", "b")}
         if tap_major is not None:
             info["tap_major"] = tap_major
-    return KernelSource([src], [step], [], "gemm", need, info)
+    if split == 1:
+        return KernelSource([src], [step], [], "gemm", need, info)
+    from .kernelgen import fold_stage
+
+    ks2, steps2, partial_len = fold_stage(kernel, numerics, name, split, pitch, slice_major=True)
+    info["stage2"] = ks2.info
+    need.update({gid_: b_ for gid_, b_ in ks2.min_input_bytes.items() if gid_ != kernel.nargs})
+    return KernelSource([src] + ks2.sources, [step] + steps2, [partial_len * 4], "gemm+fold", need, info)

@@ -1043,7 +1043,7 @@ def splitGraphDataflow(jaxpr: Jaxpr, maxArgs: int) -> Set[Var]:
 
 @dataclass
 class JitStep:
-    kind: str                      # "malloc" | "execute" | "free"
+    kind: str                      # "malloc" | "execute" | "free" | "incref"
     kernel: Optional[Kernel] = None    # an "execute" step runs either a Kernel (one output) ...
     inputs: List[int] = field(default_factory=list)
     output: int = -1
@@ -1084,12 +1084,9 @@ class JitProgram:
                 backend.dispatch(exe, [scope[i] for i in step.inputs], [scope[step.output]])
             elif step.kind == "free":
                 backend.decRef(scope.pop(step.output))
-        outs = []
-        for o in self.outputs:
-            if o < self.nargs:
-                backend.incRef(scope[o])
-            outs.append(scope[o])
-        return outs
+            elif step.kind == "incref":
+                backend.incRef(scope[step.output])
+        return [scope[o] for o in self.outputs]
 
     def prepare(self, backend) -> Dict[int, Any]:
         return {k: (backend.prepareRoutineSync(s.routine) if s.routine is not None else backend.prepareKernelSync(s.kernel))
@@ -1230,12 +1227,27 @@ def jitCompile(jaxpr: Jaxpr, consts: Sequence[ConstArray] = (), maxArgs: int = 6
 
     outputs: List[int] = []
     for out in jaxpr.outs:
-        if not isinstance(out, Var):
-            raise NotImplementedError("jit: literal outputs")
+        if isinstance(out, Lit):  # a literal output is realised by a nullary kernel (pushLit, src/frontend/jit.ts:176-183)
+            kernel = Kernel(0, out.aval.size, AluExp.const(out.aval.dtype, out.value))
+            out_id = next_id[0]
+            next_id[0] += 1
+            steps.append(JitStep("malloc", output=out_id, size=kernel.bytes))
+            steps.append(JitStep("execute", kernel=kernel, inputs=[], output=out_id))
+            outputs.append(out_id)
+            continue
         jv = ctx[out]
         if jv[0] != "imm":
             raise RuntimeError("internal: Expected imm, since outs are black nodes")
         outputs.append(jv[1])
+
+    # Every returned slot carries a reference of its own: an input returned directly, or an id returned a second
+    # time, gets an "incref" step (src/frontend/jit.ts:449-458).
+    needs_ref = set(range(nargs))
+    for o in outputs:
+        if o in needs_ref:
+            steps.append(JitStep("incref", output=o))
+        else:
+            needs_ref.add(o)
 
     # Free every intermediate after its last use (JitProgramBuilder.insertFreeSteps).
     last_use: Dict[int, int] = {}

@@ -153,8 +153,17 @@ class _Body:
         return "\n".join(cg.take_lines()), value
 
 
+# "wasm": the reference Wasm backend's polynomial transcendentals, operation for operation (f32 maps within 2 ulp of
+# the checker).  "fast": the same, except exp and reciprocal on the hardware's exp2 / rcp instructions (within rel
+# 1e-5 of the checker; what keeps a fused softmax-style row kernel off the VALU limit).  "native": device libm.
+NUMERICS = ("wasm", "fast", "native")
+
+
 def _prelude(numerics: str) -> str:
-    return f"#define JH_WASM_NUMERICS {1 if numerics == 'wasm' else 0}\n" + template("prelude.hip.inc") + "\n"
+    if numerics not in NUMERICS:
+        raise ValueError(f"numerics must be one of {NUMERICS}")
+    return (f"#define JH_WASM_NUMERICS {1 if numerics in ('wasm', 'fast') else 0}\n#define JH_FAST_NUMERICS {1 if numerics == 'fast' else 0}\n"
+            + template("prelude.hip.inc") + "\n")
 
 
 IDENT = {"gidx": "gidx", "ridx": "ridx"}
@@ -277,14 +286,29 @@ def _gen_reduce(kernel: Kernel, t: TuneResult, numerics: str, name: str, row: bo
     grid_x = max(1, min(grid_x, (256 * 16) // split + 1))
     step1 = LaunchStep(name, (grid_x, split, 1), (block, 1, 1), 0,
                        [("in", i) for i in range(kernel.nargs)] + [("scratch", 0)])
+    pitch = 1 if row else _partial_pitch(size, V)
+    ks2, steps2, partial_len = fold_stage(kernel, numerics, name, split, pitch, slice_major=not row)
+    p["stage2"] = ks2.info
+    need.update({g: b for g, b in ks2.min_input_bytes.items() if g != kernel.nargs})
+    return KernelSource([src] + ks2.sources, [step1] + steps2, [partial_len * byteWidth(re.dtype)],
+                        klass + "+fold", need, p)
+
+
+def fold_stage(kernel: Kernel, numerics: str, name: str, split: int, pitch: int, slice_major: bool,
+               first_module: int = 1):
+    """Second stage of a reduction whose reduce axis was cut into `split` slices: a Kernel over the IR that folds the
+    partial accumulators (in scratch buffer 0) in slice order and applies the caller's epilogue.  Partials are laid out
+    `[slice][pitch]` (slice-major, `pitch` >= size) or `[output][split]`.  Returns (its KernelSource, its launch steps
+    with the scratch buffer bound and module indices shifted by `first_module`, the partial buffer's length in elements)."""
+    re = kernel.reduction
+    size = kernel.size
     gid_partial = kernel.nargs
-    if row:  # partial[gidx][slice]
-        idx = AluExp.add(AluExp.mul(AluVar.gidx, AluExp.i32(split)), AluVar.ridx)
-        partial_len = size * split
-    else:  # partial[slice][gidx], rows padded to the vector width
-        pitch = _partial_pitch(size, V)
+    if slice_major:  # partial[slice][gidx], rows padded to the vector width
         idx = AluExp.add(AluExp.mul(AluVar.ridx, AluExp.i32(pitch)), AluVar.gidx)
         partial_len = pitch * split
+    else:  # partial[gidx][slice]
+        idx = AluExp.add(AluExp.mul(AluVar.gidx, AluExp.i32(split)), AluVar.ridx)
+        partial_len = size * split
     stage2 = Kernel(kernel.nargs + 1, size,
                     AluExp.globalIndex(re.dtype, gid_partial, partial_len, idx),
                     Reduction(re.dtype, re.op, split, re.epilogue))
@@ -292,8 +316,5 @@ def _gen_reduce(kernel: Kernel, t: TuneResult, numerics: str, name: str, row: bo
     steps2 = []
     for s in ks2.steps:
         mapped = [("scratch", 0) if a == ("in", gid_partial) else a for a in s.args]
-        steps2.append(LaunchStep(s.name, s.grid, s.block, s.shared, mapped, module=s.module + 1))
-    p["stage2"] = ks2.info
-    need.update({g: b for g, b in ks2.min_input_bytes.items() if g != gid_partial})
-    return KernelSource([src] + ks2.sources, [step1] + steps2, [partial_len * byteWidth(re.dtype)],
-                        klass + "+fold", need, p)
+        steps2.append(LaunchStep(s.name, s.grid, s.block, s.shared, mapped, module=s.module + first_module))
+    return ks2, steps2, partial_len

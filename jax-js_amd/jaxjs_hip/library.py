@@ -169,6 +169,28 @@ def argmax(a: Tracer, axis: int):
     return length.sub(idx.max(axis))
 
 
+def argmin(a: Tracer, axis: int):
+    """First index of the minimum: the same construction on `a == min(a)` (numpy.ts:497-524)."""
+    axis = axis + a.ndim if axis < 0 else axis
+    n = a.shape[axis]
+    isMin = J.equal(a, a.min(axis, keepdims=True))
+    length = J.scalar(n, DType.Int32)
+    rev = arange_const(n, 0, -1, DType.Int32, shape=[n] + [1] * (a.ndim - axis - 1))
+    idx = isMin.astype(DType.Int32).mul(rev)
+    return length.sub(idx.max(axis))
+
+
+def logsumexp(x: Tracer, axis=None, keepdims: bool = False):
+    """max + log(sum(exp(x - max))) (nn.ts:332-345)."""
+    xMax = x.max(axis, keepdims=True)
+    shifted = x.sub(xMax)
+    result = xMax.add(J.log(J.exp(shifted).sum(axis, keepdims=True)))
+    if keepdims:
+        return result
+    ax = J._normalize_axis(axis, x.ndim)
+    return result.reshape([n for i, n in enumerate(x.shape) if i not in ax])
+
+
 def dotProductAttention(query: Tracer, key: Tracer, value: Tracer, isCausal: bool = False, scale: Optional[float] = None,
                         fused: bool = False):
     """[B,L,N,H] attention with equal query and key/value head counts (nn.ts:478-583).  `fused=True` hands the whole

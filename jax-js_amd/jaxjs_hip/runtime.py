@@ -62,6 +62,7 @@ _SIGNATURES = {
                                   ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_size_t),
                                   ctypes.c_char_p, ctypes.c_size_t]),
     "jh_code_free": (None, [ctypes.c_void_p]),
+    "jh_compiler_version": (ctypes.c_int, [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]),
     "jh_module_load": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p)]),
     "jh_module_unload": (ctypes.c_int, [ctypes.c_void_p]),
     "jh_module_function": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_char_p, ctypes.POINTER(ctypes.c_void_p)]),
@@ -113,12 +114,33 @@ def check(rc: int, what: str) -> None:
         raise HipRuntimeError(f"{what} failed (status {rc}): {msg}")
 
 
+_toolchain: Optional[str] = None
+
+
+def toolchain_tag() -> str:
+    """What a cached code object depends on besides its source and options: the run-time compiler's version and this
+    library's ABI version.  (The target architecture is one of the options.)"""
+    global _toolchain
+    if _toolchain is None:
+        lib = load_library()
+        major, minor = ctypes.c_int(), ctypes.c_int()
+        check(lib.jh_compiler_version(ctypes.byref(major), ctypes.byref(minor)), "jh_compiler_version")
+        _toolchain = f"hiprtc-{major.value}.{minor.value}/abi-{lib.jh_abi_version()}"
+    return _toolchain
+
+
+DISK_CACHE = os.environ.get("JAXHIP_NO_DISK_CACHE") != "1"  # False: every prepare goes through hiprtc
+
+
 def compile_source(source: str, name: str = "kernel.hip", options: Optional[Sequence[str]] = None,
-                   use_cache: bool = True) -> bytes:
-    """HIP source -> gfx950 code object through hiprtc, with an on-disk cache keyed by content."""
+                   use_cache: Optional[bool] = None) -> bytes:
+    """HIP source -> gfx950 code object through hiprtc, with an on-disk cache keyed by compiler version, options
+    and source text."""
     lib = load_library()
+    if use_cache is None:
+        use_cache = DISK_CACHE
     opts = list(options if options is not None else COMPILE_OPTIONS)
-    key = hashlib.sha256(("\0".join(opts) + "\0" + source).encode()).hexdigest()[:32]
+    key = hashlib.sha256((toolchain_tag() + "\0" + "\0".join(opts) + "\0" + source).encode()).hexdigest()[:32]
     path = os.path.join(CACHE_DIR, key + ".hsaco")
     if use_cache and os.path.exists(path):
         with open(path, "rb") as f:
@@ -194,6 +216,28 @@ class Device:
         else:
             check(self.lib.jh_memcpy_d2h(None, None, 0, 0), "jh_memcpy_d2h")
         return out
+
+    def host_alloc(self, nbytes: int) -> int:
+        """Pinned host memory (the destination of asynchronous reads)."""
+        p = ctypes.c_void_p()
+        check(self.lib.jh_host_alloc(nbytes, ctypes.byref(p)), f"jh_host_alloc({nbytes})")
+        return p.value or 0
+
+    def host_free(self, ptr: int) -> None:
+        if ptr:
+            check(self.lib.jh_host_free(ctypes.c_void_p(ptr)), "jh_host_free")
+
+    def d2h_async(self, host_ptr: int, src: int, offset: int, nbytes: int) -> int:
+        """Queue a device -> pinned-host copy behind everything issued so far; returns the completion event."""
+        ev = ctypes.c_void_p()
+        check(self.lib.jh_memcpy_d2h_async(ctypes.c_void_p(host_ptr), ctypes.c_void_p(src), offset, nbytes, ctypes.byref(ev)),
+              "jh_memcpy_d2h_async")
+        return ev.value
+
+    def event_done(self, ev: int) -> bool:
+        done = ctypes.c_int()
+        check(self.lib.jh_event_query(ctypes.c_void_p(ev), ctypes.byref(done)), "jh_event_query")
+        return bool(done.value)
 
     def d2d(self, dst: int, src: int, nbytes: int) -> None:
         check(self.lib.jh_memcpy_d2d(ctypes.c_void_p(dst), ctypes.c_void_p(src), nbytes), "jh_memcpy_d2d")

@@ -28,9 +28,18 @@ from typing import Dict, List, Optional, Sequence, Tuple
 from .alu import AluExp, AluGroup, AluOp, AluVar, DType, Kernel, Reduction, byteWidth, isFloatDtype
 from .shape import ShapeTracker, unravelAlu
 
-CU_COUNT = 256          # MI355X: 8 XCDs x 32 CUs
+CU_COUNT = 256          # MI355X: 8 XCDs x 32 CUs; replaced by the device's own count once a backend is up
 WAVE = 64
 MAX_GRID_BLOCKS = CU_COUNT * 16
+
+
+def set_compute_units(n: int) -> None:
+    """Take the CU count from the initialised device (`jh_get_device_info`); 256 stays the value for ahead-of-time
+    generation without a device."""
+    global CU_COUNT, MAX_GRID_BLOCKS
+    if n and n > 0:
+        CU_COUNT = int(n)
+        MAX_GRID_BLOCKS = CU_COUNT * 16
 # Map kernels get one block per 256 lane groups rather than a capped grid-stride launch: blocks are dispatched in
 # order, so the chip walks the buffers front to back (open DRAM pages are used up before they close), whereas a
 # block that strides by the whole grid touches a new page every trip: 5.0-5.3 -> 5.9-6.3 TB/s on streams of 400 MB
@@ -486,11 +495,13 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
     if split > 1 and V > 1:
         lx_line = 8  # 8 lanes x 16 bytes = one 128-byte line per row
         blk = 1024
-        if col_strip:  # (lanes per strip, block size, unroll): tuning override
-            lx_line, blk, unroll = col_strip
+        rows_split = 1
+        if col_strip:  # (lanes per strip, block size, unroll[, blocks along the reduce axis]): tuning override
+            lx_line, blk, unroll = col_strip[:3]
+            rows_split = col_strip[3] if len(col_strip) > 3 else 1
         strips = -(-groups // lx_line)
         if strips >= CU_COUNT // 2 and R // (blk // lx_line) >= 8:
-            lx, T, split, unroll = lx_line, blk // lx_line, 1, (unroll if col_strip else 8)
+            lx, T, split, unroll = lx_line, blk // lx_line, rows_split, (unroll if col_strip else 8)
     t.klass = "reduce_col"
     t.vector_loads = along_g if V > 1 else {}
     t.params = dict(V=V, T=T, lx=lx, block=lx * T, split=split, unroll=unroll)

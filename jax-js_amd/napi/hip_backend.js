@@ -92,14 +92,37 @@ class HipBackend {
     return addon.d2h(s.ptr, start, count);
   }
 
+  // Asynchronous read (src/backend.ts:182-186; src/backend/webgpu/reader.ts maps a staging buffer the same way): the
+  // copy into pinned host memory is queued behind every earlier dispatch, and the promise resolves from the event
+  // loop once the copy's completion event has passed -- the thread is never blocked on the device, so a caller that
+  // awaits a result goes on preparing and dispatching other work.
   read(slot, start, count) {
-    // The stream is in order, so a blocking copy issued now observes every earlier dispatch.  A build with
-    // jh_memcpy_d2h_async + eventQuery polling on setImmediate keeps the event loop free; the contract is the same.
-    try {
-      return Promise.resolve(this.readSync(slot, start, count));
-    } catch (e) {
-      return Promise.reject(e);
-    }
+    return new Promise((resolve, reject) => {
+      let pending;
+      try {
+        const s = this._get(slot);
+        start = start === undefined ? 0 : start;
+        count = count === undefined ? s.size - start : count;
+        if (start < 0 || count < 0 || start + count > s.size) throw new RangeError('read outside of the buffer');
+        pending = addon.d2hAsync(s.ptr, start, count);
+      } catch (e) {
+        reject(e);
+        return;
+      }
+      const poll = () => {
+        try {
+          if (!addon.eventQuery(pending.event)) {
+            setImmediate(poll);
+            return;
+          }
+          addon.eventDestroy(pending.event);
+          resolve(pending.data);
+        } catch (e) {
+          reject(e);
+        }
+      };
+      poll();
+    });
   }
 
   // -- kernels -----------------------------------------------------------------------------------------

@@ -163,6 +163,51 @@ napi_value D2H(napi_env env, napi_callback_info info) {  // d2h(src, offset, byt
   return out;
 }
 
+void free_pinned(napi_env, void* data, void*) {  // finalizer of the array buffers d2hAsync hands out
+  if (data) (void)jh_host_free(data);
+}
+
+// d2hAsync(src, offset, bytes) -> {event: BigInt, data: Uint8Array}.  The copy into pinned host memory is queued behind
+// every earlier launch and the call returns at once; `data` holds the bytes once eventQuery(event) reports true.  The
+// pinned memory belongs to the returned array buffer and is released when that is collected.
+napi_value D2HAsync(napi_env env, napi_callback_info info) {
+  Args a(env, info);
+  uint64_t src, off, bytes;
+  if (a.argc < 3 || !get_u64(env, a.argv[0], &src) || !get_u64(env, a.argv[1], &off) || !get_u64(env, a.argv[2], &bytes)) {
+    napi_throw_type_error(env, nullptr, "d2hAsync(src, offset, bytes)"); return nullptr;
+  }
+  void* host = nullptr;
+  if (bytes) JH_OK(jh_host_alloc((size_t)bytes, &host));
+  jh_event ev = nullptr;
+  if (jh_memcpy_d2h_async(host, (jh_devptr)(uintptr_t)src, (size_t)off, (size_t)bytes, &ev) != 0) {
+    if (host) (void)jh_host_free(host);
+    napi_throw_error(env, nullptr, jh_last_error());
+    return nullptr;
+  }
+  napi_value ab, arr, out;
+  napi_status st = bytes ? napi_create_external_arraybuffer(env, host, (size_t)bytes, free_pinned, nullptr, &ab)
+                         : napi_create_arraybuffer(env, 0, &host, &ab);
+  if (st != napi_ok) {
+    (void)jh_event_sync(ev); (void)jh_event_destroy(ev);
+    if (bytes && host) (void)jh_host_free(host);
+    napi_throw_error(env, nullptr, "jaxhip: cannot wrap pinned memory in an ArrayBuffer");
+    return nullptr;
+  }
+  NAPI_OK(napi_create_typedarray(env, napi_uint8_array, (size_t)bytes, ab, 0, &arr));
+  NAPI_OK(napi_create_object(env, &out));
+  NAPI_OK(napi_set_named_property(env, out, "event", make_u64(env, (uint64_t)(uintptr_t)ev)));
+  NAPI_OK(napi_set_named_property(env, out, "data", arr));
+  return out;
+}
+
+napi_value CompilerVersion(napi_env env, napi_callback_info) {  // "major.minor" of hiprtc (part of a code-object cache key)
+  int major = 0, minor = 0;
+  JH_OK(jh_compiler_version(&major, &minor));
+  napi_value out;
+  napi_create_string_utf8(env, (std::to_string(major) + "." + std::to_string(minor)).c_str(), NAPI_AUTO_LENGTH, &out);
+  return out;
+}
+
 napi_value Compile(napi_env env, napi_callback_info info) {  // compile(source, name, options: string[]) -> Buffer
   Args a(env, info);
   std::string source, name;
@@ -347,7 +392,7 @@ NAPI_MODULE_INIT() {
       {"moduleFunction", ModuleFunction}, {"launch", Launch}, {"sync", Sync}, {"eventCreate", EventCreate},
       {"eventRecord", EventRecord}, {"eventQuery", EventQuery}, {"eventElapsedMs", EventElapsed},
       {"eventDestroy", EventDestroy}, {"graphBegin", GraphBegin}, {"graphEnd", GraphEnd}, {"graphLaunch", GraphLaunch},
-      {"graphDestroy", GraphDestroy}, {"abiVersion", AbiVersion},
+      {"graphDestroy", GraphDestroy}, {"abiVersion", AbiVersion}, {"d2hAsync", D2HAsync}, {"compilerVersion", CompilerVersion},
   };
   for (const auto& e : table) {
     napi_value fn;

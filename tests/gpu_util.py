@@ -13,13 +13,30 @@ _backend = None
 
 
 def backend():
+    """The backend the parity tests run on: Wasm-faithful numerics, so that f32 maps can be held to 2 ulp of the
+    checker.  (The backend's default, "fast", is covered by `fast_backend()` under the rel 1e-5 bar.)"""
     global _backend
     if _backend is None:
         from jaxjs_hip import getBackend, init
 
-        init("hip")
+        init("hip", numerics="wasm")
         _backend = getBackend("hip")
     return _backend
+
+
+_fast = None
+
+
+def fast_backend():
+    """A second backend object on the same device with the default ("fast") numerics."""
+    global _fast
+    if _fast is None:
+        from jaxjs_hip.backend import HipBackend
+
+        backend()
+        _fast = HipBackend()
+        assert _fast.numerics == "fast"
+    return _fast
 
 
 def device_run(kernel, inputs, **tune_opts):

@@ -272,3 +272,84 @@ def test_dispatch_order_and_buffer_reuse(be):
         cur = nxt
     np.testing.assert_array_equal(np.frombuffer(be.readSync(cur), np.int32), np.full(n, 50, np.int32))
     be.decRef(cur)
+
+
+def test_read_is_asynchronous(be):
+    """`read` (src/backend.ts:182-186) queues its copy behind the pending dispatches and yields to the event loop until it
+    has landed: another coroutine runs, and dispatches more work, while the read is still pending; the bytes are those
+    of the dispatches queued before the read (not of the later ones)."""
+    n = 1 << 26
+    heavy = be.prepareKernelSync(Kernel(0, n, AluExp.sin(AluExp.cast(DType.Float32, AluVar.gidx))))
+    st = ShapeTracker.fromShape([1024])
+    inc = be.prepareKernelSync(Kernel(1, 1024, AluExp.add(AluExp.globalView(DType.Int32, 0, st, [AluVar.gidx]), AluExp.i32(1))))
+    big = be.malloc(n * 4)
+    a = be.malloc(4096, u8(np.zeros(1024, np.int32)))
+    b = be.malloc(4096)
+    state = dict(turns=0, done=False, dispatched_while_pending=0)
+
+    async def other_work():
+        while not state["done"]:
+            state["turns"] += 1
+            if state["dispatched_while_pending"] < 3:  # the host keeps issuing work while the read is in flight
+                be.dispatch(inc, [b], [a])
+                state["dispatched_while_pending"] += 1
+            await asyncio.sleep(0)
+
+    async def main():
+        for _ in range(300):  # tens of milliseconds of device work ahead of the read
+            be.dispatch(heavy, [], [big])
+        be.dispatch(inc, [a], [b])  # b = 1 everywhere
+        task = asyncio.ensure_future(other_work())
+        raw = await be.read(b)
+        state["done"] = True
+        await task
+        part = await be.read(b, 8, 16)
+        return raw, part
+
+    try:
+        raw, part = asyncio.run(main())
+        assert state["turns"] > 1 and state["dispatched_while_pending"] == 3, state
+        np.testing.assert_array_equal(np.frombuffer(raw, np.int32), np.ones(1024, np.int32))
+        assert len(part) == 16
+        np.testing.assert_array_equal(np.frombuffer(be.readSync(a), np.int32), np.full(1024, 2, np.int32))
+        assert len(asyncio.run(be.read(be_zero := be.malloc(0)))) == 0
+        be.decRef(be_zero)
+        with pytest.raises(ValueError, match="outside buffer"):
+            asyncio.run(be.read(a, 4000, 200))
+    finally:
+        for s in (big, a, b):
+            be.decRef(s)
+
+
+def test_routine_executables_are_cached_and_released(be):
+    """prepareRoutineSync returns one executable per distinct routine (no scratch or module is allocated twice), and an
+    executable that the cache lets go gives its scratch and code objects back; using it afterwards raises."""
+    from jaxjs_hip.routine import Routine, Routines, RoutineType
+    F = DType.Float32
+    mk = lambda n: Routine(Routines.Cholesky, RoutineType([[n, n]], [F], [[n, n]], [F]))  # noqa: E731
+    e1, e2 = be.prepareRoutineSync(mk(256)), be.prepareRoutineSync(mk(256))
+    assert e1 is e2 and e1.data.scratch, "right-looking Cholesky owns a double-precision scratch copy"
+    assert be.prepareRoutineSync(mk(192)) is not e1
+    a = np.random.default_rng(3).standard_normal((256, 256))
+    spd = (a @ a.T + 256 * np.eye(256)).astype(np.float32)
+    x, y = be.malloc(spd.nbytes, u8(spd)), be.malloc(spd.nbytes)
+    try:
+        be.dispatch(e1, [x], [y])
+        got = np.frombuffer(be.readSync(y), np.float32).reshape(256, 256)
+        np.testing.assert_allclose(np.tril(got) @ np.tril(got).T, spd, rtol=1e-4, atol=1e-3)
+        limit, be.cacheLimit = be.cacheLimit, 0
+        try:
+            k = Kernel(0, 4, AluExp.cast(DType.Float32, AluExp.add(AluVar.gidx, AluExp.i32(77))))
+            fresh = be.prepareKernelSync(k)  # over the limit: everything prepared earlier (and this one) is let go
+        finally:
+            be.cacheLimit = limit
+        assert e1.data.released and fresh.data.released and not e1.data.scratch and not e1.data.modules
+        with pytest.raises(ValueError, match="released"):
+            be.dispatch(e1, [x], [y])
+        e3 = be.prepareRoutineSync(mk(256))  # prepared again from the on-disk code objects
+        assert e3 is not e1
+        be.dispatch(e3, [x], [y])
+        np.testing.assert_array_equal(np.frombuffer(be.readSync(y), np.float32).reshape(256, 256), got)
+    finally:
+        be.decRef(x)
+        be.decRef(y)

@@ -32,7 +32,7 @@ def test_library_exports_every_declared_symbol():
     exported = sorted(set(re.findall(r" T (jh_[a-z0-9_]+)", out)))
     assert exported == _declared()
     lib = load_library()
-    assert lib.jh_abi_version() == 1
+    assert lib.jh_abi_version() == 2
     for name in EXPORTED_SYMBOLS:
         assert getattr(lib, name) is not None
 

@@ -106,15 +106,22 @@ def test_gemm_fused_epilogue_bias_relu_f32_out():
     np.testing.assert_allclose(got.reshape(M, N), ref, rtol=1e-4, atol=1e-4)
 
 
+def _tile_row_sample(n, bm=256):
+    """Three rows of every block-tile row: the first, one in the second 128-row wave half, the last."""
+    return sorted({t * bm + r for t in range(n // bm) for r in (0, bm // 2 + 3, bm - 1)})
+
+
 def test_gemm_8192_cubed_sampled():
-    """Headline shape.  Full f64 verification would take minutes on the host; rows are independent, so a
-    sample of 24 rows spread over all tile rows (and every column) is compared with exact dot products."""
+    """Headline shape.  Full f64 verification would take minutes on the host; rows are independent, so rows
+    t*256 + {0, 131, 255} for every one of the 32 tile rows (both 128-row wave halves, every column, so every
+    workgroup of the launch) are compared with exact dot products."""
     n = 8192
     A = RNG.uniform(-1, 1, (n, n)).astype(np.float16)
     B = RNG.uniform(-1, 1, (n, n)).astype(np.float16)
     got, ks = device_run(matmulKernel(n, n, n, DType.Float16), [A, B])
-    assert ks.klass == "gemm"
-    rows = sorted(set(list(range(0, n, 353)) + [255, 256, n - 1]))
+    assert ks.klass == "gemm" and (ks.info["BM"], ks.info["BN"]) == (256, 256) and ks.info["direct_lds"], ks.info
+    rows = _tile_row_sample(n)
+    assert len(rows) == 96
     _check(got.reshape(n, n)[rows], A[rows], B, n)
 
 
@@ -126,8 +133,73 @@ def test_gemm_8192_cubed_nt_sampled():
     Bt = RNG.uniform(-1, 1, (n, n)).astype(np.float16)
     got, ks = device_run(matmulKernel(n, n, n, DType.Float16, b_transposed=True), [A, Bt])
     assert ks.klass == "gemm" and ks.info["BK"] == 64 and ks.info["ring"] == 5, ks.info
-    rows = sorted(set(list(range(0, n, 353)) + [255, 256, n - 1]))
+    rows = _tile_row_sample(n)
     _check(got.reshape(n, n)[rows], A[rows], Bt.T, n)
+
+
+def _f32_out(base, K):
+    """The same contraction with the f32 accumulator stored as it is (no rounding to the operand type)."""
+    return Kernel(base.nargs, base.size, base.exp_raw, Reduction(DType.Float32, AluOp.Add, K, AluVar.acc(DType.Float32)))
+
+
+def test_gemm_8192_cubed_every_element_exact():
+    """Entries in {-1, 0, 1}: every product and every partial sum is an integer below 2^24, so the f32 accumulator is
+    exact in any summation order and the whole 8192 x 8192 result must equal the host product bit for bit (the
+    integer-exact style of test/numpy.test.ts:1510-1660), in both layouts of B."""
+    n = 8192
+    A = RNG.integers(-1, 2, (n, n)).astype(np.float16)
+    B = RNG.integers(-1, 2, (n, n)).astype(np.float16)
+    ref = A.astype(np.float32) @ B.astype(np.float32)  # exact for these inputs whatever the BLAS blocking
+    assert np.array_equal(ref[:4].astype(np.float64), A[:4].astype(np.float64) @ B.astype(np.float64))
+    got, ks = device_run(_f32_out(matmulKernel(n, n, n, DType.Float16), n), [A, B])
+    assert ks.klass == "gemm" and got.dtype == np.float32 and ks.info["tiles"] == 1024, ks.info
+    np.testing.assert_array_equal(got.reshape(n, n), ref)
+    got, ks = device_run(_f32_out(matmulKernel(n, n, n, DType.Float16, b_transposed=True), n), [A, np.ascontiguousarray(B.T)])
+    assert ks.klass == "gemm" and ks.info["ring"] == 5, ks.info
+    np.testing.assert_array_equal(got.reshape(n, n), ref)
+
+
+# The dense-GEMM sweep of the benchmark configuration: square 2048 / 4096 / 8192 and the skinny 128 x 14336 x 4096,
+# in f16 and f32.  Each case pins the launch shape the tuner picks for it (block tile, k split, workgroups) and is
+# checked against f64 dot products under the K-scaled bound on a row sample that meets every block-tile row.
+SWEEP = [
+    (DType.Float16, 2048, 2048, 2048, dict(BM=128, BN=128, tiles=256, direct_lds=True)),
+    (DType.Float16, 4096, 4096, 4096, dict(BM=256, BN=256, tiles=256, direct_lds=True)),
+    (DType.Float16, 128, 14336, 4096, None),
+    (DType.Float32, 1024, 1024, 1024, None),
+    (DType.Float32, 2048, 2048, 2048, dict(BM=128, BN=64, tiles=512)),
+    (DType.Float32, 4096, 4096, 4096, dict(BM=128, BN=128, tiles=1024)),
+    (DType.Float32, 8192, 8192, 8192, dict(BM=128, BN=128, tiles=4096)),
+    (DType.Float32, 128, 14336, 4096, None),
+]
+
+
+# Shapes whose launch fills less than the chip with one workgroup per output tile: the tuner cuts their k axis.
+SWEEP_SPLIT = {
+    (DType.Float16, 128, 14336, 4096): dict(),
+    (DType.Float32, 1024, 1024, 1024): dict(),
+    (DType.Float32, 128, 14336, 4096): dict(),
+}
+
+
+@pytest.mark.parametrize("dt,M,N,K,want", SWEEP, ids=lambda v: v.value if isinstance(v, DType) else (None if isinstance(v, dict) or v is None else str(v)))
+def test_gemm_sweep_shapes(dt, M, N, K, want):
+    from jaxjs_hip.kernelgen import generate
+
+    npdt = np.float16 if dt == DType.Float16 else np.float32
+    A = RNG.uniform(-1, 1, (M, K)).astype(npdt)
+    B = RNG.uniform(-1, 1, (K, N)).astype(npdt)
+    k = matmulKernel(M, N, K, dt)
+    got, ks = device_run(k, [A, B])
+    assert ks.klass.startswith("gemm"), ks.klass
+    want = want if want is not None else SWEEP_SPLIT[(dt, M, N, K)]
+    assert {key: ks.info[key] for key in want} == want, ks.info
+    assert ks.info == generate(k).info  # the launch that ran is the tuner's default choice
+    bm = ks.info["BM"]
+    rows = _tile_row_sample(M, bm) if M >= 2 * bm else list(range(M))
+    if len(rows) > 128:
+        rows = rows[::len(rows) // 96]
+    _check(got.reshape(M, N)[rows], A[rows], B, K, out_f16=(dt == DType.Float16))
 
 
 # Direct-to-LDS pipeline variants: (M, N, K, B stored [N, K], tile options).  K values give 1, 2, 3, 5, 6 and 17

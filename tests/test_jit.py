@@ -471,3 +471,37 @@ def test_concatenate_stack_and_split():
         run_typed(lambda a: J.split(a, 1, [2, 3]), [x], [F32])
     with pytest.raises(TypeError):
         run_typed(lambda a, b: J.concatenate([a, b], 0), [x, x[:, :2]], [F32, F32])
+
+
+# ---- output references (src/frontend/jit.ts:449-458) --------------------------------------------------
+
+def _run_keeping_outputs(fn, *arrays):
+    prog = J.jit(fn, [ShapedArray(tuple(a.shape), F32) for a in arrays])
+    be = OracleBackend()
+    ins = [be.malloc(a.nbytes, a.tobytes()) for a in arrays]
+    outs = prog.execute(be, ins)
+    return prog, be, ins, outs
+
+
+def test_output_returned_twice_carries_two_references():
+    """`return [y, y]`: both entries name one slot, and each can be released on its own."""
+    x = f32([1, 2, 3])
+    prog, be, ins, outs = _run_keeping_outputs(lambda a: (lambda y: [y, y])(a.mul(a)), x)
+    assert outs[0] == outs[1] and sum(1 for s in prog.steps if s.kind == "incref") == 1
+    be.decRef(outs[0])
+    np.testing.assert_array_equal(np.frombuffer(be.readSync(outs[1]), np.float32), [1, 4, 9])  # still alive
+    be.decRef(outs[1])
+    be.decRef(ins[0])
+    assert be.live_slots() == 0
+
+
+def test_input_returned_twice_beside_a_result():
+    """`return [x, y, x]`: the input gains one reference per appearance and stays the caller's as well."""
+    x = f32([1, 2, 3])
+    prog, be, ins, outs = _run_keeping_outputs(lambda a: [a, a.add(1), a], x)
+    assert outs[0] == ins[0] and outs[2] == ins[0] and sum(1 for s in prog.steps if s.kind == "incref") == 2
+    for o in outs:
+        be.decRef(o)
+    np.testing.assert_array_equal(np.frombuffer(be.readSync(ins[0]), np.float32), x)  # the caller's own reference
+    be.decRef(ins[0])
+    assert be.live_slots() == 0

@@ -10,7 +10,7 @@ import subprocess
 import numpy as np
 import pytest
 
-from jaxjs_hip import AluExp, AluOp, DType, ShapeTracker
+from jaxjs_hip import AluExp, AluOp, AluVar, DType, Kernel, ShapeTracker
 from jaxjs_hip.alu import numpyDtype
 from jaxjs_hip.lowering import mapKernel, matmulKernel, matvecKernel, reduceKernel
 from jaxjs_hip.plan import exportPlan, exportRoutinePlan
@@ -24,7 +24,7 @@ needs_node = pytest.mark.skipif(NODE is None or not os.path.exists(os.path.join(
 
 EXPORTS = ["init", "shutdown", "deviceInfo", "malloc", "free", "h2d", "d2h", "compile", "moduleLoad", "moduleUnload",
            "moduleFunction", "launch", "sync", "eventCreate", "eventRecord", "eventQuery", "eventElapsedMs", "eventDestroy",
-           "graphBegin", "graphEnd", "graphLaunch", "graphDestroy", "abiVersion"]
+           "graphBegin", "graphEnd", "graphLaunch", "graphDestroy", "abiVersion", "d2hAsync", "compilerVersion"]
 
 
 @needs_node
@@ -33,7 +33,7 @@ def test_addon_loads_and_exports_every_binding():
                          cwd=NAPI, capture_output=True, text=True, timeout=60)
     assert out.returncode == 0, out.stderr
     keys, abi = json.loads(out.stdout)
-    assert sorted(keys) == sorted(EXPORTS) and abi == 1
+    assert sorted(keys) == sorted(EXPORTS) and abi == 2
 
 
 @needs_node
@@ -87,12 +87,19 @@ def test_javascript_backend_replays_plans(tmp_path):
         pytest.skip("warm-up run: nothing to execute")
     payload = [dict(name=n, plan=exportPlan(k), inputs=[base64.b64encode(np.ascontiguousarray(x).tobytes()).decode() for x in xs])
                for n, k, xs in cases]
+    # the kernel behind the asynchronous-read check: no inputs, 2^26 floats written per launch (tens of microseconds)
+    big = Kernel(0, 1 << 26, AluExp.sin(AluExp.cast(DType.Float32, AluVar.gidx)))
+    payload.append(dict(name="async_read", plan=exportPlan(big), inputs=[], asyncOnly=True))
     src, dst = tmp_path / "cases.json", tmp_path / "results.json"
     src.write_text(json.dumps(payload))
     out = subprocess.run([NODE, os.path.join(NAPI, "run_plan.js"), str(src), str(dst)], capture_output=True, text=True, timeout=300)
     assert out.returncode == 0, out.stdout + out.stderr
     res = json.loads(dst.read_text())
     assert res["protocol"] is True and "gfx950" in res["device"]["arch"]
+    # `read` is asynchronous: pending when it returns, the event loop turns while 400 launches drain, same bytes
+    ar = res["asyncRead"]
+    assert ar["pendingAtReturn"] and ar["loopTurnsWhilePending"] > 0 and ar["bytesEqual"] and ar["rangedEqual"], ar
+    assert ar["emptyLength"] == 0 and ar["unknownSlotRejects"], ar
     classes = set()
     for (name, k, xs), r in zip(cases, res["cases"]):
         assert r["name"] == name

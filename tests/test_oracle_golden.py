@@ -214,31 +214,55 @@ def test_erf_values():  # src/alu.test.ts:115-137
         assert abs(oracle.wasm_builtin("erfc", x) - L.jo_js_erfc(float(np.float32(x)))) < 5e-7
 
 
-def test_wasm_exp_bounds():  # wasm/builtins.test.ts:20-42: rel < 2e-7 on moderate inputs, edge cases
-    for x in [-10, -5, -2, -1, -0.5, 0, 0.5, 1, 2, 5, 10, 0.001, -0.001, 3.14159]:
-        got, want = oracle.wasm_builtin("exp", x), math.exp(float(np.float32(x)))
-        assert abs(got - want) / want < 2e-6, x
+def _rel(got, want):  # relativeError of wasm/builtins.test.ts:15-17
+    return abs(got - want) / max(abs(want), 1e-3)
+
+
+def test_wasm_exp_bounds():
+    """wasm/builtins.test.ts:19-42: the reference's own sample list under its own bound (rel < 2e-7), edge cases.
+    A wrong high-order Taylor coefficient shows at x = 0.3 .. 0.35 (r^6/720 ~ 1e-6 there)."""
+    for x in [-5, -2, -1, -0.5, 0, 0.001, 0.01, 0.1, 0.2, 0.3, 0.4, 0.5, 0.6, 0.9, 0.99, 1, 2, 3, 5, 10]:
+        assert _rel(oracle.wasm_builtin("exp", x), math.exp(x)) < 2e-7, x
+    assert oracle.wasm_builtin("exp", math.inf) == math.inf
+    assert oracle.wasm_builtin("exp", -math.inf) == 0.0
+    assert math.isnan(oracle.wasm_builtin("exp", math.nan))
     assert oracle.wasm_builtin("exp", 0.0) == 1.0
     assert oracle.wasm_builtin("exp", 1000.0) == math.inf  # test/numpy.test.ts:2803-2830
     assert oracle.wasm_builtin("exp", -1000.0) == 0.0
-    assert math.isnan(oracle.wasm_builtin("exp", math.nan))
     xs = np.linspace(-80, 80, 4001).astype(np.float32)
     rel = max(abs(oracle.wasm_builtin("exp", float(x)) - math.exp(float(x))) / math.exp(float(x)) for x in xs)
     assert rel < 1e-5  # grows with |x| because k*ln2 is formed in f32
 
 
-def test_wasm_log_bounds():  # wasm/builtins.test.ts:44-64
-    for x in [0.001, 0.1, 0.5, 1, 2, 2.718281828, 10, 100, 1000, 1e10]:
-        got, want = oracle.wasm_builtin("log", x), math.log(float(np.float32(x)))
-        assert abs(got - want) <= 2e-5 * max(1.0, abs(want)), x
+def test_wasm_log_bounds():
+    """wasm/builtins.test.ts:44-64: the reference's sample list under its bound (rel < 5e-7), edge cases."""
+    for x in [0.01, 0.1, 0.5, 1, 1.5, 2, math.e, 5, 10, 100]:
+        assert _rel(oracle.wasm_builtin("log", x), math.log(float(np.float32(x)))) < 5e-7, x
     assert oracle.wasm_builtin("log", 1.0) == 0.0
     assert oracle.wasm_builtin("log", 0.0) == -math.inf
     assert math.isnan(oracle.wasm_builtin("log", -1.0))
     assert oracle.wasm_builtin("log", math.inf) == math.inf
+    assert math.isnan(oracle.wasm_builtin("log", math.nan))
     # Series truncated at t^7: the worst case is a mantissa just below 2 with exponent 0.
     worst = max(abs(oracle.wasm_builtin("log", float(x)) - math.log(float(x))) / abs(math.log(float(x)))
                 for x in np.linspace(1.5, 1.999, 200).astype(np.float32))
     assert 1e-6 < worst < 3e-5
+
+
+def test_wasm_sincos_atan_reference_lists():
+    """wasm/builtins.test.ts:66-167 on the reference's own points and bounds: sin/cos abs < 5e-7, atan rel < 2e-6."""
+    pi = math.pi
+    for x in [-2 * pi, -pi, -pi / 2, -pi / 4, 0, pi / 6, pi / 4, pi / 3, pi / 2, pi, 3 * pi / 2, 2 * pi, 5, 10, -5, -10]:
+        assert abs(oracle.wasm_builtin("sin", x) - math.sin(x)) < 5e-7, x
+        assert abs(oracle.wasm_builtin("cos", x) - math.cos(x)) < 5e-7, x
+    for f in ("sin", "cos"):
+        for x in (math.inf, -math.inf, math.nan):
+            assert math.isnan(oracle.wasm_builtin(f, x))
+    for x in [-1000, -100, -50, -10, -5, -2, -1, -0.5, -0.1, -0.01, 0, 0.01, 0.1, 0.5, 1, 2, 5, 10, 50, 100, 1000]:
+        assert _rel(oracle.wasm_builtin("atan", x), math.atan(x)) < 2e-6, x
+    assert oracle.wasm_builtin("atan", math.inf) == pytest.approx(pi / 2, abs=5e-3)   # toBeCloseTo: two decimals
+    assert oracle.wasm_builtin("atan", -math.inf) == pytest.approx(-pi / 2, abs=5e-3)
+    assert math.isnan(oracle.wasm_builtin("atan", math.nan))
 
 
 def test_wasm_sincos_atan_bounds():  # wasm/builtins.test.ts:66-167
