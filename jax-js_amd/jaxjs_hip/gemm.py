@@ -27,14 +27,25 @@ def choose_tile(g: dict) -> Dict[str, int]:
     def tiles(bm, bn):
         return -(-g["M"] // bm) * -(-g["N"] // bn) * nb
 
+    CU = tuner.CU_COUNT
+    plain_k = not (g.get("a_gather") or g.get("b_gather")) and g["a_k0"] == g["K"] and g["b_k0"] == g["K"]
     if g["dtype"] == DType.Float32:
         # The f32 matrix pipe is 16x slower than the f16 one, so LDS traffic matters little and filling
         # every CU matters most: take the largest tile that still yields two workgroups per CU (the
-        # second one hides the first one's staging latency).
+        # second one hides the first one's staging latency).  Slabs are 32 deep (measured 3-6 % over 16 on
+        # 2048^3 and 4096^3: half the barriers); gather operands keep the 16-deep slabs they were tuned with.
+        bk = 32 if plain_k else 16
         for bm, bn in ((128, 128), (128, 64), (64, 64)):
-            if g["M"] >= bm and g["N"] >= bn and tiles(bm, bn) >= 2 * tuner.CU_COUNT:
-                return dict(BM=bm, BN=bn)
-        return dict(BM=64, BN=64)
+            if g["M"] >= bm and g["N"] >= bn and tiles(bm, bn) >= 2 * CU:
+                return dict(BM=bm, BN=bn, BK=bk)
+        # Fewer tiles than that: 128x64 tiles with the k axis cut over blockIdx.y until the launch has at least 1.5
+        # workgroups per CU (1024^3: 128 tiles x 4 slices, 37.9 -> 31.1 us; 128x14336x4096: 224 x 2, 222 -> 172 us).
+        if plain_k and g["M"] >= 128 and g["N"] >= 64:
+            split = 1
+            while tiles(128, 64) * split < 1.5 * CU and split < 8 and g["K"] % (split * 2 * bk) == 0 and g["K"] // (split * 2) >= 256:
+                split *= 2
+            return dict(BM=128, BN=64, BK=bk, SPLITK=split)
+        return dict(BM=64, BN=64, BK=bk)
     # f16: estimated time = (tiles the busiest CU runs) x (tile area) x (K + fixed per-tile overhead) / efficiency.
     # Efficiencies are measured rates of each tile shape relative to 256x256 on large problems (MI355X):
     # 128x256 0.84, 256x128 0.79, 128x128 0.72 with two workgroups resident per CU (0.64 alone).  The fixed
@@ -57,8 +68,19 @@ def choose_tile(g: dict) -> Dict[str, int]:
             eff = 0.64
         cost = per_cu * bm * bn * (g["K"] + 100) / eff
         if best is None or cost < best[0]:
-            best = (cost, dict(BM=bm, BN=bn, **extra))
-    return best[1]
+            best = (cost, dict(BM=bm, BN=bn, **extra), per_cu)
+    tile, per_cu = dict(best[1]), best[2]
+    both_k = g["a_sk"] == 1 and g["b_sk"] == 1
+    if (tile["BM"], tile["BN"]) == (128, 128) and per_cu == 1 and plain_k and g["K"] % 64 == 0:
+        # One 128x128 workgroup per CU (or fewer): nothing shares the CU's LDS, so the slabs can be 64 deep in four
+        # stages (128 KiB: twice the bytes in flight per workgroup; 2048^3 20.7 -> 19.6 us, 128x14336x4096 35.2 -> 27.4 us).
+        if not both_k:
+            tile.update(BK=64, STAGES=4)
+        # Half the CUs or fewer would get a workgroup: cut the k axis in two (128x14336x4096: 27.4 -> 26.0 us with
+        # the fold launch included; four slices cost more in partial sums than they gain)
+        if tiles(128, 128) * 2 <= CU and g["K"] >= 2048 and g["K"] % 128 == 0:
+            tile["SPLITK"] = 2
+    return tile
 
 
 def _strip_casts(e: AluExp) -> AluExp:
@@ -498,7 +520,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     # measured +7..21 % on every tile shape.  An operand that runs along m or n is fetched in whole lines either way,
     # and the shorter pipeline that 64-deep slabs leave room for then costs more than it gains.
     both_k = g["a_sk"] == 1 and g["b_sk"] == 1 and g["K"] % 64 == 0 and g["K"] >= 128
-    dBK = tile.get("BK", 64 if both_k and tile.get("PIPE", 1) else 32)
+    dBK = tile.get("BK", 64 if both_k and tile.get("PIPE", 1) else 32) if g["dtype"] == DType.Float16 else 32
     if dBK not in (32, 64):
         raise ValueError(f"direct-to-LDS slab depth must be 32 or 64, got {dBK}")
     full = g["M"] % BM == 0 and g["N"] % BN == 0 and g["K"] % dBK == 0 and BM >= 128 and BN >= 128
@@ -516,6 +538,10 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         span = 2 * max((BM - 1) * abs(g["a_sm"]) + dBK * abs(g["a_sk"]), (BN - 1) * abs(g["b_sn"]) + dBK * abs(g["b_sk"]))
         sched["SADDR"] = 1 if tile.get("SADDR", 1) and span < 2 ** 31 and g["a_sm"] >= 0 and g["a_sk"] >= 0 and g["b_sn"] >= 0 and g["b_sk"] >= 0 else 0
         sched.update(PIN=tile.get("PIN", 1), BAR_AT=tile.get("BAR_AT", 2), READ_AHEAD=tile.get("RA", 1), LOADS_LATE=tile.get("LATE", 1))
+        # Tile walk: groups of 4 tile rows (8192^3: 865 -> 853 us against groups of 8, 873 with 16; one group spanning
+        # all rows loses a third).  C leaves through nontemporal stores: it is not read again by the launch and
+        # should not displace operand lines from the caches (+0.5..1 % on 8192^3, 3 % on 128x14336x4096).
+        sched.update(GROUP_M=int(tile.get("GM", 4)), NT_STORE=int(tile.get("NTS", 1)))
         sched["RING"] = ring = tile.get("RING", ring_default)
         if ring and (ring != 5 or BM != BN or not sched["PIPE"]):
             raise ValueError("the unit ring is five units of a square block tile under the phase-pipelined loop")

@@ -265,7 +265,7 @@ def _gen_reduce(kernel: Kernel, t: TuneResult, numerics: str, name: str, row: bo
             epi_value = tail_value = "0"
         src = _prelude(numerics) + fill(template("reduce_col.hip.inc"), dict(
             SIZE=size, R=R, V=V, T=T, LX=p["lx"], SPLIT=split, SLICE=slice_len, PITCH=_partial_pitch(size, V),
-            UNROLL=p.get("unroll", 4),
+            UNROLL=p.get("unroll", 4), INTERLEAVE=p.get("interleave", 0),
             REDUCE=_reduce_text(re.op, re.dtype), NAME=name, PARAMS=params, ACC_T=acc_t, OUT_T=out_t,
             IDENTITY=ident, VECTOR_LOADS=hoisted, LANE_BODY=lane_body, LANE_VALUE=lane_value,
             SCALAR_BODY=scalar_body, SCALAR_VALUE=scalar_value,

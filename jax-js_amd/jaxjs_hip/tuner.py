@@ -403,7 +403,8 @@ def _grid_for(blocks_needed: int) -> int:
 
 
 def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True,
-            gemm_tile: Optional[tuple] = None, col_strip: Optional[tuple] = None) -> TuneResult:
+            gemm_tile: Optional[tuple] = None, col_strip: Optional[tuple] = None,
+            row_lanes: Optional[int] = None) -> TuneResult:
     """Pick the kernel class and its parameters for one Kernel on MI355X."""
     t = tuneNullopt(kernel)
     re = kernel.reduction
@@ -459,6 +460,8 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
         T = max(min(t_hi, 16), min(_pow2_floor(max(vec_iters // 8, 1)), t_hi))
         while T < t_hi and size * T < CU_COUNT * 512:
             T *= 2
+        if row_lanes:  # tuning override: lanes per output row
+            T = int(row_lanes)
         block = max(T, 256)
         rows = block // T
         split = 1
@@ -488,7 +491,7 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
     if allow_split and groups * T < CU_COUNT * 512 and R // T >= 64:
         want = (CU_COUNT * 1024) // max(groups * T, 1)
         split = max(1, min(want, R // (T * 16), 1024))
-    unroll = 4
+    unroll, interleave = 4, 0
     # Few column groups but a long fold: instead of two launches (slices + fold), give each block a strip
     # only one 128-byte line wide and ALL of the reduce axis -- 1024 lanes as 8 column lanes x 128 row slots,
     # 8 independent vector loads in flight per lane.  Enough strips for half the CUs already saturates HBM.
@@ -496,15 +499,16 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
         lx_line = 8  # 8 lanes x 16 bytes = one 128-byte line per row
         blk = 1024
         rows_split = 1
-        if col_strip:  # (lanes per strip, block size, unroll[, blocks along the reduce axis]): tuning override
+        if col_strip:  # (lanes per strip, block size, unroll[, blocks along the reduce axis[, interleaved rows]]): tuning override
             lx_line, blk, unroll = col_strip[:3]
             rows_split = col_strip[3] if len(col_strip) > 3 else 1
+            interleave = col_strip[4] if len(col_strip) > 4 else 0
         strips = -(-groups // lx_line)
         if strips >= CU_COUNT // 2 and R // (blk // lx_line) >= 8:
             lx, T, split, unroll = lx_line, blk // lx_line, rows_split, (unroll if col_strip else 8)
     t.klass = "reduce_col"
     t.vector_loads = along_g if V > 1 else {}
-    t.params = dict(V=V, T=T, lx=lx, block=lx * T, split=split, unroll=unroll)
+    t.params = dict(V=V, T=T, lx=lx, block=lx * T, split=split, unroll=unroll, interleave=interleave)
     t.params["grid"] = _grid_for((groups + lx - 1) // lx)
     t.epi_vector_loads = classify_loads(t.epilogue, "gidx", V) if V > 1 else {}
     return t

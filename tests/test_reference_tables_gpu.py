@@ -16,21 +16,29 @@ from jaxjs_hip.jit import ShapedArray
 from jit_util import run_program
 
 pytestmark = pytest.mark.gpu
+if WARM_ONLY:  # every comparison below would see the empty placeholder
+    pytestmark = [pytest.mark.gpu, pytest.mark.xfail(reason="warm-up run: compiled only", strict=False)]
 F32, F16, I32 = DType.Float32, DType.Float16, DType.Int32
 NP = {F32: np.float32, F16: np.float16, I32: np.int32}
 
 
 @pytest.fixture(params=["wasm", "fast"])
 def be(request):
+    if WARM_ONLY:
+        return request.param
     return backend() if request.param == "wasm" else fast_backend()
 
 
 def run(be, fn, *arrays, dtype=F32):
     arrays = [np.asarray(a, dtype=NP[dtype]) for a in arrays]
     prog = J.jit(fn, [ShapedArray(tuple(a.shape), dtype) for a in arrays])
-    if WARM_ONLY:
-        from test_programs_gpu import warm
-        warm(prog)
+    if WARM_ONLY:  # compile this program's kernels into the on-disk cache and move on to the next program
+        from jaxjs_hip.kernelgen import generate
+        from jaxjs_hip.runtime import compile_source
+        for k in prog.kernels + [c.kernel() for c in prog.consts]:
+            for src in generate(k, be).sources:
+                compile_source(src)
+        return np.zeros(0)
     outs = run_program(be, prog, arrays)
     return outs[0] if len(outs) == 1 else outs
 
