@@ -123,6 +123,23 @@ int jh_module_function(jh_module module, const char *kernel_name, jh_function *o
 int jh_launch(jh_function fn, uint32_t grid_x, uint32_t grid_y, uint32_t grid_z, uint32_t block_x,
               uint32_t block_y, uint32_t block_z, uint32_t shared_bytes, void **args);
 
+/*
+ * `jh_launch` for callers that cannot allocate (a launch recorded under graph capture, a serving loop, a harness that
+ * forbids hipMalloc).  No counterpart in the reference.  Kernels whose reduce axis is cut over several workgroups
+ * (two-stage reductions, split-k GEMMs) write partial accumulators to a scratch buffer that the host side normally
+ * allocates per executable; here the kernel argument number `scratch_arg` is instead pointed at a buffer that lives
+ * inside the library (a file-scope device array of `jh_static_scratch_bytes` = 32 MiB per GPU, held until the process
+ * ends): the 8-byte cell `args[scratch_arg]` points at is overwritten with its device address, then the launch is
+ * queued exactly like `jh_launch`.  `scratch_bytes` is what the kernel will address; more than the buffer holds is an
+ * error and nothing is launched.  Calls no hipMalloc/hipFree.  Every call on a GPU shares that GPU's buffer, which
+ * keeps the previous call's contents (these kernels write every partial before reading it, so nothing needs clearing);
+ * launches that use it must not overlap -- on this library's single in-order stream they never do.
+ */
+int jh_launch_static_scratch(jh_function fn, uint32_t grid_x, uint32_t grid_y, uint32_t grid_z, uint32_t block_x,
+                             uint32_t block_y, uint32_t block_z, uint32_t shared_bytes, void **args,
+                             uint32_t scratch_arg, size_t scratch_bytes);
+int jh_static_scratch_bytes(size_t *bytes);
+
 /* Same launch repeated `count` times back to back (benchmark loops without per-call host overhead). */
 int jh_launch_repeat(jh_function fn, uint32_t grid_x, uint32_t grid_y, uint32_t grid_z, uint32_t block_x,
                      uint32_t block_y, uint32_t block_z, uint32_t shared_bytes, void **args, int count);

@@ -15,9 +15,18 @@
 #include <cstring>
 #include <string>
 
+// Scratch memory of `jh_launch_static_scratch`: one array per GPU, inside the library's own code object, so the entry
+// point never allocates.  In host code the array's name is only a stand-in: the device address is looked up once
+// per device (hipGetSymbolAddress in jh_init) and that pointer is what kernels receive.
+#define JH_STATIC_SCRATCH_BYTES (32u << 20)
+static __device__ __align__(256) unsigned char jh_static_scratch[JH_STATIC_SCRATCH_BYTES];
+
 namespace {
 
 thread_local std::string g_last_error;
+
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices] = {};  // device address of jh_static_scratch on each GPU this process has initialised
 
 struct Runtime {
   bool ready = false;
@@ -66,6 +75,16 @@ int jh_init(int device) {
   JH_HIP(hipSetDevice(device));
   // Default priority on purpose: work on streams of different priorities has hung on this pool.
   JH_HIP(hipStreamCreateWithFlags(&g_rt.stream, hipStreamNonBlocking));
+  if (device < kMaxDevices && !g_scratch_ptr[device]) {
+    void *p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(jh_static_scratch));  // this device's copy of the array
+    if (e != hipSuccess || !p) {
+      (void)hipStreamDestroy(g_rt.stream);
+      g_rt.stream = nullptr;
+      return fail((int)e ? (int)e : -9, "hipGetSymbolAddress(jh_static_scratch) failed: %s", hipGetErrorString(e));
+    }
+    g_scratch_ptr[device] = p;
+  }
   g_rt.device = device;
   g_rt.ready = true;
   return 0;
@@ -266,6 +285,26 @@ int jh_launch(jh_function fn, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx
     return fail(-8, "invalid block %ux%ux%u", bx, by, bz);
   JH_HIP(hipModuleLaunchKernel((hipFunction_t)fn, gx, gy, gz, bx, by, bz, shared_bytes, g_rt.stream, args, nullptr));
   return 0;
+}
+
+int jh_static_scratch_bytes(size_t *bytes) {
+  if (!bytes) return fail(-5, "null output");
+  *bytes = JH_STATIC_SCRATCH_BYTES;
+  return 0;
+}
+
+int jh_launch_static_scratch(jh_function fn, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, uint32_t by, uint32_t bz,
+                             uint32_t shared_bytes, void **args, uint32_t scratch_arg, size_t scratch_bytes) {
+  JH_NEED_INIT();
+  if (!fn || !args) return fail(-5, "null kernel or argument list");
+  if (scratch_bytes > JH_STATIC_SCRATCH_BYTES)
+    return fail(-10, "kernel needs %zu bytes of scratch, the static scratch buffer holds %u", scratch_bytes,
+                (unsigned)JH_STATIC_SCRATCH_BYTES);
+  if (g_rt.device >= kMaxDevices || !g_scratch_ptr[g_rt.device]) return fail(-9, "no static scratch on device %d", g_rt.device);
+  if (!args[scratch_arg]) return fail(-5, "argument %u has no cell to receive the scratch address", scratch_arg);
+  // The kernel takes the looked-up device address, never the array's name.
+  *(void **)args[scratch_arg] = g_scratch_ptr[g_rt.device];
+  return jh_launch(fn, gx, gy, gz, bx, by, bz, shared_bytes, args);
 }
 
 int jh_launch_repeat(jh_function fn, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, uint32_t by, uint32_t bz,

@@ -374,6 +374,37 @@ class HipBackend:
             else:
                 self.dev.launch(fn, step.grid, step.block, step.shared, argv, repeat)
 
+    def dispatchStaticScratch(self, exe: Executable, inputs: Sequence[int], outputs: Sequence[int]) -> None:
+        """`dispatch` of a Kernel through `jh_launch_static_scratch`: launch steps that take a scratch buffer get the
+        library's static one instead of the buffer allocated with the executable, so nothing is allocated on the way.
+        For callers that must not allocate; results are bit-identical to `dispatch` (same kernels, same fold order)."""
+        ins = [self._get(s) for s in inputs]
+        outs = [self._get(s) for s in outputs]
+        kernel, prep = exe.source, exe.data
+        if isinstance(kernel, Routine) or prep.released or len(outs) != 1:
+            raise ValueError("dispatchStaticScratch takes a live prepared Kernel and one output")
+        if len(ins) < kernel.nargs or outs[0]["size"] < kernel.bytes:
+            raise ValueError("inputs or output do not fit the kernel")
+        for gid, need in prep.ks.min_input_bytes.items():
+            if ins[gid]["size"] < need:
+                raise ValueError(f"input {gid} holds {ins[gid]['size']} bytes, kernel addresses {need}")
+        if len(prep.ks.scratch_bytes) > 1:
+            raise ValueError("a kernel with several scratch buffers cannot share the one static buffer")
+        if kernel.size == 0:
+            return
+        lib = self.dev.lib
+        for step, head, (cells, argv, patch) in zip(prep.ks.steps, prep.launch_head, prep.bound):
+            for c, kind, i in patch:
+                cells[c] = ins[i]["ptr"] if kind == "in" else outs[0]["ptr"]
+            where = [c for c, (kind, _) in enumerate(step.args) if kind == "scratch"]
+            if where:
+                rc = lib.jh_launch_static_scratch(*head, argv, where[0], prep.ks.scratch_bytes[0])
+                cells[where[0]] = prep.scratch[0]  # the cell was overwritten: restore it for ordinary dispatches
+            else:
+                rc = lib.jh_launch(*head, argv)
+            if rc:
+                check(rc, "jh_launch_static_scratch")
+
     def sync(self) -> None:
         """Completion fence (what `read(slot, 0, 0)` stands for in src/frontend/array.ts:827)."""
         self.dev.sync()

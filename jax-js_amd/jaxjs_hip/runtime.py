@@ -67,6 +67,9 @@ _SIGNATURES = {
     "jh_module_unload": (ctypes.c_int, [ctypes.c_void_p]),
     "jh_module_function": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_char_p, ctypes.POINTER(ctypes.c_void_p)]),
     "jh_launch": (ctypes.c_int, [ctypes.c_void_p] + [ctypes.c_uint32] * 7 + [ctypes.POINTER(ctypes.c_void_p)]),
+    "jh_launch_static_scratch": (ctypes.c_int, [ctypes.c_void_p] + [ctypes.c_uint32] * 7 +
+                                 [ctypes.POINTER(ctypes.c_void_p), ctypes.c_uint32, ctypes.c_size_t]),
+    "jh_static_scratch_bytes": (ctypes.c_int, [ctypes.POINTER(ctypes.c_size_t)]),
     "jh_launch_repeat": (ctypes.c_int, [ctypes.c_void_p] + [ctypes.c_uint32] * 7 +
                          [ctypes.POINTER(ctypes.c_void_p), ctypes.c_int]),
     "jh_sync": (ctypes.c_int, []),
