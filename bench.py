@@ -14,6 +14,7 @@ import argparse
 import ctypes
 import json
 import os
+import re
 import sys
 import time
 
@@ -409,8 +410,9 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-settle", action="store_true", help="skip the clock-settling launches before the warm-up steps")
-    ap.add_argument("--only", choices=["all", "gemm", "copy"], default="all",
-                    help="gemm: headline kernel only; copy: a plain f32 copy kernel of known size (counter calibration)")
+    ap.add_argument("--only", choices=["all", "gemm", "copy", "hbm"], default="all",
+                    help="gemm: headline kernel only; copy: a plain f32 copy kernel of known size (counter calibration); "
+                         "hbm: headline + the HBM-bound secondary workloads only (matvecs, row kernels, map)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -440,7 +442,7 @@ def main():
     A = hostrand.uniform(1004, (n, n), dtype=np.float16)
     B = hostrand.uniform(1005, (n, n), dtype=np.float16, stream=1)
     kern = matmulKernel(n, n, n, DType.Float16)
-    exe = be.prepareKernelSync(kern)
+    exe = be.prepareKernelSync(kern, name=f"jh_gemm_f16_{n}_headline")
     a, b = upload(be, A), upload(be, B)
     c = be.malloc(kern.bytes)
     settled = 0 if args.no_settle else settle(be, exe, [a, b], c)
@@ -475,7 +477,8 @@ def main():
         steps, warm = max(args.steps, 20), max(args.warmup, 5)
 
         def run(name, kernel, bufs, work, unit, peak):
-            ex = be.prepareKernelSync(kernel)
+            # the entry point carries the workload's name, so a profiler's per-kernel rows can be told apart
+            ex = be.prepareKernelSync(kernel, name="jh_" + re.sub(r"[^A-Za-z0-9]+", "_", name).strip("_"))
             slots = [upload(be, x) for x in bufs]
             o = be.malloc(kernel.bytes)
             # The clocks idle down while the host prepares inputs: warm up for ~30 ms of device work and time
@@ -540,6 +543,11 @@ def main():
         kmap = mapKernel([rows, L], [(f, st)], lambda v: AluExp.mul(AluExp.exp(v), AluExp.f32(0.5)))
         run("map_exp_f32[8192,4096]", kmap, [X], 2 * xb, "GB/s", PEAK_HBM_GBS)
         del X
+        if args.only == "hbm":
+            result["extra"] = extra
+            result["cpu_baseline"] = None
+            print(json.dumps(result))
+            return
 
         for (mm, nn, kk, dt, tag, peak) in [
             (1024, 1024, 1024, DType.Float32, "c1_matmul_f32_1024", PEAK_F32_MATRIX_TFLOPS),

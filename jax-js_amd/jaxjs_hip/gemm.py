@@ -539,9 +539,10 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         sched["SADDR"] = 1 if tile.get("SADDR", 1) and span < 2 ** 31 and g["a_sm"] >= 0 and g["a_sk"] >= 0 and g["b_sn"] >= 0 and g["b_sk"] >= 0 else 0
         sched.update(PIN=tile.get("PIN", 1), BAR_AT=tile.get("BAR_AT", 2), READ_AHEAD=tile.get("RA", 1), LOADS_LATE=tile.get("LATE", 1))
         # Tile walk: groups of 4 tile rows (8192^3: 865 -> 853 us against groups of 8, 873 with 16; one group spanning
-        # all rows loses a third).  C leaves through nontemporal stores: it is not read again by the launch and
-        # should not displace operand lines from the caches (+0.5..1 % on 8192^3, 3 % on 128x14336x4096).
-        sched.update(GROUP_M=int(tile.get("GM", 4)), NT_STORE=int(tile.get("NTS", 1)))
+        # all rows loses a third).  Nontemporal C stores only for the f32 partials of a k split, where a wave's store
+        # covers whole 128-byte lines (128x14336x4096: 26.1 -> 25.3 us): with 2-byte outputs they gain nothing once the
+        # walk is in groups of 4 and the half-line writes cost a third more HBM write traffic (WRITE_SIZE 132 -> 176 MiB).
+        sched.update(GROUP_M=int(tile.get("GM", 4)), NT_STORE=int(tile.get("NTS", 1 if split > 1 else 0)))
         sched["RING"] = ring = tile.get("RING", ring_default)
         if ring and (ring != 5 or BM != BN or not sched["PIPE"]):
             raise ValueError("the unit ring is five units of a square block tile under the phase-pipelined loop")
