@@ -10,6 +10,7 @@ from .alu import (AluExp, AluGroup, AluOp, AluVar, DType, Kernel, Reduction, acc
 from .errors import HipRuntimeError, SlotError, UnsupportedOpError, UnsupportedRoutineError
 from .routine import Routine, Routines, RoutineType, ScatterOp
 from .shape import ShapeTracker, View, unravelAlu
+from .tracing import isTracing, startTrace, stopTrace
 
 devices = ["hip"]
 _backends = {}

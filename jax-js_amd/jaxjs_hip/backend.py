@@ -25,9 +25,11 @@ from __future__ import annotations
 
 import asyncio
 import ctypes
+import time
 from collections import OrderedDict
 from typing import Dict, List, Optional, Sequence
 
+from . import tracing
 from .alu import Kernel, byteWidth
 from .errors import HipRuntimeError, SlotError, UnsupportedRoutineError
 from .kernelgen import NUMERICS, KernelSource, generate
@@ -127,8 +129,13 @@ class HipBackend:
         self._pool_limit = 8 << 30
         self._exes: "OrderedDict[tuple, Executable]" = OrderedDict()
         self.cacheLimit = 4096
+        self._preparing: Dict[tuple, "asyncio.Future"] = {}  # prepares in flight, by cache key
+        self._compile_pool = None
         self._staging: Dict[int, List[int]] = {}  # capacity -> free pinned host buffers for asynchronous reads
-        self.trace: Optional[list] = None       # when a list: (label, start_event, stop_event) per dispatch
+        self.trace: Optional[list] = None       # when a list: (label, start_event, stop_event) per launch step
+        self._trace_base = None                 # (event, host ms) pair fixing the profiler hook's time base
+        self._trace_pending: list = []          # (TraceInfo, start event, stop event) per traced dispatch
+        self._trace_registered = False
 
     # -- memory -----------------------------------------------------------------------------------
     @staticmethod
@@ -252,8 +259,10 @@ class HipBackend:
         return self._get(slot)["ptr"]
 
     # -- kernels ----------------------------------------------------------------------------------
-    def _build(self, source, ks: KernelSource) -> Executable:
-        modules = [self.dev.load_module(compile_source(src, f"{ks.klass}.hip")) for src in ks.sources]
+    def _build(self, source, ks: KernelSource, blobs=None) -> Executable:
+        if blobs is None:
+            blobs = [compile_source(src, f"{ks.klass}.hip") for src in ks.sources]
+        modules = [self.dev.load_module(b) for b in blobs]
         functions = [self.dev.function(modules[s.module], s.name) for s in ks.steps]
         scratch = [self.dev.malloc(self._rounded(b)) for b in ks.scratch_bytes]
         return Executable(source, _Prepared(ks, functions, scratch, modules))
@@ -286,8 +295,40 @@ class HipBackend:
             return exe
         return self._remember(key, self._build(kernel, generate(kernel, self.numerics, **tune_opts)))
 
-    async def prepareKernel(self, kernel: Kernel) -> Executable:
-        return self.prepareKernelSync(kernel)
+    async def _prepare_async(self, key: tuple, source, make_plan) -> Executable:
+        """Asynchronous prepare (src/backend.ts:192-203; `createComputePipelineAsync` in src/backend/webgpu.ts:705-744):
+        source generation runs here, the hiprtc compilations run on worker threads (the C call releases the
+        interpreter lock), so a caller that awaits many kernels at once (src/frontend/array.ts:792-797) gets them
+        compiled side by side.  Idempotent: concurrent requests for one kernel share one compilation."""
+        exe = self._cached(key)
+        if exe is not None:
+            return exe
+        pending = self._preparing.get(key)
+        if pending is not None:
+            return await asyncio.shield(pending)
+        loop = asyncio.get_running_loop()
+        fut = loop.create_future()
+        self._preparing[key] = fut
+        try:
+            ks = make_plan()
+            if self._compile_pool is None:
+                from concurrent.futures import ThreadPoolExecutor
+                self._compile_pool = ThreadPoolExecutor(max_workers=8, thread_name_prefix="jaxhip-compile")
+            blobs = await asyncio.gather(*[loop.run_in_executor(self._compile_pool, compile_source, src, f"{ks.klass}.hip")
+                                           for src in ks.sources])
+            exe = self._cached(key) or self._remember(key, self._build(source, ks, blobs))
+            fut.set_result(exe)
+            return exe
+        except BaseException as e:
+            fut.set_exception(e)
+            fut.exception()  # mark as retrieved: waiters, if any, re-raise it themselves
+            raise
+        finally:
+            del self._preparing[key]
+
+    async def prepareKernel(self, kernel: Kernel, **tune_opts) -> Executable:
+        key = (kernel.key(), self.numerics, tuple(sorted(tune_opts.items())))
+        return await self._prepare_async(key, kernel, lambda: generate(kernel, self.numerics, **tune_opts))
 
     def prepareRoutineSync(self, routine: Routine) -> Executable:
         from .routine import SUPPORTED_ROUTINES
@@ -305,7 +346,13 @@ class HipBackend:
         return self._remember(key, self._build(routine, ks))
 
     async def prepareRoutine(self, routine: Routine) -> Executable:
-        return self.prepareRoutineSync(routine)
+        from .routine import SUPPORTED_ROUTINES
+        from .routinegen import generateRoutine
+
+        if routine.name not in SUPPORTED_ROUTINES:
+            raise UnsupportedRoutineError(routine.name, "hip")
+        key = ("routine", routineKey(routine), self.numerics)
+        return await self._prepare_async(key, routine, lambda: generateRoutine(routine, self.numerics))
 
     def _dispatch_routine(self, exe: Executable, ins, outs) -> None:
         """Launch a routine's native plan (several kernels on the one in-order stream)."""
@@ -334,7 +381,54 @@ class HipBackend:
             if rc:
                 check(rc, "jh_launch")
 
+    # -- profiler hook (src/backend/webgpu/tracing.ts: a timestamp pair around every pass) -----------
+    def _trace_begin(self):
+        """While tracing is on: an event ahead of the executable's launches; the first one also fixes the time base
+        (a synchronised event paired with the host clock) and registers the flush."""
+        if self._trace_base is None:
+            self.dev.sync()
+            ev = self.dev.event()
+            self.dev.record(ev)
+            self.dev.sync()
+            self._trace_base = (ev, time.perf_counter() * 1e3)
+            if not self._trace_registered:
+                tracing.onFlushTrace(self._trace_flush)
+                self._trace_registered = True
+        e0 = self.dev.event()
+        self.dev.record(e0)
+        return e0
+
+    def _trace_end(self, exe: Executable, e0) -> None:
+        e1 = self.dev.event()
+        self.dev.record(e1)
+        self._trace_pending.append((tracing.traceSourceInfo(exe.source), e0, e1))
+
+    def _trace_flush(self) -> None:
+        """Resolve the pending event pairs into host-clock times and emit them (run by `stopTrace`)."""
+        if self._trace_base is None:
+            return
+        base_ev, base_ms = self._trace_base
+        self.dev.sync()
+        for info, e0, e1 in self._trace_pending:
+            t0 = base_ms + self.dev.elapsed_ms(base_ev, e0)
+            t1 = base_ms + self.dev.elapsed_ms(base_ev, e1)
+            tracing.emitTrace("hip", info, t0, t1)
+            self.dev.destroy_event(e0)
+            self.dev.destroy_event(e1)
+        self.dev.destroy_event(base_ev)
+        self._trace_pending, self._trace_base = [], None
+
     def dispatch(self, exe: Executable, inputs: Sequence[int], outputs: Sequence[int], repeat: int = 1) -> None:
+        if tracing.isTracing():
+            e0 = self._trace_begin()
+            try:
+                self._dispatch(exe, inputs, outputs, repeat)
+            finally:
+                self._trace_end(exe, e0)
+            return
+        self._dispatch(exe, inputs, outputs, repeat)
+
+    def _dispatch(self, exe: Executable, inputs: Sequence[int], outputs: Sequence[int], repeat: int = 1) -> None:
         ins = [self._get(s) for s in inputs]
         outs = [self._get(s) for s in outputs]
         if isinstance(exe.source, Routine):

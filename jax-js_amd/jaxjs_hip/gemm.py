@@ -566,7 +566,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         sched = dict(COMMIT_A=tile.get("CA", 2), COMMIT_B=tile.get("CB", 3), FETCH_A=tile.get("FA", 0),
                      FETCH_B=tile.get("FB", 1), IGLP=tile.get("IGLP", -1), SCHED_FENCE=tile.get("FENCE", 0))
     else:
-        sched = dict(BK=fBK)
+        sched = dict(BK=fBK, FRAG_FENCE=int(tile.get("FENCE", 1)))
     if not dlds:
         sched.update(GATHER_FNS="\n".join(gather_fns), A_GATHER=gather_flags["a"], B_GATHER=gather_flags["b"],
                      GATHER_A_CALL=gather_calls["a"], GATHER_B_CALL=gather_calls["b"],

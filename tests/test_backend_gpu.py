@@ -353,3 +353,87 @@ def test_routine_executables_are_cached_and_released(be):
     finally:
         be.decRef(x)
         be.decRef(y)
+
+
+def test_prepare_kernel_compiles_concurrently(be, monkeypatch):
+    """`prepareKernel` awaited for many kernels at once (src/frontend/array.ts:792-797): the compilations overlap on
+    worker threads, two requests for one kernel share one compilation, and the executables compute what the
+    synchronous path's do."""
+    import threading
+    import jaxjs_hip.backend as B
+    from jaxjs_hip import runtime
+    monkeypatch.setattr(runtime, "DISK_CACHE", False)
+    active, peak, calls, lock = [0], [0], [0], threading.Lock()
+    orig = B.compile_source
+
+    def counting(src, nm="kernel.hip", *a, **kw):
+        with lock:
+            active[0] += 1
+            calls[0] += 1
+            peak[0] = max(peak[0], active[0])
+        try:
+            return orig(src, nm, *a, **kw)
+        finally:
+            with lock:
+                active[0] -= 1
+    monkeypatch.setattr(B, "compile_source", counting)
+    fresh = B.HipBackend(numerics="wasm")
+    n = 4096
+    st = ShapeTracker.fromShape([n])
+    x = AluExp.globalView(DType.Float32, 0, st, [AluVar.gidx])
+    kernels = [Kernel(1, n, AluExp.add(AluExp.mul(x, AluExp.f32(float(c))), AluExp.sin(x))) for c in range(2, 8)]
+
+    async def main():
+        return await asyncio.gather(*[fresh.prepareKernel(k) for k in kernels + kernels[:2]])
+    exes = asyncio.run(main())
+    assert calls[0] == len(kernels) and peak[0] >= 2, (calls, peak)
+    assert exes[6] is exes[0] and exes[7] is exes[1] and len({id(e) for e in exes[:6]}) == 6
+    assert fresh.prepareKernelSync(kernels[3]) is exes[3] and asyncio.run(fresh.prepareKernel(kernels[3])) is exes[3]
+    data = np.linspace(-3, 3, n).astype(np.float32)
+    a, o = fresh.malloc(n * 4, u8(data)), fresh.malloc(n * 4)
+    try:
+        fresh.dispatch(exes[5], [a], [o])
+        got = np.frombuffer(fresh.readSync(o), np.float32)
+        np.testing.assert_allclose(got, data * 7 + np.sin(data), rtol=1e-5, atol=1e-6)
+    finally:
+        fresh.decRef(a)
+        fresh.decRef(o)
+        fresh.clearCache()
+
+
+def test_profiler_hook_emits_one_measure_per_dispatch(be):
+    """startTrace / stopTrace (src/tracing.ts:15-36): every dispatch between them becomes one record shaped like the
+    reference's `performance.measure` entries, in dispatch order, with device times that nest inside the host's."""
+    import time
+    from jaxjs_hip import tracing
+    n = 1 << 22
+    st = ShapeTracker.fromShape([n])
+    k_map = Kernel(1, n, AluExp.exp(AluExp.globalView(DType.Float32, 0, st, [AluVar.gidx])))
+    k_red = Kernel(1, 1, AluExp.globalView(DType.Float32, 0, st, [AluVar.ridx]), Reduction(DType.Float32, AluOp.Add, n))
+    e_map, e_red = be.prepareKernelSync(k_map), be.prepareKernelSync(k_red)
+    a, b, c = be.malloc(n * 4, u8(np.zeros(n, np.float32))), be.malloc(n * 4), be.malloc(4)
+    seen = []
+    tracing.setTraceSink(seen.append)
+    try:
+        be.dispatch(e_map, [a], [b])  # not traced
+        t_before = time.perf_counter() * 1e3
+        tracing.startTrace()
+        assert tracing.isTracing()
+        be.dispatch(e_map, [a], [b])
+        be.dispatch(e_red, [b], [c])
+        tracing.stopTrace()
+        t_after = time.perf_counter() * 1e3
+        assert not tracing.isTracing() and [r["name"] for r in seen] == ["Kernel[4.19M]", "Kernel[1]"]
+        dev0, dev1 = seen[0]["detail"]["devtools"], seen[1]["detail"]["devtools"]
+        assert dev0["trackGroup"] == "JAX Profiler" and dev0["track"] == "hip" and dev0["color"] == "primary"
+        assert dev1["color"] == "secondary" and ("reduction", f"Add:{n}") in dev1["properties"]
+        assert dict(dev0["properties"])["size"] == str(n) and dict(dev0["properties"])["nargs"] == "1"
+        assert t_before <= seen[0]["start"] < seen[0]["end"] <= seen[1]["start"] + 0.05 and seen[1]["end"] <= t_after + 0.5
+        assert 0.001 < seen[0]["end"] - seen[0]["start"] < 5.0
+        assert np.frombuffer(be.readSync(c), np.float32)[0] == n  # the traced work ran: sum of exp(0)
+        be.dispatch(e_map, [a], [b])  # after stopTrace: nothing more is recorded
+        assert len(seen) == 2
+    finally:
+        tracing.setTraceSink(None)
+        for s in (a, b, c):
+            be.decRef(s)
