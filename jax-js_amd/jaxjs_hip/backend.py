@@ -254,6 +254,10 @@ class HipBackend:
         else:
             self.dev.host_free(host)
 
+    def live_slots(self) -> int:
+        """Slots currently allocated through this backend object (leak checks)."""
+        return len(self._slots)
+
     def slotPointer(self, slot: int) -> int:
         """Device address of a slot (for the benchmark harness)."""
         return self._get(slot)["ptr"]

@@ -373,6 +373,14 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
             return None
         oexp = operand_exps[gid].rewrite(_retarget_operand).simplify()
         gather_oexp[tag] = oexp
+        if tag == "b" and g["dtype"] == DType.Float16 and not g.get("a_gather") and split == 1 and tile.get("CONV", 1) and not tile.get("TAPMAJOR", 0):
+            # A stride-1 window walk over an image (verified on the operand's own index expression): the patch-in-LDS
+            # convolution template instead of an im2col tile built element by element.
+            from .convgen import gen_conv
+
+            conv = gen_conv(kernel, g, oexp, numerics, name, params, names, epi_fn, epi_args, _min_bytes(t.epilogue), tile)
+            if conv is not None:
+                return conv
         gcg = HipExpCodegen(names, {"row": "row", "k": "k", "b0": "b0", "b1": "b1", "b2": "b2"}, "  ", prefix=f"g{tag}", numerics=numerics)
         gcg.countReferences(oexp)
         gval = strip_parens(gcg.run(oexp))

@@ -230,6 +230,19 @@ F16_CONV_CASES = [
     dict(x=(2, 8, 7, 7), w=(32, 8, 3, 3), strides=[1, 1], padding="SAME", loader="element"),
     dict(x=(2, 8, 32, 32), w=(32, 8, 3, 3), strides=[2, 2], padding="SAME", loader="element"),
     dict(x=(2, 8, 16, 16), w=(32, 8, 1, 1), strides=[1, 1], padding="VALID", loader=None),
+    # stride-1 window walks with at least 16 input and 64 output channels and an output width that is a multiple of 4:
+    # the patch-in-LDS convolution template (image rows resident in LDS, one copy per window column)
+    dict(x=(2, 16, 16, 16), w=(64, 16, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),
+    dict(x=(3, 32, 8, 24), w=(64, 32, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),
+    dict(x=(2, 16, 28, 28), w=(64, 16, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),      # 4-element fill vectors
+    dict(x=(2, 16, 30, 30), w=(64, 16, 3, 3), strides=[1, 1], padding="VALID", loader="patch"),     # output narrower than the image
+    dict(x=(1, 32, 20, 40), w=(64, 32, 5, 5), strides=[1, 1], padding=[(3, 1), (0, 4)], loader="patch"),
+    dict(x=(2, 64, 12, 12), w=(128, 64, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),     # two channel tiles, ragged last position tile
+    dict(x=(1, 16, 56, 56), w=(256, 16, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),     # 128-channel tiles
+    dict(x=(2, 128, 14, 12), w=(64, 128, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),    # several channel slabs
+    dict(x=(2, 16, 64), w=(64, 16, 3), strides=[1], padding="SAME", loader="patch"),                # one spatial dim
+    dict(x=(2, 16, 16, 16), w=(32, 16, 3, 3), strides=[1, 1], padding="SAME", loader="rows8"),      # 32 output channels: generic loaders
+    dict(x=(2, 16, 32, 32), w=(64, 16, 3, 3), strides=[2, 2], padding="SAME", loader="element"),    # strided: generic loaders
 ]
 
 
@@ -247,6 +260,9 @@ def test_f16_convolution_loader_choice(case):
         assert "gather" not in ks.info or set(ks.info["gather"].values()) == {"none"}
     else:
         assert ks.klass.startswith("gemm") and case["loader"] in ks.info["gather"].values(), ks.info
+        if case["loader"] == "patch":
+            cv = ks.info["conv"]
+            assert (cv["KH"] * cv["KW"], cv["C"]) == (int(np.prod(case["w"][2:])), case["w"][1]) and len(ks.steps) == 2
         # the optional tap-major k order (k' = tap * C + c) applies to every one of them
         tm = generate(_f16_conv_program(case).kernels[0], gemm_tile=(("TAPMAJOR", 1),))
         assert tm.info["tap_major"]["T"] == int(np.prod(case["w"][2:])) and any(v.startswith("tap-major rows") for v in tm.info["gather"].values())

@@ -1,0 +1,61 @@
+"""The table tests of `test_jit.py` (the reference's nn / numpy / lax-linalg / random tables replayed through traced
+programs) run again with the hip backend in place of the CPU checker: same programs, same expected values, every
+kernel and routine on the GPU (Wasm-faithful numerics, so the tables' own tolerances apply unchanged)."""
+import pytest
+
+import test_jit as T
+from gpu_util import WARM_ONLY, backend
+
+pytestmark = pytest.mark.gpu
+
+# Tests of test_jit.py that only look at program structure (no backend involved) are left out.
+TABLE_TESTS = [
+    "test_elementwise_chain_is_one_kernel", "test_reduction_fuses_unary_and_literal_epilogue",
+    "test_reduction_epilogue_stops_at_broadcasting_operand_and_second_use", "test_two_reductions_never_share_a_kernel",
+    "test_dot_operand_with_reuse_is_materialised", "test_row_softmax_argmax_program_is_four_row_reductions_plus_one_constant",
+    "test_max_args_splits_wide_expressions", "test_softmax_table", "test_gelu_tables", "test_tanh_matches_libm_and_saturates",
+    "test_standardize_table", "test_attention_tables", "test_causal_attention_closed_form", "test_matmul_integer_cases_are_exact",
+    "test_einsum_layouts_of_attention", "test_gpt2_block_program_structure_and_values_f32",
+    "test_routine_outputs_and_operands_are_dispatch_boundaries", "test_solve_is_lu_plus_two_triangular_solves",
+    "test_triangular_solve_variants_match_the_reference_tables", "test_cholesky_upper_eigh_and_fft_along_an_axis",
+    "test_eigh_svd_and_diagonal_reference_tables", "test_random_bits_and_split_match_jax", "test_uniform_and_normal_distributions",
+    "test_gather_take_and_take_along_axis", "test_concatenate_stack_and_split",
+    "test_output_returned_twice_carries_two_references", "test_input_returned_twice_beside_a_result",
+]
+
+
+_shared = None
+
+
+def _hip():
+    """One backend object for all table tests (each test releases its own slots, so its leak check still holds)."""
+    global _shared
+    if _shared is None:
+        from jaxjs_hip.backend import HipBackend
+        backend()  # device up
+        _shared = HipBackend(numerics="wasm")
+    return _shared
+
+
+class _CompileOnly(T.OracleBackend):
+    """Warm-up stand-in: compiles what the hip backend would run into the on-disk cache, computes on the CPU checker."""
+
+    def prepareKernelSync(self, kernel):
+        from jaxjs_hip.kernelgen import generate
+        from jaxjs_hip.runtime import compile_source
+        for src in generate(kernel, "wasm").sources:
+            compile_source(src)
+        return super().prepareKernelSync(kernel)
+
+    def prepareRoutineSync(self, routine):
+        from jaxjs_hip.routinegen import generateRoutine
+        from jaxjs_hip.runtime import compile_source
+        for src in generateRoutine(routine, "wasm").sources:
+            compile_source(src)
+        return super().prepareRoutineSync(routine)
+
+
+@pytest.mark.parametrize("name", TABLE_TESTS)
+def test_table_on_the_gpu(name, monkeypatch):
+    monkeypatch.setattr(T, "OracleBackend", _CompileOnly if WARM_ONLY else (lambda *a, **kw: _hip()))
+    getattr(T, name)()
