@@ -269,6 +269,8 @@ class HipBackend:
         modules = [self.dev.load_module(b) for b in blobs]
         functions = [self.dev.function(modules[s.module], s.name) for s in ks.steps]
         scratch = [self.dev.malloc(self._rounded(b)) for b in ks.scratch_bytes]
+        for i in ks.zeroed_scratch:
+            self.dev.h2d(scratch[i], bytes(ks.scratch_bytes[i]))
         return Executable(source, _Prepared(ks, functions, scratch, modules))
 
     def _cached(self, key: tuple):

@@ -59,6 +59,8 @@ class KernelSource:
     # Minimum byte size each input slot must have (from the lengths the index analysis assumed).
     min_input_bytes: Dict[int, int] = field(default_factory=dict)
     info: Dict[str, object] = field(default_factory=dict)
+    # Scratch buffers (indices) that must hold zeros before the executable's first launch; the kernels leave them zeroed.
+    zeroed_scratch: List[int] = field(default_factory=list)
 
 
 def _used_args(nargs: int, *exps: Optional[AluExp]) -> List[Optional[DType]]:
