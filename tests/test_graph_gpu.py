@@ -97,3 +97,29 @@ def test_graph_replay_of_programs_with_routine_steps():
         a = block_inputs(batch, seq, d, d_ff, np.float16, seed=200 + r)
         return [a[n] for n in order]
     _check_program(block, arrays)
+
+
+def test_graph_replay_of_a_k_split_folded_inside_the_launch():
+    """An f32 matmul small enough that its k axis is cut over workgroups and folded inside the launch (per-tile counters
+    that every launch must leave at zero): replays of the captured graph equal the eager run bit for bit."""
+    from jaxjs_hip import jit as J
+    from jaxjs_hip import library as L
+    from jaxjs_hip.alu import DType
+    from jaxjs_hip.jit import ShapedArray
+    M, K, N = 256, 2048, 192
+    prog = J.jit(lambda a, b: L.matmul(a, b), [ShapedArray((M, K), DType.Float32), ShapedArray((K, N), DType.Float32)])
+    if WARM_ONLY:
+        from jaxjs_hip.kernelgen import generate
+        from jaxjs_hip.runtime import compile_source
+        for k in prog.kernels:
+            for src in generate(k).sources:
+                compile_source(src)
+        pytest.skip("warm-up run: compiled only")
+    be = backend()
+    info = be.prepareKernelSync(prog.kernels[0]).data.ks.info
+    assert info.get("fused_fold") and info["splitk"] > 1, info
+
+    def operands(r):
+        rng = np.random.default_rng(300 + r)
+        return [rng.uniform(-1, 1, (M, K)).astype(np.float32), rng.uniform(-1, 1, (K, N)).astype(np.float32)]
+    _check_program(prog, operands)
