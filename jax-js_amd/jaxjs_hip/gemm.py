@@ -78,10 +78,12 @@ def choose_tile(g: dict) -> Dict[str, int]:
         # stages (128 KiB: twice the bytes in flight per workgroup; 2048^3 20.7 -> 19.6 us, 128x14336x4096 35.2 -> 27.4 us).
         if not both_k:
             tile.update(BK=64, STAGES=4)
-        # Half the CUs or fewer would get a workgroup: cut the k axis in two (128x14336x4096: 27.4 -> 26.0 us with
-        # the fold launch included; four slices cost more in partial sums than they gain)
+        # Half the CUs or fewer would get a workgroup: cut the k axis in two, four when a quarter or fewer would, the
+        # slices folded inside the launch by the last one to arrive (128x14336x4096: 27.4 -> 26.0 us with a fold
+        # launch, 24.7 folded in the launch; 128x4096x4096: 16.1 us in two slices, 13.9 in four; with 112 tiles four
+        # slices cost more in partial sums than they gain).
         if tiles(128, 128) * 2 <= CU and g["K"] >= 2048 and g["K"] % 128 == 0:
-            tile["SPLITK"] = 2
+            tile.update(SPLITK=4 if tiles(128, 128) * 4 <= CU and g["K"] >= 4096 and g["K"] % 256 == 0 else 2, FUSEK=1)
     return tile
 
 
@@ -309,7 +311,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     if split > 1:
         KS = K_full // split
         g = dict(g, K=KS, a_k0=KS, b_k0=KS)
-        fusek = split if tile.get("FUSEK", 0) and g["dtype"] == DType.Float32 else 0
+        fusek = split if tile.get("FUSEK", 0) else 0
         if not fusek:
             out_t = "float"
 
@@ -557,7 +559,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         # all rows loses a third).  Nontemporal C stores only for the f32 partials of a k split, where a wave's store
         # covers whole 128-byte lines (128x14336x4096: 26.1 -> 25.3 us): with 2-byte outputs they gain nothing once the
         # walk is in groups of 4 and the half-line writes cost a third more HBM write traffic (WRITE_SIZE 132 -> 176 MiB).
-        sched.update(GROUP_M=int(tile.get("GM", 4)), NT_STORE=int(tile.get("NTS", 1 if split > 1 else 0)))
+        sched.update(GROUP_M=int(tile.get("GM", 4)), NT_STORE=int(tile.get("NTS", 1 if split > 1 and not fusek else 0)), FUSEK=fusek)
         sched["RING"] = ring = tile.get("RING", ring_default)
         if ring and (ring != 5 or BM != BN or not sched["PIPE"]):
             raise ValueError("the unit ring is five units of a square block tile under the phase-pipelined loop")
@@ -597,6 +599,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         A_K0=g["a_k0"], A_SK1=g["a_sk1"], B_K0=g["b_k0"], B_SK1=g["b_sk1"],
         C_SM=g["c_sm"], C_SN=g["c_sn"], EPILOGUE_ARGS=epi_args))
     tiles = -(-g["M"] // BM) * -(-g["N"] // BN) * nbatch
+    if fusek and g["dtype"] == DType.Float16 and not dlds:
+        raise ValueError("an in-launch fold of a k split needs the direct-to-LDS f16 template or the f32 template")
     out_args = [("out", 0), ("scratch", 0), ("scratch", 1)] if fusek else [("scratch", 0) if split > 1 else ("out", 0)]
     step = LaunchStep(name, (tiles, split, 1), (nthreads, 1, 1), 0, [("in", i) for i in range(kernel.nargs)] + out_args)
     need = _min_bytes(t.epilogue)

@@ -165,8 +165,8 @@ def test_gemm_8192_cubed_every_element_exact():
 SWEEP = [
     (DType.Float16, 2048, 2048, 2048, dict(BM=128, BN=128, BK=64, stages=4, tiles=256, splitk=1, direct_lds=True)),
     (DType.Float16, 4096, 4096, 4096, dict(BM=256, BN=256, BK=32, tiles=256, splitk=1, direct_lds=True)),
-    # fewer tiles than CUs: the k axis is cut over blockIdx.y, f32 partials in scratch, fold kernel applies the epilogue
-    (DType.Float16, 128, 14336, 4096, dict(BM=128, BN=128, BK=64, stages=4, tiles=112, splitk=2, direct_lds=True)),
+    # fewer tiles than CUs: the k axis is cut over blockIdx.y, f32 partials in scratch, folded inside the launch
+    (DType.Float16, 128, 14336, 4096, dict(BM=128, BN=128, BK=64, stages=4, tiles=112, splitk=2, direct_lds=True, fused_fold=True)),
     # f32 k splits are folded inside the launch by the last slice to arrive at the tile's counter
     (DType.Float32, 1024, 1024, 1024, dict(BM=128, BN=64, BK=32, tiles=128, splitk=4, fused_fold=True)),
     (DType.Float32, 2048, 2048, 2048, dict(BM=128, BN=64, BK=32, tiles=512, splitk=1)),
@@ -193,6 +193,43 @@ def test_gemm_sweep_shapes(dt, M, N, K, want):
     if len(rows) > 128:
         rows = rows[::len(rows) // 96]
     _check(got.reshape(M, N)[rows], A[rows], B, K, out_f16=(dt == DType.Float16))
+
+
+@pytest.mark.parametrize("M,N,K,split,bt", [(384, 640, 1024, 4, False), (128, 1792, 2048, 2, False), (256, 256, 4096, 8, True), (640, 128, 512, 2, True)])
+def test_gemm_f16_in_launch_fold_matches_the_fold_kernel_bit_for_bit(M, N, K, split, bt):
+    """The same check for the direct-to-LDS f16 template (15, 14, 4 and 5 tiles; B stored [K,N] and [N,K])."""
+    from gpu_util import WARM_ONLY, backend
+    k = matmulKernel(M, N, K, DType.Float16, b_transposed=bt)
+    tiles = dict(BM=128, BN=128, SPLITK=split)
+    opts = [dict(gemm_tile=tuple(sorted(dict(tiles, FUSEK=f).items()))) for f in (0, 1)]
+    if WARM_ONLY:
+        from jaxjs_hip.kernelgen import generate
+        from jaxjs_hip.runtime import compile_source
+        from jaxjs_hip.tuner import tuneHip
+        for o in opts:
+            for src in generate(k, tune=tuneHip(k, **o)).sources:
+                compile_source(src)
+        pytest.skip("warm-up run: compiled only")
+    be = backend()
+    A = RNG.uniform(-1, 1, (M, K)).astype(np.float16)
+    B = RNG.uniform(-1, 1, (K, N)).astype(np.float16)
+    Bs = np.ascontiguousarray(B.T) if bt else B
+    sa, sb, so = be.malloc(A.nbytes, A.tobytes()), be.malloc(Bs.nbytes, Bs.tobytes()), be.malloc(k.bytes)
+    try:
+        two, one = (be.prepareKernelSync(k, **o) for o in opts)
+        assert two.data.ks.klass == "gemm+fold" and one.data.ks.klass == "gemm" and one.data.ks.info["fused_fold"]
+        assert one.data.ks.info["direct_lds"] and one.data.ks.info["splitk"] == split and len(one.data.ks.steps) == 1
+        be.dispatch(two, [sa, sb], [so])
+        want = np.frombuffer(be.readSync(so), np.float16).copy()
+        _check(want.reshape(M, N), A, B, K)
+        for it in range(40):
+            be.dispatch(one, [sa, sb], [so])
+            if it % 8 == 7 or it < 2:
+                got = np.frombuffer(be.readSync(so), np.float16)
+                np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16), err_msg=f"launch {it}")
+    finally:
+        for s_ in (sa, sb, so):
+            be.decRef(s_)
 
 
 @pytest.mark.parametrize("M,N,K,split", [(384, 320, 1024, 4), (1024, 1024, 1024, 4), (128, 192, 2048, 8), (640, 64, 512, 2)])

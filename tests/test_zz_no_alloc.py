@@ -51,7 +51,8 @@ def test_static_scratch_matches_allocated_scratch_twice_in_a_row():
         A = rng.uniform(-1, 1, (M, K)).astype(np.float16)
         B = rng.uniform(-1, 1, (K, N)).astype(np.float16)
         k = matmulKernel(M, N, K, DType.Float16)
-        a, b, ks = _both_ways(be, k, [A, B], gemm_tile=(("SPLITK", 4),))
+        # the fold of the slices by a second kernel: the in-launch fold keeps counters in a second scratch buffer
+        a, b, ks = _both_ways(be, k, [A, B], gemm_tile=(("FUSEK", 0), ("SPLITK", 4)))
         assert ks.klass == "gemm+fold" and ks.info["splitk"] == 4
         np.testing.assert_array_equal(a, b)
         ref = A.astype(np.float64) @ B.astype(np.float64)
@@ -81,6 +82,24 @@ def test_static_scratch_rejects_oversized_requests_without_launching():
     try:
         with pytest.raises(Exception, match="static scratch"):
             be.dispatchStaticScratch(big, [a, b], [o])
+    finally:
+        for s in (a, b, o):
+            be.decRef(s)
+
+
+def test_static_scratch_refuses_executables_with_state_in_a_second_scratch_buffer():
+    """A k split folded inside the launch keeps per-tile arrival counters in a second scratch buffer that must start at
+    zero: one shared static buffer cannot serve it, and the host layer says so before anything is launched."""
+    if WARM_ONLY:
+        pytest.skip("warm-up run")
+    be = backend()
+    k = matmulKernel(1024, 1024, 1024, F32)
+    exe = be.prepareKernelSync(k)
+    assert exe.data.ks.info.get("fused_fold") and len(exe.data.ks.scratch_bytes) == 2
+    a, b, o = be.malloc(4 << 20), be.malloc(4 << 20), be.malloc(k.bytes)
+    try:
+        with pytest.raises(ValueError, match="several scratch buffers"):
+            be.dispatchStaticScratch(exe, [a, b], [o])
     finally:
         for s in (a, b, o):
             be.decRef(s)
