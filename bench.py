@@ -575,7 +575,8 @@ def main():
         extra["c5_gpt2_block_b8_l1024_f16"] = bench_program_gpt2(be, hostrand, timed)
         extra["c5_gpt2_block_b8_l1024_f16_fused_attention"] = bench_program_gpt2_fused(be, hostrand, timed)
 
-        # Convolution through the view algebra (no implicit-GEMM class yet: the kernel takes a generic reduce class).
+        # Convolution through the view algebra: the traced reduce Kernel is recognised as an implicit GEMM (f16 stride-1
+        # windows: image patch resident in LDS; f32: gather loaders).
         from jaxjs_hip import jit as J, library as Lb
         from jaxjs_hip.jit import ShapedArray
         for cdt, npdt, tag in ((DType.Float16, np.float16, "f16"), (DType.Float32, np.float32, "f32")):
