@@ -96,9 +96,10 @@ def match_conv(oexp: AluExp, extent: int, K: int, batch: list) -> Optional[dict]
         return None
     idx, ok = first
     # Probes.  The window width is where consecutive taps stop being consecutive elements, and what the next window
-    # row advances by is the image width; the output width is where consecutive positions stop being consecutive --
-    # or, when output and image are equally wide (the index is then linear in the position), whichever divisor of
-    # the position count makes the padding mask come out right.  Every candidate is checked against the whole table.
+    # row advances by is the image width (a window of one row says nothing about it: every divisor of the plane is
+    # tried); the output width is where consecutive positions stop being consecutive -- or, when output and image are
+    # equally wide (the index is then linear in the position), whichever divisor of the position count makes the
+    # padding mask come out right.  Every candidate is checked against the whole table.
     d_tap = np.diff(idx[0, :])
     tbreaks = np.nonzero(d_tap != 1)[0]
     KW = int(tbreaks[0]) + 1 if len(tbreaks) else T
@@ -107,34 +108,36 @@ def match_conv(oexp: AluExp, extent: int, K: int, batch: list) -> Optional[dict]
     KH = T // KW
     d_row = np.diff(idx[:, 0])
     breaks = np.nonzero(d_row != 1)[0]
-    if KH > 1:
-        W = int(idx[0, KW] - idx[0, 0])
-    elif len(breaks):
-        W = int(idx[int(breaks[0]) + 1, 0] - idx[0, 0])
-    else:
-        W = cs
-    if W <= 0 or cs % W:
-        return None
-    H = cs // W
     base = int(idx[0, 0])  # = -(PH * W + PW): position 0 with tap 0 sits PH rows and PW columns before the plane
     if base > 0:
         return None
-    PH, PW = (-base) // W, (-base) % W
-    candidates = [int(breaks[0]) + 1] if len(breaks) else [W] + [d for d in range(extent, 0, -1) if extent % d == 0 and d != W]
+    if KH > 1:
+        widths = [int(idx[0, KW] - idx[0, 0])]
+    else:
+        widths = [d for d in range(cs, 0, -1) if cs % d == 0]
+    ky, kx = taps // KW, taps % KW
     found = None
-    for OW in candidates:
-        if extent % OW:
+    for W in widths:
+        if W <= 0 or cs % W:
             continue
-        oy, ox = rows // OW, rows % OW
-        ky, kx = taps // KW, taps % KW
-        iy, ix = oy + ky - PH, ox + kx - PW
-        valid = (iy >= 0) & (iy < H) & (ix >= 0) & (ix < W)
-        model = iy * W + ix
-        if np.array_equal(ok, valid) and np.array_equal(idx[valid], model[valid]) and (cond is not None or valid.all()):
-            found = OW
+        H = cs // W
+        PH, PW = (-base) // W, (-base) % W
+        candidates = [int(breaks[0]) + 1] if len(breaks) else [W] + [d for d in range(extent, 0, -1) if extent % d == 0 and d != W]
+        for OW in candidates:
+            if extent % OW:
+                continue
+            oy, ox = rows // OW, rows % OW
+            iy, ix = oy + ky - PH, ox + kx - PW
+            valid = (iy >= 0) & (iy < H) & (ix >= 0) & (ix < W)
+            model = iy * W + ix
+            if np.array_equal(ok, valid) and np.array_equal(idx[valid], model[valid]) and (cond is not None or valid.all()):
+                found = (W, H, PH, PW, OW)
+                break
+        if found:
             break
     if found is None:
         return None
+    W, H, PH, PW, found = found
     OW, OH = found, extent // found
     SB = 0
     if nb > 1:

@@ -241,6 +241,14 @@ F16_CONV_CASES = [
     dict(x=(1, 16, 56, 56), w=(256, 16, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),     # 128-channel tiles
     dict(x=(2, 128, 14, 12), w=(64, 128, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),    # several channel slabs
     dict(x=(2, 16, 64), w=(64, 16, 3), strides=[1], padding="SAME", loader="patch"),                # one spatial dim
+    dict(x=(1, 16, 16, 16), w=(64, 16, 7, 7), strides=[1, 1], padding="SAME", loader="patch"),      # shifts of 3: two dwords from each neighbour
+    dict(x=(2, 16, 12, 16), w=(64, 16, 1, 3), strides=[1, 1], padding="SAME", loader="patch"),      # one window row
+    dict(x=(2, 16, 12, 16), w=(64, 16, 3, 1), strides=[1, 1], padding="SAME", loader="patch"),      # one window column: no shifted copies
+    dict(x=(1, 48, 8, 8), w=(64, 48, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),        # three slabs; one fill vector per row
+    dict(x=(1, 256, 8, 8), w=(64, 256, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),      # sixteen slabs: the paired loop
+    dict(x=(1, 16, 8, 112), w=(64, 16, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),      # 14 fill vectors per row, 4 rows per wave
+    dict(x=(8, 16, 8, 4), w=(64, 16, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),        # one tile per image, mostly padding
+    dict(x=(1, 16, 12, 32), w=(64, 16, 5, 5), strides=[1, 1], padding="SAME", loader="patch"),      # shifts of 2 to either side
     dict(x=(2, 16, 16, 16), w=(32, 16, 3, 3), strides=[1, 1], padding="SAME", loader="rows8"),      # 32 output channels: generic loaders
     dict(x=(2, 16, 32, 32), w=(64, 16, 3, 3), strides=[2, 2], padding="SAME", loader="element"),    # strided: generic loaders
 ]
