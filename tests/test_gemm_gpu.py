@@ -106,6 +106,56 @@ def test_gemm_fused_epilogue_bias_relu_f32_out():
     np.testing.assert_allclose(got.reshape(M, N), ref, rtol=1e-4, atol=1e-4)
 
 
+def _random_gemm_cases():
+    """Seeded shapes around the tile chooser's decision points: few tiles with a long k axis (k splits folded inside
+    the launch), tile counts around the CU count, short k, ragged extents; f16 (NN and NT) and f32, with a row-bias
+    + ReLU epilogue on every other case (the fold applies the caller's epilogue, loads included)."""
+    rng = np.random.default_rng(2024)
+    cases = []
+    for i in range(36):
+        dt = DType.Float32 if i % 3 == 2 else DType.Float16
+        if i % 4 == 0:  # small grids, long k: split candidates
+            M, N, K = int(rng.choice([128, 256, 384])), int(rng.choice([128, 256, 512, 1024])), int(rng.choice([2048, 4096, 8192]))
+        elif i % 4 == 1:  # around one tile per CU
+            M, N, K = int(rng.choice([1024, 2048, 1536])), int(rng.choice([2048, 1024, 2560])), int(rng.choice([256, 512, 1024]))
+        elif i % 4 == 2:  # ragged
+            M, N, K = int(rng.integers(33, 700)), int(rng.integers(5, 90)) * 8, int(rng.integers(3, 60)) * 8
+        else:  # short k, many tiles
+            M, N, K = int(rng.choice([4096, 2048])), int(rng.choice([512, 768, 2304])), int(rng.choice([64, 96, 192]))
+        cases.append((dt, M, N, K, bool(i % 2 and dt == DType.Float16 and i % 4 != 2), bool(i % 2 == 0)))
+    return cases
+
+
+@pytest.mark.parametrize("dt,M,N,K,bt,bias", _random_gemm_cases(), ids=lambda v: v.value if isinstance(v, DType) else str(int(v)) if not isinstance(v, bool) else ("T" if v else "F"))
+def test_gemm_random_shapes_with_and_without_epilogue(dt, M, N, K, bt, bias):
+    npdt = np.float16 if dt == DType.Float16 else np.float32
+    A = RNG.uniform(-1, 1, (M, K)).astype(npdt)
+    B = RNG.uniform(-1, 1, (K, N)).astype(npdt)
+    base = matmulKernel(M, N, K, dt, b_transposed=bt)
+    bufs = [A, np.ascontiguousarray(B.T) if bt else B]
+    if bias:
+        bv = RNG.uniform(-1, 1, N).astype(np.float32)
+        acc = AluVar.acc(DType.Float32)
+        n_idx = unravelAlu([M, N], AluVar.gidx)[1]
+        b = AluExp.globalView(DType.Float32, 2, ShapeTracker.fromShape([N]), [n_idx])
+        k = Kernel(3, M * N, base.exp_raw, Reduction(DType.Float32, AluOp.Add, K, AluExp.max(AluExp.add(acc, b), AluExp.f32(0))))
+        bufs.append(bv)
+    else:
+        k = base
+    got, ks = device_run(k, bufs)
+    assert ks.klass.startswith("gemm"), (ks.klass, ks.info)
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    mag = np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)
+    bound = 2 * K * np.finfo(np.float32).eps * mag
+    if bias:
+        ref = np.maximum(ref + bv, 0)
+        bound = bound + 4 * np.finfo(np.float32).eps * (np.abs(ref) + 1)
+    elif dt == DType.Float16:
+        bound = bound + np.abs(ref) * 2.0**-11 + 2.0**-24
+    err = np.abs(got.astype(np.float64).reshape(ref.shape) - ref)
+    assert np.all(err <= bound), f"max excess {np.max(err - bound)} with {ks.info}"
+
+
 def _tile_row_sample(n, bm=256):
     """Three rows of every block-tile row: the first, one in the second 128-row wave half, the last."""
     return sorted({t * bm + r for t in range(n // bm) for r in (0, bm // 2 + 3, bm - 1)})
