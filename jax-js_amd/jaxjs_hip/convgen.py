@@ -179,7 +179,7 @@ def gen_conv(kernel, g: dict, oexp: AluExp, numerics: str, name: str, params: st
     if cv is None:
         return None
     O, C, OW = g["M"], cv["C"], cv["OW"]
-    if OW % 4 or C % 16 or O % 64 or g["c_sn"] != 1 and False:
+    if OW % 4 or C % 16 or O % 64:  # 8-byte aligned row offsets in LDS, whole MFMA k steps, whole 64-channel tiles
         return None
     BM = int(tile.get("CBM", 128 if O % 128 == 0 and O >= 256 else 64))
     # 256 positions per tile (wave tile 32 x 128: four MFMAs per A fragment) unless the image is smaller than that
