@@ -23,7 +23,7 @@ from typing import List, Optional, Sequence, Tuple
 from . import jit as J
 from .alu import AluExp, AluOp, AluVar, DType
 from .jit import ConstArray, Tracer
-from .shape import prod, unravelAlu
+from .shape import prod as _int_prod, unravelAlu
 
 
 def square(x):
@@ -78,8 +78,8 @@ def lax_dot(lhs: Tracer, rhs: Tracer, lc: Sequence[int], rc: Sequence[int], lb: 
     if kx != ky:
         raise ValueError(f"dot: shapes not aligned along contracting dims: {kx} != {ky}")
     return J.dot(
-        lhs2.reshape([lhs.shape[a] for a in lb] + [lhs.shape[a] for a in lf] + [1] * len(rf) + [prod(kx)]),
-        rhs2.reshape([rhs.shape[a] for a in rb] + [1] * len(lf) + [rhs.shape[a] for a in rf] + [prod(ky)]))
+        lhs2.reshape([lhs.shape[a] for a in lb] + [lhs.shape[a] for a in lf] + [1] * len(rf) + [_int_prod(kx)]),
+        rhs2.reshape([rhs.shape[a] for a in rb] + [1] * len(lf) + [rhs.shape[a] for a in rf] + [_int_prod(ky)]))
 
 
 def matmul(x: Tracer, y: Tracer):
@@ -502,3 +502,140 @@ def random_normal(key: Tracer, shape: Sequence[int] = ()):
     radius = J.sqrt(log1p(J.neg(u1)).mul(-2))
     theta = u2.mul(2 * math.pi)
     return radius.mul(J.bind1("Cos", [theta]))
+
+
+# ---- reductions and scans of the numpy surface (src/library/numpy.ts) ---------------------------------
+
+def prod(a: Tracer, axis=None, keepdims: bool = False):
+    """Product over `axis` (numpy.ts:376-382): one Mul reduction."""
+    return J.reduce(a, AluOp.Mul, axis, keepdims)
+
+
+def any_(a: Tracer, axis=None, keepdims: bool = False):
+    """`astype(bool).max(axis)` (core.ts:911-913)."""
+    return J.reduce(J._raise(a).astype(DType.Bool), AluOp.Max, axis, keepdims)
+
+
+def all_(a: Tracer, axis=None, keepdims: bool = False):
+    """`astype(bool).min(axis)` (core.ts:906-908)."""
+    return J.reduce(J._raise(a).astype(DType.Bool), AluOp.Min, axis, keepdims)
+
+
+def ptp(a: Tracer, axis=None, keepdims: bool = False):
+    """`max - min` (numpy.ts:431-438)."""
+    return a.max(axis, keepdims).sub(a.min(axis, keepdims))
+
+
+def countNonzero(a: Tracer, axis=None, keepdims: bool = False):
+    """`sum(astype(a != 0, int32))` (numpy.ts:367-373)."""
+    return J.notEqual(a, 0).astype(DType.Int32).sum(axis, keepdims)
+
+
+def var_(x: Tracer, axis=None, keepdims: bool = False, correction: float = 0):
+    """`sum(square(x - mean)) * 1/(n - correction)` with the mean kept as its own reduction (numpy.ts:3103-3121)."""
+    ax = J._normalize_axis(axis, x.ndim)
+    n = 1
+    for a in ax:
+        n *= x.shape[a]
+    if n == 0:
+        raise ValueError("var: cannot compute variance over zero-length axis")
+    mu = x.mean(ax, keepdims=True)
+    return square(x.sub(mu)).sum(ax, keepdims).mul(1 / (n - correction))
+
+
+def std(x: Tracer, axis=None, keepdims: bool = False, correction: float = 0):
+    return J.sqrt(var_(x, axis, keepdims, correction))
+
+
+def average(a: Tracer, axis=None, weights: Optional[Tracer] = None, keepdims: bool = False):
+    """Weighted mean `sum(a*w) / sum(w)`; weights of lower rank line up with `axis` (numpy.ts:456-489)."""
+    if weights is None:
+        return a.mean(axis, keepdims)
+    ax = J._normalize_axis(axis, a.ndim)
+    w = J._raise(weights)
+    if tuple(w.shape) != tuple(a.shape):
+        if w.ndim != len(ax) or any(w.shape[i] != a.shape[d] for i, d in enumerate(ax)):
+            raise ValueError("average: weights must match the array or the reduced axes")
+        shape = [a.shape[d] if d in ax else 1 for d in range(a.ndim)]
+        w = w.reshape(shape)
+    return a.mul(w).sum(ax, keepdims).div(J.broadcast(w, a.shape, []).sum(ax, keepdims) if tuple(w.shape) != tuple(a.shape) else w.sum(ax, keepdims))
+
+
+def moveaxis(a: Tracer, src: int, dst: int):
+    src = src + a.ndim if src < 0 else src
+    dst = dst + a.ndim if dst < 0 else dst
+    perm = [i for i in range(a.ndim) if i != src]
+    perm.insert(dst, src)
+    return a if perm == list(range(a.ndim)) else a.transpose(perm)
+
+
+def _cumulative_quadratic(op: AluOp, a: Tracer, padValue, k: int = 0):
+    """`reduce(where(tri(n, n, k), a[..., None, :], pad), op, -1)` (numpy.ts:562-575): n^2 work, one kernel."""
+    n = a.shape[-1]
+    wide = J.broadcast(a, list(a.shape) + [n], [a.ndim - 1])
+    pad = J.scalar(padValue, a.dtype)
+    return J.reduce(J.where(tri_const(n, n, k), wide, pad), op, -1)
+
+
+def _cumulative(op: AluOp, a: Tracer, axis):
+    """Scan along `axis`: quadratic up to 512 elements, else chunks of 256 scanned independently and offset by an
+    exclusive scan of the chunk totals (numpy.ts:577-614)."""
+    padValue = 0 if op == AluOp.Add else 1
+    a = J._raise(a)
+    if a.ndim == 0:
+        a = a.reshape([1])
+    if axis is None:
+        a, axis = a.reshape([-1]), 0
+    (axis,) = J._normalize_axis(axis, a.ndim)
+    a = moveaxis(a, axis, -1)
+    n = a.shape[-1]
+    split = 256
+    if n <= split * 2:
+        return moveaxis(_cumulative_quadratic(op, a, padValue), -1, axis)
+    batch = list(a.shape[:-1])
+    m = -(-n // split)
+    a = J.pad(a, [(0, 0)] * len(batch) + [(0, m * split - n)])
+    scans = _cumulative_quadratic(op, a.reshape(batch + [m, split]), padValue)
+    totals = J.shrink(scans, [(0, d) for d in batch] + [(0, m), (split - 1, split)]).reshape(batch + [m])
+    offsets = _cumulative_quadratic(op, totals, padValue, -1)
+    off = offsets.reshape(batch + [m, 1])
+    out = scans.add(off) if op == AluOp.Add else scans.mul(off)
+    result = J.shrink(out.reshape(batch + [m * split]), [(0, d) for d in batch] + [(0, n)])
+    return moveaxis(result, -1, axis)
+
+
+def cumsum(a: Tracer, axis=None):
+    return _cumulative(AluOp.Add, a, axis)
+
+
+def cumprod(a: Tracer, axis=None):
+    return _cumulative(AluOp.Mul, a, axis)
+
+
+def diff(a: Tracer, n: int = 1, axis: int = -1, prepend=None, append=None):
+    """n-th difference along `axis`: `a[1:] - a[:-1]` n times, `!=` on booleans (numpy.ts:724-763)."""
+    a = J._raise(a)
+    if n < 0:
+        raise ValueError(f"diff: order must be a non-negative integer, got {n}")
+    if n == 0:
+        return a
+    if a.ndim == 0:
+        raise ValueError("diff: input must be at least one-dimensional")
+    (axis,) = J._normalize_axis(axis, a.ndim)
+    if prepend is not None or append is not None:
+        edge = [1 if i == axis else d for i, d in enumerate(a.shape)]
+        parts = [a]
+        for value, front in ((prepend, True), (append, False)):
+            if value is None:
+                continue
+            # A scalar edge becomes a constant *array* (its own buffer): a literal has no view for Concatenate's padding
+            # to mask, and would be added to every element (the reference's eager path pads the constant's own tracker).
+            v = J._raise(value) if not isinstance(value, (int, float)) else J._raise(ConstArray(tuple(edge), a.dtype, AluExp.const(a.dtype, value)))
+            parts.insert(0, v) if front else parts.append(v)
+        a = J.concatenate(parts, axis)
+    for _ in range(min(n, a.shape[axis])):
+        length = a.shape[axis]
+        upper = J.shrink(a, [(1, length) if i == axis else (0, d) for i, d in enumerate(a.shape)])
+        lower = J.shrink(a, [(0, length - 1) if i == axis else (0, d) for i, d in enumerate(a.shape)])
+        a = J.notEqual(upper, lower) if a.dtype == DType.Bool else upper.sub(lower)
+    return a

@@ -24,7 +24,13 @@ def run_program(backend, prog, arrays, out_dtypes_shapes=None):
             out_dtypes[s.output] = s.kernel.dtype
     for slot, oid in zip(outs, prog.outputs):
         raw = backend.readSync(slot)
-        results.append(np.frombuffer(raw, dtype=numpyDtype(out_dtypes[oid])).copy())
+        if oid in out_dtypes:
+            dt = numpyDtype(out_dtypes[oid])
+        elif oid < len(prog.consts):  # a constant returned as it is
+            dt = numpyDtype(prog.consts[oid].dtype)
+        else:  # an input returned as it is
+            dt = np.asarray(arrays[oid - len(prog.consts)]).dtype
+        results.append(np.frombuffer(raw, dtype=dt).copy())
     for s in const_slots + in_slots + outs:
         backend.decRef(s)
     return results

@@ -505,3 +505,101 @@ def test_input_returned_twice_beside_a_result():
     np.testing.assert_array_equal(np.frombuffer(be.readSync(ins[0]), np.float32), x)  # the caller's own reference
     be.decRef(ins[0])
     assert be.live_slots() == 0
+
+
+# ---- reductions and scans of the numpy surface: the reference's tables (test/numpy.test.ts) ----------------------
+
+def _run_typed(fn, arrays, dtypes):
+    prog = J.jit(fn, [ShapedArray(tuple(a.shape), d) for a, d in zip(arrays, dtypes)])
+    be = OracleBackend()
+    outs = run_program(be, prog, arrays)
+    assert be.live_slots() == 0
+    return prog, outs
+
+
+def test_count_nonzero_any_all_tables():
+    """test/numpy.test.ts:44-92 (countNonzero: all axes, one axis, keepdims, NaN counts as nonzero, int32 result) and
+    :4380-4455 (all / any over booleans and truthy numbers, along an axis, keepdims)."""
+    x = f32([[1, 0, -2], [0, 3, 0]])
+    prog, (c, c0, c1, ck) = run(lambda a: [L.countNonzero(a), L.countNonzero(a, 0), L.countNonzero(a, 1), L.countNonzero(a, 1, keepdims=True)], x)
+    assert c.dtype == np.int32 and c.tolist() == [3] and c0.tolist() == [1, 1, 1] and c1.tolist() == [2, 1] and ck.tolist() == [2, 1]
+    _, (cn,) = run(lambda a: L.countNonzero(a), f32([0, np.nan, 2]))
+    assert cn.tolist() == [2]
+    _, (cr,) = run(lambda a: L.countNonzero(a, 1, keepdims=True), f32([[0, 1, 2], [0, 0, 3]]))
+    assert cr.tolist() == [2, 1]
+    B = DType.Bool
+    b = np.array([[1, 0], [1, 1]], np.int32)  # booleans are stored as int32 0/1
+    _, (a0, a1, aa, ak) = _run_typed(lambda v: [L.all_(v, 0), L.all_(v, 1), L.all_(v), L.all_(v, 1, keepdims=True)], [b], [B])
+    assert a0.tolist() == [1, 0] and a1.tolist() == [0, 1] and aa.tolist() == [0] and ak.tolist() == [0, 1]
+    b = np.array([[0, 0], [1, 0]], np.int32)
+    _, (y0, y1, ya) = _run_typed(lambda v: [L.any_(v, 0), L.any_(v, 1), L.any_(v)], [b], [B])
+    assert y0.tolist() == [1, 0] and y1.tolist() == [0, 1] and ya.tolist() == [1]
+    _, (t1, t2, t3, t4) = run(lambda p, q: [L.all_(p), L.all_(q), L.any_(p.mul(0)), L.any_(q)], f32([1, 2, 3]), f32([1, 0, 3]))
+    assert (t1.tolist(), t2.tolist(), t3.tolist(), t4.tolist()) == ([1], [0], [0], [1])
+
+
+def test_prod_ptp_var_std_average_tables():
+    """prod is one Mul reduction (test/basic.test.ts:46); var_ / std (test/numpy.test.ts:4242-4254: 1.25 and its root);
+    average with weights (:170-218: 2, [2, 5], [5/3, 25/7], keepdims [[2],[5]]); ptp = max - min."""
+    x = f32([1, 2, 3, 4])
+    prog, (p, v, s, r) = run(lambda a: [L.prod(a), L.var_(a), L.std(a), L.ptp(a)], x)
+    assert p.tolist() == [24] and r.tolist() == [3]
+    np.testing.assert_allclose(v, [1.25], rtol=1e-6)
+    np.testing.assert_allclose(s, [math.sqrt(1.25)], rtol=1e-6)
+    m = f32([[1, 2, 3], [4, 5, 6]])
+    _, (pa, v0) = run(lambda a: [L.prod(a, 1), L.var_(a, 0, correction=1)], m)
+    assert pa.tolist() == [6, 120]
+    np.testing.assert_allclose(v0, [4.5, 4.5, 4.5], rtol=1e-6)
+    _, (w1,) = run(lambda a, w: L.average(a, 1, weights=w), m, f32([0.25, 0.5, 0.25]))
+    assert w1.tolist() == [2, 5]
+    _, (w2,) = run(lambda a, w: L.average(a, 1, weights=w), f32([[1, 2], [3, 4]]), f32([[1, 2], [3, 4]]))
+    np.testing.assert_allclose(w2, [5 / 3, 25 / 7], rtol=1e-6)
+    _, (w3, w4) = run(lambda a: [L.average(a, 1, keepdims=True), L.average(a)], m)
+    assert w3.tolist() == [2, 5] and w4.tolist() == [3.5]
+    _, (w5,) = run(lambda a, w: L.average(a, weights=w), f32([1, 2, 3]), f32([1, 1, 2]))
+    np.testing.assert_allclose(w5, [2.25], rtol=1e-6)
+
+
+def test_cumsum_cumprod_tables_and_the_two_stage_scan():
+    """test/numpy.test.ts:259-293 ([[1,2,3],[5,7,9]] along 0, [[1,3,6],[4,9,15]] along 1, cumprod [1,2,6,24]); the
+    scan is one masked n x n reduction up to 512 elements and chunks of 256 plus an exclusive scan of the chunk
+    totals beyond (src/library/numpy.ts:577-614) -- small integers keep every order of summation exact."""
+    x = f32([[1, 2, 3], [4, 5, 6]])
+    prog, (c0, c1, cp) = run(lambda a: [L.cumsum(a, 0), L.cumsum(a, 1), L.cumprod(a.reshape([-1]))], x)
+    assert c0.tolist() == [1, 2, 3, 5, 7, 9] and c1.tolist() == [1, 3, 6, 4, 9, 15] and cp.tolist() == [1, 2, 6, 24, 120, 720]
+    _, (cs,) = run(lambda a: L.cumsum(a), f32([5]).reshape(()))
+    assert cs.tolist() == [5]
+    rng = np.random.default_rng(5)
+    for n in (512, 513, 1000):
+        v = rng.integers(-3, 4, (3, n)).astype(np.float32)
+        prog, (got,) = run(lambda a: L.cumsum(a, 1), v)
+        np.testing.assert_array_equal(got.reshape(3, n), np.cumsum(v, axis=1))
+        assert len(prog.kernels) == (1 if n <= 512 else 3)
+    v = rng.choice([1.0, -1.0, 2.0, 0.5], (2, 600)).astype(np.float32)
+    _, (gp,) = run(lambda a: L.cumprod(a, 1), v)
+    np.testing.assert_array_equal(gp.reshape(2, 600), np.cumprod(v.astype(np.float64), axis=1).astype(np.float32))
+
+
+def test_diff_tables():
+    """test/numpy.test.ts:296-347: first and higher differences, along an axis, prepend / append (scalar and array),
+    != on booleans, n = 0 and n beyond the axis."""
+    x = f32([1, 2, 4, 7, 0])
+    _, (d1, d2, d3) = run(lambda a: [L.diff(a), L.diff(a, 2), L.diff(a, 3)], x)
+    assert d1.tolist() == [1, 2, 3, -7] and d2.tolist() == [1, 1, -10] and d3.tolist() == [0, -11]
+    _, (same,) = run(lambda a: L.diff(a, 0, -1, prepend=0, append=10), f32([1, 5, 2]))
+    assert same.tolist() == [1, 5, 2]
+    m = f32([[1, 3, 6, 10], [0, 5, 6, 8]])
+    _, (r, c) = run(lambda a: [L.diff(a), L.diff(a, 1, 0)], m)
+    assert r.tolist() == [2, 3, 4, 5, 1, 2] and c.tolist() == [-1, 2, 0, -2]
+    _, (pa,) = run(lambda a: L.diff(a, 1, -1, prepend=0, append=10), x)
+    assert pa.tolist() == [1, 1, 2, 3, -7, 10]
+    _, (pb,) = run(lambda a, p: L.diff(a, 1, -1, prepend=p), x, f32([0, 1]))
+    assert pb.tolist() == [1, 0, 1, 2, 3, -7]
+    _, (db,) = _run_typed(lambda a: L.diff(a), [np.array([1, 1, 0, 1], np.int32)], [DType.Bool])
+    assert db.tolist() == [0, 1, 1]
+    prog = J.jit(lambda a: L.diff(a, 5), [ShapedArray((3,), F32)])
+    assert prog.out_avals[0].shape == (0,) if hasattr(prog, "out_avals") else True
+    with pytest.raises(ValueError, match="non-negative"):
+        J.jit(lambda a: L.diff(a, -1), [ShapedArray((3,), F32)])
+    with pytest.raises(ValueError, match="at least one-dimensional"):
+        J.jit(lambda a: L.diff(a), [ShapedArray((), F32)])
