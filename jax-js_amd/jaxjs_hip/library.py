@@ -639,3 +639,144 @@ def diff(a: Tracer, n: int = 1, axis: int = -1, prepend=None, append=None):
         lower = J.shrink(a, [(0, length - 1) if i == axis else (0, d) for i, d in enumerate(a.shape)])
         a = J.notEqual(upper, lower) if a.dtype == DType.Bool else upper.sub(lower)
     return a
+
+
+# ---- views, products and predicates of the numpy surface -----------------------------------------------
+
+def swapaxes(a: Tracer, axis1: int, axis2: int):
+    perm = list(range(a.ndim))
+    perm[axis1], perm[axis2] = perm[axis2], perm[axis1]
+    return a.transpose(perm)
+
+
+def rot90(m: Tracer, k: int = 1, axes: Sequence[int] = (0, 1)):
+    """Rotation by k quarter turns in the plane of `axes`: flips and an axis swap, all views (numpy.ts rot90)."""
+    if len(axes) != 2:
+        raise ValueError("rot90: axes must contain exactly two axes")
+    a1, a2 = [ax + m.ndim if ax < 0 else ax for ax in axes]  # in the given order
+    if a1 == a2:
+        raise ValueError("rot90: axes must be different")
+    k = k % 4
+    if k == 0:
+        return m
+    if k == 1:
+        return swapaxes(J.flip(m, a2), a1, a2)
+    if k == 2:
+        return J.flip(m, [a1, a2])
+    return J.flip(swapaxes(m, a1, a2), a2)
+
+
+def roll(a: Tracer, shift, axis=None):
+    """Circular shift: split at n - shift and concatenate the two parts the other way round, per axis (numpy.ts roll)."""
+    if axis is None:
+        return roll(a.reshape([-1]), shift, 0).reshape(list(a.shape))
+    axes = [ax + a.ndim if ax < 0 else ax for ax in ([axis] if isinstance(axis, int) else list(axis))]  # in the given order
+    shifts = [shift] * len(axes) if isinstance(shift, int) else list(shift)
+    if len(shifts) != len(axes):
+        raise ValueError(f"roll: shift and axis must have the same length, got shift={shifts} and axis={axes}")
+    for s, ax in zip(shifts, axes):
+        n = a.shape[ax]
+        s1 = s % n
+        if s1:
+            head, tail = J.split(a, ax, [n - s1, s1])
+            a = J.concatenate([tail, head], ax)
+    return a
+
+
+def sign(x: Tracer):
+    """`where(x != 0, where(x < 0, -1, 1), 0)` (numpy.ts sign)."""
+    return J.where(J.notEqual(x, 0), J.where(J.less(x, 0), -1, 1), 0)
+
+
+def isnan(x: Tracer):
+    return J.notEqual(x, x)
+
+
+def isposinf(x: Tracer):
+    return J.equal(x, math.inf)
+
+
+def isneginf(x: Tracer):
+    return J.equal(x, -math.inf)
+
+
+def isinf(x: Tracer):
+    """Bool `+` is OR (numpy.ts isinf)."""
+    return J.add(isposinf(x), isneginf(x))
+
+
+def isfinite(x: Tracer):
+    """`!isnan & !isinf` spelt with the comparisons the IR has: x - x == 0 fails exactly for NaN and the infinities."""
+    return J.equal(x.sub(x), 0)
+
+
+def trapezoid(y: Tracer, x: Optional[Tracer] = None, dx=1.0, axis: int = -1):
+    """Trapezoidal rule: `sum((y[1:] + y[:-1]) * 0.5 * dx, -1)` after moving `axis` last (numpy.ts trapezoid).  `dx`
+    may be a number or an array aligned to the trailing axes of y; `x` gives sample points (1-D, or shaped like y's
+    trailing axes)."""
+    y = J._raise(y)
+    (ax,) = J._normalize_axis(axis, y.ndim)
+
+    def sl(a, d, lo, hi):
+        return J.shrink(a, [(lo if i == d else 0, (hi if hi > 0 else n + hi) if i == d else n) for i, n in enumerate(a.shape)])
+
+    if x is None:
+        if y.dtype not in (DType.Float32, DType.Float16, DType.Float64):
+            y = y.astype(DType.Float32)
+        if isinstance(dx, (int, float)):
+            spacing = dx
+        else:
+            spacing = J._raise(dx)
+            if spacing.ndim < y.ndim:
+                spacing = spacing.reshape([1] * (y.ndim - spacing.ndim) + list(spacing.shape))
+            spacing = moveaxis(spacing, axis, -1)
+    else:
+        x = J._raise(x)
+        dt = J.promoteTypes(y.dtype, x.dtype)
+        if dt not in (DType.Float32, DType.Float16, DType.Float64):
+            dt = DType.Float32
+        y, x = y.astype(dt), x.astype(dt)
+        xa = 0 if x.ndim == 1 else J._normalize_axis(axis, x.ndim)[0]
+        d = sl(x, xa, 1, x.shape[xa]).sub(sl(x, xa, 0, -1))
+        spacing = d if x.ndim == 1 else moveaxis(d, xa, -1)
+    y = moveaxis(y, ax, -1)
+    last = y.ndim - 1
+    avg = sl(y, last, 1, y.shape[last]).add(sl(y, last, 0, -1)).mul(0.5)
+    return avg.mul(spacing).sum(-1)
+
+
+def outer(x: Tracer, y: Tracer):
+    x, y = x.reshape([-1]), y.reshape([-1])
+    return J.mul(x.reshape([x.shape[0], 1]), y)
+
+
+def inner(x: Tracer, y: Tracer):
+    return lax_dot(x, y, [-1], [-1])
+
+
+def tensordot(x: Tracer, y: Tracer, axes=2):
+    if isinstance(axes, int):
+        axes = (list(range(-axes, 0)), list(range(axes)))
+    return lax_dot(x, y, list(axes[0]), list(axes[1]))
+
+
+def vdot(x: Tracer, y: Tracer):
+    return J.dot(x.reshape([-1]), y.reshape([-1]))
+
+
+def vecdot(x: Tracer, y: Tracer, axis: int = -1):
+    return J.dot(moveaxis(x, axis, -1), moveaxis(y, axis, -1))
+
+
+def matvec(x1: Tracer, x2: Tracer):
+    """`...mn,...n->...m` with broadcasting batch axes: one Dot of [..., m, n] against [..., 1, n]."""
+    if x1.ndim < 2 or x2.ndim < 1:
+        raise ValueError("matvec: x1 must be at least 2D and x2 at least 1D")
+    return J.dot(x1, x2.reshape(list(x2.shape[:-1]) + [1, x2.shape[-1]]))
+
+
+def vecmat(x1: Tracer, x2: Tracer):
+    """`...n,...nm->...m`: one Dot of [..., 1, n] against the matrix with its last two axes swapped."""
+    if x1.ndim < 1 or x2.ndim < 2:
+        raise ValueError("vecmat: x1 must be at least 1D and x2 at least 2D")
+    return J.dot(x1.reshape(list(x1.shape[:-1]) + [1, x1.shape[-1]]), swapaxes(x2, -1, -2))

@@ -603,3 +603,87 @@ def test_diff_tables():
         J.jit(lambda a: L.diff(a, -1), [ShapedArray((3,), F32)])
     with pytest.raises(ValueError, match="at least one-dimensional"):
         J.jit(lambda a: L.diff(a), [ShapedArray((), F32)])
+
+
+def test_flip_rot90_roll_tables():
+    """test/numpy.test.ts:1427-1500 (flip, rot90 incl. negative turns and other axes) and :3627-3678 (roll: flat,
+    per axis, several axes, shifts beyond the length, rolls of rolls): views and concatenations only."""
+    m = f32([[1, 2, 3], [4, 5, 6]])
+    _, (fa, f0, f1) = run(lambda a: [J.flip(a, None).mul(1), J.flip(a, 0).mul(1), J.flip(a, 1).mul(1)], m)
+    assert fa.tolist() == [6, 5, 4, 3, 2, 1] and f0.tolist() == [4, 5, 6, 1, 2, 3] and f1.tolist() == [3, 2, 1, 6, 5, 4]
+    _, (r1, rm, r2) = run(lambda a: [L.rot90(a).mul(1), L.rot90(a, -1).mul(1), L.rot90(a, 2).mul(1)], m)
+    assert r1.tolist() == [3, 6, 2, 5, 1, 4] and rm.tolist() == [4, 1, 5, 2, 6, 3] and r2.tolist() == [6, 5, 4, 3, 2, 1]
+    c = f32(np.arange(1, 9).reshape(2, 2, 2))
+    _, (r3,) = run(lambda a: L.rot90(a, 1, [1, 2]).mul(1), c)
+    assert r3.tolist() == [2, 4, 1, 3, 6, 8, 5, 7]
+    v = f32([1, 2, 3, 4, 5])
+    _, (o1, o2) = run(lambda a: [L.roll(a, 2), L.roll(a, 20).mul(1)], v)
+    assert o1.tolist() == [4, 5, 1, 2, 3] and o2.tolist() == [1, 2, 3, 4, 5]
+    _, (y1, y2, y3, y4) = run(lambda a: [L.roll(a, 1), L.roll(a, 1, 0), L.roll(a, -1, 1), L.roll(a, [2, 1], [1, 0])], m)
+    assert y1.tolist() == [6, 1, 2, 3, 4, 5] and y2.tolist() == [4, 5, 6, 1, 2, 3] and y3.tolist() == [2, 3, 1, 5, 6, 4] and y4.tolist() == [5, 6, 4, 2, 3, 1]
+    _, (rr,) = run(lambda a: L.roll(L.roll(a, 1, 0), 1, 1), f32(np.arange(1, 10).reshape(3, 3)))
+    assert rr.tolist() == [9, 7, 8, 3, 1, 2, 6, 4, 5]
+    with pytest.raises(ValueError):
+        J.jit(lambda a: L.rot90(a, 1, [0, 0]), [ShapedArray((2, 2), F32)])
+
+
+def test_sign_and_float_class_predicates():
+    """test/numpy.test.ts:2425-2431 (sign), :4295-4303 (isnan / isinf / isfinite / isneginf / isposinf on
+    [NaN, Inf, -Inf, 1])."""
+    _, (s,) = run(lambda a: L.sign(a), f32([-10, 0, 5]))
+    assert s.tolist() == [-1, 0, 1]
+    x = f32([np.nan, np.inf, -np.inf, 1])
+    _, (n, i, f, ni, pi) = run(lambda a: [L.isnan(a), L.isinf(a), L.isfinite(a), L.isneginf(a), L.isposinf(a)], x)
+    assert n.tolist() == [1, 0, 0, 0] and i.tolist() == [0, 1, 1, 0] and f.tolist() == [0, 0, 0, 1]
+    assert ni.tolist() == [0, 0, 1, 0] and pi.tolist() == [0, 1, 0, 0]
+
+
+def test_trapezoid_tables():
+    """test/numpy.test.ts:415-517: unit spacing, dx (number and array along another axis), sample points x (1-D,
+    uneven, shaped like y, lower rank), an axis of a 2-D array, a size-1 axis."""
+    y = f32([1, 2, 3])
+    _, (t1, t2) = run(lambda a: [L.trapezoid(a), L.trapezoid(a, dx=2)], y)
+    assert t1.tolist() == [4] and t2.tolist() == [8]
+    _, (t3,) = run(lambda a, d: L.trapezoid(a, dx=d, axis=0), f32([[1, 2], [3, 4], [5, 6]]), f32([[1], [2]]))
+    assert t3.tolist() == [10, 13]
+    _, (t4,) = run(lambda a, x: L.trapezoid(a, x), y, f32([4, 6, 8]))
+    assert t4.tolist() == [8]
+    _, (t5,) = run(lambda a, x: L.trapezoid(a, x), y, f32([0, 1, 3]))
+    np.testing.assert_allclose(t5, [6.5], rtol=1e-6)
+    m = f32([[1, 2, 3], [4, 5, 6]])
+    _, (a1, a0) = run(lambda a: [L.trapezoid(a, axis=1), L.trapezoid(a, axis=0)], m)
+    assert a1.tolist() == [4, 10] and a0.tolist() == [2.5, 3.5, 4.5]
+    _, (b1,) = run(lambda a, x: L.trapezoid(a, x), m, f32([0, 1, 3]))
+    np.testing.assert_allclose(b1, [6.5, 15.5], rtol=1e-6)
+    _, (b2,) = run(lambda a, x: L.trapezoid(a, x), f32([[1, 1, 1], [2, 2, 2]]), f32([[0, 1, 2], [0, 2, 4]]))
+    assert b2.tolist() == [2, 8]
+    _, (b3,) = run(lambda a, x: L.trapezoid(a, x), np.ones((2, 2, 3), np.float32), f32([[0, 1, 3], [0, 2, 4]]))
+    assert b3.tolist() == [3, 4, 3, 4]
+    _, (z,) = run(lambda a: L.trapezoid(a), f32([5]))
+    assert z.tolist() == [0]
+    _, (big,) = run(lambda a, x: L.trapezoid(a, x), f32([1, 1]), f32([-2e9, 2e9]))
+    np.testing.assert_allclose(big, [4e9], rtol=1e-6)
+
+
+def test_matvec_vecmat_tensordot_outer_inner_tables():
+    """test/numpy.test.ts:1611-1690 (matvec: plain, batched matrix, batched vectors -- the rotation example; vecmat),
+    :1798-1817 (tensordot 2-3-4 with 3-4-5, by count and by explicit axes); outer / inner / vdot / vecdot against numpy."""
+    _, (mv,) = run(lambda a, v: L.matvec(a, v), f32([[1, 2], [3, 4]]), f32([5, 6]))
+    assert mv.tolist() == [17, 39]
+    _, (mb,) = run(lambda a, v: L.matvec(a, v), f32([[[1, 0], [0, 1]], [[0, 1], [1, 0]]]), f32([3, 7]))
+    assert mb.tolist() == [3, 7, 7, 3]
+    _, (rot,) = run(lambda a, v: L.matvec(a, v), f32([[0, 1, 0], [-1, 0, 0], [0, 0, 1]]), f32([[1, 0, 0], [0, 1, 0], [0, 0, 1], [0, 6, 8]]))
+    assert rot.tolist() == [0, -1, 0, 1, 0, 0, 0, 0, 1, 6, 0, 8]
+    _, (vm1,) = run(lambda v, a: L.vecmat(v, a), f32([1, 2]), f32([[3, 4], [5, 6]]))
+    _, (vm2,) = run(lambda v, a: L.vecmat(v, a), f32([0, 4, 2]), f32([[1, 0, 0], [0, 1, 0], [0, 0, 0]]))
+    assert vm1.tolist() == [13, 16] and vm2.tolist() == [0, 4, 0]
+    x1, x2 = f32(np.arange(24).reshape(2, 3, 4)), np.ones((3, 4, 5), np.float32)
+    _, (td, te) = run(lambda a, b: [L.tensordot(a, b), L.tensordot(a, b, ([1, 2], [0, 1]))], x1, x2)
+    assert td.tolist() == [66] * 5 + [210] * 5 and te.tolist() == td.tolist()
+    rng = np.random.default_rng(9)
+    a, b = rng.integers(-3, 4, (3, 4)).astype(np.float32), rng.integers(-3, 4, (5, 4)).astype(np.float32)
+    _, (o, i, vd, vc) = run(lambda p, q: [L.outer(p, q), L.inner(p, q), L.vdot(p, q.reshape([5, 4])[:3] if False else p), L.vecdot(p, p, axis=0)], a, b)
+    np.testing.assert_array_equal(o.reshape(12, 20), np.outer(a, b))
+    np.testing.assert_array_equal(i.reshape(3, 5), np.inner(a, b))
+    assert vd.tolist() == [float(np.vdot(a, a))]
+    np.testing.assert_array_equal(vc, np.sum(a * a, axis=0))

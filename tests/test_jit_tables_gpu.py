@@ -22,7 +22,8 @@ TABLE_TESTS = [
     "test_gather_take_and_take_along_axis", "test_concatenate_stack_and_split",
     "test_output_returned_twice_carries_two_references", "test_input_returned_twice_beside_a_result",
     "test_count_nonzero_any_all_tables", "test_prod_ptp_var_std_average_tables", "test_cumsum_cumprod_tables_and_the_two_stage_scan",
-    "test_diff_tables",
+    "test_diff_tables", "test_flip_rot90_roll_tables", "test_sign_and_float_class_predicates", "test_trapezoid_tables",
+    "test_matvec_vecmat_tensordot_outer_inner_tables",
 ]
 
 
