@@ -106,8 +106,12 @@ def match_conv(oexp: AluExp, extent: int, K: int, batch: list) -> Optional[dict]
     if T % KW:
         return None
     KH = T // KW
+    # consecutive output positions advance by the column stride; the first break ends an output row
     d_row = np.diff(idx[:, 0])
-    breaks = np.nonzero(d_row != 1)[0]
+    SX = int(d_row[0]) if len(d_row) else 1
+    if SX < 1:
+        return None
+    breaks = np.nonzero(d_row != SX)[0]
     base = int(idx[0, 0])  # = -(PH * W + PW): position 0 with tap 0 sits PH rows and PW columns before the plane
     if base > 0:
         return None
@@ -122,22 +126,29 @@ def match_conv(oexp: AluExp, extent: int, K: int, batch: list) -> Optional[dict]
             continue
         H = cs // W
         PH, PW = (-base) // W, (-base) % W
-        candidates = [int(breaks[0]) + 1] if len(breaks) else [W] + [d for d in range(extent, 0, -1) if extent % d == 0 and d != W]
+        candidates = [int(breaks[0]) + 1] if len(breaks) else [-(-W // SX)] + [d for d in range(extent, 0, -1) if extent % d == 0 and d != -(-W // SX)]
         for OW in candidates:
-            if extent % OW:
+            if OW <= 0 or extent % OW:
                 continue
+            # the row stride: from the first position of the second output row, else (one output row) 1
+            SY = 1
+            if extent > OW:
+                step = int(idx[OW, 0]) - base
+                if step <= 0 or step % W:
+                    continue
+                SY = step // W
             oy, ox = rows // OW, rows % OW
-            iy, ix = oy + ky - PH, ox + kx - PW
+            iy, ix = SY * oy + ky - PH, SX * ox + kx - PW
             valid = (iy >= 0) & (iy < H) & (ix >= 0) & (ix < W)
             model = iy * W + ix
             if np.array_equal(ok, valid) and np.array_equal(idx[valid], model[valid]) and (cond is not None or valid.all()):
-                found = (W, H, PH, PW, OW)
+                found = (W, H, PH, PW, OW, SY)
                 break
         if found:
             break
     if found is None:
         return None
-    W, H, PH, PW, found = found
+    W, H, PH, PW, found, SY = found
     OW, OH = found, extent // found
     SB = 0
     if nb > 1:
@@ -154,7 +165,7 @@ def match_conv(oexp: AluExp, extent: int, K: int, batch: list) -> Optional[dict]
     length = node.arg[1]
     if (nb - 1) * SB + (C - 1) * cs + H * W > length:
         return None
-    return dict(gid=node.arg[0], length=length, T=T, C=C, SC=cs, SB=SB, NB=nb, OW=OW, OH=OH, KW=KW, KH=KH, W=W, H=H, PH=PH, PW=PW)
+    return dict(gid=node.arg[0], length=length, T=T, C=C, SC=cs, SB=SB, NB=nb, OW=OW, OH=OH, KW=KW, KH=KH, W=W, H=H, PH=PH, PW=PW, SX=SX, SY=SY)
 
 
 def _pitch(elems: int) -> int:
@@ -179,32 +190,52 @@ def gen_conv(kernel, g: dict, oexp: AluExp, numerics: str, name: str, params: st
     if cv is None:
         return None
     O, C, OW = g["M"], cv["C"], cv["OW"]
-    if OW % 4 or C % 16 or O % 64:  # 8-byte aligned row offsets in LDS, whole MFMA k steps, whole 64-channel tiles
+    if C % 16 or O % 64:  # whole MFMA k steps, whole 64-channel tiles
         return None
-    BM = int(tile.get("CBM", 128 if O % 128 == 0 and O >= 256 else 64))
-    # 256 positions per tile (wave tile 32 x 128: four MFMAs per A fragment) unless the image is smaller than that
-    BN = int(tile.get("CBN", 256 if g["N"] >= 256 else 128))
+    # Output rows are walked at a width of whole 4-position groups (8-byte aligned row offsets in LDS): the up to three
+    # extra columns per row are computed and dropped.  Positions, tiles and the patch pitch all use this width.
+    OWP = -(-OW // 4) * 4
+    NV = cv["OH"] * OWP
+    # 256 positions per tile (wave tile 32 x 128: four MFMAs per A fragment) unless the image is smaller than that;
+    # 128 output channels per tile from 256 channels on, as long as that still gives every CU a tile (small images:
+    # [32,256,14,14] 44 -> 29 us, [32,512,7,7] 84 -> 52 us with 64)
+    from . import tuner
+    BN = int(tile.get("CBN", 256 if NV >= 256 else 128))
+    wide = O % 128 == 0 and O >= 256 and -(-NV // BN) * (O // 128) * cv["NB"] >= tuner.CU_COUNT
+    BM = int(tile.get("CBM", 128 if wide else 64))
     WM, WN = 2, 2
     if O % BM or BM % (32 * WM) or BN % (32 * WN) or BN % 4:
         return None
-    # rows of the image a tile can touch: the output rows its BN consecutive positions span, plus the window's height
-    n_tiles = -(-g["N"] // BN)
-    spans = max(((t * BN + BN - 1) // OW) - ((t * BN) // OW) + 1 for t in range(n_tiles))
-    R = spans + cv["KH"] - 1
-    P = _pitch(R * OW)
-    G = 8 if OW % 8 == 0 else 4
-    smax = max(cv["PW"], cv["KW"] - 1 - cv["PW"])
-    if cv["W"] < G or smax >= G:
+    # output rows a tile's BN consecutive positions span; the image rows behind them live in SY planes (by row % SY) of
+    # RP rows each: plane rows from floor(-PH / SY) to floor((KH - 1 - PH) / SY) past the tile's first and last row
+    n_tiles = -(-NV // BN)
+    spans = max((min(t * BN + BN - 1, NV - 1) // OWP) - ((t * BN) // OWP) + 1 for t in range(n_tiles))
+    SX, SY = cv["SX"], cv["SY"]
+    qmin, qmax = (-cv["PH"]) // SY, (cv["KH"] - 1 - cv["PH"]) // SY
+    RP = spans + qmax - qmin
+    R = SY * RP
+    P = _pitch(R * OWP)
+    GO = 8 if OWP % 8 == 0 and SX == 1 and cv["W"] >= 8 else 4   # output columns per fill vector (16- or 8-byte LDS stores)
+    G = GO * SX                                  # image elements per fill vector
+    SR = cv["KW"] - 1 - cv["PW"]
+    # neighbour-exchange fill: rows of whole aligned vectors that line up with the output columns
+    xch = G in (4, 8) and OWP == OW and cv["W"] % G == 0 and cv["W"] == SX * OW and OW // GO <= 64 and cv["PW"] < G and SR - SX + 1 < G
+    # otherwise (stride 1 only): unaligned vector loads, clamped into the row and shifted into place; a group may hang
+    # over the row's start by PW and over its end by the window's reach plus the columns the walking width adds
+    smax = max(cv["PW"], SR) if xch else max(cv["PW"], max(0, OWP - cv["W"] + SR))
+    if not xch and (SX != 1 or SY != 1 or cv["W"] < G or smax >= G):
         return None
     # channels per slab: 16 (one MFMA k step per tap) measured fastest on every shape tried -- short slabs keep the fill of
     # the next patch and the MFMAs of this one in step, and leave LDS for a second workgroup per CU
-    CS = int(tile.get("CCS", 16))
+    # (32 when the patch is small and there are many slabs to walk: 3-4 % on the 14x14 and 7x7 shapes)
+    CS = int(tile.get("CCS", 32 if C % 32 == 0 and C >= 128 and cv["KW"] * 32 * P * 2 <= 40 * 1024 else 16))
     if not CS or C % CS or cv["KW"] * CS * P * 2 > 160 * 1024:
         return None
     sb_c = g["batch"][0][3] if g["batch"] else 0
     src = _prelude(numerics) + fill(template("conv_f16.hip.inc"), dict(
-        OW=OW, OH=cv["OH"], W=cv["W"], H=cv["H"], KH=cv["KH"], KW=cv["KW"], PH=cv["PH"], PW=cv["PW"], C=C, O=O,
+        OW=OW, OWP=OWP, OH=cv["OH"], W=cv["W"], H=cv["H"], KH=cv["KH"], KW=cv["KW"], PH=cv["PH"], PW=cv["PW"], C=C, O=O,
         SC=cv["SC"], SB=cv["SB"], NB=cv["NB"], BM=BM, BN=BN, WM=WM, WN=WN, CS=CS, R=R, P=P, G=G, SMAX=smax,
+        SX=SX, SY=SY, RP=RP, QMIN=qmin, XCH=int(xch),
         EPILOGUE_FN=epi_fn, EPILOGUE_ARGS=epi_args, NAME=name, PARAMS=params, IMG_PTR=names[cv["gid"]],
         A_OFF=g["a_off"], A_SM=g["a_sm"], A_SK=g["a_sk"], C_SM=g["c_sm"], C_SN=g["c_sn"], C_SB=sb_c))
     T = cv["T"]
@@ -218,5 +249,5 @@ def gen_conv(kernel, g: dict, oexp: AluExp, numerics: str, name: str, params: st
     need[g["gid_a"]] = max(need.get(g["gid_a"], 0), g["a_len"] * 2)
     need[cv["gid"]] = max(need.get(cv["gid"], 0), ((cv["NB"] - 1) * cv["SB"] + (C - 1) * cv["SC"] + cv["H"] * cv["W"]) * 2)
     info = dict(BM=BM, BN=BN, WM=WM, WN=WN, BK=16, direct_lds=False, tiles=tiles, M=O, N=g["N"], K=g["K"], nbatch=cv["NB"], splitk=1,
-                conv=dict(cv, CS=CS, R=R, P=P, G=G), gather=dict(a="none", b="patch"))
+                conv=dict(cv, CS=CS, R=R, P=P, G=G, OWP=OWP, exchange=bool(xch)), gather=dict(a="none", b="patch"))
     return KernelSource([src], [prep, main], [total_w * 2], "gemm", need, info)

@@ -250,7 +250,23 @@ F16_CONV_CASES = [
     dict(x=(8, 16, 8, 4), w=(64, 16, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),        # one tile per image, mostly padding
     dict(x=(1, 16, 12, 32), w=(64, 16, 5, 5), strides=[1, 1], padding="SAME", loader="patch"),      # shifts of 2 to either side
     dict(x=(2, 16, 16, 16), w=(32, 16, 3, 3), strides=[1, 1], padding="SAME", loader="rows8"),      # 32 output channels: generic loaders
-    dict(x=(2, 16, 32, 32), w=(64, 16, 3, 3), strides=[2, 2], padding="SAME", loader="element"),    # strided: generic loaders
+    # output widths that are not a multiple of 4: rows are walked at the next multiple, the extra columns dropped
+    dict(x=(2, 16, 14, 14), w=(64, 16, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),
+    dict(x=(3, 32, 7, 7), w=(64, 32, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),
+    dict(x=(2, 16, 10, 10), w=(64, 16, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),
+    dict(x=(2, 16, 15, 15), w=(64, 16, 3, 3), strides=[1, 1], padding="VALID", loader="patch"),
+    dict(x=(2, 16, 9, 6), w=(64, 16, 3, 3), strides=[1, 1], padding="SAME", loader="patch"),
+    dict(x=(2, 16, 9, 5), w=(64, 16, 3, 3), strides=[1, 1], padding="SAME", loader="element"),       # overhang of a whole vector: generic loaders
+    dict(x=(1, 16, 33, 21), w=(64, 16, 5, 5), strides=[1, 1], padding="SAME", loader="patch"),
+    # strided window walks: copies pick every second column, rows live in planes by parity
+    dict(x=(2, 16, 32, 32), w=(64, 16, 3, 3), strides=[2, 2], padding="SAME", loader="patch"),
+    dict(x=(2, 16, 32, 32), w=(64, 16, 3, 3), strides=[2, 2], padding=[(1, 1), (1, 1)], loader="patch"),  # left and top padding
+    dict(x=(2, 16, 16, 32), w=(64, 16, 3, 3), strides=[1, 2], padding="SAME", loader="patch"),
+    dict(x=(2, 16, 32, 16), w=(64, 16, 3, 3), strides=[2, 1], padding="SAME", loader="patch"),
+    dict(x=(1, 32, 32, 32), w=(64, 32, 5, 5), strides=[2, 2], padding="SAME", loader="patch"),            # a dword from the right neighbour
+    dict(x=(3, 32, 56, 56), w=(128, 32, 3, 3), strides=[2, 2], padding="SAME", loader="patch"),           # several position tiles per image
+    dict(x=(2, 16, 24, 24), w=(64, 16, 3, 3), strides=[3, 3], padding="SAME", loader="element"),          # other strides: generic loaders
+    dict(x=(2, 16, 33, 32), w=(64, 16, 3, 3), strides=[2, 2], padding="VALID", loader="element"),         # image wider than 2 x output
 ]
 
 
