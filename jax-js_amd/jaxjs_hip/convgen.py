@@ -220,10 +220,10 @@ def gen_conv(kernel, g: dict, oexp: AluExp, numerics: str, name: str, params: st
     SR = cv["KW"] - 1 - cv["PW"]
     # neighbour-exchange fill: rows of whole aligned vectors that line up with the output columns
     xch = G in (4, 8) and OWP == OW and cv["W"] % G == 0 and cv["W"] == SX * OW and OW // GO <= 64 and cv["PW"] < G and SR - SX + 1 < G
-    # otherwise (stride 1 only): unaligned vector loads, clamped into the row and shifted into place; a group may hang
-    # over the row's start by PW and over its end by the window's reach plus the columns the walking width adds
-    smax = max(cv["PW"], SR) if xch else max(cv["PW"], max(0, OWP - cv["W"] + SR))
-    if not xch and (SX != 1 or SY != 1 or cv["W"] < G or smax >= G):
+    # otherwise: unaligned vector loads, clamped into the row and shifted into place; a vector may hang over the row's
+    # start by PW and over its end by the window's reach plus the columns the walking width adds
+    smax = max(cv["PW"], SR) if xch else max(cv["PW"], max(0, SX * (OWP - GO) + SR - (cv["W"] - G)))
+    if not xch and (G not in (4, 8) or cv["W"] < G or smax >= G):
         return None
     # channels per slab: 16 (one MFMA k step per tap) measured fastest on every shape tried -- short slabs keep the fill of
     # the next patch and the MFMAs of this one in step, and leave LDS for a second workgroup per CU

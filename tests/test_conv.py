@@ -266,7 +266,11 @@ F16_CONV_CASES = [
     dict(x=(1, 32, 32, 32), w=(64, 32, 5, 5), strides=[2, 2], padding="SAME", loader="patch"),            # a dword from the right neighbour
     dict(x=(3, 32, 56, 56), w=(128, 32, 3, 3), strides=[2, 2], padding="SAME", loader="patch"),           # several position tiles per image
     dict(x=(2, 16, 24, 24), w=(64, 16, 3, 3), strides=[3, 3], padding="SAME", loader="element"),          # other strides: generic loaders
-    dict(x=(2, 16, 33, 32), w=(64, 16, 3, 3), strides=[2, 2], padding="VALID", loader="element"),         # image wider than 2 x output
+    # strided and not whole vectors: unaligned loads, every second element kept
+    dict(x=(2, 16, 33, 32), w=(64, 16, 3, 3), strides=[2, 2], padding="VALID", loader="patch"),
+    dict(x=(2, 32, 28, 28), w=(64, 32, 3, 3), strides=[2, 2], padding="SAME", loader="patch"),            # 28 -> 14
+    dict(x=(3, 16, 14, 14), w=(128, 16, 3, 3), strides=[2, 2], padding=[(1, 1), (1, 1)], loader="patch"), # 14 -> 7
+    dict(x=(2, 16, 20, 12), w=(64, 16, 3, 3), strides=[2, 1], padding="SAME", loader="patch"),
 ]
 
 
