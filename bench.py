@@ -587,6 +587,14 @@ def main():
                 [hostrand.normal(1007, cx, 1.0, npdt), hostrand.normal(1007, cw, 0.05, npdt, stream=1)],
                 2.0 * 32 * 64 * 56 * 56 * 64 * 9, "TFLOP/s", PEAK_F16_TFLOPS if cdt == DType.Float16 else PEAK_F32_MATRIX_TFLOPS)
 
+        # ResNet-shaped f16 layers (batch 32): 3x3 at 28x28x256 and 14x14x256, and the stride-2 3x3 that halves 56x56.
+        for cx, cw, st in (((32, 256, 28, 28), (256, 256, 3, 3), 1), ((32, 256, 14, 14), (256, 256, 3, 3), 1),
+                           ((32, 64, 56, 56), (128, 64, 3, 3), 2)):
+            cprog = J.jit(lambda a, b: Lb.convGeneralDilated(a, b, [st, st], "SAME"), [ShapedArray(cx, DType.Float16), ShapedArray(cw, DType.Float16)])
+            run(f"conv3x3_s{st}_f16[{','.join(map(str, cx))}]x[{','.join(map(str, cw))}]", cprog.kernels[0],
+                [hostrand.normal(1007, cx, 1.0, np.float16), hostrand.normal(1007, cw, 0.05, np.float16, stream=1)],
+                2.0 * cx[0] * cw[0] * (cx[2] // st) * (cx[3] // st) * cw[1] * 9, "TFLOP/s", PEAK_F16_TFLOPS)
+
         # Routines: sort / argsort of f32 [8192, 4096] rows (native bitonic network in LDS).
         from jaxjs_hip.routine import Routine, Routines, RoutineType
         rows, L = 8192, 4096
