@@ -493,6 +493,18 @@ def exp(x): return bind1("Exp", [x])
 def log(x): return bind1("Log", [x])
 def sqrt(x): return bind1("Sqrt", [x])
 def erfc(x): return bind1("Erfc", [x])
+def erf(x): return bind1("Erf", [x])
+def sin(x): return bind1("Sin", [x])
+def cos(x): return bind1("Cos", [x])
+def asin(x): return bind1("Asin", [x])
+def atan(x): return bind1("Atan", [x])
+def floor(x): return bind1("Floor", [x])
+def ceil(x): return bind1("Ceil", [x])
+def idiv(x, y): return bind1("Idiv", [x, y])
+def mod(x, y): return bind1("Mod", [x, y])  # sign of the numerator (core.ts:43)
+def bitCombine(x, y, op: str): return bind1("BitCombine", [x, y], dict(op=op))  # core.ts:189-195
+def bitShift(x, y, op: str): return bind1("BitShift", [x, y], dict(op=op))  # core.ts:197-199
+def bitcast(x, dtype: DType): return bind1("Bitcast", [x], dict(dtype=dtype))
 def stopGradient(x): return bind1("StopGradient", [x])
 def maximum(x, y): return bind1("Max", [x, y])
 def minimum(x, y): return bind1("Min", [x, y])
@@ -645,7 +657,7 @@ def trace(fn: Callable[..., Any], avals: Sequence[ShapedArray]) -> Tuple[Jaxpr, 
     try:
         ins = [Var(a) for a in avals]
         outs = fn(*[Tracer(v) for v in ins])
-        if isinstance(outs, Tracer):
+        if isinstance(outs, (Tracer, ConstArray, int, float, bool)):
             outs = [outs]
         out_atoms = [_raise(o).atom for o in outs]
     finally:
@@ -840,6 +852,8 @@ JIT_RULES: Dict[str, Callable] = {
     "Mod": _broadcasted(lambda e, p: AluExp.mod(e[0], e[1])),
     "Min": _broadcasted(lambda e, p: AluExp.min(e[0], e[1])),
     "Max": _broadcasted(lambda e, p: AluExp.max(e[0], e[1])),
+    "BitCombine": _broadcasted(lambda e, p: AluExp.bitCombine(e[0], e[1], p["op"])),
+    "BitShift": _broadcasted(lambda e, p: AluExp.bitShift(e[0], e[1], p["op"])),
     "Neg": _unop(lambda a, p: AluExp.sub(AluExp.const(a.dtype, 0), a)),
     "Reciprocal": _unop(lambda a, p: AluExp.reciprocal(a)),
     "Floor": _unop(lambda a, p: AluExp.floor(a)),

@@ -13,6 +13,23 @@ the backend is handed, so it is kept literally:
   eigh (unsorted), fft along an axis                  src/library/lax-linalg.ts:52-100; numpy-fft.ts:50-66, 126-157
   stack, take, takeAlongAxis, absolute, clip, log1p   src/library/numpy.ts:971-985, 1493-1567, 2433-2452, 2854-2884
   random: bits, split, uniform, exponential, normal   src/library/random.ts:53-135, 350-356, 511-525
+  reductions and scans: prod, any, all, ptp, var, std, average, cumsum, cumprod, diff, trapezoid
+                                                      src/library/numpy.ts:358-500, 560-772, 3100-3140
+  element-wise: logical / bitwise / shifts, signbit, copysign, fmin / fmax, division family (trueDivide, floorDivide,
+  fmod, remainder, divmod, modf, trunc), rint / round, exp2 / log2 / log10 / expm1 / logaddexp, power / floatPower /
+  cbrt, sinc, tan, acos, atan2, hypot, sinh ... arctanh, nanToNum and the float class predicates
+                                                      src/library/numpy.ts:159-225, 2433-3100, 3194-3253
+  creation (lazy constants): full / zeros / ones, eye, arange, tri / tril / triu, linspace / logspace / geomspace,
+  bartlett / hann / blackman                          src/frontend/array.ts:1484-1790; numpy.ts:2524-2566
+  shapes and joins: ravel, squeeze, expandDims, broadcastTo, repeat, tile, pad, split family, concatenate, stack
+  family, unstack, append, flip / rot90 / roll, swapaxes, moveaxis
+                                                      src/library/numpy.ts:253-275, 792-1330, 1474-1492
+  selection and comparison: select, arrayEqual, arrayEquiv, isin, diag / diagflat / diagIndices / trace, meshgrid,
+  indices, ediff1d                                    src/library/numpy.ts:774-790, 1350-1450, 1583-1727, 2312-2385, 3176-3192
+  products and polynomials: dot, inner, outer, tensordot, vdot, vecdot, matvec, vecmat, cross, vander, polyval, polyadd,
+  polysub, polymul, convolve, correlate, cov, corrcoef, unwrap
+                                                      src/library/numpy.ts:1729-1815, 1988-2310, 2933-2980, 3141-3174
+Not restated: fromfunction and applyAlongAxis (they are built on vmap, a transformation this layer does not have).
 """
 
 from __future__ import annotations
@@ -392,7 +409,7 @@ def fft(real: Tracer, imag: Tracer, axis: int = -1, inverse: bool = False):
 
 
 def stack(xs: Sequence[Tracer], axis: int = 0):
-    xs = [J._raise(x) for x in xs]
+    xs = [_as_array(x) for x in xs]
     if not xs:
         raise ValueError("Need at least one array to stack")
     if any(tuple(x.shape) != tuple(xs[0].shape) for x in xs):
@@ -706,8 +723,11 @@ def isinf(x: Tracer):
 
 
 def isfinite(x: Tracer):
-    """`!isnan & !isinf` spelt with the comparisons the IR has: x - x == 0 fails exactly for NaN and the infinities."""
-    return J.equal(x.sub(x), 0)
+    """`(isnan | isinf) != true` (numpy.ts:3250-3253)."""
+    x = J._raise(x)
+    if x.dtype not in (DType.Float32, DType.Float16, DType.Float64):
+        return J.equal(x, x)
+    return J.notEqual(J.add(isnan(x), isinf(x)), True)
 
 
 def trapezoid(y: Tracer, x: Optional[Tracer] = None, dx=1.0, axis: int = -1):
@@ -780,3 +800,1002 @@ def vecmat(x1: Tracer, x2: Tracer):
     if x1.ndim < 1 or x2.ndim < 2:
         raise ValueError("vecmat: x1 must be at least 1D and x2 at least 2D")
     return J.dot(x1.reshape(list(x1.shape[:-1]) + [1, x1.shape[-1]]), swapaxes(x2, -1, -2))
+
+
+# ---- element-wise arithmetic, as the reference spells it (src/library/numpy.ts) -----------------------------------
+
+_FLOATS = (DType.Float32, DType.Float16, DType.Float64)
+
+
+def _floatish(x: Tracer) -> Tracer:
+    return x if x.dtype in _FLOATS else x.astype(DType.Float32)
+
+
+def logicalAnd(x, y):  # numpy.ts:159-162: bool `*` is AND
+    return J.mul(J._raise(x).astype(DType.Bool), J._raise(y).astype(DType.Bool))
+
+
+def logicalOr(x, y):  # numpy.ts:164-167: bool `+` is OR
+    return J.add(J._raise(x).astype(DType.Bool), J._raise(y).astype(DType.Bool))
+
+
+def logicalXor(x, y):  # numpy.ts:169-172
+    return J.notEqual(J._raise(x).astype(DType.Bool), J._raise(y).astype(DType.Bool))
+
+
+def logicalNot(x):  # numpy.ts:174-177
+    return J.notEqual(J._raise(x).astype(DType.Bool), True)
+
+
+def bitwiseAnd(x, y):
+    return J.bitCombine(x, y, "and")
+
+
+def bitwiseOr(x, y):
+    return J.bitCombine(x, y, "or")
+
+
+def bitwiseXor(x, y):
+    return J.bitCombine(x, y, "xor")
+
+
+def invert(x: Tracer):
+    """XOR with all ones of the operand's own dtype (numpy.ts:194-211)."""
+    x = J._raise(x)
+    if x.dtype == DType.Bool:
+        ones = True
+    elif x.dtype == DType.Uint32:
+        ones = J.scalar(0xFFFFFFFF, DType.Uint32)
+    elif x.dtype == DType.Int32:
+        ones = J.scalar(-1, DType.Int32)
+    else:
+        raise TypeError(f"invert: unsupported dtype {x.dtype}")
+    return J.bitCombine(x, ones, "xor")
+
+
+def leftShift(x, y):
+    return J.bitShift(x, y, "shl")
+
+
+def rightShift(x, y):
+    return J.bitShift(x, y, "shr")
+
+
+def signbit(x: Tracer):
+    """Bool and uint32 have no sign; int32 compares with 0; floats read the top bit of their f32 image through a
+    bitcast, which keeps -0 and the sign of a NaN (numpy.ts:2470-2485)."""
+    x = J._raise(x)
+    if x.dtype in (DType.Bool, DType.Uint32):
+        return J.notEqual(x, x)  # all false, shaped like x
+    if x.dtype == DType.Int32:
+        return J.less(x, 0)
+    return J.less(J.bitcast(x.astype(DType.Float32), DType.Int32), J.scalar(0, DType.Int32))
+
+
+def copysign(x: Tracer, y: Tracer):  # numpy.ts:2490-2492 (so a zero y gives 0)
+    return absolute(x).mul(sign(y))
+
+
+def fmax(x1: Tracer, x2: Tracer):  # numpy.ts:2501-2503
+    return J.where(J.add(J.greater(x1, x2), isnan(x2)), x1, x2)
+
+
+def fmin(x1: Tracer, x2: Tracer):  # numpy.ts:2512-2514
+    return J.where(logicalOr(J.less(x1, x2), isnan(x2)), x1, x2)
+
+
+def heaviside(x1: Tracer, x2):  # numpy.ts:2574-2576
+    return J.where(J.less(x1, 0), 0, J.where(J.equal(x1, 0), x2, 1))
+
+
+def tan(x: Tracer):
+    return J.sin(x).div(J.cos(x))
+
+
+def sinc(x: Tracer):  # numpy.ts:2600-2604
+    pix = x.mul(math.pi)
+    return J.where(J.equal(x, 0), 1, J.sin(pix).div(pix))
+
+
+def acos(x: Tracer):
+    return J._raise(math.pi / 2).sub(J.asin(x))
+
+
+def hypot(x1: Tracer, x2: Tracer):
+    return J.sqrt(square(x1).add(square(x2)))
+
+
+def atan2(y: Tracer, x: Tracer):
+    """Half-angle form: 2*atan(y / (r + x)) for x >= 0 and 2*atan((r - x) / y) for x < 0 (numpy.ts:2636-2647)."""
+    r = J.sqrt(square(x).add(square(y)))
+    xNeg = J.less(x, 0)
+    numer = J.where(xNeg, r.sub(x), y)
+    denom = J.where(xNeg, y, r.add(x))
+    return J.atan(numer.div(denom)).mul(2)
+
+
+def trueDivide(x, y):  # numpy.ts:2669-2677
+    x, y = J._raise(x), J._raise(y)
+    if x.dtype not in _FLOATS and y.dtype not in _FLOATS:
+        x, y = x.astype(DType.Float32), y.astype(DType.Float32)
+    return x.div(y)
+
+
+def fmod(x: Tracer, y: Tracer):  # numpy.ts:2700-2702
+    x, y = J._raise(x), J._raise(y)
+    return x.sub(J.mul(y, J.idiv(x, y)))
+
+
+def remainder(x: Tracer, y: Tracer):
+    """Sign of the divisor: `mod(mod(x, y) + y, y)` over the numerator-signed Mod primitive (numpy.ts:2708-2712)."""
+    return J.mod(J.add(J.mod(x, y), y), y)
+
+
+def floorDivide(x, y):  # numpy.ts:2684-2694
+    x, y = J._raise(x), J._raise(y)
+    if x.dtype in _FLOATS or y.dtype in _FLOATS:
+        return J.floor(trueDivide(x, y))
+    return J._raise(x).sub(remainder(x, y)).div(y)
+
+
+def divmod_(x, y):
+    return [floorDivide(x, y), remainder(x, y)]
+
+
+def trunc(x):
+    return J.idiv(x, 1)  # numpy.ts:2731-2733
+
+
+def modf(x: Tracer):
+    x = _floatish(J._raise(x))
+    whole = trunc(x)
+    return [x.sub(whole), whole]
+
+
+def rint(x: Tracer):
+    """Round half to even from floor(x + 0.5), stepping back when the fraction is exactly one half and the rounded
+    value is odd (numpy.ts:2774-2781)."""
+    rounded = J.floor(x.add(0.5))
+    half = J.equal(x.sub(J.floor(x)), 0.5)
+    odd = J.notEqual(remainder(rounded, 2), 0)
+    return J.where(J.mul(half, odd), rounded.sub(1), rounded)
+
+
+def round_(a: Tracer, decimals: int = 0):  # numpy.ts:2757-2766
+    if decimals == 0:
+        return rint(a)
+    factor = 10 ** decimals
+    return rint(a.mul(factor)).mul(1 / factor)
+
+
+def exp2(p):
+    return J.exp(J.mul(p, math.log(2)))
+
+
+def log2(x):
+    return J.log(x).mul(math.log2(math.e))
+
+
+def log10(x):
+    return J.log(x).mul(math.log10(math.e))
+
+
+def ldexp(x1, x2):
+    return J.mul(x1, exp2(x2))
+
+
+def expm1(x: Tracer):
+    """Series through x^7 (Horner) for |x| <= 0.1 (0.01 in f64), exp(x) - 1 elsewhere (numpy.ts:2827-2852)."""
+    x = _floatish(J._raise(x))
+    cutoff = 0.01 if x.dtype == DType.Float64 else 0.1
+    useSeries = J.lessEqual(absolute(x), cutoff)
+    sx = clip(x, -cutoff, cutoff)
+    series = (sx.mul(1 / 5040).add(1 / 720).mul(sx).add(1 / 120).mul(sx).add(1 / 24).mul(sx).add(1 / 6).mul(sx)
+              .add(1 / 2).mul(sx).add(1).mul(sx))
+    return J.where(useSeries, series, J.exp(x).sub(1))
+
+
+def logaddexp(x1: Tracer, x2: Tracer):  # numpy.ts:2890-2893
+    xmax = J.maximum(x1, x2)
+    return J.log(J.exp(J._raise(x1).sub(xmax)).add(J.exp(J._raise(x2).sub(xmax)))).add(xmax)
+
+
+def logaddexp2(x1: Tracer, x2: Tracer):  # numpy.ts:2899-2902
+    xmax = J.maximum(x1, x2)
+    return log2(exp2(J._raise(x1).sub(xmax)).add(exp2(J._raise(x2).sub(xmax)))).add(xmax)
+
+
+def deg2rad(x):
+    return J.mul(x, math.pi / 180)
+
+
+def rad2deg(x):
+    return J.mul(x, 180 / math.pi)
+
+
+def power(x1, x2):
+    """exp(x2 * log|x1|) with the sign put back for odd integer exponents and NaN for a negative base with a
+    non-integer exponent (numpy.ts:2982-2999)."""
+    x1, x2 = J._raise(x1), J._raise(x2)
+    x2i = trunc(x2)
+    shouldBeNaN = J.mul(J.notEqual(x2, x2i), J.less(x1, 0))
+    resultSign = J.where(J.notEqual(J.mod(x2i, 2), 0), J.where(J.less(x1, 0), -1, 1), 1)
+    return J.where(shouldBeNaN, math.nan, J.exp(J.log(absolute(x1)).mul(x2)).mul(resultSign))
+
+
+def resultType(*xs) -> DType:
+    """The promoted dtype of the operands, shapes aside (numpy.ts:342-355)."""
+    avals = [J.ShapedArray((), t.dtype, t.aval.weak) for t in (J._raise(x) for x in xs)]
+    out = avals[0]
+    for a in avals[1:]:
+        out = J.promoteAvals(out, a)
+    return out.dtype
+
+
+def floatPower(x1, x2):  # numpy.ts:3007-3015
+    x1, x2 = J._raise(x1), J._raise(x2)
+    dt = J.promoteAvals(x1.aval, x2.aval).dtype
+    if dt not in _FLOATS:
+        dt = DType.Float32
+    return power(x1.astype(dt), x2.astype(dt))
+
+
+def cbrt(x: Tracer):  # numpy.ts:3018-3022
+    sgn = J.where(J.less(x, 0), -1, 1)
+    return sgn.mul(J.exp(J.log(x.mul(sgn)).mul(1 / 3)))
+
+
+def sinh(x: Tracer):
+    ex = J.exp(x)
+    return ex.sub(J.reciprocal(ex)).mul(0.5)
+
+
+def cosh(x: Tracer):
+    ex = J.exp(x)
+    return ex.add(J.reciprocal(ex)).mul(0.5)
+
+
+def arcsinh(x: Tracer):
+    return J.log(x.add(J.sqrt(square(x).add(1))))
+
+
+def arccosh(x: Tracer):
+    return J.log(x.add(J.sqrt(square(x).sub(1))))
+
+
+def arctanh(x: Tracer):
+    return J.log(J.add(1, x).div(J._raise(1).sub(x))).mul(0.5)
+
+
+_FINFO_MAX = {DType.Float32: 3.4028234663852886e38, DType.Float16: 65504.0, DType.Float64: 1.7976931348623157e308}
+
+
+def nanToNum(x: Tracer, nan=0.0, posinf=None, neginf=None):
+    """NaN -> `nan`, +-Inf -> `posinf` / `neginf` (default: the dtype's largest finite values) (numpy.ts:3225-3244)."""
+    x = J._raise(x)
+    x = J.where(isnan(x), nan, x)
+    if x.dtype in _FLOATS:
+        hi, lo = _FINFO_MAX[x.dtype], -_FINFO_MAX[x.dtype]
+    else:
+        hi, lo = {DType.Int32: (2**31 - 1, -2**31), DType.Uint32: (2**32 - 1, 0), DType.Bool: (1, 0)}[x.dtype]
+    x = J.where(isposinf(x), hi if posinf is None else posinf, x)
+    return J.where(isneginf(x), lo if neginf is None else neginf, x)
+
+
+# ---- array creation: lazy constants (src/frontend/array.ts:1484-1790) ---------------------------------------------
+
+def full(shape: Sequence[int], value, dtype: Optional[DType] = None) -> ConstArray:
+    if dtype is None:
+        dtype = DType.Bool if isinstance(value, bool) else DType.Float32
+    return ConstArray(tuple(shape), dtype, AluExp.const(dtype, value))
+
+
+def zeros(shape: Sequence[int], dtype: DType = DType.Float32) -> ConstArray:
+    return full(shape, 0, dtype)
+
+
+def ones(shape: Sequence[int], dtype: DType = DType.Float32) -> ConstArray:
+    return full(shape, 1, dtype)
+
+
+def zerosLike(a: Tracer, dtype: Optional[DType] = None, shape: Optional[Sequence[int]] = None) -> ConstArray:
+    return full(a.shape if shape is None else shape, 0, dtype or a.dtype)
+
+
+def onesLike(a: Tracer, dtype: Optional[DType] = None, shape: Optional[Sequence[int]] = None) -> ConstArray:
+    return full(a.shape if shape is None else shape, 1, dtype or a.dtype)
+
+
+def eye(numRows: int, numCols: Optional[int] = None, dtype: DType = DType.Float32):
+    """`idx % (cols + 1) < 1` cast to the dtype; with fewer columns than rows the transpose of the wide case, since that
+    is no modular expression of the index any more (array.ts:1515-1547)."""
+    numCols = numRows if numCols is None else numCols
+    if numCols < numRows:
+        return J.transpose(J._raise(eye(numCols, numRows, dtype)))
+    if numRows == 0:
+        return zeros([0, numCols], dtype)
+    exp = AluExp.cmplt(AluExp.mod(AluVar.gidx, AluExp.i32(numCols + 1)), AluExp.i32(1))
+    return ConstArray((numRows, numCols), dtype, AluExp.cast(dtype, exp))
+
+
+def arange(start, stop=None, step=1, dtype: DType = DType.Int32) -> ConstArray:
+    """`start + cast(idx) * step` in the result dtype, so a fractional step in int32 adds zeros (array.ts:1570-1612)."""
+    if stop is None:
+        start, stop = 0, start
+    if step == 0:
+        raise ValueError(f"Invalid step for arange: {step}. Step must be non-zero.")
+    size = max(0, math.ceil((stop - start) / step))
+    if size == 0:
+        return zeros([0], dtype)
+    exp = AluExp.add(AluExp.const(dtype, start), AluExp.mul(AluExp.cast(dtype, AluVar.gidx), AluExp.const(dtype, step)))
+    return ConstArray((size,), dtype, exp)
+
+
+def tri(n: int, m: Optional[int] = None, k: int = 0, dtype: DType = DType.Float32):
+    """`arange(k, n + k)[:, None] >= arange(m)` (array.ts:1614-1635)."""
+    m = n if m is None else m
+    for name, v in (("n", n), ("m", m)):
+        if not isinstance(v, int) or v < 0:
+            raise ValueError(f"tri: {name} must be a non-negative integer, got {v}")
+    if not isinstance(k, int):
+        raise ValueError(f"tri: k must be an integer, got {k}")
+    rows, cols = J._raise(arange(k, n + k, 1)), J._raise(arange(0, m, 1))
+    return J.greaterEqual(rows.reshape([n, 1]), cols).astype(dtype)
+
+
+def tril(a: Tracer, k: int = 0):
+    a = J._raise(a)
+    if a.ndim < 2:
+        raise ValueError(f"tril: input array must be at least 2D, got {a.ndim}D")
+    return J.where(tri(a.shape[-2], a.shape[-1], k, DType.Bool), a, zerosLike(a))
+
+
+def triu(a: Tracer, k: int = 0):
+    a = J._raise(a)
+    if a.ndim < 2:
+        raise ValueError(f"tril: input array must be at least 2D, got {a.ndim}D")
+    return J.where(tri(a.shape[-2], a.shape[-1], k - 1, DType.Bool), zerosLike(a), a)
+
+
+def linspace(start: float, stop: float, num: int = 50, endpoint: bool = True, dtype: DType = DType.Float32) -> ConstArray:
+    """`cast(f32(start) + f32(delta / denom) * f32(idx))` (array.ts:1673-1729)."""
+    if not isinstance(num, int) or num < 0:
+        raise ValueError(f"Invalid num for linspace: {num}. Must be non-negative integer.")
+    if num == 0:
+        return zeros([0], dtype)
+    if num == 1:
+        return full([1], start, dtype)
+    if start == stop:
+        return full([num], start, dtype)
+    denom = num - 1 if endpoint else num
+    exp = AluExp.cast(dtype, AluExp.add(AluExp.f32(start), AluExp.mul(AluExp.f32((stop - start) / denom), AluExp.cast(DType.Float32, AluVar.gidx))))
+    return ConstArray((num,), dtype, exp)
+
+
+def logspace(start: float, stop: float, num: int = 50, endpoint: bool = True, base: float = 10, dtype: DType = DType.Float32):
+    return J.exp(J.mul(linspace(start, stop, num, endpoint, dtype), math.log(base)))  # array.ts:1731-1743
+
+
+def geomspace(start: float, stop: float, num: int = 50, endpoint: bool = True, dtype: DType = DType.Float32):
+    if start == 0 or stop == 0 or (start > 0) != (stop > 0):
+        raise ValueError(f"geomspace: start ({start}) and stop ({stop}) must be nonzero and have the same sign")
+    comp = dtype if dtype in _FLOATS else DType.Float32
+    y = logspace(math.log10(abs(start)), math.log10(abs(stop)), num, endpoint, 10, comp)
+    result = y.mul(-1) if start < 0 else y
+    return result.astype(dtype)
+
+
+def _window_size(name: str, M):
+    if not isinstance(M, int) or M < 0:
+        raise ValueError(f"Invalid window size for {name}: {M}. Must be a non-negative integer.")
+
+
+def bartlett(M: int):  # numpy.ts:2524-2532
+    _window_size("bartlett", M)
+    if M <= 1:
+        return ones([M])
+    return J._raise(1).sub(absolute(J._raise(linspace(-1, 1, M))))
+
+
+def hann(M: int):
+    return J.cos(linspace(0, 2 * math.pi, M)).mul(-0.5).add(0.5)
+
+
+def blackman(M: int):  # numpy.ts:2552-2566
+    _window_size("blackman", M)
+    if M <= 1:
+        return ones([M])
+    return J.cos(linspace(0, 2 * math.pi, M)).mul(-0.5).add(J.cos(linspace(0, 4 * math.pi, M)).mul(0.08)).add(0.42)
+
+
+# ---- shapes, joins and selections (src/library/numpy.ts:792-1500) --------------------------------------------------
+
+def _as_array(x):
+    """A Python number becomes a 0-d constant array (what the reference's fudgeArray makes of it) rather than a literal
+    inlined into the expression: Pad and Concatenate act on views, and a bare literal has none."""
+    if isinstance(x, bool):
+        return J._raise(full([], x))
+    if isinstance(x, (int, float)):
+        return J._raise(full([], float(x)))
+    return J._raise(x)
+
+
+def ravel(a):
+    return _as_array(a).reshape([-1])
+
+
+def squeeze(a: Tracer, axis=None):
+    a = J._raise(a)
+    if axis is None:
+        axis = [i for i, d in enumerate(a.shape) if d == 1]
+    axis = J._normalize_axis(axis, a.ndim)
+    if any(a.shape[i] != 1 for i in axis):
+        raise ValueError("Cannot squeeze axis with size != 1")
+    return a.reshape([d for i, d in enumerate(a.shape) if i not in axis])
+
+
+def expandDims(a: Tracer, axis):
+    a = J._raise(a)
+    axis = [axis] if isinstance(axis, int) else list(axis)
+    nd = a.ndim + len(axis)
+    norm = [x + nd if x < 0 else x for x in axis]
+    if any(x < 0 or x >= nd for x in norm):
+        raise ValueError(f"expandDims: axis {axis} out of bounds for array of dimension {nd}")
+    if len(set(norm)) != len(norm):
+        raise ValueError("expandDims: repeated axis")
+    src = iter(a.shape)
+    return a.reshape([1 if i in norm else next(src) for i in range(nd)])
+
+
+def broadcastTo(a, shape: Sequence[int]):
+    a = J._raise(a)
+    if len(shape) < a.ndim:
+        raise ValueError(f"broadcastTo: target shape {list(shape)} has fewer dimensions than input array: {a.ndim}")
+    return J.broadcast(a, list(shape), list(range(len(shape) - a.ndim)))
+
+
+def broadcastArrays(*xs):
+    xs = [J._raise(x) for x in xs]
+    shape: Sequence[int] = ()
+    for x in xs:
+        shape = J.generalBroadcast(tuple(shape), tuple(x.shape))
+    return [broadcastTo(x, shape) for x in xs]
+
+
+def repeat(a: Tracer, repeats: int, axis: Optional[int] = None):
+    """Each element `repeats` times in a row: broadcast a new axis after `axis`, then merge it (numpy.ts:1254-1276)."""
+    if not isinstance(repeats, int) or repeats < 0:
+        raise ValueError(f"repeat: repeats must be a non-negative integer, got {repeats}")
+    a = J._raise(a)
+    if axis is None:
+        a, axis = ravel(a), 0
+    (axis,) = J._normalize_axis(axis, a.ndim)
+    if repeats == 1:
+        return a
+    wide = list(a.shape[:axis + 1]) + [repeats] + list(a.shape[axis + 1:])
+    final = list(a.shape[:axis]) + [a.shape[axis] * repeats] + list(a.shape[axis + 1:])
+    return J.broadcast(a, wide, [axis + 1]).reshape(final)
+
+
+def tile(a: Tracer, reps):
+    """Whole-array copies: a new leading axis per repeated dimension, then merged (numpy.ts:1283-1310)."""
+    a = J._raise(a)
+    reps = [reps] if isinstance(reps, int) else list(reps)
+    if any(not isinstance(r, int) or r < 0 for r in reps):
+        raise ValueError(f"tile: reps must be non-negative integers, got {reps}")
+    ndiff = len(reps) - a.ndim
+    if ndiff > 0:
+        a = a.reshape([1] * ndiff + list(a.shape))
+    if ndiff < 0:
+        reps = [1] * (-ndiff) + reps
+    wide, axes = [], []
+    for i in range(a.ndim):
+        if reps[i] > 1:
+            wide.append(reps[i])
+            axes.append(len(wide) - 1)
+        wide.append(a.shape[i])
+    final = [d * r for d, r in zip(a.shape, reps)]
+    if any(r == 0 for r in reps):
+        return zeros(final, a.dtype)
+    return J.broadcast(a, wide, axes).reshape(final)
+
+
+def pad(x: Tracer, width):
+    """Width as one number, one pair (both for every axis), a pair per axis, or {axis: pair} (core.ts:500-527)."""
+    x = J._raise(x)
+    nd = x.ndim
+    is_pair = lambda w: isinstance(w, (list, tuple)) and len(w) == 2 and all(isinstance(v, int) for v in w)
+    if isinstance(width, int):
+        w = [(width, width)]
+    elif is_pair(width):
+        w = [tuple(width)]
+    elif isinstance(width, dict):
+        w = [(0, 0)] * nd
+        for k, v in width.items():
+            w[J._normalize_axis(int(k), nd)[0]] = tuple(v)
+    elif not all(is_pair(p) for p in width):
+        raise TypeError(f"Invalid pad() type: {width}")
+    else:
+        w = [tuple(p) for p in width]
+    if len(w) == 1:
+        w = [w[0]] * nd
+    elif len(w) != nd:
+        raise ValueError(f"Invalid pad(): expected {nd} axes, got {len(w)}")
+    return J.pad(x, w)
+
+
+def _split_by_sizes(a: Tracer, sizes: List[int], axis: int):
+    """Groups of at most eight outputs per Split (numpy.ts:912-935)."""
+    results: List[Tracer] = []
+    i = 0
+    while i < len(sizes):
+        if i + 8 >= len(sizes):
+            results.extend(J.split(a, axis, sizes[i:]))
+            break
+        outs = J.split(a, axis, sizes[i:i + 7] + [sum(sizes[i + 7:])])
+        results.extend(outs[:-1])
+        a = outs[-1]
+        i += 7
+    return results
+
+
+def split(a: Tracer, indicesOrSections, axis: int = 0):
+    a = J._raise(a)
+    (axis,) = J._normalize_axis(axis, a.ndim)
+    size = a.shape[axis]
+    if isinstance(indicesOrSections, int):
+        if size % indicesOrSections != 0:
+            raise ValueError(f"Array of size {size} cannot be split into {indicesOrSections} equal parts")
+        sizes = [size // indicesOrSections] * indicesOrSections
+    else:
+        bounds = [0] + [i + size if i < 0 else i for i in indicesOrSections] + [size]
+        sizes = [bounds[i + 1] - bounds[i] for i in range(len(bounds) - 1)]
+    return _split_by_sizes(a, sizes, axis)
+
+
+def arraySplit(a: Tracer, indicesOrSections, axis: int = 0):
+    a = J._raise(a)
+    (axis,) = J._normalize_axis(axis, a.ndim)
+    if not isinstance(indicesOrSections, int):
+        return split(a, indicesOrSections, axis)
+    size = a.shape[axis]
+    part, rem = divmod(size, indicesOrSections)
+    return _split_by_sizes(a, [part + 1] * rem + [part] * (indicesOrSections - rem), axis)
+
+
+def dsplit(a: Tracer, indicesOrSections):
+    if J._raise(a).ndim < 3:
+        raise ValueError("dsplit only works on arrays of 3 or more dimensions")
+    return split(a, indicesOrSections, 2)
+
+
+def hsplit(a: Tracer, indicesOrSections):
+    a = J._raise(a)
+    if a.ndim == 0:
+        raise ValueError("hsplit only works on arrays of 1 or more dimensions")
+    return split(a, indicesOrSections, 1 if a.ndim > 1 else 0)
+
+
+def vsplit(a: Tracer, indicesOrSections):
+    return split(a, indicesOrSections, 0)
+
+
+def concatenate(xs: Sequence[Tracer], axis: int = 0):
+    """In groups of eight operands per Concatenate (numpy.ts:937-962)."""
+    xs = [J._raise(x) for x in xs]
+    if not xs:
+        raise ValueError("Need at least one array to concatenate")
+    (axis,) = J._normalize_axis(axis, xs[0].ndim)
+    for x in xs[1:]:
+        if x.ndim != xs[0].ndim or any(j != axis and d != xs[0].shape[j] for j, d in enumerate(x.shape)):
+            raise ValueError(f"Cannot concatenate arrays {list(xs[0].shape)} and {list(x.shape)} along axis {axis}")
+    result = xs[0]
+    for i in range(1, len(xs), 7):
+        result = J.concatenate([result] + xs[i:i + 7], axis)
+    return result
+
+
+def unstack(x: Tracer, axis: int = 0):
+    x = J._raise(x)
+    if x.ndim == 0:
+        raise ValueError("unstack requires arrays with rank > 0")
+    (axis,) = J._normalize_axis(axis, x.ndim)
+    if x.shape[axis] == 0:
+        return []
+    return [squeeze(p, axis) for p in split(x, x.shape[axis], axis)]
+
+
+def _same_rank(xs, name):
+    xs = [_as_array(x) for x in xs]
+    if not xs:
+        raise ValueError(f"Need at least one array to {name}")
+    if any(x.ndim != xs[0].ndim for x in xs):
+        raise ValueError(f"Cannot stack different ranks: {[x.ndim for x in xs]}")
+    return xs, xs[0].ndim
+
+
+def hstack(xs):
+    xs, nd = _same_rank(xs, "hstack")
+    return stack(xs) if nd == 0 else concatenate(xs, 0 if nd == 1 else 1)
+
+
+def vstack(xs):
+    xs, nd = _same_rank(xs, "vstack")
+    if nd == 0:
+        return stack(xs).reshape([-1, 1])
+    return stack(xs) if nd == 1 else concatenate(xs, 0)
+
+
+def dstack(xs):
+    xs, nd = _same_rank(xs, "dstack")
+    if nd == 0:
+        return stack(xs).reshape([1, 1, -1])
+    if nd == 1:
+        r = stack(xs, -1)
+        return r.reshape([1] + list(r.shape))
+    return stack(xs, -1) if nd == 2 else concatenate(xs, 2)
+
+
+def columnStack(xs):
+    xs, nd = _same_rank(xs, "columnStack")
+    if nd == 0:
+        return stack(xs).reshape([1, -1])
+    return stack(xs, -1) if nd == 1 else concatenate(xs, 1)
+
+
+def append(arr, values, axis: Optional[int] = None):
+    if axis is None:
+        return concatenate([ravel(arr), ravel(values)], 0)
+    return concatenate([_as_array(arr), _as_array(values)], axis)
+
+
+def select(condlist, choicelist, defaultValue=0):
+    """The first true condition picks: nested `where` from the last pair inwards (numpy.ts:1583-1603)."""
+    if len(condlist) != len(choicelist):
+        raise ValueError(f"select: condlist must have length equal to choicelist ({len(condlist)} vs {len(choicelist)})")
+    if not condlist:
+        raise ValueError("select: condlist must be non-empty")
+    out = J._raise(defaultValue)
+    for c, v in zip(reversed(condlist), reversed(choicelist)):
+        out = J.where(J._raise(c).astype(DType.Bool), v, out)
+    return out
+
+
+def arrayEqual(a1, a2, equalNaN: bool = False):
+    a1, a2 = J._raise(a1), J._raise(a2)
+    if tuple(a1.shape) != tuple(a2.shape):
+        return full([], False)
+    if equalNaN:
+        return all_(J.where(J.mul(isnan(a1), isnan(a2)), True, J.equal(a1, a2)))
+    return all_(J.equal(a1, a2))
+
+
+def arrayEquiv(a1, a2):
+    try:
+        b1, b2 = broadcastArrays(a1, a2)
+    except (ValueError, TypeError):
+        return full([], False)
+    return all_(J.equal(b1, b2))
+
+
+def isin(element, testElements, invert: bool = False):
+    """any(element[:, None] == test[None, :], 1) over the raveled operands (numpy.ts:3176-3192)."""
+    element = J._raise(element)
+    outShape = list(element.shape)
+    if _int_prod(outShape) == 0:
+        return element.astype(DType.Bool)
+    test = ravel(testElements)
+    if test.shape[0] == 0:  # nothing to compare with: the reduction's identity
+        result = full([_int_prod(outShape)], False)
+    else:
+        result = any_(J.equal(expandDims(ravel(element), 1), test), 1)
+    return J._raise(logicalNot(result) if invert else result).reshape(outShape)
+
+
+def ediff1d(ary, toEnd=None, toBegin=None):
+    """Differences of the raveled array, with `toBegin` / `toEnd` cast to its dtype on either side (numpy.ts:774-790)."""
+    arr = ravel(ary)
+    n = arr.shape[0]
+    d = J.shrink(arr, [(min(n, 1), n)]).sub(J.shrink(arr, [(0, max(n - 1, 0))]))
+    parts = [d]
+    if toBegin is not None:
+        parts.insert(0, ravel(toBegin).astype(arr.dtype))
+    if toEnd is not None:
+        parts.append(ravel(toEnd).astype(arr.dtype))
+    return parts[0] if len(parts) == 1 else concatenate(parts, 0)
+
+
+def diag(v: Tracer, k: int = 0):
+    """1-D: where(eye(n) == 1, v, 0) padded out to the k-th diagonal; 2-D: that diagonal (numpy.ts:1365-1393)."""
+    a = J._raise(v)
+    if not isinstance(k, int):
+        raise ValueError(f"k must be an integer, got {k}")
+    if a.ndim == 1:
+        n = a.shape[0]
+        ret = J.where(J.equal(eye(n), 1), a, zerosLike(a))
+        if k > 0:
+            return J.pad(ret, [(0, k), (k, 0)])
+        if k < 0:
+            return J.pad(ret, [(-k, 0), (0, -k)])
+        return ret
+    if a.ndim == 2:
+        return diagonal(a, k)
+    raise ValueError("numpy.diag only supports 1D and 2D arrays")
+
+
+def diagflat(v: Tracer, k: int = 0):
+    return diag(ravel(v), k)
+
+
+def diagIndices(n: int, ndim: int = 2):
+    if not isinstance(n, int) or n < 0:
+        raise ValueError(f"n must be a nonnegative integer, got {n}")
+    if not isinstance(ndim, int) or ndim < 0:
+        raise ValueError(f"ndim must be a nonnegative integer, got {ndim}")
+    index = arange(n)
+    return [index] * ndim
+
+
+def diagIndicesFrom(arr: Tracer):
+    a = J._raise(arr)
+    if a.ndim < 2:
+        raise ValueError(f"diagIndicesFrom: input array must be at least 2D, got {a.ndim}D")
+    if any(d != a.shape[0] for d in a.shape):
+        raise ValueError(f"diagIndicesFrom: all dimensions of input must be equal, got shape {list(a.shape)}")
+    return diagIndices(a.shape[0], a.ndim)
+
+
+def trace(a: Tracer, offset: int = 0, axis1: int = 0, axis2: int = 1):
+    return diagonal(a, offset, axis1, axis2).sum(-1)
+
+
+def meshgrid(xs: Sequence[Tracer], indexing: str = "xy"):
+    """Coordinate grids by broadcasting alone; "xy" swaps the first two (numpy.ts:2312-2345)."""
+    xs = [J._raise(x) for x in xs]
+    for x in xs:
+        if x.ndim != 1:
+            raise ValueError(f"meshgrid: all inputs must be 1D arrays, got {x.ndim}D array")
+    if len(xs) <= 1:
+        return xs
+    if indexing == "xy":
+        rb, ra, *rest = meshgrid([xs[1], xs[0]] + xs[2:], "ij")
+        return [ra, rb] + rest
+    shape = [x.shape[0] for x in xs]
+    return [J.broadcast(x, shape, [j for j in range(len(xs)) if j != i]) for i, x in enumerate(xs)]
+
+
+def indices(dimensions: Sequence[int], dtype: DType = DType.Int32, sparse: bool = False):
+    if any(not isinstance(d, int) or d < 0 for d in dimensions):
+        raise ValueError(f"indices: dimensions must be non-negative integers, got {list(dimensions)}")
+    out = []
+    for i, dim in enumerate(dimensions):
+        shape = [1] * len(dimensions)
+        shape[i] = dim
+        x = J._raise(arange(0, dim, 1, dtype)).reshape(shape)
+        out.append(x if sparse else broadcastTo(x, list(dimensions)))
+    if sparse:
+        return out
+    return stack(out) if out else zeros([0], dtype)
+
+
+def cumulativeProd(x: Tracer, axis: Optional[int] = None, includeInitial: bool = False):
+    x = J._raise(x)
+    if x.ndim == 0:
+        x = x.reshape([1])
+    if x.ndim > 1 and axis is None:
+        raise ValueError("cumulativeProd: axis is required for arrays of ndim > 1")
+    (axis,) = J._normalize_axis(axis or 0, x.ndim)
+    if includeInitial:
+        x = concatenate([onesLike(x, shape=[1 if i == axis else d for i, d in enumerate(x.shape)]), x], axis)
+    return _cumulative(AluOp.Mul, x, axis)
+
+
+def cumulativeSum(x: Tracer, axis: Optional[int] = None, includeInitial: bool = False):
+    x = J._raise(x)
+    if x.ndim == 0:
+        x = x.reshape([1])
+    if x.ndim > 1 and axis is None:
+        raise ValueError("cumulativeSum: axis is required for arrays of ndim > 1")
+    (axis,) = J._normalize_axis(axis or 0, x.ndim)
+    if includeInitial:
+        x = concatenate([zerosLike(x, shape=[1 if i == axis else d for i, d in enumerate(x.shape)]), x], axis)
+    return _cumulative(AluOp.Add, x, axis)
+
+
+def vander(x: Tracer, n: Optional[int] = None, increasing: bool = False):
+    """Powers of x as a running product over n - 1 copies, highest power first unless `increasing` (numpy.ts:2014-2034)."""
+    x = J._raise(x)
+    if x.ndim != 1:
+        raise ValueError(f"vander: input must be 1D, got {x.ndim}D")
+    n = x.shape[0] if n is None else n
+    if not isinstance(n, int) or n < 0:
+        raise ValueError(f"vander: n must be a non-negative integer, got {n}")
+    rows = x.shape[0]
+    if n <= 1:
+        return onesLike(x, shape=[rows, n])
+    tiled = broadcastTo(x.reshape([rows, 1]), [rows, n - 1])
+    result = cumulativeProd(tiled, axis=1, includeInitial=True)
+    return result if increasing else J.flip(result, 1)
+
+
+def polyval(p: Tracer, x: Tracer):
+    p, x = J._raise(p), J._raise(x)
+    if p.ndim == 0:
+        raise ValueError(f"polyval: coefficients must have at least one dimension, got {p.ndim}D")
+    n = p.shape[0]
+    powers = J._raise(vander(ravel(x), n)).reshape(list(x.shape) + [n])
+    return vecdot(moveaxis(p, 0, -1), powers)
+
+
+def _poly_align(a1, a2, name):
+    a1, a2 = J._raise(a1), J._raise(a2)
+    if a1.ndim == 0 or a2.ndim == 0:
+        raise ValueError(f"{name}: both inputs must be at least 1D arrays, got {a1.ndim}D and {a2.ndim}D")
+    swapped = a2.shape[0] > a1.shape[0]
+    base, update = (a2, a1) if swapped else (a1, a2)
+    update = broadcastTo(update, [update.shape[0]] + list(base.shape[1:]))
+    leading = base.shape[0] - update.shape[0]
+    if leading > 0:
+        update = pad(update, {0: (leading, 0)})
+    return base, update, swapped
+
+
+def polyadd(a1, a2):  # numpy.ts:2071-2102
+    base, update, _ = _poly_align(a1, a2, "polyadd")
+    return J.add(base, update)
+
+
+def polysub(a1, a2):  # numpy.ts:2109-2137
+    base, update, swapped = _poly_align(a1, a2, "polysub")
+    return update.sub(base) if swapped else base.sub(update)
+
+
+def _conv_impl(name: str, x: Tracer, y: Tracer, mode: str):
+    """1-D convolution / correlation through the Conv primitive: the longer operand is the signal
+    (numpy.ts:2255-2287)."""
+    x, y = J._raise(x), J._raise(y)
+    if x.ndim != 1 or y.ndim != 1:
+        raise ValueError(f"{name}: both inputs must be 1D arrays, got {x.ndim}D and {y.ndim}D")
+    flipOutput = False
+    if x.shape[0] < y.shape[0]:
+        x, y = y, x
+        flipOutput = name == "correlate"
+    if name == "convolve":
+        y = J.flip(y, None)
+    if mode == "valid":
+        padding = "VALID"
+    elif mode == "same":
+        padding = "SAME_LOWER"
+    elif mode == "full":
+        padding = [(y.shape[0] - 1, y.shape[0] - 1)]
+    else:
+        raise ValueError(f'{name}: invalid mode {mode}, expected "full", "same", or "valid"')
+    z = convGeneralDilated(x.reshape([1, 1, x.shape[0]]), y.reshape([1, 1, y.shape[0]]), [1], padding)
+    z = z.reshape([z.shape[-1]])
+    return J.flip(z, None) if flipOutput else z
+
+
+def convolve(x, y, mode: str = "full"):
+    return _conv_impl("convolve", x, y, mode)
+
+
+def correlate(x, y, mode: str = "valid"):
+    return _conv_impl("correlate", x, y, mode)
+
+
+def polymul(a1, a2):  # numpy.ts:2144-2168
+    a1, a2 = J._raise(a1), J._raise(a2)
+    if a1.ndim != 1 or a2.ndim != 1:
+        raise ValueError(f"polymul: both inputs must be 1D arrays, got {a1.ndim}D and {a2.ndim}D")
+    dt = resultType(a1, a2)
+    if dt not in _FLOATS:
+        dt = DType.Float32
+    a1, a2 = a1.astype(dt), a2.astype(dt)
+    if a1.shape[0] == 0:
+        a1 = J._raise(zeros([1], dt))
+    if a2.shape[0] == 0:
+        a2 = J._raise(zeros([1], dt))
+    return convolve(a1, a2, "full")
+
+
+def cross(a, b, axisa: int = -1, axisb: int = -1, axisc: int = -1, axis: Optional[int] = None):
+    """2- and 3-component cross products along an axis; 2-component operands gain a zero third component
+    (numpy.ts:2176-2229)."""
+    a, b = J._raise(a), J._raise(b)
+    if axis is not None:
+        axisa = axisb = axisc = axis
+    a, b = moveaxis(a, axisa, -1), moveaxis(b, axisb, -1)
+    da, db = a.shape[-1], b.shape[-1]
+    if da not in (2, 3) or db not in (2, 3):
+        raise ValueError(f"cross: incompatible dimensions for cross product (got {da} and {db})")
+    if da == 2 and db == 2:
+        a0, a1 = split(a, 2, -1)
+        b0, b1 = split(b, 2, -1)
+        return squeeze(a0.mul(b1).sub(a1.mul(b0)), -1)
+    if da == 2:
+        a = concatenate([a, zeros(list(a.shape[:-1]) + [1])], -1)
+    if db == 2:
+        b = concatenate([b, zeros(list(b.shape[:-1]) + [1])], -1)
+    a0, a1, a2 = split(a, 3, -1)
+    b0, b1, b2 = split(b, 3, -1)
+    c0 = a1.mul(b2).sub(a2.mul(b1))
+    c1 = a2.mul(b0).sub(a0.mul(b2))
+    c2 = a0.mul(b1).sub(a1.mul(b0))
+    return moveaxis(concatenate([c0, c1, c2], -1), -1, axisc)
+
+
+def dot(x, y):
+    """Scalar operands multiply; a 1-D y contracts with x's last axis; otherwise x's last axis against y's second to
+    last (numpy.ts:1764-1782)."""
+    x, y = J._raise(x), J._raise(y)
+    if x.ndim == 0 or y.ndim == 0:
+        return J.mul(x, y)
+    if y.ndim == 1:
+        return J.dot(x, y)
+    return lax_dot(x, y, [-1], [-2])
+
+
+def cov(x, y=None, rowvar: bool = True):
+    """Rows are variables, columns observations: centre each row, then `x @ x.T / (N - 1)` (numpy.ts:3141-3160)."""
+    x = J._raise(x)
+    if x.ndim == 1:
+        x = x.reshape([1, x.shape[0]])
+    if y is not None:
+        y = J._raise(y)
+        if y.ndim == 1:
+            y = y.reshape([1, y.shape[0]])
+        x = vstack([x, y])
+    if not rowvar:
+        x = x.transpose()
+    N = x.shape[1]
+    x = x.sub(x.mean(1, keepdims=True))
+    return dot(x, x.transpose()).div(N - 1)
+
+
+def corrcoef(x, y=None):
+    c = cov(x, y)
+    variances = diag(c)
+    return c.div(J.sqrt(outer(variances, variances)))
+
+
+def _round_to(dtype: DType, v: float) -> float:
+    import numpy as _np
+    if dtype == DType.Float64:
+        return float(v)
+    with _np.errstate(over="ignore"):  # beyond the dtype's range the rounded constant is an infinity, as Math.fround gives
+        return float(_np.float16(v)) if dtype == DType.Float16 else float(_np.float32(v))
+
+
+def unwrap(p, discont: Optional[float] = None, axis: int = -1, period: float = 2 * math.pi):
+    """Jumps of more than `discont` between neighbours are replaced by their complement modulo `period`; the scalar
+    constants are rounded to the array's dtype first so that a delta of exactly period / 2 falls the same way on every
+    backend (numpy.ts:2933-2980)."""
+    x = _floatish(J._raise(p))
+    (axis,) = J._normalize_axis(axis, x.ndim)
+    n = x.shape[axis]
+    if n <= 1:
+        return x
+    T = _round_to(x.dtype, period)
+    interval = _round_to(x.dtype, T / 2)
+    disc = _round_to(x.dtype, T / 2 if discont is None else discont)
+    head, tail = J.split(x, axis, [1, n - 1])
+    dd = tail.sub(J.shrink(x, [(0, n - 1) if i == axis else (0, d) for i, d in enumerate(x.shape)]))
+    r = J.mod(dd.add(interval), T)
+    pymod = J.where(J.less(r, 0), r.add(T), r) if T >= 0 else J.where(J.greater(r, 0), r.add(T), r)
+    ddmod = pymod.sub(interval)
+    ddmod = J.where(logicalAnd(J.equal(ddmod, -interval), J.greater(dd, 0)), interval, ddmod)
+    correction = J.where(J.less(absolute(dd), disc), 0, ddmod.sub(dd))
+    return concatenate([head, tail.add(cumsum(correction, axis))], axis)
+
+
+def applyOverAxes(func, a, axes: Sequence[int]):
+    a = J._raise(a)
+    for axis in axes:
+        b = func(a, axis)
+        if b.ndim == a.ndim:
+            a = b
+        elif b.ndim == a.ndim - 1:
+            a = expandDims(b, axis)
+        else:
+            raise ValueError("function must return array of the correct shape")
+    return a

@@ -687,3 +687,598 @@ def test_matvec_vecmat_tensordot_outer_inner_tables():
     np.testing.assert_array_equal(i.reshape(3, 5), np.inner(a, b))
     assert vd.tolist() == [float(np.vdot(a, a))]
     np.testing.assert_array_equal(vc, np.sum(a * a, axis=0))
+
+
+I32, U32, BOOL = DType.Int32, DType.Uint32, DType.Bool
+
+
+def test_min_max_fmin_fmax_abs_signbit_tables():
+    """test/numpy.test.ts:2279-2306 (minimum, also of bools), :2307-2345 (fmin ignores one NaN, broadcasts), :2347-2412
+    (maximum, fmax incl. infinities), :2414-2423 (absolute), :2438-2484 (signbit: signed zero, the sign of a NaN, int32,
+    uint32 and bool inputs)."""
+    x, y = f32([1, 2, 3]), f32([4, 2, 0])
+    _, (mn, mx, fn, fx) = run(lambda a, b: [J.minimum(a, b), J.maximum(a, b), L.fmin(a, b), L.fmax(a, b)], x, y)
+    assert mn.tolist() == [1, 2, 0] and mx.tolist() == [4, 2, 3] and fn.tolist() == [1, 2, 0] and fx.tolist() == [4, 2, 3]
+    _, (mb,) = _run_typed(lambda a, b: J.minimum(a, b), [np.array([1, 0, 1], np.int32), np.array([0, 0, 1], np.int32)], [BOOL, BOOL])
+    assert mb.tolist() == [0, 0, 1]
+    nan, inf = np.nan, np.inf
+    _, (a,) = run(lambda p, q: L.fmin(p, q), f32([nan, 2, nan, -inf]), f32([5, nan, nan, 3]))
+    np.testing.assert_array_equal(a, f32([5, 2, nan, -inf]))
+    _, (b,) = run(lambda p, q: L.fmin(p, q), f32([[1, 5], [4, 2]]), f32([3]))
+    assert b.tolist() == [1, 3, 3, 2]
+    _, (c,) = run(lambda p, q: L.fmax(p, q), f32([[1, 5], [4, 2]]), f32([3, 3]))
+    assert c.tolist() == [3, 5, 4, 3]
+    _, (d,) = run(lambda p, q: L.fmax(p, q), f32([1, nan, nan, 5]), f32([nan, 3, nan, 2]))
+    np.testing.assert_array_equal(d, f32([1, 3, nan, 5]))
+    _, (e,) = run(lambda p, q: L.fmax(p, q), f32([-inf, inf, nan]), f32([2, nan, -inf]))
+    np.testing.assert_array_equal(e, f32([2, inf, -inf]))
+    _, (ab,) = run(lambda p: L.absolute(p), f32([-1, 2, -3]))
+    assert ab.tolist() == [1, 2, 3]
+    _, (sb,) = run(lambda p: L.signbit(p), f32([-inf, -3, -0.0, 0, 2, inf]))
+    assert sb.tolist() == [1, 1, 1, 0, 0, 0]
+    bits = np.array([0xFFC00000, 0x7FC00000], np.uint32).view(np.float32)
+    _, (sn,) = run(lambda p: L.signbit(p), bits)
+    assert sn.tolist() == [1, 0]
+    _, (si,) = _run_typed(lambda p: L.signbit(p), [np.array([-2, 0, 3], np.int32)], [I32])
+    _, (su,) = _run_typed(lambda p: L.signbit(p), [np.array([0, 1, 0xFFFFFFFF], np.uint32)], [U32])
+    _, (sl,) = _run_typed(lambda p: L.signbit(p), [np.array([0, 1], np.int32)], [BOOL])
+    assert si.tolist() == [1, 0, 0] and su.tolist() == [0, 0, 0] and sl.tolist() == [0, 0]
+
+
+def test_division_family_tables():
+    """test/numpy.test.ts:2486-2527 (reciprocal, divide, 1/0 = Inf), :2529-2560 (floorDivide rounds towards -Inf, f32
+    and int32), :2562-2609 (fmod keeps the numerator's sign, remainder the divisor's), :2611-2646 (divmod and
+    x == q*y + r), :2648-2682 (modf: both parts carry the input's sign; int32 is promoted)."""
+    _, (r, dv, z) = run(lambda a, b: [J.reciprocal(a), L.trueDivide(a, b), J._raise(a).mul(0).add(9).div(a.mul(0))], f32([1, 2, 3]), f32([4, 5, 6]))
+    np.testing.assert_allclose(r, [1, 0.5, 1 / 3], rtol=1e-6)
+    np.testing.assert_allclose(dv, [0.25, 0.4, 0.5], rtol=1e-6)
+    assert z.tolist() == [np.inf] * 3
+    x, y = [7, 7, -7, -7], [3, -3, 3, -3]
+    _, (q, rm) = run(lambda a, b: L.divmod_(a, b), f32(x), f32(y))
+    assert q.tolist() == [2, -3, -3, 2] and rm.tolist() == [1, -2, 2, -1]
+    _, (q2,) = run(lambda a, b: L.floorDivide(a, b), f32([5, -5, 10, -10]), f32([2, 2, 3, 3]))
+    assert q2.tolist() == [2, -3, 3, -4]
+    prog, (qi, ri) = _run_typed(lambda a, b: L.divmod_(a, b), [np.array(x, np.int32), np.array(y, np.int32)], [I32, I32])
+    assert qi.dtype == np.int32 and qi.tolist() == [2, -3, -3, 2] and ri.dtype == np.int32 and ri.tolist() == [1, -2, 2, -1]
+    _, (fm, rr) = run(lambda a, b: [L.fmod(a, b), L.remainder(a, b)], f32([5, 7, -9, -11]), f32([3, -4, 2, -3]))
+    assert fm.tolist() == [2, 3, -1, -2]
+    _, (r2,) = run(lambda a, b: L.remainder(a, b), f32([5, 5, -5, -5]), f32([3, -3, 3, -3]))
+    assert r2.tolist() == [2, -1, 1, -2]
+    _, (rec,) = run(lambda a, b: (lambda qr: J.add(J.mul(qr[0], b), qr[1]))(L.divmod_(a, b)), f32([5, -5, 10, -10]), f32([3, 3, 4, 4]))
+    assert rec.tolist() == [5, -5, 10, -10]
+    _, (fr, wh) = run(lambda a: L.modf(a), f32([3.5, -3.5, 0, 1.25, -2.75, 2.75]))
+    np.testing.assert_allclose(fr, [0.5, -0.5, 0, 0.25, -0.75, 0.75], atol=1e-6)
+    assert wh.tolist() == [3, -3, 0, 1, -2, 2]
+    v = f32([1.7, -4.2, 100.001, -0.5])
+    _, (back,) = run(lambda a: (lambda fw: J.add(fw[0], fw[1]))(L.modf(a)), v)
+    np.testing.assert_allclose(back, v, atol=1e-6)
+    _, (fi, wi) = _run_typed(lambda a: L.modf(a), [np.array([5, -3], np.int32)], [I32])
+    assert fi.dtype == np.float32 and wi.dtype == np.float32 and fi.tolist() == [0, 0] and wi.tolist() == [5, -3]
+
+
+def test_exponential_and_power_tables():
+    """test/numpy.test.ts:2803-2853 (exp over [-1000, 1000], exp2), :2855-2871 (expm1 near 0, rtol 2e-5), :2873-2910
+    (log, log(0), log2/log10), :2912-2928 (log1p), :2930-2946 (logaddexp, logaddexp2 without overflow), :2948-2960
+    (sqrt), :2962-2979 (cbrt of negatives), :2981-3006 (power: negative bases, power of zero), :3008-3039 (floatPower)."""
+    _, (e,) = run(lambda a: J.exp(a), f32([-1000, -100, -50, -10, 0, 10, 50, 100, 1000]))
+    np.testing.assert_allclose(e, f32([0, 3.720075976020836e-44, 1.9287498479639178e-22, 4.5399929762484854e-5, 1, 22026.465794806718,
+                                      5.184705528587072e21, 2.6881171418161356e43, np.inf]), rtol=1e-5, atol=1e-8)
+    _, (e2,) = run(lambda a: L.exp2(a), f32([10, 0]))
+    np.testing.assert_allclose(e2, [1024, 1], rtol=1e-5)
+    vals = [-1, -0.1, -0.01, -1e-4, -1e-8, 0, 1e-8, 1e-4, 0.01, 0.1, 1]
+    _, (em,) = run(lambda a: L.expm1(a), f32(vals))
+    np.testing.assert_allclose(em, np.expm1(np.array(vals)), rtol=2e-5, atol=0)
+    _, (lg, l2, l10) = run(lambda a: [J.log(a), L.log2(a), L.log10(a)], f32([1, 2, 4, 8, 0, math.e]))
+    np.testing.assert_allclose(lg[[0, 5]], [0, 1], atol=1e-6)
+    assert lg[4] == -np.inf
+    np.testing.assert_allclose(l2[:4], [0, 1, 2, 3], rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(l10[:4], np.log10([1, 2, 4, 8]), rtol=1e-5, atol=1e-6)
+    v1 = [-0.9, -0.2, -0.1, -0.01, -1e-4, -1e-8, 0, 1e-8, 1e-4, 0.01, 0.1, 0.2, 1]
+    _, (lp,) = run(lambda a: L.log1p(a), f32(v1))
+    np.testing.assert_allclose(lp, np.log1p(np.array(v1)), rtol=2e-5, atol=0)
+    _, (la, la2) = run(lambda a, b: [L.logaddexp(a, b), L.logaddexp2(a.mul(0).add(1000), b.mul(0).add(1000))], f32([1, 2, 3]), f32([4, 5, 6]))
+    np.testing.assert_allclose(la, np.logaddexp([1, 2, 3], [4, 5, 6]), rtol=1e-5)
+    np.testing.assert_allclose(la2, [1001] * 3, rtol=1e-5)
+    _, (sq,) = run(lambda a: J.sqrt(a), f32([-1, -4, 9, 1, 4]))
+    np.testing.assert_array_equal(sq, f32([np.nan, np.nan, 3, 1, 2]))
+    _, (cb,) = run(lambda a: L.cbrt(a), f32([-8, -1, 0, 1, 8]))
+    np.testing.assert_allclose(cb, [-2, -1, 0, 1, 2], rtol=1e-5, atol=1e-6)
+    _, (p3,) = run(lambda a: L.power(a, 3), f32([-1, 2, 3, 4]))
+    np.testing.assert_allclose(p3, [-1, 8, 27, 64], rtol=1e-5)
+    _, (pe, pn, p0) = run(lambda a, h, z: [L.power(3, a), L.power(-3, h), L.power(0, z)], f32([-2, 0, 0.5, 1, 2]), f32([0.5, 1.5, 2.5]), f32([-2, -1, 0, 0.5, 1, 2]))
+    np.testing.assert_allclose(pe, [1 / 9, 1, math.sqrt(3), 3, 9], rtol=1e-5)
+    assert np.isnan(pn).all()
+    np.testing.assert_array_equal(p0, f32([np.inf, np.inf, np.nan, 0, 0, 0]))
+    prog, (fp,) = _run_typed(lambda a, b: L.floatPower(a, b), [np.array([1, 2, 3, 4], np.int32), f32(3).reshape(())], [I32, F32])
+    assert fp.dtype == np.float32
+    np.testing.assert_allclose(fp, [1, 8, 27, 64], rtol=1e-5)
+    _, (fq, fr) = run(lambda a, b: [L.floatPower(a, 2), L.floatPower(b, 0.5)], f32([1.5, 2.5]), f32([4, 9, 16]))
+    np.testing.assert_allclose(fq, [2.25, 6.25], rtol=1e-5)
+    np.testing.assert_allclose(fr, [2, 3, 4], rtol=1e-5)
+
+
+def test_trigonometric_and_hyperbolic_tables():
+    """test/numpy.test.ts:4035-4056 (sinh / cosh / tanh over [-1, 1000]), :4058-4088 (sinc: 1 at 0, 0 at integers,
+    symmetric), :4118-4152 (atan, asin, acos to 5 digits), :4154-4166 (atan2 in all quadrants and on the axes)."""
+    vals = [-1, -0.7, 0, 0.5, 1.7, 10, 50, 100, 1000]
+    with np.errstate(over="ignore"):
+        _, (sh, ch, th) = run(lambda a: [L.sinh(a), L.cosh(a), L.tanh(a)], f32(vals))
+        np.testing.assert_allclose(sh, np.sinh(f32(vals)), rtol=1e-5, atol=1e-7)
+        np.testing.assert_allclose(ch, np.cosh(f32(vals)), rtol=1e-5)
+    np.testing.assert_allclose(th, np.tanh(vals), rtol=1e-5, atol=1e-7)
+    _, (ti,) = run(lambda a: L.tanh(a), f32([np.inf]))
+    assert ti.tolist() == [1]
+    _, (sc,) = run(lambda a: L.sinc(a), f32([0, 0.5, 1, 2, 3, -1, -2, -3, 0.1, -0.1, 1.5, -1.5, 2.5, -2.5]))
+    np.testing.assert_allclose(sc[:3], [1, 2 / math.pi, 0], atol=2e-7)
+    np.testing.assert_allclose(sc[3:8], 0, atol=1e-5)
+    np.testing.assert_array_equal(sc[8::2], sc[9::2])
+    av = [-1000, -100, -10, -1, 0, 1, 10, 100, 1000, np.inf]
+    _, (at,) = run(lambda a: J.atan(a), f32(av))
+    np.testing.assert_allclose(at, np.arctan(av), atol=5e-6)
+    sv = [-1, -0.7, 0, 0.5, 1]
+    _, (as_, ac) = run(lambda a: [J.asin(a), L.acos(a)], f32(sv))
+    np.testing.assert_allclose(as_, np.arcsin(sv), atol=5e-6)
+    np.testing.assert_allclose(ac, np.arccos(sv), atol=5e-6)
+    yy, xx = [3, 5, -7, -2, 4, -6, 0, 0, 1.5, -2.5], [4, -2, -3, 8, 0, 0, 5, -9, 1.5, -2.5]
+    _, (a2,) = run(lambda p, q: L.atan2(p, q), f32(yy), f32(xx))
+    np.testing.assert_allclose(a2, np.arctan2(yy, xx), atol=5e-6)
+    _, (hy, tn) = run(lambda p, q: [L.hypot(p, q), L.tan(p)], f32([3, 5]), f32([4, 12]))
+    np.testing.assert_allclose(hy, [5, 13], rtol=1e-6)
+    np.testing.assert_allclose(tn, np.tan([3.0, 5.0]), rtol=1e-4)
+
+
+def test_nan_to_num_rounding_and_copysign_tables():
+    """test/numpy.test.ts:4305-4341 (nanToNum: defaults and overrides), :5152-5165 (copysign; a zero sign source gives
+    0), :5167-5190 (round: half to even, decimals, negative decimals; rint)."""
+    nan, inf = np.nan, np.inf
+    _, (a, b) = run(lambda p: [L.nanToNum(p), L.nanToNum(p, nan=99)], f32([1, nan, 3]))
+    assert a.tolist() == [1, 0, 3] and b.tolist() == [1, 99, 3]
+    _, (c, d, e) = run(lambda p: [L.nanToNum(p, posinf=999), L.nanToNum(p, neginf=-999), L.nanToNum(p)], f32([1, inf, -inf]))
+    assert c.tolist() == [1, 999, np.finfo(np.float32).min] and d.tolist() == [1, np.finfo(np.float32).max, -999]
+    np.testing.assert_allclose(e[1:], [3.40282347e38, -3.40282347e38], rtol=1e-7)
+    _, (f,) = run(lambda p: L.nanToNum(p, nan=0, posinf=100, neginf=-100), f32([nan, inf, -inf, 42]))
+    assert f.tolist() == [0, 100, -100, 42]
+    _, (cs, cz) = run(lambda p, q: [L.copysign(p, q), L.copysign(p, q.mul(0))], f32([1, -2, 3, -4]), f32([-1, 1, -1, 1]))
+    assert cs.tolist() == [-1, 2, -3, 4] and cz.tolist() == [0, 0, 0, 0]
+    _, (r0, ri) = run(lambda p: [L.round_(p, 0), L.rint(p)], f32([1.4, 1.5, 2.5, 3.5, -0.5, 3.6]))
+    np.testing.assert_allclose(r0, [1, 2, 2, 4, 0, 4], atol=1e-6)
+    np.testing.assert_allclose(ri, [1, 2, 2, 4, 0, 4], atol=1e-6)
+    _, (r2,) = run(lambda p: L.round_(p, 2), f32([1.234, 2.567, 3.891]))
+    np.testing.assert_allclose(r2, [1.23, 2.57, 3.89], rtol=1e-6)
+    _, (rn,) = run(lambda p: L.round_(p, -2), f32([123, 456, 789]))
+    np.testing.assert_allclose(rn, [100, 500, 800], rtol=1e-6)
+
+
+def test_logical_and_bitwise_tables():
+    """test/numpy.test.ts:5038-5081 (logical and / or / xor / not over numbers and booleans), :5083-5130 (bitwise and /
+    or / xor on uint32 and bool, invert on uint32 / bool / int32), :5132-5150 (shifts; the right shift is logical)."""
+    a, b = f32([1, 0, 3, 0]), np.array([0, 0, 1, 0], np.int32)
+    _, (an,) = _run_typed(lambda p, q: L.logicalAnd(p, q), [a, b], [F32, BOOL])
+    assert an.tolist() == [0, 0, 1, 0]
+    _, (af,) = run(lambda p, q: L.logicalAnd(p, q), f32([1.5, 0.0, -2.0]), f32([0.5, 0.0, 1.0]))
+    assert af.tolist() == [1, 0, 1]
+    _, (o, x, n) = run(lambda p, q: [L.logicalOr(p, q), L.logicalXor(p, q), L.logicalNot(p)], a, f32([0, 0, 1, 0]))
+    assert o.tolist() == [1, 0, 1, 0] and x.tolist() == [1, 0, 0, 0] and n.tolist() == [0, 1, 0, 1]
+    u = lambda *v: np.array(v, np.uint32)
+    _, (ba,) = _run_typed(lambda p, q: L.bitwiseAnd(p, q), [u(0xFF00FF00, 0x0F0F0F0F), u(0x00FF00FF, 0xF0F0F0F0)], [U32, U32])
+    _, (bo,) = _run_typed(lambda p, q: L.bitwiseOr(p, q), [u(0xFF00FF00, 7), u(0x00FF00FF, 3)], [U32, U32])
+    _, (bx,) = _run_typed(lambda p, q: L.bitwiseXor(p, q), [u(0xAAAAAAAA, 7), u(0x55555555, 3)], [U32, U32])
+    assert ba.tolist() == [0, 0] and bo.tolist() == [0xFFFFFFFF, 7] and bx.tolist() == [0xFFFFFFFF, 4]
+    _, (bb,) = _run_typed(lambda p, q: L.bitwiseAnd(p, q), [np.array([1, 1, 0, 0], np.int32), np.array([1, 0, 1, 0], np.int32)], [BOOL, BOOL])
+    assert bb.tolist() == [1, 0, 0, 0]
+    _, (iu,) = _run_typed(lambda p: L.invert(p), [u(0, 0xFFFFFFFF)], [U32])
+    _, (ib,) = _run_typed(lambda p: L.invert(p), [np.array([1, 0], np.int32)], [BOOL])
+    _, (ii,) = _run_typed(lambda p: L.invert(p), [np.array([0, -3], np.int32)], [I32])
+    assert iu.tolist() == [0xFFFFFFFF, 0] and ib.tolist() == [0, 1] and ii.tolist() == [-1, 2]
+    with pytest.raises(TypeError):
+        J.jit(lambda p: L.invert(p), [ShapedArray((2,), F32)])
+    _, (sl,) = _run_typed(lambda p, q: L.leftShift(p, q), [u(1, 1, 1), u(0, 8, 16)], [U32, U32])
+    _, (sr,) = _run_typed(lambda p, q: L.rightShift(p, q), [u(256, 65536, 0xFFFF0000), u(0, 1, 8)], [U32, U32])
+    assert sl.tolist() == [1, 256, 65536] and sr.tolist() == [256, 32768, 0x00FFFF00]
+
+
+def run0(fn):
+    """A program without inputs: everything comes from lazy constants."""
+    return run(fn)[1]
+
+
+def test_creation_tables():
+    """test/numpy.test.ts:563-590 (eye: square, wide, scaled), :833-884 (tri, triu, tril), :886-926 (arange incl. empty
+    ranges and a fractional step in int32), :928-953 (linspace), :955-985 (logspace), :987-1032 (geomspace), :143-175
+    (bartlett), :4090-4116 (blackman)."""
+    e3, e23, e35, e32 = run0(lambda: [J._raise(L.eye(3)).mul(1), J._raise(L.eye(2, 3)).mul(1), J._raise(L.eye(3, 5)).mul(-42), J._raise(L.eye(3, 2)).mul(1)])
+    np.testing.assert_array_equal(e3.reshape(3, 3), np.eye(3))
+    np.testing.assert_array_equal(e23.reshape(2, 3), np.eye(2, 3))
+    np.testing.assert_array_equal(e35.reshape(3, 5), -42 * np.eye(3, 5))
+    np.testing.assert_array_equal(e32.reshape(3, 2), np.eye(3, 2))
+    t3, t24 = run0(lambda: [L.tri(3), L.tri(2, 4, 1)])
+    np.testing.assert_array_equal(t3.reshape(3, 3), np.tri(3))
+    np.testing.assert_array_equal(t24.reshape(2, 4), np.tri(2, 4, 1))
+    x = np.arange(24, dtype=np.int32).reshape(2, 3, 4)
+    _, (up, lo) = _run_typed(lambda a: [L.triu(a), L.tril(a)], [x], [I32])
+    np.testing.assert_array_equal(up.reshape(x.shape), np.triu(x))
+    np.testing.assert_array_equal(lo.reshape(x.shape), np.tril(x))
+    a5, a0, an, a2, a3, a3n, a3m = run0(lambda: [J._raise(c).add(0) for c in (L.arange(5), L.arange(0), L.arange(-10), L.arange(50, 60), L.arange(0, 10, 2), L.arange(10, 0, -2), L.arange(0, -10, -2))])
+    assert a5.tolist() == [0, 1, 2, 3, 4] and a0.tolist() == [] and an.tolist() == [] and a2.tolist() == list(range(50, 60))
+    assert a3.tolist() == [0, 2, 4, 6, 8] and a3n.tolist() == [10, 8, 6, 4, 2] and a3m.tolist() == [0, -2, -4, -6, -8]
+    fi, ff = run0(lambda: [J._raise(L.arange(0, 1, 0.2)).add(0), J._raise(L.arange(0, 1, 0.2, F32)).add(0)])
+    assert fi.tolist() == [0, 0, 0, 0, 0]
+    np.testing.assert_allclose(ff, [0, 0.2, 0.4, 0.6, 0.8], rtol=1e-6)
+    l5, l3, l2, l1, l50 = run0(lambda: [J._raise(L.linspace(0, 1, n)).add(0) for n in (5, 3, 2, 1, 50)])
+    assert l5.tolist() == [0, 0.25, 0.5, 0.75, 1] and l3.tolist() == [0, 0.5, 1] and l2.tolist() == [0, 1] and l1.tolist() == [0]
+    assert l50.shape == (50,) and l50[0] == 0 and l50[49] == 1 and abs(l50[25] - 25 / 49) < 1e-6
+    g10, g2, gne, g50 = run0(lambda: [L.logspace(0, 2, 3), L.logspace(0, 3, 4, True, 2), L.logspace(0, 2, 4, False), L.logspace(0, 1)])
+    np.testing.assert_allclose(g10, [1, 10, 100], rtol=1e-5)
+    np.testing.assert_allclose(g2, [1, 2, 4, 8], rtol=1e-5)
+    np.testing.assert_allclose(gne, [1, 10 ** 0.5, 10, 10 ** 1.5], rtol=1e-5)
+    assert g50.shape == (50,) and abs(g50[0] - 1) < 1e-5 and abs(g50[49] - 10) < 1e-4
+    q = run0(lambda: [L.geomspace(1, 1000, 4), L.geomspace(1, 256, 9), L.geomspace(1000, 1, 4), L.geomspace(-1000, -1, 4), L.geomspace(1, 10000, 4, False)])
+    for got, want in zip(q, ([1, 10, 100, 1000], [2 ** i for i in range(9)], [1000, 100, 10, 1], [-1000, -100, -10, -1], [1, 10, 100, 1000])):
+        np.testing.assert_allclose(got, want, rtol=1e-5)
+    for bad in ((0, 10), (1, 0), (-1, 10)):
+        with pytest.raises(ValueError):
+            L.geomspace(*bad, 5)
+    b5, b4, b9, b1, b2 = run0(lambda: [J._raise(L.bartlett(n)).mul(1) for n in (5, 4, 9, 1, 2)])
+    np.testing.assert_allclose(b5, [0, 0.5, 1, 0.5, 0], atol=1e-7)
+    np.testing.assert_allclose(b4, [0, 2 / 3, 2 / 3, 0], rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(b9, np.bartlett(9), atol=1e-6)
+    assert b1.tolist() == [1] and b2.tolist() == [0, 0]
+    (bs,) = run0(lambda: L.bartlett(5).sum())
+    np.testing.assert_allclose(bs, [2], rtol=1e-6)
+    k5, k10, k1 = run0(lambda: [J._raise(L.blackman(n)).mul(1) for n in (5, 10, 1)])
+    np.testing.assert_allclose(k5, [0, 0.34, 1, 0.34, 0], atol=1e-6)
+    np.testing.assert_allclose(k10, np.blackman(10), atol=1e-6)
+    assert k1.tolist() == [1]
+    for fn in (L.bartlett, L.blackman):
+        for bad in (-1, 0.5):
+            with pytest.raises(ValueError, match="non-negative integer"):
+                fn(bad)
+
+
+def test_diag_family_tables():
+    """test/numpy.test.ts:592-628 (diag: build from 1-D, read from 2-D, off-diagonals), :630-682 (diagflat), :684-724
+    (diagIndices, also used to gather the diagonal), :726-774 (diagonal over chosen axes, trace), :776-831
+    (diagIndicesFrom)."""
+    _, (d,) = run(lambda v: L.diag(v), f32([1, 2, 3]))
+    np.testing.assert_array_equal(d.reshape(3, 3), np.diag([1, 2, 3]))
+    m = f32(np.arange(1, 10).reshape(3, 3))
+    _, (d0, d1) = run(lambda a: [L.diag(a).mul(1), L.diag(a, 1).mul(1)], m)
+    assert d0.tolist() == [1, 5, 9] and d1.tolist() == [2, 6]
+    _, (u, l) = run(lambda v: [L.diag(v, 1), L.diag(v, -2)], f32([1, 2]))
+    np.testing.assert_array_equal(u.reshape(3, 3), np.diag([1, 2], 1))
+    np.testing.assert_array_equal(l.reshape(4, 4), np.diag([1, 2], -2))
+    _, (f0, f1) = run(lambda a: [L.diagflat(a), L.diagflat(a, 1)], f32([[1, 2], [3, 4]]))
+    np.testing.assert_array_equal(f0.reshape(4, 4), np.diagflat([[1, 2], [3, 4]]))
+    np.testing.assert_array_equal(f1.reshape(5, 5), np.diagflat([[1, 2], [3, 4]], 1))
+    _, (fm,) = run(lambda a: L.diagflat(a, -1), f32([1, 2]))
+    np.testing.assert_array_equal(fm.reshape(3, 3), np.diagflat([1, 2], -1))
+    rows, cols = L.diagIndices(3)
+    assert rows is cols and rows.dtype == I32 and len(L.diagIndices(2, 3)) == 3 and L.diagIndices(3, 0) == []
+    r3, = run0(lambda: J._raise(rows).add(0))
+    assert r3.tolist() == [0, 1, 2]
+    _, (g,) = run(lambda a: J.gather(a, [J._raise(i) for i in L.diagIndicesFrom(a)], [0, 1], 0), m)
+    assert g.tolist() == [1, 5, 9]
+    with pytest.raises(ValueError, match="nonnegative integer"):
+        L.diagIndices(-1)
+    with pytest.raises(ValueError, match="nonnegative integer"):
+        L.diagIndices(3, -1)
+    with pytest.raises(ValueError, match="all dimensions of input must be equal"):
+        J.jit(lambda a: L.diagIndicesFrom(a), [ShapedArray((3, 4), F32)])
+    with pytest.raises(ValueError, match="at least 2D"):
+        J.jit(lambda a: L.diagIndicesFrom(a), [ShapedArray((3,), F32)])
+    a = f32(np.arange(12).reshape(3, 2, 2))
+    _, (p, q, r, s) = run(lambda t: [L.diagonal(t, 0, 1, 2).mul(1), L.diagonal(t, 0, 0, 1).mul(1), L.diagonal(t, 1, 0, 1).mul(1), L.diagonal(t, 1, 1, 0).mul(1)], a)
+    np.testing.assert_array_equal(p.reshape(3, 2), np.diagonal(a, 0, 1, 2))
+    np.testing.assert_array_equal(q.reshape(2, 2), np.diagonal(a, 0, 0, 1))
+    np.testing.assert_array_equal(r.reshape(2, 1), np.diagonal(a, 1, 0, 1))
+    np.testing.assert_array_equal(s.reshape(2, 2), np.diagonal(a, 1, 1, 0))
+    _, (t0, t1) = run(lambda t: [L.trace(t), L.trace(t, 1)], f32(np.arange(9).reshape(3, 3)))
+    assert t0.tolist() == [12] and t1.tolist() == [6]
+
+
+def test_where_select_equality_and_membership_tables():
+    """test/numpy.test.ts:1034-1075 (where incl. scalar broadcasting), :1077-1164 (select: first match wins, default,
+    numeric conditions, broadcasting, dtype promotion, errors), :1166-1183 (equal / notEqual), :1185-1247 (arrayEqual
+    with and without equalNaN, arrayEquiv), :1249-1335 (isin: invert, flattened test set, empty operands, NaN)."""
+    x, y, z = f32([1, 2, 3]), f32([4, 5, 6]), np.array([1, 0, 1], np.int32)
+    _, (w,) = _run_typed(lambda a, b, c: J.where(c, a, b), [x, y, z], [F32, F32, BOOL])
+    assert w.tolist() == [1, 5, 3]
+    _, (w1, w2, w3) = _run_typed(lambda c, v: [J.where(c, 1, 3), J.where(False, 1, v), J.where(True, 7, v)], [np.array([1, 0, 1, 1], np.int32), f32([10, 11, 12, 13])], [BOOL, F32])
+    assert w1.tolist() == [1, 3, 1, 1] and w2.tolist() == [10, 11, 12, 13] and w3.tolist() == [7, 7, 7, 7]
+    ar = np.arange(6, dtype=np.int32)
+    _, (s1, s2, s3) = _run_typed(lambda a: [L.select([J.less(a, 3), J.greater(a, 3)], [J.neg(a), L.square(a)], 42),
+                                            L.select([J.lessEqual(a, 4), J.greater(a, 3)], [a, L.square(a)], 55),
+                                            L.select([J.greater(a, 1)], [a])], [ar], [I32])
+    assert s1.tolist() == [0, -1, -2, 42, 16, 25] and s2.tolist() == [0, 1, 2, 3, 4, 25] and s3.tolist() == [0, 0, 2, 3, 4, 5]
+    _, (s4,) = run(lambda p, q: L.select([p, q], [10, 20], 30), f32([0, 1, -2]), f32([1, 0, 0]))
+    assert s4.tolist() == [20, 10, 10]
+    _, (s5,) = _run_typed(lambda c, d, v: L.select([c, d], [1, v], -1), [np.array([[1, 0], [0, 1]], np.int32), np.array([0, 1], np.int32), f32([[10], [20]])], [BOOL, BOOL, F32])
+    assert s5.tolist() == [1, 10, -1, 1]
+    prog, (s6,) = _run_typed(lambda a, c: L.select([J.less(a, 1)], [c], 2), [np.arange(3, dtype=np.int32), f32([0.5, 1.5, 2.5])], [I32, F32])
+    assert s6.dtype == np.float32 and s6.tolist() == [0.5, 2, 2]
+    with pytest.raises(ValueError, match="condlist must have length equal to choicelist"):
+        L.select([True], [])
+    with pytest.raises(ValueError, match="non-empty"):
+        L.select([], [])
+    _, (eq, ne) = run(lambda a, b: [J.equal(a, b), J.notEqual(a, b)], f32([1, 2, 3, 4]), f32([4, 5, 3, 4]))
+    assert eq.tolist() == [0, 0, 1, 1] and ne.tolist() == [1, 1, 0, 0]
+    nan = np.nan
+    _, (e1, e2, e3, e4) = run(lambda a, b, c, d: [L.arrayEqual(a, a.mul(1)), L.arrayEqual(a, b), L.arrayEqual(c, d), L.arrayEqual(c, d, equalNaN=True)], f32([1, 2, 3]), f32([1, 2, 4]), f32([1, nan]), f32([1, nan]))
+    assert (e1.tolist(), e2.tolist(), e3.tolist(), e4.tolist()) == ([1], [0], [0], [1])
+    _, (e5,) = run(lambda a, b: J._raise(L.arrayEqual(a, b)).add(False), f32([1, 2, 3]), f32([1, 2]))
+    assert e5.tolist() == [0]
+    _, (q1, q2, q3) = run(lambda a, b, c: [L.arrayEquiv(a, c), L.arrayEquiv(b, c), J._raise(L.arrayEquiv(c, c.reshape([1, 2]).sum(1))).add(False)], f32([[1, 2], [1, 2]]), f32([[1, 2], [3, 4]]), f32([1, 2]))
+    assert q1.tolist() == [1] and q2.tolist() == [0]
+    _, (q4,) = run(lambda a, b: J._raise(L.arrayEquiv(a, b)).add(False), f32([1, 2, 3]), f32([1, 2]))
+    assert q4.tolist() == [0]
+    el, te = f32([[0, 2], [4, 6]]), f32([1, 2, 4, 8])
+    _, (i1, i2) = run(lambda a, b: [L.isin(a, b), L.isin(a, b, invert=True)], el, te)
+    assert i1.tolist() == [0, 1, 1, 0] and i2.tolist() == [1, 0, 0, 1]
+    _, (i3,) = run(lambda a, b: L.isin(a, b), f32([1, 2, 3, 4]), f32([[1, 3], [5, 7]]))
+    assert i3.tolist() == [1, 0, 1, 0]
+    _, (i4, i5) = run(lambda a, b: [J._raise(L.isin(a, b)).add(False), L.isin(a, b, invert=True)], f32([1, 2]), f32([]))
+    assert i4.tolist() == [0, 0] and i5.tolist() == [1, 1]
+    _, (i6,) = run(lambda a, b: L.isin(a, b), np.zeros((2, 0), np.float32), f32([1]))
+    assert i6.tolist() == []
+    _, (i7,) = run(lambda a, b: L.isin(a, b), f32([nan, 1]), f32([nan, 1]))
+    assert i7.tolist() == [0, 1]
+    _, (i8,) = _run_typed(lambda a, b: L.isin(a, b), [np.array([1, 2], np.int32), f32([2.0, 3.5])], [I32, F32])
+    assert i8.tolist() == [0, 1]
+
+
+def _i32(x):
+    return np.asarray(x, dtype=np.int32)
+
+
+def _parts(fn, x, dtypes=None):
+    """Run a function returning a list of pieces of one int32 array; pieces come back as flat lists."""
+    _, outs = _run_typed(fn, [x], [I32])
+    return [o.tolist() for o in outs]
+
+
+def test_pad_and_split_family_tables():
+    """test/numpy.test.ts:3105-3185 (pad: one width, per-axis pairs, {axis: pair}, arity errors, after a prior op),
+    :3187-3288 (split: equal parts, along an axis, at indices incl. empty sections, 20 parts), :3290-3340 (arraySplit),
+    :3342-3391 (unstack), :3393-3572 (dsplit / hsplit / vsplit)."""
+    _, (p1,) = run(lambda a: L.pad(a, 1), f32([1, 2, 3]))
+    _, (p2, p3) = run(lambda a: [L.pad(a, 1), L.pad(a.add(2), 1)], f32([[1, 2], [3, 4]]))
+    assert p1.tolist() == [0, 1, 2, 3, 0]
+    np.testing.assert_array_equal(p2.reshape(4, 4), np.pad([[1, 2], [3, 4]], 1))
+    np.testing.assert_array_equal(p3.reshape(4, 4), np.pad(np.array([[3, 4], [5, 6]]), 1))
+    _, (p4,) = run(lambda a: L.pad(a, [[1, 2], [3, 0]]), f32([[1]]))
+    np.testing.assert_array_equal(p4.reshape(4, 4), np.pad([[1]], [[1, 2], [3, 0]]))
+    seen = {}
+    J.jit(lambda a: seen.setdefault("y", L.pad(a, {1: (0, 2), -1: (3, 0)})), [ShapedArray((2, 3, 4, 5), F32)])
+    assert tuple(seen["y"].shape) == (2, 5, 4, 8)
+    for bad in ([], [[0, 1], [1, 2]]):
+        with pytest.raises((ValueError, TypeError)):
+            J.jit(lambda a: L.pad(a, bad), [ShapedArray((1, 2, 3), F32)])
+    J.jit(lambda a: L.pad(a, [[0, 1]]), [ShapedArray((1, 2, 3), F32)])
+    x6, x10, x12 = _i32(np.arange(6)), _i32(np.arange(10)), _i32(np.arange(12))
+    assert _parts(lambda a: L.split(a, 3), x6) == [[0, 1], [2, 3], [4, 5]]
+    for shape, ax in (([4, 3], 0), ([3, 4], 1), ([3, 4], -1)):
+        m = x12.reshape(shape)
+        got = _parts(lambda a: L.split(a, 2, ax), m)
+        assert got == [p.ravel().tolist() for p in np.split(m, 2, ax)]
+    assert _parts(lambda a: L.split(a, [3, 7]), x10) == [[0, 1, 2], [3, 4, 5, 6], [7, 8, 9]]
+    assert _parts(lambda a: L.split(a, [0, 0, 3]), _i32(np.arange(5))) == [[], [], [0, 1, 2], [3, 4]]
+    for n in (2, 3):
+        with pytest.raises(ValueError):
+            J.jit(lambda a: L.split(a, n), [ShapedArray((5,), I32)])
+    assert _parts(lambda a: (lambda ab: [J.add(ab[0], ab[1])])(L.split(a, 2)), x6) == [[3, 5, 7]]
+    assert _parts(lambda a: L.split(a, 20), _i32(np.arange(20))) == [[i] for i in range(20)]
+    assert _parts(lambda a: L.arraySplit(a, 3), _i32(np.arange(8))) == [[0, 1, 2], [3, 4, 5], [6, 7]]
+    assert _parts(lambda a: L.arraySplit(a, 5), _i32(np.arange(3))) == [[0], [1], [2], [], []]
+    assert _parts(lambda a: L.arraySplit(a, 3, -1), x10.reshape(2, 5)) == [[0, 1, 5, 6], [2, 3, 7, 8], [4, 9]]
+    assert _parts(lambda a: L.arraySplit(a, [2, 5]), _i32(np.arange(7))) == [[0, 1], [2, 3, 4], [5, 6]]
+    assert _parts(lambda a: [p.add(0) for p in L.arraySplit(a, [])], _i32(np.arange(5))) == [[0, 1, 2, 3, 4]]
+    assert _parts(lambda a: [L.concatenate(list(reversed(L.arraySplit(a, 3))))], _i32(np.arange(8))) == [[6, 7, 3, 4, 5, 0, 1, 2]]
+    m32 = x6.reshape(3, 2)
+    assert _parts(lambda a: L.unstack(a), m32) == [[0, 1], [2, 3], [4, 5]]
+    assert _parts(lambda a: L.unstack(a, -1), m32) == [[0, 2, 4], [1, 3, 5]]
+    assert _parts(lambda a: L.unstack(a), _i32([5, 7, 9])) == [[5], [7], [9]]
+    assert _parts(lambda a: [L.stack(L.unstack(a, 1), 1)], x12.reshape(2, 3, 2)) == [x12.tolist()]
+    assert _parts(lambda a: [L.stack(list(reversed(L.unstack(a))))], m32) == [[4, 5, 2, 3, 0, 1]]
+    with pytest.raises(ValueError):
+        J.jit(lambda a: L.unstack(a), [ShapedArray((), F32)])
+    assert J.jit(lambda a: L.unstack(a) + [a], [ShapedArray((0, 3), F32)]) is not None
+    x16 = _i32(np.arange(16)).reshape(2, 2, 4)
+    assert _parts(lambda a: L.dsplit(a, 2), x16) == [p.ravel().tolist() for p in np.dsplit(x16, 2)]
+    x8 = _i32(np.arange(8)).reshape(1, 2, 4)
+    assert _parts(lambda a: L.dsplit(a, [1, 3]), x8) == [[0, 4], [1, 2, 5, 6], [3, 7]]
+    assert _parts(lambda a: (lambda ab: [L.concatenate([ab[1], ab[0]], 2)])(L.dsplit(a, 2)), x8) == [[2, 3, 0, 1, 6, 7, 4, 5]]
+    with pytest.raises(ValueError, match="3 or more dimensions"):
+        J.jit(lambda a: L.dsplit(a, 3), [ShapedArray((2, 3), F32)])
+    assert _parts(lambda a: L.hsplit(a, 2), x12.reshape(3, 4)) == [[0, 1, 4, 5, 8, 9], [2, 3, 6, 7, 10, 11]]
+    assert _parts(lambda a: L.hsplit(a, 3), x6) == [[0, 1], [2, 3], [4, 5]]
+    assert _parts(lambda a: L.hsplit(a, 2), _i32(np.arange(8)).reshape(2, 2, 2)) == [[0, 1, 4, 5], [2, 3, 6, 7]]
+    assert _parts(lambda a: L.hsplit(a, [1, 4]), x12.reshape(2, 6)) == [[0, 6], [1, 2, 3, 7, 8, 9], [4, 5, 10, 11]]
+    with pytest.raises(ValueError):
+        J.jit(lambda a: L.hsplit(a, 2), [ShapedArray((2, 5), F32)])
+    with pytest.raises(ValueError, match="1 or more dimensions"):
+        J.jit(lambda a: L.hsplit(a, 1), [ShapedArray((), F32)])
+    assert _parts(lambda a: L.vsplit(a, 2), x12.reshape(4, 3)) == [list(range(6)), list(range(6, 12))]
+    assert _parts(lambda a: L.vsplit(a, [1, 3]), x12.reshape(4, 3)) == [[0, 1, 2], [3, 4, 5, 6, 7, 8], [9, 10, 11]]
+    assert _parts(lambda a: (lambda ab: [J.add(ab[0], ab[1])])(L.vsplit(a, 2)), _i32(np.arange(8)).reshape(4, 2)) == [[4, 6, 8, 10]]
+    with pytest.raises(ValueError):
+        J.jit(lambda a: L.vsplit(a, 2), [ShapedArray((5, 3), F32)])
+
+
+def test_joins_repeats_and_reshapes_tables():
+    """test/numpy.test.ts:3574-3625 (concatenate, shape mismatch, stack / vstack / hstack / dstack of scalars and
+    vectors), :4168-4203 (repeat), :4205-4240 (tile), :4458-4526 (expandDims), :4914-4949 (append), :363-413 (ediff1d),
+    :2054-2095 (meshgrid), :2097-2160 (indices)."""
+    a, b = f32([1, 2, 3]), f32([4, 5, 6])
+    _, (c,) = run(lambda p, q: L.concatenate([p, q]), a, b)
+    assert c.tolist() == [1, 2, 3, 4, 5, 6]
+    two = [ShapedArray((2, 3), F32), ShapedArray((3, 2), F32)]
+    for ax in (0, 1):
+        with pytest.raises(ValueError):
+            J.jit(lambda p, q: L.concatenate([p, q], ax), two)
+    J.jit(lambda p, q: L.concatenate([p, q.transpose()]), two)
+    _, (cj,) = run(lambda p, q, r: L.concatenate([J.flip(p, None), q, r]), f32([1, 2]), f32([3, 4]), f32([5]))
+    assert cj.tolist() == [2, 1, 3, 4, 5]
+    s = float  # numbers become 0-d arrays, as the reference's fudgeArray makes of them
+    st0, st1, vs, hs, ds = run0(lambda: [L.stack([s(2), s(3)]), L.stack([s(2), s(3)], -1), L.vstack([s(1), s(2), s(3)]), L.hstack([s(1), s(2), s(3)]), L.dstack([s(1), s(2), s(3)])])
+    assert st0.tolist() == [2, 3] and st1.tolist() == [2, 3] and vs.tolist() == [1, 2, 3] and hs.tolist() == [1, 2, 3] and ds.tolist() == [1, 2, 3]
+    for ax in (1, 2):
+        with pytest.raises((ValueError, IndexError)):
+            J.jit(lambda: L.stack([s(2), s(3)], ax), [])
+    one = np.ones(3, np.float32)
+    prog, (v2, h2, d2, c2) = run(lambda p, q: [L.vstack([p, q]), L.hstack([p, q]), L.dstack([p, q]), L.columnStack([p, q])], a, one)
+    np.testing.assert_array_equal(v2.reshape(2, 3), np.vstack([a, one]))
+    np.testing.assert_array_equal(h2, np.hstack([a, one]))
+    np.testing.assert_array_equal(d2.reshape(1, 3, 2), np.dstack([a, one]))
+    np.testing.assert_array_equal(c2.reshape(3, 2), np.column_stack([a, one]))
+    m = f32([[1, 2], [3, 4]])
+    _, (r1, r2, r3, r4) = run(lambda p, q: [L.repeat(p, 2), L.repeat(q, 2, 0), L.repeat(q, 3, 1), L.repeat(q, 2)], a, m)
+    assert r1.tolist() == [1, 1, 2, 2, 3, 3] and r4.tolist() == [1, 1, 2, 2, 3, 3, 4, 4]
+    np.testing.assert_array_equal(r2.reshape(4, 2), np.repeat(m, 2, 0))
+    np.testing.assert_array_equal(r3.reshape(2, 6), np.repeat(m, 3, 1))
+    _, (t1, t2, t3, t4) = run(lambda p, q: [L.tile(p, 2), L.tile(q, [2, 1]), L.tile(q, 3), L.tile(p, [2, 2])], a, m)
+    assert t1.tolist() == [1, 2, 3, 1, 2, 3]
+    np.testing.assert_array_equal(t2.reshape(4, 2), np.tile(m, [2, 1]))
+    np.testing.assert_array_equal(t3.reshape(2, 6), np.tile(m, 3))
+    np.testing.assert_array_equal(t4.reshape(2, 6), np.tile(a, [2, 2]))
+    shapes = {}
+    def ed(p, q):
+        outs = [L.expandDims(p, 0), L.expandDims(p, 1), L.expandDims(p, -1), L.expandDims(p, [0, 2]), L.expandDims(q, 0), L.expandDims(q, 2)]
+        shapes["s"] = [tuple(o.shape) for o in outs]
+        return [o.mul(1) for o in outs]
+    run(ed, a, m)
+    assert shapes["s"] == [(1, 3), (3, 1), (3, 1), (1, 3, 1), (1, 2, 2), (2, 2, 1)]
+    for bad in (3, -4, [0, 0]):
+        with pytest.raises(ValueError):
+            J.jit(lambda p: L.expandDims(p, bad), [ShapedArray((3,), F32)])
+    _, (ap, ap0, ap1) = run(lambda p, q, r: [L.append(p, q), L.append(p, q, 0), L.append(p, r, 1)], m, f32([[5, 6]]), f32([[5], [6]]))
+    assert ap.tolist() == [1, 2, 3, 4, 5, 6] and ap0.tolist() == [1, 2, 3, 4, 5, 6] and ap1.tolist() == [1, 2, 5, 3, 4, 6]
+    x = f32([1, 2, 4, 7, 0])
+    _, (e1, e2, e3) = run(lambda p, q, r: [L.ediff1d(p), L.ediff1d(q), L.ediff1d(p, toBegin=-99, toEnd=r)], x, f32([[1, 2, 4], [1, 6, 24]]), f32([88, 99]))
+    assert e1.tolist() == [1, 2, 3, -7] and e2.tolist() == [1, 2, -3, 5, 18] and e3.tolist() == [-99, 1, 2, 3, -7, 88, 99]
+    prog, (e4,) = _run_typed(lambda p, r: L.ediff1d(p, toBegin=-99.5, toEnd=r), [_i32(np.arange(4)), f32([1.5, 2.5])], [I32, F32])
+    assert e4.dtype == np.int32 and e4.tolist() == [-99, 1, 1, 1, 1, 2]
+    _, (e5, e6) = run(lambda p: [L.ediff1d(p), L.ediff1d(p, toBegin=1, toEnd=2)], f32([5]))
+    assert e5.tolist() == [] and e6.tolist() == [1, 2]
+    X, Y = f32([1, 2, 3]), f32([4, 5])
+    _, (gx, gy, ix, iy) = run(lambda p, q: [o.mul(1) for o in L.meshgrid([p, q]) + L.meshgrid([p, q], "ij")], X, Y)
+    wx, wy = np.meshgrid(X, Y)
+    vx, vy = np.meshgrid(X, Y, indexing="ij")
+    for got, want in ((gx, wx), (gy, wy), (ix, vx), (iy, vy)):
+        np.testing.assert_array_equal(got.reshape(want.shape), want)
+    prog3 = J.jit(lambda p, q, r: [o.mul(1) for o in L.meshgrid([p, q, r])], [ShapedArray((2,), F32), ShapedArray((3,), F32), ShapedArray((4,), F32)])
+    g23, g4, sr, sc, gf = run0(lambda: [L.indices([2, 3]), L.indices([4])] + [o.add(0) for o in L.indices([2, 3], sparse=True)] + [L.indices([2, 2], F32)])
+    np.testing.assert_array_equal(g23.reshape(2, 2, 3), np.indices([2, 3]))
+    assert g23.dtype == np.int32 and g4.tolist() == [0, 1, 2, 3] and sr.tolist() == [0, 1] and sc.tolist() == [0, 1, 2]
+    assert gf.dtype == np.float32 and gf.tolist() == np.indices([2, 2]).ravel().tolist()
+    assert L.indices([], sparse=True) == [] and tuple(L.indices([]).shape) == (0,)
+    for bad in ([2, -1], [1.5]):
+        with pytest.raises(ValueError, match="non-negative integers"):
+            L.indices(bad)
+
+
+def test_polynomial_convolution_and_statistics_tables():
+    """test/numpy.test.ts:3680-3713 (vander), :3715-3779 (polyval: scalar and array points, dtype kept, empty and
+    batched coefficients), :3781-3944 (polyadd / polysub: alignment, empty operands, batches, promotion), :3946-4005
+    (polymul), :4343-4378 (convolve / correlate in the three modes), :522-561 (cross), :4242-4290 (var, std, cov)."""
+    _, (v1, v2) = run(lambda a, b: [L.vander(a), L.vander(b, 4, increasing=True)], f32([0, 2, 3]), f32([1, 2, 3]))
+    np.testing.assert_allclose(v1.reshape(3, 3), np.vander([0, 2, 3]), rtol=1e-6)
+    np.testing.assert_allclose(v2.reshape(3, 4), np.vander([1, 2, 3], 4, increasing=True), rtol=1e-6)
+    seen = {}
+    J.jit(lambda a: seen.setdefault("v", L.vander(a, 0)), [ShapedArray((3,), F32)])
+    assert tuple(seen["v"].shape) == (3, 0)
+    with pytest.raises(ValueError, match="input must be 1D"):
+        J.jit(lambda a: L.vander(a), [ShapedArray((2, 2), F32)])
+    p = f32([3, 0, 1])
+    _, (pv0, pv1) = run(lambda c, x0, x1: [L.polyval(c, x0), L.polyval(c, x1)], p, f32(5).reshape(()), f32([0, 1, 2]))
+    assert pv0.tolist() == [76]
+    np.testing.assert_allclose(pv1, [1, 4, 13], rtol=1e-6)
+    _, (pi,) = _run_typed(lambda c, x: L.polyval(c, x), [_i32([1, 2]), _i32([3, 4])], [I32, I32])
+    assert pi.dtype == np.int32 and pi.tolist() == [5, 6]
+    _, (pm,) = _run_typed(lambda c, x: L.polyval(c, x), [_i32([1, 2]), f32([0.5, 1.5])], [I32, F32])
+    assert pm.dtype == np.float32 and pm.tolist() == [2.5, 3.5]
+    _, (pc,) = run(lambda c, x: L.polyval(c, x), f32([7]), np.ones((2, 2), np.float32))
+    assert pc.tolist() == [7, 7, 7, 7]
+    _, (pb,) = run(lambda c, x: L.polyval(c, x), f32([[1, 2], [0, 3], [4, 5]]), f32([2, 3]))
+    np.testing.assert_allclose(pb, [8, 32], rtol=1e-6)
+    with pytest.raises(ValueError, match="at least one dimension"):
+        J.jit(lambda c, x: L.polyval(c, x), [ShapedArray((), F32), ShapedArray((), F32)])
+    a1, a2, lo, sh = f32([1, 2, 3]), f32([4, 5, 6]), f32([1, 2, 3, 4]), f32([10, 20])
+    _, (s0, s1, s2, d0, d1, d2) = run(lambda p, q, r, t: [L.polyadd(p, q), L.polyadd(r, t), L.polyadd(t, r), L.polysub(p, q), L.polysub(r, t), L.polysub(t, r)], a1, a2, lo, sh)
+    assert s0.tolist() == [5, 7, 9] and s1.tolist() == [1, 2, 13, 24] and s2.tolist() == [1, 2, 13, 24]
+    assert d0.tolist() == [-3, -3, -3] and d1.tolist() == [1, 2, -7, -16] and d2.tolist() == [-1, -2, 7, 16]
+    _, (se, de, de2) = run(lambda p, q: [L.polyadd(p, q), L.polysub(p, q), L.polysub(q, p)], f32([1, 2]), f32([]))
+    assert se.tolist() == [1, 2] and de.tolist() == [1, 2] and de2.tolist() == [-1, -2]
+    _, (sp, dp) = run(lambda p, q: [L.polyadd(p, q), L.polysub(p, q)], a1, f32([0.5, 1.5]))
+    np.testing.assert_allclose(sp, [1, 2.5, 4.5])
+    np.testing.assert_allclose(dp, [1, 1.5, 1.5])
+    b1, b2, bt = f32([[2, 3, 1]]), f32([[5, 7, 3], [8, 2, 6]]), f32([[5, 7, 9], [8, 6, 4]])
+    _, (sb, db, sc, dc) = run(lambda p, q, r, t: [L.polyadd(p, q), L.polysub(p, q), L.polyadd(r, t), L.polysub(r, t)], b1, b2, bt, f32([2]))
+    assert sb.tolist() == [5, 7, 3, 10, 5, 7] and db.tolist() == [-5, -7, -3, -6, 1, -5]
+    assert sc.tolist() == [5, 7, 9, 10, 8, 6] and dc.tolist() == [5, 7, 9, 6, 4, 2]
+    for fn in (L.polyadd, L.polysub):
+        with pytest.raises(ValueError):
+            J.jit(lambda p, q: fn(p, q), [ShapedArray((3,), F32), ShapedArray((2, 3), F32)])
+        with pytest.raises(ValueError, match="at least 1D"):
+            J.jit(lambda p, q: fn(p, q), [ShapedArray((), F32), ShapedArray((2,), F32)])
+    _, (m0, m1, m2, m3) = run(lambda p, q, r, t: [L.polymul(p, q), L.polymul(r, t), L.polymul(t, r), L.polymul(J.shrink(r, [(1, 2)]), J.shrink(t, [(0, 1)]))], f32([2, 1, 0]), f32([0, 5, 3]), f32([1, 2]), f32([3, 4, 5]))
+    assert m0.tolist() == [0, 10, 11, 3, 0] and m1.tolist() == [3, 10, 13, 10] and m2.tolist() == [3, 10, 13, 10] and m3.tolist() == [6]
+    _, (mi,) = _run_typed(lambda p, q: L.polymul(p, q), [_i32([1, 2, 3]), _i32([4, 5, 6])], [I32, I32])
+    assert mi.dtype == np.float32 and mi.tolist() == [4, 13, 28, 27, 18]
+    _, (z0, z1, z2) = run(lambda p, q: [L.polymul(p, q), L.polymul(q, p), L.polymul(p, p)], f32([]), f32([1, 2]))
+    assert z0.tolist() == [0, 0] and z1.tolist() == [0, 0] and z2.tolist() == [0]
+    for shp in ((), (2, 2)):
+        with pytest.raises(ValueError, match="both inputs must be 1D arrays"):
+            J.jit(lambda p, q: L.polymul(p, q), [ShapedArray(shp, F32), ShapedArray((2,), F32)])
+    x, y = f32([1, 2, 3, 2, 1]), f32([4, 1, 2])
+    _, (cf, cs, cv) = run(lambda p, q: [L.convolve(p, q), L.convolve(p, q, "same"), L.convolve(p, q, "valid")], x, y)
+    assert cf.tolist() == [4, 9, 16, 15, 12, 5, 2] and cs.tolist() == [9, 16, 15, 12, 5] and cv.tolist() == [16, 15, 12]
+    _, (rv, rf, rs, rsw) = run(lambda p, q: [L.correlate(p, q), L.correlate(p, q, "full"), L.correlate(p, q, "same"), L.correlate(q, p, "full")], x, f32([4, 5, 6]))
+    assert rv.tolist() == [32, 35, 28] and rf.tolist() == [6, 17, 32, 35, 28, 13, 4] and rs.tolist() == [17, 32, 35, 28, 13]
+    assert rsw.tolist() == np.correlate([4, 5, 6], [1, 2, 3, 2, 1], "full").tolist()
+    _, (k1, k2) = run(lambda p, q: [L.correlate(p, q, "full"), L.convolve(p, q, "full")], x, f32([4, 5, 4]))
+    assert k1.tolist() == [4, 13, 26, 31, 26, 13, 4] and k2.tolist() == k1.tolist()
+    _, (c2,) = run(lambda p, q: L.cross(p, q), f32([1, 2]), f32([3, 4]))
+    _, (c3,) = run(lambda p, q: L.cross(p, q), f32([1, 2, 3]), f32([4, 5, 6]))
+    A, B = f32([[1, 2, 3], [3, 4, 3]]), f32([[2, 3, 2], [4, 5, 6]])
+    _, (cb, ca, cm) = run(lambda p, q: [L.cross(p, q), L.cross(p, q, axis=0), L.cross(J.shrink(p, [(0, 2), (0, 2)]), q)], A, B)
+    assert c2.tolist() == [-2] and c3.tolist() == [-3, 6, -3] and cb.tolist() == [-5, 4, -1, 9, -6, -1] and ca.tolist() == [-2, -2, 12]
+    np.testing.assert_array_equal(cm.reshape(2, 3), np.cross(np.pad(A[:, :2], [(0, 0), (0, 1)]), B))
+    _, (vr, sd) = run(lambda p: [L.var_(p), L.std(p)], f32([1, 2, 3, 4]))
+    np.testing.assert_allclose(vr, [1.25], rtol=1e-6)
+    np.testing.assert_allclose(sd, [math.sqrt(1.25)], rtol=1e-6)
+    _, (v1c, v2c, v3c, cc) = run(lambda p, q, r, t: [L.cov(p), L.cov(q), L.cov(r, t), L.corrcoef(q)], f32([[0, 1, 2], [0, 1, 2]]), f32([[-1, 0, 1], [1, 0, -1]]), f32([-1, 0, 1]), f32([1, 0, -1]))
+    np.testing.assert_allclose(v1c, [1, 1, 1, 1], rtol=1e-6)
+    np.testing.assert_allclose(v2c, [1, -1, -1, 1], rtol=1e-6)
+    np.testing.assert_allclose(v3c, [1, -1, -1, 1], rtol=1e-6)
+    np.testing.assert_allclose(cc, [1, -1, -1, 1], rtol=1e-6)
+
+
+def test_unwrap_tables():
+    """test/numpy.test.ts:2684-2801: the NumPy docs example, custom periods, a larger discont, the dtype-rounded period,
+    other axes (also an interior one), deltas of exactly half a period, int32 input, short inputs."""
+    pi = math.pi
+    _, (u1,) = run(lambda a: L.unwrap(a), f32([0, pi / 4, pi / 2, 3 * pi / 4 + pi, 2 * pi]))
+    np.testing.assert_allclose(u1, [0, pi / 4, pi / 2, -pi / 4, 0], atol=1e-5)
+    _, (u2, u3) = run(lambda a, b: [L.unwrap(a, None, -1, 4), L.unwrap(b, None, -1, 4)], f32([0, 1, 2, -1, 0]), f32([2, 3, 4, 5, 2, 3, 4, 5]))
+    np.testing.assert_allclose(u2, [0, 1, 2, 3, 4], rtol=1e-6)
+    np.testing.assert_allclose(u3, [2, 3, 4, 5, 6, 7, 8, 9], rtol=1e-6)
+    _, (u4, u5) = run(lambda a: [L.unwrap(a), L.unwrap(a, 4)], f32([0, 3.5]))
+    np.testing.assert_allclose(u4, [0, 3.5 - 2 * pi], rtol=1e-5)
+    np.testing.assert_allclose(u5, [0, 3.5], rtol=1e-6)
+    _, (u6,) = run(lambda a: L.unwrap(a, None, -1, 3.5e38), f32([0, 3e38]))
+    assert u6.tolist() == [0, float(np.float32(3e38))]
+    x = f32([[0, 2 * pi + 0.1, 4 * pi + 0.2], [0.5, 2 * pi + 0.6, 4 * pi + 0.7]])
+    _, (u7, u8, u9) = run(lambda a: [L.unwrap(a), L.unwrap(a.transpose(), None, 0), L.unwrap(a.transpose().reshape([1, 1, 3, 2]), None, 2)], x)
+    np.testing.assert_allclose(u7.reshape(2, 3), [[0, 0.1, 0.2], [0.5, 0.6, 0.7]], atol=1e-5)
+    np.testing.assert_allclose(u8.reshape(3, 2), [[0, 0.5], [0.1, 0.6], [0.2, 0.7]], atol=1e-5)
+    np.testing.assert_allclose(u9, u8, atol=1e-6)
+    _, (up, dn) = run(lambda a: [L.unwrap(a), L.unwrap(a.mul(-1))], f32([0, pi, 2 * pi]))
+    np.testing.assert_allclose(up, [0, pi, 2 * pi], atol=1e-5)
+    np.testing.assert_allclose(dn, [0, -pi, -2 * pi], atol=1e-5)
+    _, (ui,) = _run_typed(lambda a: L.unwrap(a, None, -1, 4), [_i32([0, 1, 2, -1, 0])], [I32])
+    assert ui.dtype == np.float32
+    np.testing.assert_allclose(ui, [0, 1, 2, 3, 4], rtol=1e-6)
+    _, (us, ue) = run(lambda a, b: [L.unwrap(a).mul(1), L.unwrap(b).mul(1)], f32([1.5]), f32([]))
+    assert us.tolist() == [1.5] and ue.tolist() == []
+    _, (uj,) = run(lambda a: L.unwrap(a), f32([0, pi - 0.1, 2 * pi + 0.5]))
+    np.testing.assert_allclose(uj, [0, pi - 0.1, 0.5], atol=1e-5)

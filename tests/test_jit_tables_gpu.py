@@ -23,7 +23,11 @@ TABLE_TESTS = [
     "test_output_returned_twice_carries_two_references", "test_input_returned_twice_beside_a_result",
     "test_count_nonzero_any_all_tables", "test_prod_ptp_var_std_average_tables", "test_cumsum_cumprod_tables_and_the_two_stage_scan",
     "test_diff_tables", "test_flip_rot90_roll_tables", "test_sign_and_float_class_predicates", "test_trapezoid_tables",
-    "test_matvec_vecmat_tensordot_outer_inner_tables",
+    "test_matvec_vecmat_tensordot_outer_inner_tables", "test_min_max_fmin_fmax_abs_signbit_tables", "test_division_family_tables",
+    "test_exponential_and_power_tables", "test_trigonometric_and_hyperbolic_tables", "test_nan_to_num_rounding_and_copysign_tables",
+    "test_logical_and_bitwise_tables", "test_creation_tables", "test_diag_family_tables",
+    "test_where_select_equality_and_membership_tables", "test_pad_and_split_family_tables", "test_joins_repeats_and_reshapes_tables",
+    "test_polynomial_convolution_and_statistics_tables", "test_unwrap_tables",
 ]
 
 
