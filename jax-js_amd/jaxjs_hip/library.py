@@ -29,6 +29,15 @@ the backend is handed, so it is kept literally:
   products and polynomials: dot, inner, outer, tensordot, vdot, vecdot, matvec, vecmat, cross, vander, polyval, polyadd,
   polysub, polymul, convolve, correlate, cov, corrcoef, unwrap
                                                       src/library/numpy.ts:1729-1815, 1988-2310, 2933-2980, 3141-3174
+  activations: relu ... mish, glu, logSoftmax, logmeanexp, log1mexp, oneHot; lax.topK; scipySpecial.logit
+                                                      src/library/nn.ts:47-380, 430-436; lax.ts:538-567; scipy-special.ts
+  numpy.linalg: cholesky (symmetrised), det, slogdet, eigh / eigvalsh, inv, lstsq, matrixPower, multiDot, solve with
+  broadcast batches, norm / vectorNorm / matrixNorm   src/library/numpy-linalg.ts:14-485
+  numpy.fft over (real, imag) pairs: fft / ifft, fftn / fft2 and inverses, rfft / irfft and n-d forms, hfft / ihfft,
+  fftfreq / rfftfreq, fftshift / ifftshift            src/library/numpy-fft.ts:105-384
+  random: ball, bernoulli, categorical, cauchy, choice, doubleSidedMaxwell, geometric, gumbel, laplace, logistic,
+  lognormal, maxwell, multivariateNormal, pareto, permutation, rademacher, randint, rayleigh, triangular, weibullMin
+                                                      src/library/random.ts:146-700
 Not restated: fromfunction and applyAlongAxis (they are built on vmap, a transformation this layer does not have).
 """
 
@@ -65,7 +74,10 @@ def gelu(x, approximate: bool = True):
     return x.mul(0.5).mul(J.erfc(J.neg(x.mul(math.sqrt(0.5)))))
 
 
-def softmax(x, axis: int = -1):
+def softmax(x, axis=-1):
+    x = J._raise(x)
+    if not J._normalize_axis(axis, x.ndim):
+        return onesLike(x)  # no axes to normalise over (nn.ts:294-296)
     xMax = x.max(axis, keepdims=True)
     unnormalized = J.exp(x.sub(J.stopGradient(xMax)))
     return unnormalized.div(unnormalized.sum(axis, keepdims=True))
@@ -175,8 +187,11 @@ def tri_const(n: int, m: Optional[int] = None, k: int = 0) -> ConstArray:
     return ConstArray((n, m), DType.Bool, J.aluCompare(cols, rows, "LessEqual"))
 
 
-def argmax(a: Tracer, axis: int):
+def argmax(a: Tracer, axis: Optional[int] = None):
     """First index of the maximum: max over isMax * (length - i), then length - that (numpy.ts:533-556)."""
+    a = J._raise(a)
+    if axis is None:
+        a, axis = a.reshape([-1]), 0  # the flattened array by default
     axis = axis + a.ndim if axis < 0 else axis
     n = a.shape[axis]
     isMax = J.equal(a, a.max(axis, keepdims=True))
@@ -186,8 +201,11 @@ def argmax(a: Tracer, axis: int):
     return length.sub(idx.max(axis))
 
 
-def argmin(a: Tracer, axis: int):
+def argmin(a: Tracer, axis: Optional[int] = None):
     """First index of the minimum: the same construction on `a == min(a)` (numpy.ts:497-524)."""
+    a = J._raise(a)
+    if axis is None:
+        a, axis = a.reshape([-1]), 0
     axis = axis + a.ndim if axis < 0 else axis
     n = a.shape[axis]
     isMin = J.equal(a, a.min(axis, keepdims=True))
@@ -199,7 +217,10 @@ def argmin(a: Tracer, axis: int):
 
 def logsumexp(x: Tracer, axis=None, keepdims: bool = False):
     """max + log(sum(exp(x - max))) (nn.ts:332-345)."""
-    xMax = x.max(axis, keepdims=True)
+    x = J._raise(x)
+    if not J._normalize_axis(axis, x.ndim):
+        return x
+    xMax = J.stopGradient(x.max(axis, keepdims=True))
     shifted = x.sub(xMax)
     result = xMax.add(J.log(J.exp(shifted).sum(axis, keepdims=True)))
     if keepdims:
@@ -277,16 +298,25 @@ def triangularSolve(a: Tracer, b: Tracer, leftSide: bool = False, lower: bool = 
 
 
 def solve(a: Tracer, b: Tracer):
-    """`numpy.linalg.solve` for equal batch dimensions: LU with partial pivoting, the permutation applied as a 0/1
-    matrix product, then a unit-lower and an upper triangular solve."""
-    n = a.shape[-1]
+    """`numpy.linalg.solve`: batch dimensions broadcast, LU with partial pivoting, the permutation applied as a 0/1
+    matrix product, then a unit-lower and an upper triangular solve (numpy-linalg.ts:274-318)."""
+    a, b = J._raise(a), J._raise(b)
+    n = a.shape[-1] if a.ndim >= 1 else 0
     if a.ndim < 2 or a.shape[-2] != n:
         raise ValueError(f"solve: a must be a batch of square matrices, got {a.shape}")
+    if b.ndim == 0:
+        raise ValueError("solve: b cannot be scalar")
     b_is_1d = b.ndim == 1
     if b_is_1d:
         b = b.reshape(list(b.shape) + [1])
-    if b.shape[-2] != n or tuple(a.shape[:-2]) != tuple(b.shape[:-2]):
+    if b.shape[-2] != n:
         raise ValueError(f"solve: leading dimension of b must match size of a, got a={a.shape}, b={b.shape}")
+    m = b.shape[-1]
+    batch = list(J.generalBroadcast(tuple(a.shape[:-2]), tuple(b.shape[:-2])))
+    if list(a.shape[:-2]) != batch:
+        a = J.broadcast(a, batch + [n, n], list(range(len(batch) + 2 - a.ndim)))
+    if list(b.shape[:-2]) != batch:
+        b = J.broadcast(b, batch + [n, m], list(range(len(batch) + 2 - b.ndim)))
     lu, _pivots, permutation = J.lu(a)
     P = J.equal(arange_const(0, n), permutation.reshape(list(permutation.shape) + [1])).astype(b.dtype)
     LPb = triangularSolve(lu, matmul(P, b), leftSide=True, lower=True, unitDiagonal=True)
@@ -1799,3 +1829,688 @@ def applyOverAxes(func, a, axes: Sequence[int]):
         else:
             raise ValueError("function must return array of the correct shape")
     return a
+
+
+# ---- activations and friends (src/library/nn.ts:47-380, 430-436), lax.topK, scipySpecial.logit ----------------------
+
+def relu(x):
+    return J.maximum(x, 0)
+
+
+def relu6(x):
+    return clip(J._raise(x), 0, 6)
+
+
+def softplus(x):
+    return J.log(J.exp(x).add(1))
+
+
+def sparsePlus(x: Tracer):
+    return J.where(J.lessEqual(x, -1), 0, J.where(J.less(x, 1), square(x.add(1)).mul(0.25), x))
+
+
+def sparseSigmoid(x: Tracer):
+    return clip(x.add(1).mul(0.5), 0, 1)
+
+
+def softSign(x: Tracer):
+    x = J._raise(x)
+    return x.div(absolute(x).add(1))
+
+
+def silu(x: Tracer):
+    return x.mul(sigmoid(x))
+
+
+def logSigmoid(x):
+    return J.neg(softplus(J.neg(x)))
+
+
+def leakyRelu(x: Tracer, negativeSlope=0.01):
+    x = J._raise(x)
+    return J.where(J.less(x, 0), x.mul(negativeSlope), x)
+
+
+def hardSigmoid(x):
+    return relu6(J.add(x, 3)).mul(1 / 6)
+
+
+def hardSilu(x: Tracer):
+    return J._raise(x).mul(hardSigmoid(x))
+
+
+def hardTanh(x):
+    return clip(J._raise(x), -1, 1)
+
+
+def elu(x: Tracer, alpha=1.0):
+    x = J._raise(x)
+    return J.where(J.less(x, 0), J.exp(x).sub(1).mul(alpha), x)
+
+
+def celu(x: Tracer, alpha=1.0):
+    x = J._raise(x)
+    return J.where(J.less(x, 0), J.exp(x.div(alpha)).sub(1).mul(alpha), x)
+
+
+def selu(x: Tracer):
+    return J.where(J.less(x, 0), expm1(x).mul(1.6732632423543772), x).mul(1.0507009873554805)
+
+
+def glu(x: Tracer, axis: int = -1):
+    x = J._raise(x)
+    (axis,) = J._normalize_axis(axis, x.ndim)
+    size = x.shape[axis]
+    if size % 2 != 0:
+        raise ValueError(f"glu: axis {axis} of shape ({list(x.shape)}) does not have even length")
+    sl = lambda lo, hi: [(lo, hi) if i == axis else (0, d) for i, d in enumerate(x.shape)]
+    return J.shrink(x, sl(0, size // 2)).mul(sigmoid(J.shrink(x, sl(size // 2, size))))
+
+
+def squareplus(x: Tracer, b=4.0):
+    x = J._raise(x)
+    return x.add(J.sqrt(square(x).add(b))).mul(0.5)
+
+
+def mish(x: Tracer):
+    x = J._raise(x)
+    return x.mul(tanh(softplus(x)))
+
+
+def logSoftmax(x: Tracer, axis=-1):
+    x = J._raise(x)
+    ax = J._normalize_axis(axis, x.ndim)
+    if not ax:
+        return zerosLike(x)
+    shifted = x.sub(J.stopGradient(x.max(ax, keepdims=True)))
+    return shifted.sub(J.log(J.exp(shifted).sum(ax, keepdims=True)))
+
+
+def logmeanexp(x: Tracer, axis=None, keepdims: bool = False):
+    x = J._raise(x)
+    ax = J._normalize_axis(axis, x.ndim)
+    if not ax:
+        return x
+    return logsumexp(x, ax, keepdims).sub(math.log(_int_prod([x.shape[a] for a in ax])))
+
+
+def log1mexp(x: Tracer):
+    """log(1 - exp(-x)): through expm1 up to log 2, through log1p beyond (nn.ts:370-376)."""
+    return J.where(J.lessEqual(x, math.log(2)), J.log(J.neg(expm1(J.neg(x)))), log1p(J.neg(J.exp(J.neg(x)))))
+
+
+def oneHot(x: Tracer, numClasses: int):
+    """Rows of the identity picked by the indices (nn.ts:430-435)."""
+    if x.dtype in _FLOATS:
+        raise TypeError(f"oneHot expects integers, got {x.dtype}")
+    return J.gather(J._raise(eye(numClasses)), [x], [0], 0)
+
+
+def logit(x: Tracer):
+    return J.log(J._raise(x).div(J._raise(1).sub(x)))  # scipy-special.ts
+
+
+def topK(x: Tracer, k: int, axis: int = -1):
+    """The k largest along `axis`, largest first, ties by smaller index: a stable ascending argsort of the reversed
+    axis, its last k entries reversed back, indices mirrored (lax.ts:538-567)."""
+    x = J._raise(x)
+    (axis,) = J._normalize_axis(axis, x.ndim)
+    size = x.shape[axis]
+    if k < 0 or k > size:
+        raise ValueError(f"topK: k must be in the range [0, {size}], got {k}")
+    if k == 0:
+        shape = [0 if i == axis else d for i, d in enumerate(x.shape)]
+        return [zerosLike(x, shape=shape), zerosLike(x, DType.Int32, shape)]
+    y, yi = J.argsort(moveaxis(J.flip(x, [axis]), axis, -1))
+
+    def extract(a):
+        a = J.shrink(a, [(0, d) for d in a.shape[:-1]] + [(a.shape[-1] - k, a.shape[-1])])
+        return J.flip(moveaxis(a, -1, axis), [axis])
+    return [extract(y), extract(J.neg(yi).add(size - 1))]
+
+
+# ---- numpy.linalg (src/library/numpy-linalg.ts) ----------------------------------------------------------------------
+
+def _check_square(name: str, shape) -> int:
+    if len(shape) < 2 or shape[-1] != shape[-2]:
+        raise ValueError(f"{name}: input must be at least 2D square matrix, got {list(shape)}")
+    return shape[-1]
+
+
+def matrixTranspose(a: Tracer):
+    a = J._raise(a)
+    if a.ndim < 2:
+        raise ValueError("matrixTranspose: input array must be at least 2D")
+    return moveaxis(a, -1, -2)
+
+
+def linalgCholesky(a: Tracer, upper: bool = False, symmetrizeInput: bool = True):
+    """`numpy.linalg.cholesky`: the input is symmetrised as (a + a^T) / 2 first (numpy-linalg.ts:14-30)."""
+    a = J._raise(a)
+    _check_square("cholesky", a.shape)
+    if symmetrizeInput:
+        a = a.add(matrixTranspose(a)).mul(0.5)
+    return cholesky(a, upper)
+
+
+def det(a: Tracer):
+    """Product of U's diagonal times (-1)^(number of row exchanges) (numpy-linalg.ts:53-62)."""
+    a = J._raise(a)
+    n = _check_square("det", a.shape)
+    lu, pivots, _perm = J.lu(a)
+    parity = J.mod(J.notEqual(pivots, arange(n)).astype(DType.Int32).sum(-1), 2)
+    sign = parity.mul(-2).add(1)
+    return prod(diagonal(lu, 0, -1, -2), -1).mul(sign)
+
+
+def slogdet(a: Tracer):
+    a = J._raise(a)
+    n = _check_square("slogdet", a.shape)
+    lu, pivots, _perm = J.lu(a)
+    parity = J.notEqual(pivots, arange(n)).astype(DType.Int32).sum(-1)
+    diag = diagonal(lu, 0, -1, -2)
+    parity = J.mod(parity.add(J.less(diag, 0).astype(DType.Int32).sum(-1)), 2)
+    return [parity.mul(-2).add(1), J.log(absolute(diag)).sum(-1)]
+
+
+def linalgEigh(a: Tracer, symmetrizeInput: bool = True):
+    """`numpy.linalg.eigh`: (eigenvalues ascending, eigenvectors) (numpy-linalg.ts:77-83)."""
+    vectors, values = eigh(a, symmetrizeInput=symmetrizeInput)
+    return [values, vectors]
+
+
+def eigvalsh(a: Tracer, symmetrizeInput: bool = True):
+    return eigh(a, symmetrizeInput=symmetrizeInput)[1]
+
+
+def inv(a: Tracer):
+    a = J._raise(a)
+    n = _check_square("inv", a.shape)
+    return solve(a, J._raise(eye(n, None, a.dtype)))
+
+
+def lstsq(a: Tracer, b: Tracer):
+    """Normal equations through a Cholesky factor: A^T (A A^T)^-1 B for wide or square A, (A^T A)^-1 A^T B for tall A
+    (numpy-linalg.ts:145-181)."""
+    a, b = J._raise(a), J._raise(b)
+    if a.ndim != 2:
+        raise ValueError(f"lstsq: 'a' must be a 2D array, got {list(a.shape)}")
+    m, n = a.shape
+    if b.ndim < 1 or b.shape[0] != m:
+        raise ValueError(f"lstsq: leading dimension of 'b' must match number of rows of 'a', got {list(b.shape)}")
+    at = matrixTranspose(a)
+    if m <= n:
+        l = linalgCholesky(matmul(a, at), symmetrizeInput=False)
+        lb = triangularSolve(l, b, leftSide=True, lower=True)
+        return matmul(at, triangularSolve(l, lb, leftSide=True, lower=True, transposeA=True))
+    l = linalgCholesky(matmul(at, a), symmetrizeInput=False)
+    lb = triangularSolve(l, matmul(at, b), leftSide=True, lower=True)
+    return triangularSolve(l, lb, leftSide=True, lower=True, transposeA=True)
+
+
+def matrixPower(a: Tracer, n: int):
+    """Binary powering; a negative exponent powers the inverse (numpy-linalg.ts:185-209)."""
+    if not isinstance(n, int):
+        raise ValueError(f"matrixPower: exponent must be an integer, got {n}")
+    a = J._raise(a)
+    m = _check_square("matrixPower", a.shape)
+    if n == 0:
+        return broadcastTo(eye(m, None, a.dtype), list(a.shape))
+    if n < 0:
+        a, n = inv(a), -n
+    result, a2k, k = None, a, 0
+    while n:
+        if k > 0:
+            a2k = matmul(a2k, a2k)
+        if n % 2 == 1:
+            result = a2k if result is None else matmul(result, a2k)
+        n //= 2
+        k += 1
+    return result
+
+
+def multiDot(arrays: Sequence[Tracer]):
+    """A chain of matrix products with 1-D ends as row / column vectors.  The reference hands the chain to its einsum,
+    which picks a contraction order; here the products are taken left to right (same value up to rounding)
+    (numpy-linalg.ts:223-246)."""
+    arrays = [J._raise(a) for a in arrays]
+    if len(arrays) < 2:
+        raise ValueError("Expected at least two arrays")
+    if arrays[0].ndim == 1:
+        r = multiDot([arrays[0].reshape([1, -1])] + arrays[1:])
+        return r.reshape(list(r.shape[1:]))
+    if arrays[-1].ndim == 1:
+        r = multiDot(arrays[:-1] + [arrays[-1].reshape([-1, 1])])
+        return r.reshape(list(r.shape[:-1]))
+    for i, a in enumerate(arrays):
+        if a.ndim != 2:
+            raise ValueError(f"multiDot: expected 2D, got {list(a.shape)} at index {i}")
+    out = arrays[0]
+    for a in arrays[1:]:
+        out = matmul(out, a)
+    return out
+
+
+def vectorNorm(x: Tracer, ord=2, axis=None, keepdims: bool = False):
+    x = J._raise(x)
+    if ord == math.inf:
+        return absolute(x).max(axis, keepdims)
+    if ord == -math.inf:
+        return absolute(x).min(axis, keepdims)
+    if ord == 0:
+        return J.notEqual(x, 0).astype(x.dtype).sum(axis, keepdims)
+    return power(power(absolute(x), ord).sum(axis, keepdims), 1 / ord)
+
+
+def matrixNorm(x: Tracer, ord="fro", keepdims: bool = False):
+    x = J._raise(x)
+    if x.ndim < 2:
+        raise ValueError(f"Input must be at least 2-dimensional. Recieved {x.ndim}-dimensional array")
+    if ord == "fro":
+        return J.sqrt(square(x).sum([-2, -1], keepdims))
+    if ord in (1, -1):
+        s = absolute(x).sum([-2], keepdims)
+        return s.max([-1], keepdims) if ord == 1 else s.min([-1], keepdims)
+    if ord in (math.inf, -math.inf):
+        s = absolute(x).sum([-1], keepdims)
+        ax = [-2 if keepdims else -1]
+        return s.max(ax, keepdims) if ord == math.inf else s.min(ax, keepdims)
+    raise ValueError(f"Order {ord} is not supported")
+
+
+def norm(x: Tracer, ord=None, axis=None, keepdims: bool = False):
+    """`numpy.linalg.norm`: the flattened 2-norm by default, vector norms over one axis, matrix norms (Frobenius, 1, inf,
+    and the singular-value ones) over a pair of axes (numpy-linalg.ts:338-412)."""
+    x = _floatish(J._raise(x))
+    nd = x.ndim
+    check = lambda a: J._normalize_axis(a, nd)[0] if -nd <= a < nd else (_ for _ in ()).throw(ValueError(f"norm: axis {a} out of bounds"))
+    if axis is None:
+        if ord is None:
+            return J.sqrt(square(x).sum(None, keepdims))
+        axes = list(range(nd))
+    elif isinstance(axis, int):
+        axes = [check(axis)]
+    else:
+        axes = [check(a) for a in axis]
+    if len(axes) == 1:
+        if isinstance(ord, str):
+            raise ValueError(f"norm: invalid order '{ord}' for vector norm")
+        return vectorNorm(x, 2 if ord is None else ord, axes[0], keepdims)
+    if len(axes) != 2:
+        raise ValueError(f"norm: axis must be null, an integer, or a pair of integers, got {axis}")
+    rowAxis, colAxis = axes
+    if rowAxis == colAxis:
+        raise ValueError(f"norm: duplicate axes {axis}")
+    if ord is None or ord in ("f", "fro"):
+        return J.sqrt(square(x).sum(axes, keepdims))
+    if ord in (1, -1):
+        sums = absolute(x).sum(rowAxis, keepdims)
+        if not keepdims and colAxis > rowAxis:
+            colAxis -= 1
+        return sums.max(colAxis, keepdims) if ord == 1 else sums.min(colAxis, keepdims)
+    if ord in (math.inf, -math.inf):
+        sums = absolute(x).sum(colAxis, keepdims)
+        if not keepdims and rowAxis > colAxis:
+            rowAxis -= 1
+        return sums.max(rowAxis, keepdims) if ord == math.inf else sums.min(rowAxis, keepdims)
+    if ord in (2, -2, "nuc"):
+        y = moveaxis(x, rowAxis, -1)
+        y = moveaxis(y, colAxis - 1 if colAxis > rowAxis else colAxis, -1)
+        sv = svdvals(y)
+        result = sv.max(-1) if ord == 2 else sv.min(-1) if ord == -2 else sv.sum(-1)
+        return expandDims(result, axes) if keepdims else result
+    raise ValueError(f"norm: invalid order '{ord}' for matrix norm")
+
+
+# ---- numpy.fft over (real, imag) pairs (src/library/numpy-fft.ts) ------------------------------------------------------
+
+def _check_pair(name: str, real: Tracer, imag: Tracer):
+    full = f"jax.numpy.fft.{name}"
+    if tuple(real.shape) != tuple(imag.shape):
+        raise ValueError(f"{full}: real and imaginary parts must have the same shape, got {list(real.shape)} and {list(imag.shape)}")
+    if real.dtype != imag.dtype:
+        raise ValueError(f"{full}: real and imaginary parts must have the same dtype, got {real.dtype} and {imag.dtype}")
+    if real.dtype not in _FLOATS:
+        raise ValueError(f"{full}: input must have a float dtype, got {real.dtype}")
+
+
+def _axes_in_order(axes, ndim: int) -> List[int]:
+    """Given order kept, duplicates refused (utils.ts normalizeAxis with sort = false)."""
+    if axes is None:
+        return list(range(ndim))
+    out: List[int] = []
+    for a in ([axes] if isinstance(axes, int) else axes):
+        if not -ndim <= a < ndim:
+            raise ValueError(f"axis {a} out of bounds for array of dimension {ndim}")
+        a = a + ndim if a < 0 else a
+        if a in out:
+            raise ValueError(f"Duplicate axis {a} passed to function")
+        out.append(a)
+    return out
+
+
+def _fft_checked(name: str, real, imag, axis: int, inverse: bool):
+    real, imag = J._raise(real), J._raise(imag)
+    _check_pair(name, real, imag)
+    (axis,) = _axes_in_order(axis, real.ndim)
+    if real.shape[axis] < 1:
+        raise ValueError(f"jax.numpy.fft.{name}: size must be a positive integer, got {real.shape[axis]}")
+    return fft(real, imag, axis, inverse)
+
+
+def fft1(real, imag, axis: int = -1):
+    """`numpy.fft.fft` of a (real, imag) pair along one axis, with the reference's input checks."""
+    return _fft_checked("fft", real, imag, axis, False)
+
+
+def ifft(real, imag, axis: int = -1):
+    return _fft_checked("ifft", real, imag, axis, True)
+
+
+def _transform_n(name, real, imag, axes, transform):
+    real, imag = J._raise(real), J._raise(imag)
+    _check_pair(name, real, imag)
+    for axis in _axes_in_order(axes, real.ndim):
+        real, imag = transform(real, imag, axis)
+    return real, imag
+
+
+def fftn(real, imag, axes=None):
+    return _transform_n("fftn", real, imag, axes, fft1)
+
+
+def fft2(real, imag, axes=(-2, -1)):
+    return fftn(real, imag, list(axes))
+
+
+def ifftn(real, imag, axes=None):
+    return _transform_n("ifftn", real, imag, axes, ifft)
+
+
+def ifft2(real, imag, axes=(-2, -1)):
+    return ifftn(real, imag, list(axes))
+
+
+def _slice_axis(a: Tracer, axis: int, start: int, end: int):
+    return J.shrink(a, [(start, end) if i == axis else (0, d) for i, d in enumerate(a.shape)])
+
+
+def rfft(a: Tracer, axis: int = -1):
+    """The non-negative half of the spectrum of a real signal: a full transform with a zero imaginary part, cut at
+    n // 2 + 1 (numpy-fft.ts:218-229)."""
+    a = J._raise(a)
+    if a.dtype not in _FLOATS:
+        raise ValueError(f"jax.numpy.fft.rfft: input must have a float dtype, got {a.dtype}")
+    (axis,) = _axes_in_order(axis, a.ndim)
+    re, im = fft1(a, zerosLike(a), axis)
+    stop = a.shape[axis] // 2 + 1
+    return _slice_axis(re, axis, 0, stop), _slice_axis(im, axis, 0, stop)
+
+
+def irfft(real, imag, axis: int = -1):
+    """Inverse of rfft for an even output length: the packed half is mirrored (conjugated) into the full Hermitian
+    spectrum first (numpy-fft.ts:237-262)."""
+    real, imag = J._raise(real), J._raise(imag)
+    _check_pair("irfft", real, imag)
+    (axis,) = _axes_in_order(axis, real.ndim)
+    m = real.shape[axis]
+    if m < 2:
+        raise ValueError(f"jax.numpy.fft.irfft: packed input length must be at least 2, got {m}")
+    mr = J.flip(_slice_axis(real, axis, 1, m - 1), [axis])
+    mi = J.flip(_slice_axis(imag, axis, 1, m - 1), [axis]).mul(-1)
+    return ifft(concatenate([real, mr], axis), concatenate([imag, mi], axis), axis)[0]
+
+
+def rfftn(a: Tracer, axes=None):
+    a = J._raise(a)
+    if a.dtype not in _FLOATS:
+        raise ValueError(f"jax.numpy.fft.rfftn: input must have a float dtype, got {a.dtype}")
+    order = _axes_in_order(axes, a.ndim)
+    if not order:
+        return a, zerosLike(a)
+    re, im = rfft(a, order[-1])
+    for axis in order[:-1]:
+        re, im = fft1(re, im, axis)
+    return re, im
+
+
+def rfft2(a: Tracer, axes=(-2, -1)):
+    return rfftn(a, list(axes))
+
+
+def irfftn(real, imag, axes=None):
+    real, imag = J._raise(real), J._raise(imag)
+    _check_pair("irfftn", real, imag)
+    order = _axes_in_order(axes, real.ndim)
+    if not order:
+        return real
+    for axis in order[:-1]:
+        real, imag = ifft(real, imag, axis)
+    return irfft(real, imag, order[-1])
+
+
+def irfft2(real, imag, axes=(-2, -1)):
+    return irfftn(real, imag, list(axes))
+
+
+def hfft(real, imag, axis: int = -1):
+    real, imag = J._raise(real), J._raise(imag)
+    _check_pair("hfft", real, imag)
+    (axis,) = _axes_in_order(axis, real.ndim)
+    n = 2 * (real.shape[axis] - 1)
+    return irfft(real, imag.mul(-1), axis).mul(n)
+
+
+def ihfft(a: Tracer, axis: int = -1):
+    a = J._raise(a)
+    (axis,) = _axes_in_order(axis, a.ndim)
+    n = a.shape[axis]
+    re, im = rfft(a, axis)
+    return re.div(n), im.mul(-1).div(n)
+
+
+def _check_frequency_args(name: str, n, d):
+    if not isinstance(n, int) or n < 1:
+        raise ValueError(f"jax.numpy.fft.{name}: n must be a positive integer, got {n}")
+    if not math.isfinite(d) or d == 0:
+        raise ValueError(f"jax.numpy.fft.{name}: d must be a finite non-zero number, got {d}")
+
+
+def fftfreq(n: int, d: float = 1.0):
+    """Sample frequencies as host float32 data, computed in double and rounded once, the way the reference builds the
+    array it uploads (numpy-fft.ts:347-356)."""
+    import numpy as _np
+    _check_frequency_args("fftfreq", n, d)
+    scale = 1 / (n * d)
+    vals = [i * scale for i in range((n - 1) // 2 + 1)] + [i * scale for i in range(-(n // 2), 0)]
+    return _np.asarray(vals, dtype=_np.float32)
+
+
+def rfftfreq(n: int, d: float = 1.0):
+    import numpy as _np
+    _check_frequency_args("rfftfreq", n, d)
+    scale = 1 / (n * d)
+    return _np.asarray([i * scale for i in range(n // 2 + 1)], dtype=_np.float32)
+
+
+def fftshift(a: Tracer, axes=None):
+    a = J._raise(a)
+    order = _axes_in_order(axes, a.ndim)
+    return roll(a, [a.shape[ax] // 2 for ax in order], order)
+
+
+def ifftshift(a: Tracer, axes=None):
+    a = J._raise(a)
+    order = _axes_in_order(axes, a.ndim)
+    return roll(a, [-(a.shape[ax] // 2) for ax in order], order)
+
+
+# ---- further distributions (src/library/random.ts:146-700), all built on uniform / normal above ------------------------
+
+def _split2(key: Tracer):
+    ka, kb = J.split(random_split(key, 2), 0, [1, 1])
+    return ka.reshape([2]), kb.reshape([2])
+
+
+def random_ball(key: Tracer, d: int, p: float = 2, shape: Sequence[int] = ()):
+    """Uniform in the unit d-ball: a normal direction scaled by u^(1/d) (random.ts:146-171)."""
+    if not isinstance(d, int) or d <= 0:
+        raise ValueError(f"ball: dimension must be a positive integer, got {d}")
+    if p != 2:
+        raise ValueError("ball: only the Euclidean p=2 case is supported")
+    k1, k2 = _split2(key)
+    z = random_normal(k1, list(shape) + [d])
+    nrm = J.sqrt(z.mul(z).sum(-1, keepdims=True))
+    radius = J.exp(J.log(random_uniform(k2, list(shape) + [1])).mul(1 / d))
+    return z.div(nrm).mul(radius)
+
+
+def random_bernoulli(key: Tracer, p=0.5, shape: Sequence[int] = ()):
+    return J.less(random_uniform(key, shape), p)
+
+
+def random_gumbel(key: Tracer, shape: Sequence[int] = ()):
+    return J.neg(J.log(J.neg(log1p(J.neg(random_uniform(key, shape))))))  # -log(-log(1 - u))
+
+
+def random_categorical(key: Tracer, logits: Tracer, axis: int = -1, shape: Optional[Sequence[int]] = None, replace: bool = True):
+    """Gumbel-max (with replacement) or Gumbel top-k (without) over `axis` of the logits (random.ts:203-262)."""
+    logits = J._raise(logits)
+    (axis,) = J._normalize_axis(axis, logits.ndim)
+    numCategories = logits.shape[axis]
+    batchShape = [d for i, d in enumerate(logits.shape) if i != axis]
+    if shape is None:
+        shape = batchShape
+    else:
+        shape = list(shape)
+        if list(J.generalBroadcast(tuple(shape), tuple(batchShape))) != shape:
+            raise ValueError(f"Shape {shape} is not broadcast-compatible with batch shape {batchShape}.")
+    prefix = shape[:len(shape) - len(batchShape)]
+    if replace:
+        noise = random_gumbel(key, prefix + list(logits.shape))
+        return argmax(noise.add(logits), axis + len(prefix))
+    k = _int_prod(prefix)
+    if k > numCategories:
+        raise ValueError(f"Number of samples without replacement ({k}) cannot exceed number of categories ({numCategories}).")
+    _values, indices = topK(random_gumbel(key, list(logits.shape)).add(logits), k, axis)
+    return J._raise(indices).reshape(shape)
+
+
+def random_cauchy(key: Tracer, shape: Sequence[int] = ()):
+    return tan(random_uniform(key, shape).sub(0.5).mul(math.pi))
+
+
+def random_randint(key: Tracer, minval: int, maxval: int, shape: Sequence[int] = (), dtype: DType = DType.Int32):
+    if not isinstance(minval, int) or not isinstance(maxval, int):
+        raise ValueError("randint: minval and maxval must be integers")
+    if minval >= maxval:
+        raise ValueError(f"Invalid range: [{minval}, {maxval}).")
+    if dtype not in (DType.Int32, DType.Uint32):
+        raise ValueError(f"randint: dtype must be int32 or uint32, got {dtype}")
+    if dtype == DType.Uint32 and minval < 0:
+        raise ValueError("randint: uint32 dtype requires minval >= 0")
+    return J.mod(random_bits(key, shape), maxval - minval).astype(dtype).add(minval)
+
+
+def random_permutation(key: Tracer, x, axis: int = 0):
+    """argsort of uniforms; an array is gathered along `axis` by that permutation (random.ts:542-566)."""
+    if isinstance(x, int):
+        if x < 0:
+            raise ValueError(f"permutation: x must be a non-negative integer, got {x}")
+        return argsort(random_uniform(key, [x])).astype(DType.Int32)
+    arr = J._raise(x)
+    (axis,) = J._normalize_axis(axis, arr.ndim)
+    return J.gather(arr, [random_permutation(key, arr.shape[axis])], [axis], axis)
+
+
+def random_choice(key: Tracer, a, shape: Sequence[int] = (), replace: bool = True, p=None, axis: int = 0):
+    shape = list(shape)
+    values = None
+    if isinstance(a, int):
+        if a < 0:
+            raise ValueError(f"choice: a must be a non-negative integer, got {a}")
+        n = a
+    else:
+        values = J._raise(a)
+        (axis,) = J._normalize_axis(axis, values.ndim)
+        n = values.shape[axis]
+    if p is not None:
+        idx = random_categorical(key, J.log(p), shape=shape, replace=replace)
+    elif replace:
+        idx = random_randint(key, 0, n, shape)
+    else:
+        k = _int_prod(shape)
+        if k > n:
+            raise ValueError(f"Number of samples without replacement ({k}) cannot exceed population size ({n}).")
+        idx = J.shrink(random_permutation(key, n), [(0, k)]).reshape(shape)
+    return idx if values is None else J.gather(values, [idx], [axis], axis)
+
+
+def random_rademacher(key: Tracer, shape: Sequence[int] = (), dtype: DType = DType.Int32):
+    if dtype in (DType.Uint32, DType.Bool):
+        raise ValueError(f"rademacher: unsupported dtype {dtype}")
+    return J.where(random_bernoulli(key, 0.5, shape), J.scalar(1, dtype), J.scalar(-1, dtype))
+
+
+def random_maxwell(key: Tracer, shape: Sequence[int] = ()):
+    z = random_normal(key, list(shape) + [3])
+    return J.sqrt(z.mul(z).sum(-1))
+
+
+def random_doubleSidedMaxwell(key: Tracer, loc, scale, shape: Sequence[int] = ()):
+    k1, k2 = _split2(key)
+    return random_rademacher(k1, shape, DType.Float32).mul(random_maxwell(k2, shape)).mul(scale).add(loc)
+
+
+def random_geometric(key: Tracer, p, shape: Sequence[int] = (), dtype: DType = DType.Int32):
+    return J.floor(log1p(J.neg(random_uniform(key, shape))).div(log1p(J.neg(J._raise(p))))).add(1).astype(dtype)
+
+
+def random_laplace(key: Tracer, shape: Sequence[int] = ()):
+    centered = random_uniform(key, shape).sub(0.5)
+    return sign(centered).mul(log1p(absolute(centered).mul(-2)).mul(-1))
+
+
+def random_logistic(key: Tracer, shape: Sequence[int] = ()):
+    u = random_uniform(key, shape)
+    return J.log(u).sub(log1p(J.neg(u)))
+
+
+def random_lognormal(key: Tracer, sigma=1, shape: Sequence[int] = ()):
+    return J.exp(random_normal(key, shape).mul(sigma))
+
+
+def random_multivariateNormal(key: Tracer, mean: Tracer, cov: Tracer, shape: Sequence[int] = ()):
+    """mean + L z with L the Cholesky factor of the covariance (random.ts:475-509)."""
+    mean, cov = J._raise(mean), J._raise(cov)
+    n = mean.shape[-1]
+    if cov.ndim < 2 or cov.shape[-1] != n or cov.shape[-2] != n:
+        raise ValueError(f"Invalid covariance shape: {list(cov.shape)}. Expected last two dimensions to be [{n}, {n}].")
+    out: Sequence[int] = tuple(shape)
+    for s in (tuple(mean.shape[:-1]), tuple(cov.shape[:-2])):
+        out = J.generalBroadcast(tuple(out), s)
+    Lc = linalgCholesky(cov)
+    z = random_normal(key, list(out) + [n])
+    return matvec(Lc, z).add(mean)
+
+
+def random_pareto(key: Tracer, b, shape: Sequence[int] = ()):
+    return J.exp(random_exponential(key, shape).div(b))
+
+
+def random_rayleigh(key: Tracer, scale=1, shape: Sequence[int] = ()):
+    return J.sqrt(random_exponential(key, shape).mul(2)).mul(scale)
+
+
+def random_triangular(key: Tracer, left, mode, right, shape: Sequence[int] = ()):
+    left, mode, right = _as_array(left), _as_array(mode), _as_array(right)
+    u = random_uniform(key, shape)
+    width, leftSpan, rightSpan = right.sub(left), mode.sub(left), right.sub(mode)
+    cond = J.less(u, leftSpan.div(width))
+    lower = left.add(J.sqrt(u.mul(width).mul(leftSpan)))
+    upper = right.sub(J.sqrt(J.neg(u).add(1).mul(width).mul(rightSpan)))
+    return J.where(cond, lower, upper)
+
+
+def random_weibullMin(key: Tracer, scale, concentration, shape: Sequence[int] = ()):
+    return J.mul(scale, J.exp(J.log(random_exponential(key, shape)).div(concentration)))

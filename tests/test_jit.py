@@ -761,8 +761,9 @@ def test_exponential_and_power_tables():
     (log, log(0), log2/log10), :2912-2928 (log1p), :2930-2946 (logaddexp, logaddexp2 without overflow), :2948-2960
     (sqrt), :2962-2979 (cbrt of negatives), :2981-3006 (power: negative bases, power of zero), :3008-3039 (floatPower)."""
     _, (e,) = run(lambda a: J.exp(a), f32([-1000, -100, -50, -10, 0, 10, 50, 100, 1000]))
-    np.testing.assert_allclose(e, f32([0, 3.720075976020836e-44, 1.9287498479639178e-22, 4.5399929762484854e-5, 1, 22026.465794806718,
-                                      5.184705528587072e21, 2.6881171418161356e43, np.inf]), rtol=1e-5, atol=1e-8)
+    with np.errstate(over="ignore"):  # e^100 is beyond float32: Inf on both sides
+        np.testing.assert_allclose(e, f32([0, 3.720075976020836e-44, 1.9287498479639178e-22, 4.5399929762484854e-5, 1, 22026.465794806718,
+                                          5.184705528587072e21, 2.6881171418161356e43, np.inf]), rtol=1e-5, atol=1e-8)
     _, (e2,) = run(lambda a: L.exp2(a), f32([10, 0]))
     np.testing.assert_allclose(e2, [1024, 1], rtol=1e-5)
     vals = [-1, -0.1, -0.01, -1e-4, -1e-8, 0, 1e-8, 1e-4, 0.01, 0.1, 1]
@@ -1282,3 +1283,449 @@ def test_unwrap_tables():
     assert us.tolist() == [1.5] and ue.tolist() == []
     _, (uj,) = run(lambda a: L.unwrap(a), f32([0, pi - 0.1, 2 * pi + 0.5]))
     np.testing.assert_allclose(uj, [0, pi - 0.1, 0.5], atol=1e-5)
+
+
+def test_reductions_views_dot_and_sort_tables():
+    """test/numpy.test.ts:24-42 (sum over several axes, keepdims, no axes), :221-257 (mean promotes int32 and bool),
+    :1337-1425 (transpose, swapaxes, reshape and its errors), :1683-1796 (dot: scalars, 1-D, 2-D, the N-D shape rule,
+    1-784-10, an affine map against a double loop), :3041-3103 (min / max), :4007-4033 (argmax, flattened by default),
+    :4585-4629 (applyOverAxes), :4631-4802 (sort / argsort: axes, NaN last, integer and bool dtypes, empty rows, 8192
+    elements, stability)."""
+    x = np.arange(24, dtype=np.int32).reshape(2, 3, 4)
+    seen = {}
+    def sums(a):
+        seen["k"] = a.sum([0, 2], keepdims=True)
+        return [a.sum([0, 2]), seen["k"], a.sum([])]
+    _, (s1, s2, s3) = _run_typed(sums, [x], [I32])
+    assert s1.tolist() == [60, 92, 124] and s2.tolist() == [60, 92, 124] and tuple(seen["k"].shape) == (1, 3, 1) and s3.tolist() == x.ravel().tolist()
+    _, (mi,) = _run_typed(lambda a: a.mean(), [_i32([1, 2, 3, 4])], [I32])
+    _, (mb,) = _run_typed(lambda a: a.mean(), [_i32([1, 0, 1])], [BOOL])
+    _, (mr,) = _run_typed(lambda a: a.mean(1), [_i32([[1, 2, 3], [4, 5, 6]])], [I32])
+    assert mi.dtype == np.float32 and abs(mi[0] - 2.5) < 1e-6 and mb.dtype == np.float32 and abs(mb[0] - 2 / 3) < 1e-6 and mr.tolist() == [2, 5]
+    m = f32([[1, 2, 3], [4, 5, 6]])
+    _, (t1, t2, sw) = run(lambda v, a, c: [v.transpose().mul(1), a.transpose().mul(1), L.swapaxes(c, 1, 2).mul(1)], f32([1, 2, 3]), m, f32(np.arange(12).reshape(2, 2, 3)))
+    assert t1.tolist() == [1, 2, 3] and t2.tolist() == [1, 4, 2, 5, 3, 6] and sw.tolist() == np.swapaxes(np.arange(12).reshape(2, 2, 3), 1, 2).ravel().tolist()
+    for bad in ([3, 2], [2, 3], [2, 2, 2], [3, -1]):
+        with pytest.raises(ValueError):
+            J.jit(lambda a: a.reshape(bad), [ShapedArray((4,), F32)])
+    _, (rs,) = run(lambda a: a.reshape([2, -1]).sum(1), f32([1, 2, 3, 4]))
+    assert rs.tolist() == [3, 7]
+    _, (d1, d2) = run(lambda a, b, p, q: [L.dot(a, b), L.dot(p, q)], f32([1, 2, 3]), f32([4, 5, 6]), f32([[1, 2], [3, 4]]), f32([[5, 6], [7, 8]]))
+    (d0,) = run0(lambda: L.dot(3, 4))
+    assert d0.tolist() == [12] and d1.tolist() == [32] and d2.tolist() == [19, 22, 43, 50]
+    J.jit(lambda a, b: seen.setdefault("d", L.dot(a, b)), [ShapedArray((2, 3, 4, 5), F32), ShapedArray((1, 4, 5, 6), F32)])
+    assert tuple(seen["d"].shape) == (2, 3, 4, 1, 4, 6)
+    _, (big,) = run(lambda a, b: L.dot(a, b), f32(np.arange(784)).reshape(1, 784), np.ones((784, 10), np.float32))
+    assert big.tolist() == [784 * 783 / 2] * 10
+    _, (mm,) = run(lambda a, b: L.dot(a, b), (f32(np.arange(200)).reshape(200, 1) * np.ones((200, 256), np.float32)), np.ones((256, 200), np.float32))
+    assert mm.shape == (40000,) and mm[0] == 0 and mm[200] == 256 and mm[-1] == 199 * 256
+    rows, depth, cols = 16, 64, 4
+    aD = f32([math.sin(i * 0.17) * 0.7 + ((i // depth) % 7) * 0.03 for i in range(rows * depth)]).reshape(rows, depth)
+    wD = f32([math.cos(i * 0.11) * 0.2 for i in range(depth * cols)]).reshape(depth, cols)
+    bD = f32([(i - 2) * 0.1 for i in range(cols)])
+    _, (aff,) = run(lambda a, w, b: L.dot(a, w).add(b), aD, wD, bD)
+    assert np.abs(aff.reshape(rows, cols) - (aD.astype(np.float64) @ wD.astype(np.float64) + bD)).max() < 1e-4
+    v, w = f32([3, 1, 4, 2]), f32([[3, 1, 4], [2, 5, 0]])
+    _, (n1, n2, n3, x1, x2, x3) = run(lambda a, b: [a.min(), b.min(0), b.min(), a.max(), b.max(0), b.max()], v, w)
+    assert (n1.tolist(), n2.tolist(), n3.tolist(), x1.tolist(), x2.tolist(), x3.tolist()) == ([1], [2, 1, 0], [0], [4], [3, 5, 4], [5])
+    _, (g1, g2, g3) = run(lambda a, b, c: [L.argmax(a), L.argmax(b, 1), L.argmax(c)], f32([0.1, 0.2, 0.3, 0.2]), f32([[0.1, -0.2, -0.3, 0.1], [0, 0.1, 0.3, 0.3]]), f32([[0.1, -0.2], [0.3, 0.1]]))
+    assert g1.tolist() == [2] and g2.tolist() == [0, 2] and g3.tolist() == [2]
+    def over(a):
+        seen["o"] = [L.applyOverAxes(lambda t, ax: t.sum(ax), a, [0, 2]), L.applyOverAxes(lambda t, ax: t.sum(ax, keepdims=True), a, [1]), L.applyOverAxes(lambda t, ax: t.sum(ax), a, [-1])]
+        return seen["o"]
+    _, (o1, o2, o3) = _run_typed(over, [x], [I32])
+    assert [tuple(o.shape) for o in seen["o"]] == [(1, 3, 1), (2, 1, 4), (2, 3, 1)]
+    assert o1.tolist() == [60, 92, 124] and o2.tolist() == [12, 15, 18, 21, 48, 51, 54, 57] and o3.tolist() == [6, 22, 38, 54, 70, 86]
+    with pytest.raises(ValueError):
+        J.jit(lambda a: L.applyOverAxes(lambda t, ax: L.expandDims(t, 0), a, [0]), [ShapedArray((2, 3), F32)])
+    nan = np.nan
+    _, (so, s0, s1_, sn) = run(lambda a, b, c: [L.sort(a), L.sort(b, 0).mul(1), L.sort(b, 1), L.sort(c)], f32([3, 1, 4, 1, 5, 9, 2, 6]), f32([[3, 1, 2], [6, 4, 5]]), f32([3, nan, 1, nan, 2]))
+    assert so.tolist() == [1, 1, 2, 3, 4, 5, 6, 9] and s0.tolist() == [3, 1, 2, 6, 4, 5] and s1_.tolist() == [1, 2, 3, 4, 5, 6]
+    np.testing.assert_array_equal(sn, f32([1, 2, 3, nan, nan]))
+    for dt, npdt in ((I32, np.int32), (U32, np.uint32)):
+        _, (si,) = _run_typed(lambda a: L.sort(a), [np.array([3, 1, 4, 1, 5], npdt)], [dt])
+        assert si.dtype == npdt and si.tolist() == [1, 1, 3, 4, 5]
+    _, (sb,) = _run_typed(lambda a: L.sort(a), [_i32([1, 0, 1, 0, 1])], [BOOL])
+    assert sb.tolist() == [0, 0, 1, 1, 1]
+    _, (sz,) = run(lambda a: L.sort(a), np.zeros((3, 0), np.float32))
+    assert sz.tolist() == []
+    lin = np.linspace(0, 1, 8192).astype(np.float32)
+    _, (sl,) = run(lambda a: L.sort(J.flip(a, None)), lin)
+    np.testing.assert_array_equal(sl, lin)
+    _, (a1, a2, a3) = run(lambda a, b, c: [L.argsort(a), L.argsort(b, 1), L.argsort(c)], f32([3, 1, 4, 2, 5]), f32([[3, 1, 2], [6, 4, 5]]), f32([3, 1, 1, nan, np.inf, 2, nan, 1, 0, -0.0, np.inf]))
+    assert a1.dtype == np.int32 and a1.tolist() == [1, 3, 0, 2, 4] and a2.tolist() == [1, 2, 0, 1, 2, 0]
+    assert a3.tolist() == [8, 9, 1, 2, 7, 5, 0, 4, 10, 3, 6]
+    _, (al,) = run(lambda a: L.argsort(J.flip(a, None)), np.linspace(0, 1, 8191).astype(np.float32))
+    assert al.tolist() == list(range(8190, -1, -1))
+
+
+def test_activation_tables():
+    """test/nn.test.ts:20-85 (relu, sigmoid, softSign, leakyRelu with and without a slope), :119-155 (softmax over two
+    axes, over none, of an empty array; log(softmax) == logSoftmax), :157-172 (logsumexp), :174-206 (log1mexp on both
+    sides of log 2 and at extreme arguments), :230-272 (oneHot for int32, 2-D and uint32 indices);
+    test/scipy-special.test.ts:24-75 (erf / erfc values, logit); the remaining activations against their definitions."""
+    x = f32([-1, 0, 1, 2])
+    _, (r, sg, ss) = run(lambda a: [L.relu(a), L.sigmoid(a), L.softSign(a)], x)
+    assert r.tolist() == [0, 0, 1, 2]
+    np.testing.assert_allclose(sg, [0.26894142, 0.5, 0.73105858, 0.88079708], rtol=1e-5)
+    np.testing.assert_allclose(ss, [-0.5, 0, 0.5, 2 / 3], rtol=1e-6)
+    v = f32([-100, -10, -1, 0, 1, 5, 10])
+    _, (l1, l2) = run(lambda a: [L.leakyRelu(a), L.leakyRelu(a, 0.2)], v)
+    np.testing.assert_allclose(l1, [-1, -0.1, -0.01, 0, 1, 5, 10], rtol=1e-6)
+    np.testing.assert_allclose(l2, [-20, -2, -0.2, 0, 1, 5, 10], rtol=1e-6)
+    _, (s2,) = run(lambda a: L.softmax(a, [0, 1]), f32([[1, 2, 3], [4, 5, 6]]))
+    np.testing.assert_allclose(s2, [0.00426978, 0.01160646, 0.03154963, 0.08576079, 0.23312202, 0.6336913], rtol=1e-5)
+    _, (sn0, sn1, sn2) = run(lambda a, b, c: [J._raise(L.softmax(a, None)).add(0), J._raise(L.softmax(b, [])).add(0), L.softmax(c)], f32(0).reshape(()), f32([1, 2, 3]), f32([]))
+    assert sn0.tolist() == [1] and sn1.tolist() == [1, 1, 1] and sn2.tolist() == []
+    w = f32([-10, -1, 1, 2])
+    _, (sm, lsm, lse) = run(lambda a: [J.log(L.softmax(a)), L.logSoftmax(a), L.logsumexp(a)], w)
+    np.testing.assert_allclose(sm, lsm, rtol=1e-5, atol=1e-6)
+    assert abs(lse[0] - 2.3490167) < 1e-5
+    _, (lse2, lme) = run(lambda a: [L.logsumexp(a), L.logmeanexp(a)], f32([[1, 2, 3, 4], [5, 6, 7, 8]]))
+    assert abs(lse2[0] - 8.45834) < 1e-4 and abs(lme[0] - (8.45834 - math.log(8))) < 1e-4
+    want = lambda vals: [math.log(-math.expm1(-t)) if t < math.log(2) else math.log1p(-math.exp(-t)) for t in vals]
+    for vals, tol in (([0.1, 0.5, 1, 2, 5, 10], 1e-5), ([1e-8, 1e-7, 1e-4, 0.1, 2, 10, 20, 50], 2e-5)):
+        _, (lm,) = run(lambda a: L.log1mexp(a), f32(vals))
+        np.testing.assert_allclose(lm, want([float(np.float32(t)) for t in vals]), rtol=tol, atol=1e-7 if tol == 1e-5 else 0)
+    _, (fx,) = run(lambda a: L.log1mexp(a), f32([math.log(2)]))
+    np.testing.assert_allclose(fx, [-math.log(2)], rtol=1e-6)
+    _, (o1,) = _run_typed(lambda i: L.oneHot(i, 3), [_i32([1, 1, 2])], [I32])
+    _, (o2,) = _run_typed(lambda i: L.oneHot(i, 3), [_i32([[0, 1], [2, 1]])], [I32])
+    _, (o3,) = _run_typed(lambda i: L.oneHot(i, 3), [np.array([0, 2, 1], np.uint32)], [U32])
+    assert o1.tolist() == [0, 1, 0, 0, 1, 0, 0, 0, 1] and o2.tolist() == [1, 0, 0, 0, 1, 0, 0, 0, 1, 0, 1, 0] and o3.tolist() == [1, 0, 0, 0, 0, 1, 0, 1, 0]
+    with pytest.raises(TypeError, match="expects integers"):
+        J.jit(lambda i: L.oneHot(i, 3), [ShapedArray((2,), F32)])
+    ev = [-10, -5, -1, -0.5, 0, 0.001, 0.1, 1, 5, 10]
+    ew = [-1, -1, -0.84270079, -0.52049988, 0, 0.00112838, 0.11246292, 0.84270079, 1, 1]
+    _, (ef, ec) = run(lambda a: [J.erf(a), J.erfc(a)], f32(ev))
+    np.testing.assert_allclose(ef, ew, rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(ec, [1 - t for t in ew], rtol=1e-5, atol=1e-7)
+    _, (lg,) = run(lambda a: L.logit(a), f32([0.01, 0.1, 0.25, 0.5, 0.75, 0.9, 0.99]))
+    np.testing.assert_allclose(lg, [-4.59511985, -2.19722458, -1.09861229, 0, 1.09861229, 2.19722458, 4.59511985], rtol=1e-5, atol=1e-7)
+    z = f32([-3, -1.5, -1, -0.25, 0, 0.5, 1, 2.5, 7])
+    d = z.astype(np.float64)
+    sig = lambda t: 1 / (1 + np.exp(-t))
+    fns = [(L.relu6, np.clip(d, 0, 6)), (L.softplus, np.log1p(np.exp(d))), (L.sparsePlus, np.where(d <= -1, 0, np.where(d < 1, (d + 1) ** 2 / 4, d))),
+           (L.sparseSigmoid, np.clip((d + 1) / 2, 0, 1)), (L.silu, d * sig(d)), (L.logSigmoid, -np.log1p(np.exp(-d))), (L.hardSigmoid, np.clip(d + 3, 0, 6) / 6),
+           (L.hardSilu, d * np.clip(d + 3, 0, 6) / 6), (L.hardTanh, np.clip(d, -1, 1)), (L.elu, np.where(d < 0, np.expm1(d), d)),
+           (lambda a: L.celu(a, 2.0), np.where(d < 0, 2 * np.expm1(d / 2), d)), (L.selu, 1.0507009873554805 * np.where(d < 0, 1.6732632423543772 * np.expm1(d), d)),
+           (L.squareplus, (d + np.sqrt(d * d + 4)) / 2), (L.mish, d * np.tanh(np.log1p(np.exp(d))))]
+    _, outs = run(lambda a: [f(a) for f, _ in fns], z)
+    for got, (_, ref) in zip(outs, fns):
+        np.testing.assert_allclose(got, ref, rtol=2e-5, atol=2e-6)
+    _, (gl,) = run(lambda a: L.glu(a), f32([[1, 2, 3, 4], [-1, 0, 1, 2]]))
+    np.testing.assert_allclose(gl, (np.array([[1, 2], [-1, 0]]) * sig(np.array([[3.0, 4.0], [1.0, 2.0]]))).ravel(), rtol=1e-5)
+    with pytest.raises(ValueError, match="even length"):
+        J.jit(lambda a: L.glu(a), [ShapedArray((3,), F32)])
+
+
+def test_top_k_tables():
+    """test/lax.test.ts:14-77: values and indices, ties keep the original order, k = n, k = 0, either axis of a 2-D
+    array, NaN ranks highest, invalid k."""
+    _, (v, i) = run(lambda a: L.topK(a, 3), f32([3, 1, 4, 1, 5, 9, 2, 6]))
+    assert v.tolist() == [9, 6, 5] and i.tolist() == [5, 7, 4]
+    _, (v, i) = run(lambda a: L.topK(a, 4), f32([1, 3, 2, 3, 3, 0]))
+    assert v.tolist() == [3, 3, 3, 2] and i.tolist() == [1, 3, 4, 2]
+    _, (v, i) = run(lambda a: L.topK(a, 3), f32([5, 2, 8]))
+    assert v.tolist() == [8, 5, 2] and i.tolist() == [2, 0, 1]
+    _, (v, i) = run(lambda a: L.topK(a, 0), f32([1, 2, 3]))
+    assert v.tolist() == [] and i.tolist() == [] and i.dtype == np.int32
+    m = f32([[3, 1, 4], [1, 5, 9]])
+    _, (v, i, v0, i0) = run(lambda a: L.topK(a, 2) + L.topK(a, 1, 0), m)
+    assert v.tolist() == [4, 3, 9, 5] and i.tolist() == [2, 0, 2, 1] and v0.tolist() == [3, 5, 9] and i0.tolist() == [0, 1, 1]
+    _, (v, i) = run(lambda a: L.topK(a, 2), f32([1.5, np.nan, 3.5, 2.1]))
+    np.testing.assert_array_equal(v, f32([np.nan, 3.5]))
+    assert i.tolist() == [1, 2]
+    for bad in (-1, 4):
+        with pytest.raises(ValueError):
+            J.jit(lambda a: L.topK(a, bad), [ShapedArray((3,), F32)])
+
+
+def test_numpy_linalg_tables():
+    """test/numpy-linalg.test.ts:227-244 (det), :246-294 (inv, batched), :296-310 (matrixPower), :312-366 (multiDot),
+    :368-514 (lstsq: tall, wide, square, several right-hand sides, shape errors), :516-526 (slogdet), :528-550 (solve,
+    batched), :72-126 (eigvalsh), :552-596 (vectorNorm), :597-713 (matrixNorm), :715-859 (norm: flattened, vector,
+    matrix over axis pairs, singular-value norms, errors)."""
+    a2 = f32([[4, 7], [2, 6]])
+    _, (d, sg, ld, ai) = run(lambda a: [L.det(a)] + L.slogdet(a) + [L.matmul(a, L.inv(a))], a2)
+    np.testing.assert_allclose(d, [10], rtol=1e-5)
+    np.testing.assert_allclose(sg, [1])
+    np.testing.assert_allclose(ld, [math.log(10)], rtol=1e-5)
+    np.testing.assert_allclose(ai.reshape(2, 2), np.eye(2), atol=1e-6)
+    rng = np.random.default_rng(0)
+    big = rng.uniform(0, 1, (15, 15)).astype(np.float32)
+    _, (db, sb, lb) = run(lambda a: [L.det(a)] + L.slogdet(a), big)
+    sgn, logabs = np.linalg.slogdet(big.astype(np.float64))
+    np.testing.assert_allclose(db, [np.linalg.det(big.astype(np.float64))], rtol=2e-3)
+    assert sb.tolist() == [sgn] and abs(lb[0] - logabs) < 1e-3
+    bat = rng.uniform(0, 1, (2, 3, 4, 4)).astype(np.float32)
+    _, (ib,) = run(lambda a: L.matmul(a, L.inv(a)), bat)
+    np.testing.assert_allclose(ib.reshape(2, 3, 4, 4), np.broadcast_to(np.eye(4), (2, 3, 4, 4)), atol=1e-4)
+    sym = f32([[2, 1], [1, 3]])
+    _, (p0, p3, pm) = run(lambda a: [J._raise(L.matrixPower(a, 0)).mul(1), L.matrixPower(a, 3), L.matrixPower(a, -2)], sym)
+    np.testing.assert_array_equal(p0.reshape(2, 2), np.eye(2))
+    np.testing.assert_allclose(p3.reshape(2, 2), np.linalg.matrix_power(sym.astype(np.float64), 3), rtol=1e-5)
+    np.testing.assert_allclose(pm.reshape(2, 2), np.linalg.matrix_power(sym.astype(np.float64), -2), rtol=1e-4)
+    A, B, C = f32([[1, 2], [3, 4]]), f32([[5, 6, 7], [8, 9, 10]]), f32([[11, 12], [13, 14], [15, 16]])
+    _, (m3, m2) = run(lambda a, b, c: [L.multiDot([a, b, c]), L.multiDot([a, b])], A, B, C)
+    np.testing.assert_allclose(m3.reshape(2, 2), A @ B @ C, rtol=1e-6)
+    np.testing.assert_allclose(m2.reshape(2, 3), A @ B, rtol=1e-6)
+    seen = {}
+    _, (mv,) = run(lambda x, a, b, y: seen.setdefault("m", L.multiDot([x, a, b, y])), f32([1, 2]), f32([[1, 2, 3], [4, 5, 6]]), f32([[1, 0], [0, 1], [1, 1]]), f32([2, 3]))
+    assert tuple(seen["m"].shape) == () and mv.tolist() == [129]
+    tall, wide = f32([[1, 2], [3, 4], [5, 6]]), f32([[1, 2, 3], [4, 5, 6]])
+    for a, b in ((tall, f32([[1], [2], [3]])), (tall, f32([[1, 2], [3, 4], [5, 6]]))):
+        _, (x,) = run(lambda p, q: L.lstsq(p, q), a, b)
+        x = x.reshape(2, -1)
+        np.testing.assert_allclose(a.T @ a @ x, a.T @ b, rtol=1e-4, atol=1e-4)
+    for a, b in ((wide, f32([[1], [2]])), (wide, f32([[1, 2], [3, 4]])), (sym, f32([[5], [7]]))):
+        _, (x,) = run(lambda p, q: L.lstsq(p, q), a, b)
+        np.testing.assert_allclose(a @ x.reshape(a.shape[1], -1), b, rtol=1e-4, atol=1e-4)
+    for shapes in (((3,), (3,)), ((2, 2), (3,))):
+        with pytest.raises(ValueError):
+            J.jit(lambda p, q: L.lstsq(p, q), [ShapedArray(s, F32) for s in shapes])
+    _, (sx,) = run(lambda p, q: L.solve(p, q), f32([[3, 2], [1, 2]]), f32([5, 4]))
+    np.testing.assert_allclose(sx, [0.5, 1.75], rtol=1e-5)
+    Ab, Xb = rng.uniform(0, 1, (10, 15, 15)).astype(np.float32), rng.uniform(0, 1, (10, 15, 5)).astype(np.float32)
+    _, (xp,) = run(lambda p, q: L.solve(p, q), Ab, (Ab.astype(np.float64) @ Xb).astype(np.float32))
+    np.testing.assert_allclose(xp.reshape(Xb.shape), Xb, rtol=1e-2, atol=1e-3)
+    _, (xb,) = run(lambda p, q: L.solve(p, q), sym, f32(np.arange(12).reshape(3, 2, 2)))
+    np.testing.assert_allclose(xb.reshape(3, 2, 2), np.linalg.solve(sym.astype(np.float64), np.arange(12.0).reshape(3, 2, 2)), rtol=1e-5, atol=1e-6)
+    S = rng.standard_normal((6, 6)).astype(np.float32)
+    S = (S + S.T) / 2
+    _, (ev, ew, evec) = run(lambda p: [L.eigvalsh(p)] + L.linalgEigh(p), S)
+    np.testing.assert_allclose(ev, np.linalg.eigvalsh(S.astype(np.float64)), rtol=1e-4, atol=1e-5)
+    np.testing.assert_array_equal(ev, ew)
+    V = evec.reshape(6, 6)
+    np.testing.assert_allclose(V @ np.diag(ew) @ V.T, S, atol=1e-4)
+    inf = math.inf
+    v = f32([3, -4])
+    _, (n2, n1, ni, nm, n0) = run(lambda p, q: [L.vectorNorm(p), L.vectorNorm(p, 1), L.vectorNorm(p, inf), L.vectorNorm(p, -inf), L.vectorNorm(q, 0)], v, f32([0, 3, 0, -4, 5]))
+    np.testing.assert_allclose([n2[0], n1[0], ni[0], nm[0], n0[0]], [5, 7, 4, 3, 3], rtol=1e-5)
+    M = f32([[3, 4], [5, 12]])
+    _, (na, nk) = run(lambda p: [L.vectorNorm(p, axis=1), seen.setdefault("k", L.vectorNorm(p, axis=1, keepdims=True))], M)
+    np.testing.assert_allclose(na, [5, 13], rtol=1e-5)
+    np.testing.assert_allclose(nk, [5, 13], rtol=1e-5)
+    assert tuple(seen["k"].shape) == (2, 1)
+    mat, batched = f32([[1, 2], [3, 4]]), f32(np.arange(18).reshape(2, 3, 3))
+    for o, want_m, want_b in (("fro", 5.477225575051661, [14.28285686, 39.7617907]), (1, 6, [15, 42]), (-1, 4, [9, 36]), (inf, 7, [21, 48]), (-inf, 3, [3, 30])):
+        shapes = {}
+        def norms(p, q):
+            outs = [L.matrixNorm(p, o), L.matrixNorm(p, o, True), L.matrixNorm(q, o), L.matrixNorm(q, o, True)]
+            shapes["s"] = [tuple(t.shape) for t in outs]
+            return outs
+        _, (a, ak, b, bk) = run(norms, mat, batched)
+        assert shapes["s"] == [(), (1, 1), (2,), (2, 1, 1)]
+        np.testing.assert_allclose([a[0], ak[0]], [want_m, want_m], rtol=1e-5)
+        np.testing.assert_allclose(b, want_b, rtol=1e-5)
+        np.testing.assert_allclose(bk, want_b, rtol=1e-5)
+    with pytest.raises(ValueError):
+        J.jit(lambda p: L.matrixNorm(p), [ShapedArray((4,), F32)])
+    for o in (-2, 2, "nuc"):
+        with pytest.raises(ValueError):
+            J.jit(lambda p: L.matrixNorm(p, o), [ShapedArray((2, 2), F32)])
+    b24 = f32(np.arange(24).reshape(2, 3, 4))
+    _, (f1, f2, f3) = run(lambda p, q: [L.norm(p), L.norm(q), seen.setdefault("n", L.norm(q, keepdims=True))], mat, b24)
+    np.testing.assert_allclose([f1[0], f2[0], f3[0]], [5.477225575051661, 65.75712889109438, 65.75712889109438], rtol=1e-5)
+    assert tuple(seen["n"].shape) == (1, 1, 1)
+    _, (v2, v1, vi) = run(lambda p: [L.norm(p), L.norm(p, 1), L.norm(p, inf)], v)
+    np.testing.assert_allclose([v2[0], v1[0], vi[0]], [5, 7, 4], rtol=1e-5)
+    _, (ni0,) = _run_typed(lambda p: L.norm(p, 0), [_i32([3, 0, -4])], [I32])
+    _, (nb,) = _run_typed(lambda p: L.norm(p), [_i32([1, 0, 1])], [BOOL])
+    assert ni0.dtype == np.float32 and ni0.tolist() == [2] and nb.dtype == np.float32 and abs(nb[0] - math.sqrt(2)) < 1e-6
+    _, (ax1, ax2) = run(lambda p: [L.norm(p, inf, -1), L.norm(p, axis=1)], b24)
+    np.testing.assert_allclose(ax1, [3, 7, 11, 15, 19, 23])
+    np.testing.assert_allclose(ax2, np.linalg.norm(b24, axis=1).ravel(), rtol=1e-5)
+    _, ms = run(lambda p: [L.norm(p, o) for o in ("fro", "f", 1, -1, inf, -inf)], mat)
+    np.testing.assert_allclose([t[0] for t in ms], [5.477225575051661, 5.477225575051661, 6, 4, 7, 3], rtol=1e-5)
+    _, (p1, p2, p3, p4, p5) = run(lambda p: [L.norm(p, axis=[1, 2]), L.norm(p, inf, [0, 2]), L.norm(p, 1, [2, 0]), L.norm(p, -1, [2, 0]), seen.setdefault("p", L.norm(p, inf, [0, 2], True))], b24)
+    np.testing.assert_allclose(p1, [22.4944437584, 61.7899668231], rtol=1e-5)
+    assert p2.tolist() == [54, 70, 86] and p3.tolist() == [54, 70, 86] and p4.tolist() == [6, 22, 38] and p5.tolist() == [54, 70, 86]
+    assert tuple(seen["p"].shape) == (1, 3, 1)
+    tol = dict(rtol=1e-4, atol=1e-4)
+    _, (s2, sm2, sn) = run(lambda p: [L.norm(p, 2), L.norm(p, -2), L.norm(p, "nuc")], mat)
+    np.testing.assert_allclose([s2[0], sm2[0], sn[0]], [5.464985704219043, 0.36596619062625757, 5.8309518948453], **tol)
+    ab = f32([[[1, 2, 0.5], [3, 4, -1]], [[2, -1, 0], [1, 5, 2]]])
+    _, (q1, q2, q3, q4, q5) = run(lambda p: [L.norm(p, 2, [1, 2]), L.norm(p, -2, [1, 2]), L.norm(p, "nuc", [1, 2]), L.norm(p, 2, [2, 0]), seen.setdefault("q", L.norm(p, "nuc", [2, 0], True))], ab)
+    np.testing.assert_allclose(q1, [5.5123605371, 5.5095335676], **tol)
+    np.testing.assert_allclose(q2, [0.9294521555, 2.1552354553], **tol)
+    np.testing.assert_allclose(q3, [6.4418126926, 7.6647690229], **tol)
+    np.testing.assert_allclose(q4, [2.2912878475, 7.0067840776], **tol)
+    np.testing.assert_allclose(q5, [4.527355825, 9.634516349], **tol)
+    assert tuple(seen["q"].shape) == (1, 2, 1)
+    for kw, shp in ((dict(ord=3, axis=[0, 1]), (2, 2)), (dict(ord="fro", axis=0), (2, 2)), (dict(axis=[0, 0]), (2, 2)), (dict(axis=[0, 1, 2]), (2, 3, 4)), (dict(ord=2), (2, 3, 4))):
+        with pytest.raises(ValueError):
+            J.jit(lambda p: L.norm(p, **kw), [ShapedArray(shp, F32)])
+
+
+def _dft(real, imag):
+    n = len(real)
+    k = np.arange(n)
+    w = np.exp(-2j * np.pi * np.outer(k, k) / n)
+    out = w @ (np.asarray(real, np.float64) + 1j * np.asarray(imag, np.float64))
+    return out.real, out.imag
+
+
+def test_numpy_fft_tables():
+    """test/numpy-fft.test.ts:28-87 (fft against a direct DFT: powers of two, length one, mixed radix, a prime; another
+    axis), :89-124 (ifft, round trips either way), :126-166 (fftn, fft2 / ifft2), :168-231 (rfft / irfft, rfft2, rfftn /
+    irfftn, hfft / ihfft), :233-255 (fftfreq, rfftfreq, fftshift / ifftshift)."""
+    cases = [([0, 1, 2, 3], [0, 0, 0, 0]), ([1, 0, 0, 0], [0, 0, 0, 0]), ([3, 3, 3, 3], [0, 0, 0, 0]), ([3], [-2]),
+             ([1, 3, 0, -2, 5, 1, 2, -1], [2, -1, 4, 1, 0, -3, 2, 1]), ([1, 3, 0, -2, 5, 1], [2, -1, 4, 1, 0, -3]), ([4, -1, 2, 0, 3], [0, 2, -3, 1, 5])]
+    for re, im in cases:
+        _, (r, i) = run(lambda a, b: list(L.fft1(a, b)), f32(re), f32(im))
+        wr, wi = _dft(re, im)
+        np.testing.assert_allclose(r, wr, atol=1e-4)
+        np.testing.assert_allclose(i, wi, atol=1e-4)
+    _, (r, i) = run(lambda a, b: list(L.fft1(a, b, 0)), f32([[1, 2, 3, 4], [5, 6, 7, 8]]), np.zeros((2, 4), np.float32))
+    np.testing.assert_allclose(r, [6, 8, 10, 12, -4, -4, -4, -4], rtol=1e-5)
+    np.testing.assert_allclose(i, 0, atol=1e-5)
+    _, (r, i) = run(lambda a, b: list(L.ifft(a, b)), f32([6, -2, -2, -2]), f32([0, 2, 0, -2]))
+    np.testing.assert_allclose(r, [0, 1, 2, 3], atol=1e-6)
+    np.testing.assert_allclose(i, 0, atol=1e-6)
+    for re, im in (([1, 2, 3, 4, 5, 6, 7, 8], [-5, 9, 0, 3, -1, 4, 2, 8]), ([1, 2, 3, 4, 5, 6], [-5, 9, 0, 3, -1, 4])):
+        _, (r, i) = run(lambda a, b: list(L.ifft(*L.fft1(a, b))), f32(re), f32(im))
+        np.testing.assert_allclose(r, re, atol=1e-5)
+        np.testing.assert_allclose(i, im, atol=1e-5)
+    _, (r, i) = run(lambda a, b: list(L.fft1(*L.ifft(a, b))), f32([2, -1, 4, 0]), f32([1, 3, -2, 5]))
+    np.testing.assert_allclose(r, [2, -1, 4, 0], atol=1e-5)
+    np.testing.assert_allclose(i, [1, 3, -2, 5], atol=1e-5)
+    _, (r, i) = run(lambda a, b: list(L.fftn(a, b)), f32([[1, 2], [3, 4]]), np.zeros((2, 2), np.float32))
+    np.testing.assert_allclose(r, [10, -2, -4, 0], atol=1e-5)
+    np.testing.assert_allclose(i, 0, atol=1e-5)
+    R, I = f32([[1, 2, 3, 4], [5, 6, 7, 8]]), f32([[1, -1, 2, -2], [3, -3, 4, -4]])
+    _, (r, i) = run(lambda a, b: list(L.ifft2(*L.fft2(a, b))), R, I)
+    np.testing.assert_allclose(r, R.ravel(), atol=1e-5)
+    np.testing.assert_allclose(i, I.ravel(), atol=1e-5)
+    _, (r, i) = run(lambda a: list(L.rfft(a)), f32([0, 1, 2, 3]))
+    np.testing.assert_allclose(r, [6, -2, -2], atol=1e-5)
+    np.testing.assert_allclose(i, [0, 2, 0], atol=1e-5)
+    x8 = f32(np.arange(8))
+    _, (back,) = run(lambda a: L.irfft(*L.rfft(a)), x8)
+    np.testing.assert_allclose(back, x8, atol=1e-5)
+    _, (r, i) = run(lambda a: list(L.rfft2(a)), R)
+    np.testing.assert_allclose(r, [36, -4, -4, -16, 0, 0], atol=1e-5)
+    np.testing.assert_allclose(i, [0, 4, 0, 0, 0, 0], atol=1e-5)
+    _, (back2,) = run(lambda a: L.irfftn(*L.rfftn(a)), R)
+    np.testing.assert_allclose(back2, R.ravel(), atol=1e-5)
+    _, (h, hr, hi) = run(lambda a, b, c: [L.hfft(a, b)] + list(L.ihfft(c)), f32([1, 2, 4]), f32([0, 3, 0]), f32([9, 3, 1, -9]))
+    np.testing.assert_allclose(h, [9, 3, 1, -9], atol=1e-5)
+    np.testing.assert_allclose(hr, [1, 2, 4], atol=1e-5)
+    np.testing.assert_allclose(hi, [0, 3, 0], atol=1e-5)
+    np.testing.assert_allclose(L.fftfreq(4), [0, 0.25, -0.5, -0.25])
+    np.testing.assert_allclose(L.fftfreq(5, 0.5), [0, 0.4, 0.8, -0.8, -0.4], rtol=1e-6)
+    np.testing.assert_allclose(L.rfftfreq(4), [0, 0.25, 0.5])
+    np.testing.assert_allclose(L.rfftfreq(5, 0.5), [0, 0.4, 0.8], rtol=1e-6)
+    assert L.fftfreq(4).dtype == np.float32
+    _, (s4, s5, is5) = run(lambda a, b: [L.fftshift(a), L.fftshift(b), L.ifftshift(b)], f32([0, 1, 2, 3]), f32([0, 1, 2, 3, 4]))
+    assert s4.tolist() == [2, 3, 0, 1] and s5.tolist() == [3, 4, 0, 1, 2] and is5.tolist() == [2, 3, 4, 0, 1]
+    with pytest.raises(ValueError, match="same shape"):
+        J.jit(lambda a, b: list(L.fft1(a, b)), [ShapedArray((4,), F32), ShapedArray((3,), F32)])
+    with pytest.raises(ValueError, match="float dtype"):
+        J.jit(lambda a, b: list(L.fft1(a, b)), [ShapedArray((4,), I32), ShapedArray((4,), I32)])
+
+
+def _key(seed):
+    return np.array([0, seed], np.uint32)
+
+
+def _sample(fn, seed, *arrays):
+    prog = J.jit(fn, [ShapedArray((2,), U32)] + [ShapedArray(tuple(a.shape), F32) for a in arrays])
+    be = OracleBackend()
+    outs = run_program(be, prog, [_key(seed)] + list(arrays))
+    assert be.live_slots() == 0
+    return outs
+
+
+def test_random_distribution_tables():
+    """test/random.test.ts:99-131 (normal: mass within 1, 2, 3 sigma; bernoulli with an array of p), :133-346
+    (categorical: frequencies, default shape, batched and non-default axes, shape errors, without replacement), :347-520
+    (cauchy quartiles; laplace, gumbel, logistic moments; randint, rademacher, lognormal, rayleigh, pareto, weibullMin,
+    geometric, triangular, maxwell, doubleSidedMaxwell, ball), :522-575 (choice, permutation), :577-600
+    (multivariateNormal mean and covariance)."""
+    (z,) = _sample(lambda k: L.random_normal(k, [5000]), 123)
+    for s, want in ((1, 0.6827), (2, 0.9545), (3, 0.9973)):
+        assert abs((np.abs(z) <= s).mean() - want) < 0.005 * 3
+    (b,) = _sample(lambda k, p: L.random_bernoulli(k, p, [2, 500]), 2024, f32([[0.25], [0.8]]))
+    fr = b.reshape(2, 500).mean(1)
+    assert abs(fr[0] - 0.25) < 0.05 and abs(fr[1] - 0.8) < 0.05
+    probs = [0.1, 0.2, 0.3, 0.4]
+    (c,) = _sample(lambda k, lg: L.random_categorical(k, J.log(lg), shape=[10000]), 555, f32(probs))
+    assert c.dtype == np.int32
+    for i, p in enumerate(probs):
+        assert abs((c == i).mean() - p) < 0.05
+    seen = {}
+    (c0,) = _sample(lambda k, lg: seen.setdefault("c", L.random_categorical(k, lg)), 444, f32([1, 2, 3]))
+    assert tuple(seen["c"].shape) == () and 0 <= c0[0] < 3
+    (cb,) = _sample(lambda k, lg: L.random_categorical(k, lg, shape=[100, 2]), 333, f32([[10, 0, 0], [0, 0, 10]]))
+    assert (cb.reshape(100, 2) == [0, 2]).all()
+    (ca,) = _sample(lambda k, lg: L.random_categorical(k, lg, axis=0, shape=[100, 2]), 123, f32([[10, 0], [0, 10], [0, 0]]))
+    assert (ca.reshape(100, 2) == [0, 1]).all()
+    for shp, lshape in (([10, 5], (2, 3)), ([1], (4, 5))):
+        with pytest.raises(ValueError, match="(?i)incompatible shapes|not broadcast-compatible"):
+            J.jit(lambda k, lg: L.random_categorical(k, lg, shape=shp), [ShapedArray((2,), U32), ShapedArray(lshape, F32)])
+    lg5 = f32([1, 2, 3, 4, 5])
+    (cm,) = _sample(lambda k, lg: L.random_categorical(k, lg, shape=[2, 3]), 888, lg5)
+    assert cm.shape == (6,) and ((0 <= cm) & (cm < 5)).all()
+    (cw,) = _sample(lambda k, lg: L.random_categorical(k, lg, shape=[3], replace=False), 222, lg5)
+    assert len(set(cw.tolist())) == 3 and ((0 <= cw) & (cw < 5)).all()
+    with pytest.raises(ValueError, match="cannot exceed"):
+        J.jit(lambda k, lg: L.random_categorical(k, lg, shape=[5], replace=False), [ShapedArray((2,), U32), ShapedArray((3,), F32)])
+    (cbw,) = _sample(lambda k, lg: L.random_categorical(k, lg, shape=[3, 2], replace=False), 777, f32([[1, 2, 3, 4, 5], [5, 4, 3, 2, 1]]))
+    rows = cbw.reshape(2, 3)  # what topK returned per batch row, before the reference's final reshape to [3, 2]
+    assert len(set(rows[0].tolist())) == 3 and len(set(rows[1].tolist())) == 3
+    (call,) = _sample(lambda k, lg: L.random_categorical(k, lg, shape=[5], replace=False), 105, lg5)
+    assert sorted(call.tolist()) == [0, 1, 2, 3, 4]
+    (c6,) = _sample(lambda k, lg: L.random_categorical(k, lg, shape=[2, 3], replace=False), 106, f32([1, 2, 3, 4, 5, 6]))
+    assert sorted(c6.tolist()) == [0, 1, 2, 3, 4, 5]
+    ones = np.ones((2, 5, 3), np.float32)
+    for kw, want in ((dict(axis=1), (2, 3)), (dict(axis=1, shape=[10, 2, 3]), (10, 2, 3)), (dict(axis=-2, shape=[4, 2, 3]), (4, 2, 3))):
+        _sample(lambda k, lg: seen.__setitem__("s", L.random_categorical(k, lg, **kw)) or seen["s"], 100, ones)
+        assert tuple(seen["s"].shape) == want
+    (cy,) = _sample(lambda k: L.random_cauchy(k, [20000]), 999)
+    q1, med, q3 = np.sort(cy)[[5000, 10000, 15000]]
+    assert abs(med) < 0.05 and abs(q1 + 1) < 0.05 and abs(q3 - 1) < 0.05
+    (lp,) = _sample(lambda k: L.random_laplace(k, [20000]), 888)
+    assert abs(lp.mean()) < 0.05 and abs(lp.var(ddof=1) - 2) < 0.5
+    (gb,) = _sample(lambda k: L.random_gumbel(k, [20000]), 777)
+    assert abs(gb.mean() - 0.5772156649) < 0.05 and abs(gb.var(ddof=1) - math.pi ** 2 / 6) < 0.05
+    (ri,) = _sample(lambda k: L.random_randint(k, -3, 7, [5000]), 1201)
+    assert ri.dtype == np.int32 and ri.min() >= -3 and ri.max() < 7
+    assert all(abs((ri == v).mean() - 0.1) < 0.05 for v in range(-3, 7))
+    (rd,) = _sample(lambda k: L.random_rademacher(k, [5000]), 1202)
+    assert set(rd.tolist()) == {-1, 1} and abs(rd.mean()) < 0.08
+    (lo,) = _sample(lambda k: L.random_logistic(k, [10000]), 1203)
+    assert abs(lo.mean()) < 0.1 and 3.0 < lo.var(ddof=1) < 3.6
+    (ln,) = _sample(lambda k: L.random_lognormal(k, 1, [10000]), 1204)
+    assert (ln > 0).all() and 1.45 < ln.mean() < 1.85
+    (ry,) = _sample(lambda k: L.random_rayleigh(k, 2, [10000]), 1205)
+    assert (ry >= 0).all() and 2.35 < ry.mean() < 2.65
+    (pa,) = _sample(lambda k: L.random_pareto(k, 3, [10000]), 1206)
+    assert (pa >= 1).all() and 1.35 < pa.mean() < 1.65
+    (wb,) = _sample(lambda k: L.random_weibullMin(k, 2, 1, [10000]), 1207)
+    assert (wb >= 0).all() and 1.8 < wb.mean() < 2.2
+    (ge,) = _sample(lambda k: L.random_geometric(k, 0.25, [10000]), 1208)
+    assert ge.dtype == np.int32 and (ge >= 1).all() and 3.7 < ge.mean() < 4.3
+    (tr,) = _sample(lambda k: L.random_triangular(k, -1, 0, 2, [10000]), 1209)
+    assert ((tr >= -1) & (tr <= 2)).all() and 0.23 < tr.mean() < 0.43
+    (mw,) = _sample(lambda k: L.random_maxwell(k, [10000]), 1210)
+    assert (mw >= 0).all() and 1.45 < mw.mean() < 1.75
+    (dm,) = _sample(lambda k: L.random_doubleSidedMaxwell(k, 0, 1, [10000]), 1211)
+    assert abs(dm.mean()) < 0.12 and 1.45 < np.abs(dm).mean() < 1.75
+    (bl,) = _sample(lambda k: L.random_ball(k, 3, shape=[5000]), 1212)
+    r2 = (bl.reshape(5000, 3) ** 2).sum(1)
+    assert (r2 <= 1.0001).all() and 0.55 < r2.mean() < 0.65
+    (ch,) = _sample(lambda k: L.random_choice(k, 5, [200]), 1213)
+    assert ch.dtype == np.int32 and ((0 <= ch) & (ch < 5)).all()
+    (cv,) = _sample(lambda k, v: L.random_choice(k, v, [200]), 1214, f32([10, 20, 30, 40, 50]))
+    assert set(cv.tolist()) <= {10, 20, 30, 40, 50}
+    (pm,) = _sample(lambda k: L.random_permutation(k, 8), 1215)
+    (pv,) = _sample(lambda k, v: L.random_permutation(k, v), 1216, f32([10, 20, 30, 40]))
+    assert sorted(pm.tolist()) == list(range(8)) and sorted(pv.tolist()) == [10, 20, 30, 40]
+    (cn,) = _sample(lambda k: L.random_choice(k, 6, [4], replace=False), 1217)
+    assert len(set(cn.tolist())) == 4 and ((0 <= cn) & (cn < 6)).all()
+    mean, cov = f32([1, 2]), f32([[1, 0.5], [0.5, 2]])
+    (mv, mm, mc) = _sample(lambda k, m, c: (lambda y: [y, y.mean(0), L.cov(y, None, rowvar=False)])(L.random_multivariateNormal(k, m, c, [5000])), 42, mean, cov)
+    assert mv.shape == (10000,)
+    np.testing.assert_allclose(mm, mean, atol=3e-2)
+    np.testing.assert_allclose(mc.reshape(2, 2), cov, atol=5e-2)

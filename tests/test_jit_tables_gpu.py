@@ -27,7 +27,8 @@ TABLE_TESTS = [
     "test_exponential_and_power_tables", "test_trigonometric_and_hyperbolic_tables", "test_nan_to_num_rounding_and_copysign_tables",
     "test_logical_and_bitwise_tables", "test_creation_tables", "test_diag_family_tables",
     "test_where_select_equality_and_membership_tables", "test_pad_and_split_family_tables", "test_joins_repeats_and_reshapes_tables",
-    "test_polynomial_convolution_and_statistics_tables", "test_unwrap_tables",
+    "test_polynomial_convolution_and_statistics_tables", "test_unwrap_tables", "test_reductions_views_dot_and_sort_tables",
+    "test_activation_tables", "test_top_k_tables", "test_numpy_linalg_tables", "test_numpy_fft_tables", "test_random_distribution_tables",
 ]
 
 
