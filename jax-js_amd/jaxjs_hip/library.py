@@ -119,22 +119,74 @@ def matmul(x: Tracer, y: Tracer):
     return lax_dot(x, y, [-1], [-2], batch, batch)
 
 
-def einsum(subscripts: str, a: Tracer, b: Tracer):
-    """Two-operand einsum without repeated or summed-alone indices: batch = shared kept indices,
-    contraction = shared dropped indices, then a transpose to the requested order
-    (numpy.ts:1935-1990)."""
-    lhs, out = subscripts.replace(" ", "").split("->")
-    ia, ib = lhs.split(",")
-    if len(set(ia)) != len(ia) or len(set(ib)) != len(ib):
-        raise NotImplementedError("einsum: repeated indices")
-    reduced = [c for c in ia if c in ib and c not in out]
-    if any((c not in out) and not (c in ia and c in ib) for c in ia + ib):
-        raise NotImplementedError("einsum: index summed over a single operand")
-    batch = [c for c in ia if c in ib and c not in reduced]
-    res = lax_dot(a, b, [ia.index(c) for c in reduced], [ib.index(c) for c in reduced],
-                  [ia.index(c) for c in batch], [ib.index(c) for c in batch])
-    order = batch + [c for c in ia if c not in ib] + [c for c in ib if c not in ia]
-    return res.transpose([order.index(c) for c in out])
+def einsum(*args):
+    """`einsum("ij,jk->ik", a, b, ...)` or `einsum(a, [0, 1], b, [1, 2], [0, 2])`: operands are contracted pairwise in
+    the order the path search picks; before each contraction an operand's repeated indices are replaced by diagonals and
+    indices nobody else needs are summed away; each pair goes through one general dot with the shared surviving indices as
+    batch dimensions; a final transpose gives the requested order (numpy.ts:1851-1986)."""
+    from .einsum import EinsumInput, computeEinsumPath, parseEinsumExpression
+    if not args:
+        raise ValueError("einsum: must provide at least one argument")
+    if isinstance(args[0], str):
+        operands = [J._raise(x) for x in args[1:]]
+        inp = parseEinsumExpression(args[0], [list(x.shape) for x in operands])
+    else:
+        n = len(args) >> 1
+        operands = [J._raise(args[2 * i]) for i in range(n)]
+        lhs = [list(args[2 * i + 1]) for i in range(n)]
+        if len(args) % 2 == 1:
+            rhs = list(args[2 * n])
+        else:
+            count: dict = {}
+            for i in [i for idx in lhs for i in idx]:
+                count[i] = count.get(i, 0) + 1
+            rhs = sorted(i for i, c in count.items() if c == 1)
+        inp = EinsumInput([list(x.shape) for x in operands], lhs, rhs)
+    path = computeEinsumPath(inp)
+    usage: dict = {}
+    for i in [i for idx in inp.lhsIndices for i in idx] + list(inp.rhsIndex):
+        usage[i] = usage.get(i, 0) + 1
+    indices = [list(i) for i in inp.lhsIndices]
+
+    def single(ar: Tracer, index, keep=()):
+        index = list(index)
+        again = True
+        while again:
+            again = False
+            for i, idx in enumerate(index):
+                if idx in index[i + 1:]:
+                    j = index.index(idx, i + 1)
+                    ar = diagonal(ar, 0, i, j)
+                    del index[j], index[i]
+                    index.append(idx)
+                    again = True
+                    break
+        for i in range(len(index) - 1, -1, -1):
+            if usage.get(index[i], 0) == 0 and index[i] not in keep:
+                ar = ar.sum(i)
+                del index[i]
+        return ar, index
+
+    for i, j in path.path:
+        reduced = []
+        for idx in indices[i] + indices[j]:
+            usage[idx] -= 1
+            if usage[idx] == 0:
+                reduced.append(idx)
+        a, aidx = single(operands[i], indices[i], indices[j])
+        b, bidx = single(operands[j], indices[j], indices[i])
+        reduced = [idx for idx in dict.fromkeys(reduced) if idx in aidx]
+        batch = [idx for idx in aidx if idx in bidx and idx not in reduced]
+        operands.append(lax_dot(a, b, [aidx.index(x) for x in reduced], [bidx.index(x) for x in reduced],
+                                [aidx.index(x) for x in batch], [bidx.index(x) for x in batch]))
+        indices.append(batch + [x for x in aidx if x not in bidx] + [x for x in bidx if x not in aidx])
+        for idx in indices[-1]:
+            usage[idx] += 1
+    for idx in indices[len(operands) - 1]:
+        usage[idx] -= 1
+    ar, index = single(operands[-1], indices[len(operands) - 1])
+    perm = [index.index(x) for x in inp.rhsIndex]
+    return ar.transpose(perm)
 
 
 def padtypeToPads(inShape, filterShape, strides, dilation, padding: str):
@@ -2070,9 +2122,8 @@ def matrixPower(a: Tracer, n: int):
 
 
 def multiDot(arrays: Sequence[Tracer]):
-    """A chain of matrix products with 1-D ends as row / column vectors.  The reference hands the chain to its einsum,
-    which picks a contraction order; here the products are taken left to right (same value up to rounding)
-    (numpy-linalg.ts:223-246)."""
+    """A chain of matrix products with 1-D ends as row / column vectors, handed to einsum in index-list form so that its
+    path search picks the order of the products (numpy-linalg.ts:223-246)."""
     arrays = [J._raise(a) for a in arrays]
     if len(arrays) < 2:
         raise ValueError("Expected at least two arrays")
@@ -2082,13 +2133,12 @@ def multiDot(arrays: Sequence[Tracer]):
     if arrays[-1].ndim == 1:
         r = multiDot(arrays[:-1] + [arrays[-1].reshape([-1, 1])])
         return r.reshape(list(r.shape[:-1]))
+    args: list = []
     for i, a in enumerate(arrays):
         if a.ndim != 2:
             raise ValueError(f"multiDot: expected 2D, got {list(a.shape)} at index {i}")
-    out = arrays[0]
-    for a in arrays[1:]:
-        out = matmul(out, a)
-    return out
+        args += [a, [i, i + 1]]
+    return einsum(*args)
 
 
 def vectorNorm(x: Tracer, ord=2, axis=None, keepdims: bool = False):

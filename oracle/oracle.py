@@ -3,7 +3,9 @@
 TEST INFRASTRUCTURE ONLY: imported by tests/, `__graft_entry__.smoke()` and the CPU-baseline leg
 of bench.py -- never by the package.  `run_kernel` serialises the expression *as the caller
 built it* (`Kernel.exp_raw`, `Reduction.epilogue_raw`, GlobalView nodes untouched), so neither
-the host-side simplifier nor the view lowering the product uses is on the checking path.
+the host-side simplifier nor the view lowering the product uses is on the checking path.  One fold
+is applied while serialising, because the reference applies it before any of its backends runs: a
+float constant under a cast to another float type becomes that constant in the target type.
 """
 from __future__ import annotations
 
@@ -124,6 +126,12 @@ class _Program:
             self.fa.append(f)
             return i
 
+        # A float constant under a cast to another float type is that constant in the target type, not first rounded to
+        # its own: the reference folds constants in JS doubles before any backend sees them (src/alu.ts:671-675, with
+        # `evaluate` returning a Const's number as it is, :1128-1137), so `x_f64 + 3.141592653589793` adds the double.
+        _fl = (DType.Float32, DType.Float16, DType.Float64)
+        exp = exp.rewrite(lambda e: AluExp.const(e.dtype, e.src[0].arg) if e.op == AluOp.Cast and e.dtype in _fl
+                          and e.src[0].op == AluOp.Const and e.src[0].dtype in _fl else None)
         exp.fold(emit)
         # `fold` visits the root last, so the result is the last node.
         assert index[id(exp)] == len(self.op) - 1

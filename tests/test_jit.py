@@ -1729,3 +1729,158 @@ def test_random_distribution_tables():
     assert mv.shape == (10000,)
     np.testing.assert_allclose(mm, mean, atol=3e-2)
     np.testing.assert_allclose(mc.reshape(2, 2), cov, atol=5e-2)
+
+
+def test_einsum_parser_and_path_golden_vectors():
+    """src/library/numpy/einsum.test.ts:4-87 (explicit and implicit forms, ellipses, broadcasting ellipses) and :89-166
+    (flop estimates, output shapes and the chosen contraction order for matmul, traces, diagonals, chains of three and
+    five matrices)."""
+    from jaxjs_hip.einsum import computeEinsumPath, parseEinsumExpression as parse
+    def both(expr, shapes):
+        e = parse(expr, shapes)
+        return e.lhsIndices, e.rhsIndex
+    assert both("ij,jk->ik", [[], []]) == ([[0, 1], [1, 2]], [0, 2])
+    assert both("iii->i", [[]]) == ([[0, 0, 0]], [0])
+    assert both("ji->ji", [[]]) == ([[1, 0]], [1, 0])
+    assert both("ij->ji", [[]]) == ([[0, 1]], [1, 0])
+    assert both("->", [[]]) == ([[]], [])
+    assert both("ij,jk", [[], []]) == ([[0, 1], [1, 2]], [0, 2])
+    assert both("iii", [[]]) == ([[0, 0, 0]], [])
+    assert both("ji", [[]]) == ([[1, 0]], [0, 1])
+    assert both("...ij,jk->...ik", [[2, 3, 4], [4, 5]]) == ([[3, 0, 1], [1, 2]], [3, 0, 2])
+    assert both("...->", [[100]]) == ([[0]], [])
+    assert both("...ij,j", [[2, 3, 4], [4, 5]]) == ([[2, 0, 1], [1]], [2, 0])
+    assert both("..., ..., ...", [[], [1, 4], [5, 3, 4]]) == ([[], [1, 2], [0, 1, 2]], [0, 1, 2])
+    p = computeEinsumPath(parse("ij,jk->ik", [[25, 30], [30, 40]]))
+    assert p.approximateFlops == 2 * 25 * 40 * 30 and p.outputShape == [25, 40] and p.path == [(0, 1)]
+    p = computeEinsumPath(parse("ii->", [[50, 50]]))
+    assert p.approximateFlops == 50 and p.outputShape == [] and p.path == []
+    p = computeEinsumPath(parse("ii->i", [[60, 60]]))
+    assert p.approximateFlops == 60 and p.outputShape == [60] and p.path == []
+    p = computeEinsumPath(parse("ii,ii->", [[70, 70], [70, 70]]))
+    assert p.approximateFlops == 2 * 70 and p.outputShape == [] and p.path == [(0, 1)]
+    p = computeEinsumPath(parse("ij,jk,kl->il", [[10, 20], [20, 30], [30, 40]]), "optimal")
+    assert p.path == [(0, 1), (2, 3)] and p.approximateFlops == 2 * (10 * 30 * 20 + 10 * 40 * 30)
+    p = computeEinsumPath(parse("ab,bc,cd,de,ef->af", [[5, 10], [10, 15], [15, 20], [20, 25], [25, 30]]), "optimal")
+    assert p.path == [(0, 1), (2, 5), (3, 6), (4, 7)]
+
+
+def test_einsum_tables():
+    """test/numpy.test.ts:1819-2052: matmul, sums and traces of one operand, transposition, the JAX documentation's
+    examples in string and index-list form (inner and outer products, matrix-vector, ellipsis reductions, diagonals, a
+    three-index contraction, a chain of four matrices), and the shape table incl. ellipses and size-1 broadcasting."""
+    a = f32(np.arange(6).reshape(2, 3))
+    _, (c,) = run(lambda p, q: L.einsum("ik,kj->ij", p, q), a, np.ones((3, 4), np.float32))
+    assert c.tolist() == [3] * 4 + [12] * 4
+    _, outs = run(lambda p: [L.einsum("ij->", p), L.einsum(p, [0, 1], []), L.einsum("ij->j", p), L.einsum("ji->j", p), L.einsum("ii->", J.shrink(p, [(0, 2), (1, 3)])), L.einsum("ji", p)], a)
+    assert [o.tolist() for o in outs] == [[15], [15], [3, 5, 7], [3, 12], [6], [0, 3, 1, 4, 2, 5]]
+    M, x, y = f32(np.arange(16).reshape(4, 4)), f32(np.arange(4)), f32([5, 4, 3, 2])
+    e = L.einsum
+    _, outs = run(lambda m, p, q: [e("i,i", p, q), e("i,i->", p, q), e(p, [0], q, [0]), e(p, [0], q, [0], []),
+                                   e("ij,j->i", m, p), e("ij,j", m, p), e(m, [0, 1], p, [1], [0]), e(m, [0, 1], p, [1]),
+                                   e("i,j->ij", p, q), e("i,j", p, q), e(p, [0], q, [1], [0, 1]), e(p, [0], q, [1]),
+                                   e("i->", p), e(p, [0], []), e("...j->...", m), e("ii->i", m), e("ii", m)], M, x, y)
+    got = [o.tolist() for o in outs]
+    outer = np.outer(x, y).ravel().tolist()
+    assert got[:4] == [[16]] * 4 and got[4:8] == [[14, 38, 62, 86]] * 4 and got[8:12] == [outer] * 4
+    assert got[12:] == [[6], [6], [6, 22, 38, 54], [0, 5, 10, 15], [30]]
+    y2 = f32([[1, 2, 3], [4, 5, 6]])
+    _, outs = run(lambda p: [e("ij->ji", p), e("ji", p), e(p, [1, 0]), e(p, [0, 1], [1, 0])], y2)
+    assert all(o.tolist() == [1, 4, 2, 5, 3, 6] for o in outs)
+    tx, ty = f32(np.arange(30).reshape(2, 3, 5)), f32(np.arange(60).reshape(3, 4, 5))
+    _, outs = run(lambda p, q: [e("ijk,jlk->il", p, q), e("ijk,jlk", p, q), e(p, [0, 1, 2], q, [1, 3, 2], [0, 3]), e(p, [0, 1, 2], q, [1, 3, 2])], tx, ty)
+    assert all(o.tolist() == [3340, 3865, 4390, 4915, 8290, 9940, 11590, 13240] for o in outs)
+    w, cx, cy, z = f32(np.arange(5, 9).reshape(2, 2)), f32(np.arange(6).reshape(2, 3)), f32(np.arange(-2, 4).reshape(3, 2)), f32([[2, 4, 6], [3, 5, 7]])
+    _, outs = run(lambda p, q, r, t: [e("ij,jk,kl,lm->im", p, q, r, t), e(p, [0, 1], q, [1, 2], r, [2, 3], t, [3, 4])], w, cx, cy, z)
+    assert all(o.tolist() == [481, 831, 1181, 651, 1125, 1599] for o in outs)
+    table = [("", [], []), ("i,i->", [3], [3], []), ("ijj->i", [2, 3, 3], [2]), ("i,i->i", [3], [3], [3]), ("ij,j->i", [2, 3], [3], [2]),
+             ("ij,ji", [3, 4], [4, 3], []), ("ij,jk", [2, 3], [3, 4], [2, 4]), ("ij,jk->ki", [2, 3], [3, 4], [4, 2]),
+             ("abc,cde->abde", [2, 3, 4], [4, 5, 6], [2, 3, 5, 6]), ("abcd,cdef->abef", [2, 3, 4, 5], [4, 5, 6, 7], [2, 3, 6, 7]),
+             ("abcd,efcd->abef", [2, 3, 4, 5], [6, 7, 4, 5], [2, 3, 6, 7]), ("abc,bcd,efa,fab", [2, 3, 4], [3, 4, 5], [10, 6, 2], [6, 2, 3], [5, 10]),
+             ("...", [5, 1], [5, 1]), ("i...", [5, 1], [1, 5]), ("...,...->...", [2, 3, 4], [3, 4], [2, 3, 4]), ("...i,i->...", [2, 3, 4], [4], [2, 3]),
+             ("i,...i->...", [4], [2, 3, 4], [2, 3]), ("...ij,jk->...ik", [5, 2, 3], [3, 4], [5, 2, 4]),
+             ("...ij,...jk->...ik", [6, 5, 2, 3], [5, 3, 4], [6, 5, 2, 4]), ("ab...cd,cd...ef->ab...ef", [2, 3, 4, 5, 6, 7], [6, 7, 8, 9], [2, 3, 4, 5, 8, 9]),
+             ("ii->i", [3, 3], [3]), ("ii->i", [3, 1], [1]), ("i,i->i", [3], [1], [3]), ("i,i->i", [1], [3], [3]), ("ii,i->i", [3, 3], [1], [3]),
+             ("ii,i->i", [1, 1], [3], [3]), ("ij,ij->ij", [1, 10], [5, 1], [5, 10]), ("...,...->...", [1, 10], [5, 1], [5, 10])]
+    rng = np.random.default_rng(5)
+    for expr, *shapes in table:
+        ins = [rng.integers(-3, 4, s).astype(np.float32) for s in shapes[:-1]]
+        seen = {}
+        _, (got,) = run(lambda *ops: seen.setdefault("r", e(expr, *ops)), *ins)
+        assert list(seen["r"].shape) == shapes[-1], expr
+        if not _needs_broadcast(expr, shapes):
+            np.testing.assert_array_equal(got.reshape(shapes[-1]), np.einsum(expr if expr else "->", *ins))
+
+
+def _needs_broadcast(expr, shapes):
+    """Cases of the shape table that rely on size-1 broadcasting of a named index, which numpy.einsum refuses."""
+    return (expr, shapes[:-1]) in [("ii->i", [[3, 1]]), ("i,i->i", [[3], [1]]), ("i,i->i", [[1], [3]]), ("ii,i->i", [[3, 3], [1]]),
+                                   ("ii,i->i", [[1, 1], [3]]), ("ij,ij->ij", [[1, 10], [5, 1]])]
+
+
+F16, F64 = DType.Float16, DType.Float64
+
+
+def test_dtype_promotion_and_half_double_tables():
+    """test/dtype.test.ts:8-150 (uint32 wrap-around; promotion of uint32 + int32, int32 * f16, uint32 - f32, bool + int32,
+    f16 / f32; numbers are weak and take the array's dtype, also through jit), :152-195 (resultType);
+    test/dtype-f16.test.ts:35-79 (signbit of -0, sum of squares, exact erfc gelu, reductions accumulate in f32) and
+    :80-125 (a transposed convolution in f16); test/dtype-f64.test.ts:34-110 (signbit incl. the sign of a NaN, sum of
+    squares, gelu, 1e-15 differences, unwrap at a rounding tie, polymul keeps double precision)."""
+    sc = lambda v, t: np.asarray(v, t).reshape(())
+    _, (u,) = _run_typed(lambda a, b: a.sub(b), [sc(3, np.uint32), sc(5, np.uint32)], [U32, U32])
+    assert u.dtype == np.uint32 and u.tolist() == [4294967294]
+    cases = [((3, np.uint32, U32), (-2, np.int32, I32), lambda a, b: a.add(b), np.int32, 1),
+             ((3, np.int32, I32), (2.5, np.float16, F16), lambda a, b: a.mul(b), np.float16, 7.5),
+             ((4, np.uint32, U32), (1.5, np.float32, F32), lambda a, b: a.sub(b), np.float32, 2.5),
+             ((1, np.int32, BOOL), (10, np.int32, I32), lambda a, b: a.add(b), np.int32, 11),
+             ((2.5, np.float16, F16), (1.5, np.float32, F32), lambda a, b: a.div(b), np.float32, 2.5 / 1.5)]
+    for (va, na, da), (vb, nb, db), fn, want_dt, want in cases:
+        _, (c,) = _run_typed(fn, [sc(va, na), sc(vb, nb)], [da, db])
+        assert c.dtype == want_dt and abs(float(c[0]) - want) < 1e-6
+    seen = {}
+    _, (w1, w2, w3) = _run_typed(lambda a, b: [seen.setdefault("i", a.add(3)), seen.setdefault("u", b.add(2.8)), seen.setdefault("m", a.add(J.mul(3, 3)))], [sc(5, np.int32), sc(5, np.uint32)], [I32, U32])
+    assert (w1.dtype, w1.tolist(), w2.dtype, w2.tolist(), w3.dtype, w3.tolist()) == (np.int32, [8], np.uint32, [7], np.int32, [14])
+    assert not seen["i"].aval.weak and not seen["u"].aval.weak and not seen["m"].aval.weak
+    J.jit(lambda a: seen.setdefault("w", J.mul(3, 5)), [ShapedArray((), F32)])
+    assert seen["w"].dtype == F32 and seen["w"].aval.weak
+    _, (s3,) = _run_typed(lambda h: seen.setdefault("s", J.sin(3)).add(h), [sc(2, np.float16)], [F16])
+    assert seen["s"].dtype == F32 and seen["s"].aval.weak and s3.dtype == np.float16 and abs(float(s3[0]) - (math.sin(3) + 2)) < 5e-3
+    for npdt, dt in ((np.int32, I32), (np.float32, F32)):
+        _, (p,) = _run_typed(lambda a: a.add(3), [sc(4, npdt)], [dt])
+        assert p.dtype == npdt and p.tolist() == [7]
+    R = L.resultType
+    t = lambda dt, weak=False: J.Tracer(J.Lit(0, ShapedArray((), dt, weak)))
+    assert R(t(U32), t(I32)) == I32 and R(t(I32), t(F16)) == F16 and R(t(BOOL), t(I32)) == I32 and R(t(F16), t(F32)) == F32 and R(t(F32), t(F64)) == F64
+    J.jit(lambda a, b, h: seen.update(r=[R(a, 3.5), R(2, h), R(1, 2.5), R(True, 2), R(3), R(True), R(b, h), J.add(J._raise(True), 2).dtype]) or a, [ShapedArray((2,), I32), ShapedArray((2,), F32), ShapedArray((3,), F16)])
+    assert seen["r"] == [I32, F16, F32, U32, F32, BOOL, F32, U32]
+    h = lambda v: np.asarray(v, np.float16)
+    _, (sb,) = _run_typed(lambda a: L.signbit(a), [h([-1.5, -0.0, 0, 1.5])], [F16])
+    _, (sq,) = _run_typed(lambda a: a.mul(a).sum(), [h(np.arange(10))], [F16])
+    _, (ge,) = _run_typed(lambda a: L.gelu(a, approximate=False), [h([-1, 0, 1])], [F16])
+    assert sb.tolist() == [1, 1, 0, 0] and sq.dtype == np.float16 and sq.tolist() == [285] and ge.dtype == np.float16
+    np.testing.assert_allclose(ge.astype(np.float32), [-0.1587, 0.0, 0.8413], rtol=1e-3, atol=1e-6)
+    _, (dd,) = _run_typed(lambda a: L.dot(a, a), [h([100, 1, 1, 1, 1, 1, 1, 1, 1])], [F16])
+    _, (ss,) = _run_typed(lambda a: a.sum(), [h([16000, 1, 1, 1, 1, 1, 1, 1, 1])], [F16])
+    assert dd.dtype == np.float16 and dd.tolist() == [10008] and ss.dtype == np.float16 and ss.tolist() == [16008]
+    xh, kh = h([[[1, 2, 3], [4, 5, 6]]]), h([[[1, 0, -1], [2, 1, 0]], [[0, 1, 2], [-1, 0, 1]]])
+    _, (ct,) = _run_typed(lambda a, k: L.convGeneralDilated(a, k, [1], [(2, 1)], lhsDilation=[2]), [xh, kh], [F16, F16])
+    dil = np.zeros((1, 2, 5 + 3), np.float32)
+    dil[:, :, 2:7:2] = xh
+    want = np.array([[[(dil[0, :, i:i + 3] * kh[o].astype(np.float32)).sum() for i in range(6)] for o in range(2)]])
+    assert ct.dtype == np.float16
+    np.testing.assert_allclose(ct.astype(np.float32).reshape(want.shape), want, rtol=1e-3, atol=1e-3)
+    d = lambda v: np.asarray(v, np.float64)
+    _, (s64,) = _run_typed(lambda a: L.signbit(a), [d([-1.5, -0.0, 0, 1.5])], [F64])
+    nans = np.array([0xFFF8000000000000, 0x7FF8000000000000], np.uint64).view(np.float64)
+    _, (sn,) = _run_typed(lambda a: L.signbit(a), [nans], [F64])
+    _, (q64,) = _run_typed(lambda a: a.mul(a).sum(), [d(np.arange(10))], [F64])
+    _, (g64,) = _run_typed(lambda a: L.gelu(a, approximate=False), [d([-1, 0, 1])], [F64])
+    assert s64.tolist() == [1, 1, 0, 0] and sn.tolist() == [1, 0] and q64.dtype == np.float64 and q64.tolist() == [285]
+    np.testing.assert_allclose(g64, [-0.15865525, 0.0, 0.84134475], rtol=1e-5, atol=1e-7)
+    _, (df,) = _run_typed(lambda a: J.shrink(a, [(1, 2)]).sub(J.shrink(a, [(0, 1)])), [d([1 + 1e-15, 1 + 2e-15])], [F64])
+    assert abs(df[0] - 1e-15) < 5e-16
+    _, (uw,) = _run_typed(lambda a: L.unwrap(a), [d([0, -3.1415926535897936])], [F64])
+    assert uw.dtype == np.float64 and uw[1] == 3.1415926535897927
+    _, (pm,) = _run_typed(lambda a, b: L.polymul(a, b), [d([1, 1e-12]), d([1, 1])], [F64, F64])
+    assert pm.dtype == np.float64 and pm[1] == 1 + 1e-12
