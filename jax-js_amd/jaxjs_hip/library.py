@@ -203,8 +203,59 @@ def padtypeToPads(inShape, filterShape, strides, dilation, padding: str):
     return [(sz - (sz >> 1), sz >> 1) for sz in sizes]
 
 
-def convGeneralDilated(lhs: Tracer, rhs: Tracer, windowStrides: Sequence[int], padding, lhsDilation=None, rhsDilation=None):
-    """`lax.conv_general_dilated` with one feature group: lhs `[N, C, *xs]`, rhs `[O, C, *ks]` (lax.ts:268-343)."""
+def _lower_conv_transpose_1d(lhs: Tracer, rhs: Tracer, strides, padding, ld, rd):
+    """A 1-D transposed convolution (unit stride, input dilated by `stride`, non-negative padding) without dilating the
+    input: every input sample times every kernel tap as one Dot giving [N, O, K, W]; the reversed kernel axis is cut into
+    ceil(K / stride) contributions of `stride` phases each, contribution i is shifted by i input blocks (a Pad) and the
+    contributions are added; the requested output range is then cut out of the full overlap-add signal
+    (lax.ts:166-250).  None when the shape is outside that case (more than eight contributions included)."""
+    from .convolution import ConvParams, checkConvShape
+    if (lhs.ndim != 3 or rhs.ndim != 3 or len(strides) != 1 or strides[0] != 1 or len(ld) != 1 or ld[0] <= 1
+            or len(rd) != 1 or rd[0] != 1 or len(padding) != 1 or padding[0][0] < 0 or padding[0][1] < 0
+            or any(d <= 0 for d in lhs.shape) or any(d <= 0 for d in rhs.shape)):
+        return None
+    outShape = checkConvShape(list(lhs.shape), list(rhs.shape), ConvParams(0, list(strides), [tuple(p) for p in padding], list(ld), list(rd)))
+    if any(d <= 0 for d in outShape):
+        return None
+    B, C, W = lhs.shape
+    O, _, K = rhs.shape
+    stride = ld[0]
+    count = -(-K // stride)
+    if count > 8:
+        return None
+    a = lhs.transpose([0, 2, 1]).reshape([B, 1, 1, W, C])
+    b = rhs.transpose([0, 2, 1]).reshape([1, O, K, 1, C])
+    cols = J.dot(a, b)  # [B, O, K, W]
+    cols = J.flip(cols.transpose([0, 1, 3, 2]), [3])
+    cols = J.pad(cols, [(0, 0), (0, 0), (0, 0), (0, count * stride - K)]).reshape([B, O, W, count, stride])
+    terms = []
+    for index, term in enumerate(J.split(cols, 3, [1] * count)):
+        term = term.reshape([B, O, W, stride])
+        terms.append(J.pad(term, [(0, 0), (0, 0), (index, count - 1 - index), (0, 0)]))
+    out = terms[0]
+    for t in terms[1:]:
+        out = out.add(t)
+    out = out.reshape([B, O, -1])
+    full = (W - 1) * stride + K
+    out = J.shrink(out, [(0, B), (0, O), (0, full)])
+    outLen = outShape[2]
+    offset = K - 1 - padding[0][0]
+    padL, padR = max(0, -offset), max(0, offset + outLen - full)
+    out = J.pad(out, [(0, 0), (0, 0), (padL, padR)])
+    return J.shrink(out, [(0, B), (0, O), (offset + padL, offset + padL + outLen)])
+
+
+def convGeneralDilated(lhs: Tracer, rhs: Tracer, windowStrides: Sequence[int], padding, lhsDilation=None, rhsDilation=None,
+                       featureGroupCount: int = 1):
+    """`lax.conv_general_dilated`: lhs `[N, C, *xs]`, rhs `[O, C / G, *ks]`.  One feature group goes to the Conv primitive
+    (a 1-D transposed convolution through the overlap-add lowering above when it applies); G groups become a leading
+    batch axis of the primitive: lhs -> [G, N, C/G, *xs], rhs -> [G, O/G, C/G, *ks], result moved back to [N, O, *ys]
+    (lax.ts:252-343)."""
+    lhs, rhs = J._raise(lhs), J._raise(rhs)
+    if lhs.ndim < 2:
+        raise ValueError("lhs must have at least 2 dimensions")
+    if rhs.ndim < 2:
+        raise ValueError("rhs must have at least 2 dimensions")
     n = lhs.ndim - 2
     rd = list(rhsDilation) if rhsDilation is not None else [1] * n
     ld = list(lhsDilation) if lhsDilation is not None else [1] * n
@@ -212,8 +263,55 @@ def convGeneralDilated(lhs: Tracer, rhs: Tracer, windowStrides: Sequence[int], p
         if any(d != 1 for d in ld):
             raise ValueError("String padding is not supported for transposed convolutions")
         padding = padtypeToPads(lhs.shape[2:], rhs.shape[2:], windowStrides, rd, padding)
+    padding = [tuple(p) for p in padding]
     from .convolution import ConvParams
-    return J.conv(lhs, rhs, ConvParams(0, list(windowStrides), [tuple(p) for p in padding], ld, rd))
+    if featureGroupCount == 1:
+        lowered = _lower_conv_transpose_1d(lhs, rhs, list(windowStrides), padding, ld, rd)
+        if lowered is not None:
+            return lowered
+        return J.conv(lhs, rhs, ConvParams(0, list(windowStrides), padding, ld, rd))
+    G = featureGroupCount
+    N, C_in, xs = lhs.shape[0], lhs.shape[1], list(lhs.shape[2:])
+    C_out, C_per, ks = rhs.shape[0], rhs.shape[1], list(rhs.shape[2:])
+    if C_in % G != 0:
+        raise ValueError(f"featureGroupCount={G} must divide input channels={C_in}")
+    if C_out % G != 0:
+        raise ValueError(f"featureGroupCount={G} must divide output channels={C_out}")
+    if C_in // G != C_per:
+        raise ValueError(f"rhs input channels={C_per} must equal lhs input channels / groups={C_in // G}")
+    lg = moveaxis(lhs.reshape([N, G, C_in // G] + xs), 1, 0)
+    rg = rhs.reshape([G, C_out // G, C_per] + ks)
+    result = J.conv(lg, rg, ConvParams(1, list(windowStrides), padding, ld, rd))
+    return moveaxis(result, 0, 1).reshape([N, C_out] + list(result.shape[3:]))
+
+
+def _conv_transpose_padding(k: int, s: int, padding):
+    """Padding of the dilated input that makes a stride-s transposed convolution the gradient of the forward one
+    (lax.ts:444-467)."""
+    if padding == "SAME":
+        padLen = k + s - 2
+        pad1 = k - 1 if s > k - 1 else -(-padLen // 2)
+    elif padding == "VALID":
+        padLen = k + s - 2 + max(k - s, 0)
+        pad1 = k - 1
+    elif isinstance(padding, (list, tuple)):
+        pad1 = k - 1 - padding[0]
+        padLen = pad1 + k - 1 - padding[1]
+    else:
+        raise ValueError(f"convTranspose: Invalid padding type {padding}")
+    return (pad1, padLen - pad1)
+
+
+def convTranspose(lhs: Tracer, rhs: Tracer, strides: Sequence[int], padding, rhsDilation=None, transposeKernel: bool = False):
+    """`lax.conv_transpose`: unit window strides over an input dilated by `strides` (lax.ts:407-442)."""
+    lhs, rhs = J._raise(lhs), J._raise(rhs)
+    ks = list(rhs.shape[2:])
+    rd = list(rhsDilation) if rhsDilation is not None else [1] * len(ks)
+    eff = [max(0, (k - 1) * d + 1) for k, d in zip(ks, rd)]
+    pads = [_conv_transpose_padding(k, strides[i], padding if isinstance(padding, str) else padding[i]) for i, k in enumerate(eff)]
+    if transposeKernel:
+        rhs = moveaxis(J.flip(rhs, list(range(2, rhs.ndim))), 0, 1)
+    return convGeneralDilated(lhs, rhs, [1] * (lhs.ndim - 2), pads, lhsDilation=list(strides), rhsDilation=rd)
 
 
 def reduceWindow(x: Tracer, op: AluOp, window: Sequence[int], strides: Optional[Sequence[int]] = None):

@@ -82,10 +82,88 @@ def test_2d_convolution_table():
 
 
 def test_transposed_convolution_table():
-    """lhsDilation 2 with padding [2,2] (test/conv.test.ts:71-80); here through the generic Conv view algebra."""
+    """lhsDilation 2 with padding [2,2] (test/conv.test.ts:71-91): lowered to a Dot plus shifted adds, no Conv left."""
     x, k = f32([[[1, 2, 3]]]), f32([[[1, 10, 100]]])
-    _, (r,) = run(lambda a, b: L.convGeneralDilated(a, b, [1], [(2, 2)], lhsDilation=[2]), x, k)
+    fn = lambda a, b: L.convGeneralDilated(a, b, [1], [(2, 2)], lhsDilation=[2])
+    _, (r,) = run(fn, x, k)
     np.testing.assert_array_equal(r, [100, 10, 201, 20, 302, 30, 3])
+    jaxpr, _ = J.trace(fn, [ShapedArray((1, 1, 3), F32), ShapedArray((1, 1, 3), F32)])
+    prims = [e.primitive for e in jaxpr.eqns]
+    assert "Conv" not in prims and "Dot" in prims and "Shrink" in prims and "Add" in prims
+
+
+TRANSPOSED_1D = [  # test/conv.test.ts:93-146 and :205-243: dilation, padding, kernel (None = the 3-output, 2-channel one)
+    (2, (2, 1), None), (3, (0, 2), None), (2, (-1, 2), None), (2, (4, 3), [[[1, -1, 2, 0, 3]]]), (4, (1, 2), [[[2, -1]]]),
+]
+
+
+@pytest.mark.parametrize("dilation,padding,kernel", TRANSPOSED_1D)
+def test_transposed_1d_convolution_lowering_matches_direct_loops(dilation, padding, kernel):
+    if kernel is None:
+        x = f32([[[1, 2, 3, 4], [5, 6, 7, 8]], [[2, 4, 6, 8], [1, 3, 5, 7]]])
+        k = f32([[[1, 0, -1], [2, 1, 0]], [[0, 1, 2], [-1, 0, 1]], [[2, -1, 1], [1, 1, -2]]])
+    else:
+        x, k = f32([[[1, 2, 3, 4]]]), f32(kernel)
+    _, (r,) = run(lambda a, b: L.convGeneralDilated(a, b, [1], [padding], lhsDilation=[dilation]), x, k)
+    want = conv_reference(x, k, [1], [padding], [dilation])
+    np.testing.assert_array_equal(r.reshape(want.shape), want)
+
+
+def test_transposed_convolution_downstream_ops_and_integer_dtype():
+    """test/conv.test.ts:148-203: the lowered result feeds an add and a split; int32 operands stay int32."""
+    x, k = f32([[[1, 2, 3], [4, 5, 6]]]), f32([[[1, 0, -1], [2, 1, 0]], [[0, 1, 2], [-1, 0, 1]]])
+    want = conv_reference(x, k, [1], [(2, 1)], [2]) + 1
+    _, (a, b) = run(lambda p, q: L.split(L.convGeneralDilated(p, q, [1], [(2, 1)], lhsDilation=[2]).add(1), [3], 2), x, k)
+    np.testing.assert_array_equal(a.reshape(1, 2, 3), want[:, :, :3])
+    np.testing.assert_array_equal(b.reshape(1, 2, -1), want[:, :, 3:])
+    prog = J.jit(lambda p, q: L.convGeneralDilated(p, q, [1], [(2, 1)], lhsDilation=[2]), [ShapedArray((1, 2, 3), DType.Int32), ShapedArray((2, 2, 3), DType.Int32)])
+    (ri,) = run_program(OracleBackend(), prog, [x.astype(np.int32), k.astype(np.int32)])
+    assert ri.dtype == np.int32
+    np.testing.assert_array_equal(ri.reshape(want.shape), want - 1)
+
+
+def test_zero_dimensional_grouped_and_conv_transpose_tables():
+    """test/conv.test.ts:245-262 (a convolution without spatial axes is x @ y^T), :352-398 (feature groups: shapes and
+    values), :400-432 (depthwise), :545-618 (convTranspose output shapes for SAME / VALID, 1-D 2x upscale)."""
+    _, (z,) = run(lambda a, b: L.convGeneralDilated(a, b, [], "VALID"), f32([[1, 2], [3, 4], [5, 8]]), f32([[6, 4], [3, 2]]))
+    assert z.tolist() == [14, 7, 34, 17, 62, 31]
+    seen = {}
+    for xs, ws, pad, G, want in (((2, 4, 8, 8), (6, 2, 3, 3), "VALID", 2, (2, 6, 6, 6)), ((1, 4, 5, 5), (8, 1, 3, 3), "SAME", 4, (1, 8, 5, 5))):
+        J.jit(lambda a, b: seen.__setitem__("g", L.convGeneralDilated(a, b, [1, 1], pad, featureGroupCount=G)) or seen["g"], [ShapedArray(xs, F32), ShapedArray(ws, F32)])
+        assert tuple(seen["g"].shape) == want
+    x = f32([[1, 2, 3, 4], [5, 6, 7, 8]]).reshape(1, 2, 4)
+    y = f32([[1, 0, -1], [1, 1, 1]]).reshape(2, 1, 3)
+    _, (g,) = run(lambda a, b: L.convGeneralDilated(a, b, [1], "VALID", featureGroupCount=2), x, y)
+    assert g.tolist() == [-2, -2, 18, 21]
+    xd = f32([[1, 2, 3, 4, 5], [2, 3, 4, 5, 6], [3, 4, 5, 6, 7]]).reshape(1, 3, 5)
+    yd = f32([[1, -1], [1, 0], [0, 1]]).reshape(3, 1, 2)
+    _, (dw,) = run(lambda a, b: L.convGeneralDilated(a, b, [1], "VALID", featureGroupCount=3), xd, yd)
+    assert dw.tolist() == [-1, -1, -1, -1, 2, 3, 4, 5, 4, 5, 6, 7]
+    rng = np.random.default_rng(2)
+    xg, wg = rng.integers(-3, 4, (2, 6, 7, 5)).astype(np.float32), rng.integers(-3, 4, (4, 3, 3, 2)).astype(np.float32)
+    _, (gg,) = run(lambda a, b: L.convGeneralDilated(a, b, [2, 1], [(1, 1), (0, 1)], featureGroupCount=2), xg, wg)
+    halves = [conv_reference(xg[:, 3 * i:3 * i + 3], wg[2 * i:2 * i + 2], [2, 1], [(1, 1), (0, 1)]) for i in range(2)]
+    np.testing.assert_array_equal(gg.reshape(2, 4, *halves[0].shape[2:]), np.concatenate(halves, 1))
+    for bad in ((2, 5, 4), (4, 2, 3)), ((2, 4, 4), (3, 2, 3)), ((2, 4, 4), (4, 1, 3)):
+        with pytest.raises(ValueError):
+            J.jit(lambda a, b: L.convGeneralDilated(a, b, [1], "VALID", featureGroupCount=2), [ShapedArray(bad[0], F32), ShapedArray(bad[1], F32)])
+    shapes = [((1, 1, 4), (1, 1, 3), [2], "SAME", (1, 1, 8)), ((1, 1, 5), (1, 1, 3), [2], "SAME", (1, 1, 10)), ((2, 3, 6), (5, 3, 4), [3], "SAME", (2, 5, 18)),
+              ((1, 1, 4), (1, 1, 3), [2], "VALID", (1, 1, 9)), ((1, 1, 5), (1, 1, 3), [2], "VALID", (1, 1, 11)), ((2, 3, 6), (5, 3, 4), [3], "VALID", (2, 5, 19)),
+              ((1, 1, 4, 4), (1, 1, 3, 3), [2, 2], "SAME", (1, 1, 8, 8)), ((2, 3, 8, 8), (5, 3, 3, 3), [2, 2], "SAME", (2, 5, 16, 16)),
+              ((1, 2, 5, 7), (4, 2, 4, 4), [2, 3], "SAME", (1, 4, 10, 21)), ((1, 1, 4, 4), (1, 1, 3, 3), [2, 2], "VALID", (1, 1, 9, 9)),
+              ((1, 2, 5, 5), (4, 2, 4, 4), [2, 2], "VALID", (1, 4, 12, 12))]
+    for xs, ks, st, pad, want in shapes:
+        J.jit(lambda a, b: seen.__setitem__("t", L.convTranspose(a, b, st, pad)) or seen["t"], [ShapedArray(xs, F32), ShapedArray(ks, F32)])
+        assert tuple(seen["t"].shape) == want, (xs, ks, st, pad)
+    _, (up,) = run(lambda a, b: L.convTranspose(a, b, [2], "SAME"), f32([[[1, 2, 3]]]), f32([[[1, 1]]]))
+    assert up.tolist() == [1, 1, 2, 2, 3, 3]
+    xt, kt = rng.integers(-3, 4, (1, 2, 4, 3)).astype(np.float32), rng.integers(-3, 4, (3, 2, 3, 2)).astype(np.float32)
+    _, (t2,) = run(lambda a, b: L.convTranspose(a, b, [2, 3], "SAME"), xt, kt)
+    pads = [L._conv_transpose_padding(3, 2, "SAME"), L._conv_transpose_padding(2, 3, "SAME")]
+    want = conv_reference(xt, kt, [1, 1], pads, [2, 3])
+    np.testing.assert_array_equal(t2.reshape(want.shape), want)
+    _, (t3,) = run(lambda a, b: L.convTranspose(a, b, [2, 3], "SAME", transposeKernel=True), xt, np.ascontiguousarray(np.flip(kt, (2, 3)).transpose(1, 0, 2, 3)))
+    np.testing.assert_array_equal(t3, t2)
 
 
 # ---- brute force --------------------------------------------------------------------------------------------
@@ -118,7 +196,11 @@ def _conv_case(c, backend):
 @pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "x".join(map(str, c["x"])) + "*" + "x".join(map(str, c["w"])))
 def test_convolution_matches_direct_loops(case):
     prog = _conv_case(case, OracleBackend())
-    assert len(prog.kernels) == 1  # one reduce kernel over C * prod(ks)
+    lowered = len(case["x"]) == 3 and case.get("ld") and min(case["padding"][0]) >= 0  # 1-D transposed: overlap-add lowering
+    if lowered:
+        assert sum(1 for k in prog.kernels if k.reduction is not None) == 1 and len(prog.kernels) > 1  # one Dot, then shifts and adds
+    else:
+        assert len(prog.kernels) == 1  # one reduce kernel over C * prod(ks)
 
 
 def test_pooling_and_window_reductions():

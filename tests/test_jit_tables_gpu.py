@@ -68,3 +68,25 @@ class _CompileOnly(T.OracleBackend):
 def test_table_on_the_gpu(name, monkeypatch):
     monkeypatch.setattr(T, "OracleBackend", _CompileOnly if WARM_ONLY else (lambda *a, **kw: _hip()))
     getattr(T, name)()
+
+
+# The reference's convolution tables (tests/test_conv.py) on the GPU, the same way.
+CONV_TABLE_TESTS = [
+    "test_1d_convolution_tables", "test_same_and_same_lower_padding", "test_2d_convolution_table", "test_transposed_convolution_table",
+    "test_transposed_convolution_downstream_ops_and_integer_dtype", "test_zero_dimensional_grouped_and_conv_transpose_tables",
+    "test_pooling_and_window_reductions",
+]
+
+
+@pytest.mark.parametrize("name", CONV_TABLE_TESTS)
+def test_convolution_table_on_the_gpu(name, monkeypatch):
+    import test_conv as C
+    monkeypatch.setattr(C, "OracleBackend", _CompileOnly if WARM_ONLY else (lambda *a, **kw: _hip()))
+    getattr(C, name)()
+
+
+def test_transposed_1d_lowering_cases_on_the_gpu(monkeypatch):
+    import test_conv as C
+    monkeypatch.setattr(C, "OracleBackend", _CompileOnly if WARM_ONLY else (lambda *a, **kw: _hip()))
+    for case in C.TRANSPOSED_1D:
+        C.test_transposed_1d_convolution_lowering_matches_direct_loops(*case)
