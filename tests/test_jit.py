@@ -1884,3 +1884,52 @@ def test_dtype_promotion_and_half_double_tables():
     assert uw.dtype == np.float64 and uw[1] == 3.1415926535897927
     _, (pm,) = _run_typed(lambda a, b: L.polymul(a, b), [d([1, 1e-12]), d([1, 1])], [F64, F64])
     assert pm.dtype == np.float64 and pm[1] == 1 + 1e-12
+
+
+def test_cholesky_lu_eigvalsh_and_argreduce_tables():
+    """test/lax-linalg.test.ts:24-84 (Cholesky 2x2, 3x3, a 512x512 blocked case, shape errors), :276-304 (LU with partial
+    pivoting: factors, pivots, permutation; P A = L U on 30x30); test/numpy-linalg.test.ts:23-34 (cholesky symmetrises
+    its input), :72-126 (eigvalsh: plain, batched, random 16x16, the lower triangle when not symmetrising);
+    test/argreduce.test.ts:14-70 (first index on ties, negatives, all equal, every axis of a 2-D array)."""
+    for x in (f32([[2, 1], [1, 2]]), f32([[4, 2, 1], [2, 5, 3], [1, 3, 6]])):
+        _, (l,) = run(lambda a: L.cholesky(a), x)
+        l = l.reshape(x.shape)
+        assert np.all(np.triu(l, 1) == 0) and l[1, 0] != 0
+        np.testing.assert_allclose(l @ l.T, x, rtol=1e-5)
+    n = 512
+    a = np.random.default_rng(n).standard_normal((n, n)).astype(np.float32)
+    spd = (a.T.astype(np.float64) @ a + n * np.eye(n)).astype(np.float32)
+    _, (lb,) = run(lambda m: L.cholesky(m), spd)
+    lb = lb.reshape(n, n).astype(np.float64)
+    assert np.abs(lb @ lb.T - spd).max() / np.abs(spd).max() < 1e-5
+    for shp in ((2, 3), (3,)):
+        with pytest.raises((ValueError, TypeError)):
+            J.jit(lambda m: L.cholesky(m), [ShapedArray(shp, F32)])
+    xs = f32([[4, 2.01], [1.99, 5]])
+    _, (ls,) = run(lambda m: L.linalgCholesky(m), xs)
+    ls = ls.reshape(2, 2)
+    np.testing.assert_allclose(ls @ ls.T, (xs + xs.T) / 2, rtol=1e-5)
+    _, (lu, piv, perm) = run(lambda m: list(J.lu(m)), f32([[4, 3], [6, 3]]))
+    np.testing.assert_allclose(lu, [6, 3, 0.6666667, 1.0], rtol=1e-6)
+    assert piv.tolist() == [1, 1] and perm.tolist() == [1, 0] and piv.dtype == np.int32
+    A = np.random.default_rng(0).uniform(0, 1, (30, 30)).astype(np.float32)
+    _, (pa, lu2) = run(lambda m: (lambda f: [L.matmul(J.gather(J._raise(L.eye(30)), [f[2]], [0], 0), m),
+                                             L.matmul(L.tril(f[0], -1).add(L.eye(30)), L.triu(f[0]))])(J.lu(m)), A)
+    np.testing.assert_allclose(pa, lu2, rtol=1e-5, atol=1e-6)
+    _, (e1, e2, e3) = run(lambda p, q, r: [L.eigvalsh(p), L.eigvalsh(q), L.eigvalsh(r, symmetrizeInput=False)], f32([[2, 1], [1, 2]]),
+                          f32([[[2, 1], [1, 2]], [[3, 1], [1, 3]]]), f32([[2, 100], [1, 2]]))
+    np.testing.assert_allclose(e1, [1, 3], rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(e2, [1, 3, 2, 4], rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(e3, [1, 3], rtol=1e-4, atol=1e-4)
+    _, (er,) = run(lambda m: L.eigvalsh(m), np.random.default_rng(0).standard_normal((16, 16)).astype(np.float32))
+    assert np.abs(er).sum() > 1
+    _, (m1, m2, m3) = run(lambda p, q, r: [L.argmax(p), L.argmax(q), L.argmax(r)], f32([3, 5, 5, 2, 5, 1]), f32([-10, -5, -20, -5, -15]), np.ones(5, np.float32))
+    assert (m1.tolist(), m2.tolist(), m3.tolist()) == ([1], [1], [0]) and m1.dtype == np.int32
+    g = f32([[1, 2, 3], [6, 5, 4], [7, 8, 9]])
+    _, (a0, a1, a2) = run(lambda p: [L.argmax(p), L.argmax(p, 0), L.argmax(p, 1)], g)
+    assert (a0.tolist(), a1.tolist(), a2.tolist()) == ([8], [2, 2, 2], [2, 0, 2])
+    _, (n1, n2) = run(lambda p, q: [L.argmin(p), L.argmin(q)], f32([3, 1, 5, 1, 1, 2]), np.full(5, 42, np.float32))
+    assert n1.tolist() == [1] and n2.tolist() == [0]
+    h = f32([[9, 8, 7], [4, 5, 6], [3, 2, 1]])
+    _, (b0, b1, b2) = run(lambda p: [L.argmin(p), L.argmin(p, 0), L.argmin(p, 1)], h)
+    assert (b0.tolist(), b1.tolist(), b2.tolist()) == ([8], [2, 2, 2], [2, 0, 2])

@@ -29,7 +29,7 @@ TABLE_TESTS = [
     "test_where_select_equality_and_membership_tables", "test_pad_and_split_family_tables", "test_joins_repeats_and_reshapes_tables",
     "test_polynomial_convolution_and_statistics_tables", "test_unwrap_tables", "test_reductions_views_dot_and_sort_tables",
     "test_activation_tables", "test_top_k_tables", "test_numpy_linalg_tables", "test_numpy_fft_tables", "test_random_distribution_tables",
-    "test_einsum_tables", "test_dtype_promotion_and_half_double_tables",
+    "test_einsum_tables", "test_dtype_promotion_and_half_double_tables", "test_cholesky_lu_eigvalsh_and_argreduce_tables",
 ]
 
 
