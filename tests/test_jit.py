@@ -916,6 +916,8 @@ def test_creation_tables():
     q = run0(lambda: [L.geomspace(1, 1000, 4), L.geomspace(1, 256, 9), L.geomspace(1000, 1, 4), L.geomspace(-1000, -1, 4), L.geomspace(1, 10000, 4, False)])
     for got, want in zip(q, ([1, 10, 100, 1000], [2 ** i for i in range(9)], [1000, 100, 10, 1], [-1000, -100, -10, -1], [1, 10, 100, 1000])):
         np.testing.assert_allclose(got, want, rtol=1e-5)
+    (gi,) = run0(lambda: L.geomspace(1, 16, 5, True, DType.Int32))
+    assert gi.dtype == np.int32 and gi.tolist() == [1, 2, 4, 8, 16]
     for bad in ((0, 10), (1, 0), (-1, 10)):
         with pytest.raises(ValueError):
             L.geomspace(*bad, 5)
