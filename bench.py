@@ -25,6 +25,8 @@ for p in (os.path.join(ROOT, "jax-js_amd"), ROOT):
 
 import numpy as np  # noqa: E402
 
+USE_GRAPHS = True  # --no-graphs clears it
+
 PEAK_HBM_GBS = 8000.0
 PEAK_F16_TFLOPS = 2500.0
 PEAK_F32_MATRIX_TFLOPS = 157.3
@@ -221,21 +223,23 @@ def bench_program_gpt2(be, hostrand, timed):
     dev.destroy_event(e0)
     dev.destroy_event(e1)
     # The same program captured once into a HIP graph and replayed with one launch call per forward.
-    from jaxjs_hip.graph import GraphedProgram
-    gp = GraphedProgram(be, prog, [bufs[i] for i in range(prog.nargs)])
-    for _ in range(5):
-        gp.launch()
-    dev.sync()
-    e0, e1 = dev.event(), dev.event()
-    dev.record(e0)
-    for _ in range(reps):
-        gp.launch()
-    dev.record(e1)
-    dev.sync()
-    graph_ms = dev.elapsed_ms(e0, e1) / reps
-    dev.destroy_event(e0)
-    dev.destroy_event(e1)
-    gp.close()
+    graph_ms = None
+    if USE_GRAPHS:
+        from jaxjs_hip.graph import GraphedProgram
+        gp = GraphedProgram(be, prog, [bufs[i] for i in range(prog.nargs)])
+        for _ in range(5):
+            gp.launch()
+        dev.sync()
+        e0, e1 = dev.event(), dev.event()
+        dev.record(e0)
+        for _ in range(reps):
+            gp.launch()
+        dev.record(e1)
+        dev.sync()
+        graph_ms = dev.elapsed_ms(e0, e1) / reps
+        dev.destroy_event(e0)
+        dev.destroy_event(e1)
+        gp.close()
     kernels = []
     for s, ex in zip(steps, exes):
         _, est = timed(be, ex, [bufs[i] for i in s.inputs], bufs[s.output], 3, 2)
@@ -250,7 +254,7 @@ def bench_program_gpt2(be, hostrand, timed):
     for sl in bufs.values():
         be.decRef(sl)
     flops = 1.417e11
-    return {"kernels_in_program": len(steps), "ms": round(total_ms, 4), "ms_as_hip_graph": round(graph_ms, 4), "sum_of_kernel_ms": round(sum(r["ms"] for r in kernels), 4),
+    return {"kernels_in_program": len(steps), "ms": round(total_ms, 4), "ms_as_hip_graph": None if graph_ms is None else round(graph_ms, 4), "sum_of_kernel_ms": round(sum(r["ms"] for r in kernels), 4),
             "model_flops": flops, "TFLOP/s": round(flops / (total_ms * 1e-3) / 1e12, 1), "per_kernel": kernels}
 
 
@@ -298,9 +302,11 @@ def bench_program_gpt2_fused(be, hostrand, timed):
             be.decRef(o)
 
     eager_ms = measure(eager)
-    gp = GraphedProgram(be, prog, ins)
-    graph_ms = measure(gp.launch)
-    gp.close()
+    graph_ms = None
+    if USE_GRAPHS:
+        gp = GraphedProgram(be, prog, ins)
+        graph_ms = measure(gp.launch)
+        gp.close()
     # the attention launch alone, on operands of the block's shape
     step = next(s for s in prog.steps if s.kind == "execute" and s.routine is not None)
     # (q, k and v reach the routine as three strided windows of the QKV projection's [batch, seq, 3d] output)
@@ -313,7 +319,7 @@ def bench_program_gpt2_fused(be, hostrand, timed):
         be.decRef(sl)
     H = d // heads
     full = 4.0 * batch * heads * seq * seq * H
-    return {"steps_in_program": sum(1 for s in prog.steps if s.kind == "execute"), "ms": round(eager_ms, 4), "ms_as_hip_graph": round(graph_ms, 4),
+    return {"steps_in_program": sum(1 for s in prog.steps if s.kind == "execute"), "ms": round(eager_ms, 4), "ms_as_hip_graph": None if graph_ms is None else round(graph_ms, 4),
             "TFLOP/s": round(1.417e11 / (eager_ms * 1e-3) / 1e12, 1),
             "attention_alone": {"ms": round(attn_ms, 5), "TFLOP/s_full_matrix_convention": round(full / (attn_ms * 1e-3) / 1e12, 1),
                                 "TFLOP/s_causal_half": round(full / 2 / (attn_ms * 1e-3) / 1e12, 1)}}
@@ -410,10 +416,14 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-settle", action="store_true", help="skip the clock-settling launches before the warm-up steps")
+    ap.add_argument("--no-graphs", action="store_true", help="skip the HIP-graph replays of the C5 programs (for runs under a profiler "
+                                                             "whose graph-launch tracing is not to be relied on)")
     ap.add_argument("--only", choices=["all", "gemm", "copy", "hbm"], default="all",
                     help="gemm: headline kernel only; copy: a plain f32 copy kernel of known size (counter calibration); "
                          "hbm: headline + the HBM-bound secondary workloads only (matvecs, row kernels, map)")
     args = ap.parse_args()
+    global USE_GRAPHS
+    USE_GRAPHS = not args.no_graphs
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
