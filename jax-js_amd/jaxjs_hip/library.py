@@ -2662,3 +2662,18 @@ def random_triangular(key: Tracer, left, mode, right, shape: Sequence[int] = ())
 
 def random_weibullMin(key: Tracer, scale, concentration, shape: Sequence[int] = ()):
     return J.mul(scale, J.exp(J.log(random_exponential(key, shape)).div(concentration)))
+
+
+def frexp(x: Tracer):
+    """Mantissa and exponent with x = m * 2^e, through floor(log2|x|) + 1 (numpy.ts:2799-2809)."""
+    x = J._raise(x)
+    exponent = J.where(J.equal(x, 0), 0, J.floor(log2(absolute(x))).add(1).astype(DType.Int32))
+    return [x.div(exp2(exponent.astype(x.dtype))), exponent]
+
+
+def flipud(x: Tracer):
+    return J.flip(x, 0)
+
+
+def fliplr(x: Tracer):
+    return J.flip(x, 1)

@@ -1935,3 +1935,16 @@ def test_cholesky_lu_eigvalsh_and_argreduce_tables():
     h = f32([[9, 8, 7], [4, 5, 6], [3, 2, 1]])
     _, (b0, b1, b2) = run(lambda p: [L.argmin(p), L.argmin(p, 0), L.argmin(p, 1)], h)
     assert (b0.tolist(), b1.tolist(), b2.tolist()) == ([8], [2, 2, 2], [2, 0, 2])
+
+
+def test_frexp_ldexp_and_flips():
+    """numpy.ts:2788-2809 (ldexp, frexp) and :1099-1107 (flipud / fliplr) against numpy on exactly representable values."""
+    x = f32([1, 8, 0.75, -6, 0, 1024])
+    _, (m, e, back) = run(lambda a: (lambda me: me + [L.ldexp(me[0], me[1].astype(F32))])(L.frexp(a)), x)
+    wm, we = np.frexp(x)
+    np.testing.assert_allclose(m, wm, rtol=2e-6, atol=1e-7)
+    assert e.dtype == np.int32 and e.tolist() == we.tolist()
+    np.testing.assert_allclose(back, x, rtol=2e-6)
+    mm = f32([[1, 2, 3], [4, 5, 6]])
+    _, (u, l) = run(lambda a: [L.flipud(a).mul(1), L.fliplr(a).mul(1)], mm)
+    assert u.tolist() == [4, 5, 6, 1, 2, 3] and l.tolist() == [3, 2, 1, 6, 5, 4]
