@@ -1948,3 +1948,26 @@ def test_frexp_ldexp_and_flips():
     mm = f32([[1, 2, 3], [4, 5, 6]])
     _, (u, l) = run(lambda a: [L.flipud(a).mul(1), L.fliplr(a).mul(1)], mm)
     assert u.tolist() == [4, 5, 6, 1, 2, 3] and l.tolist() == [3, 2, 1, 6, 5, 4]
+
+
+def test_jit_cases_of_the_tracing_suite():
+    """test/tracing.test.ts:578-625 (the jit() cases that need no other transformation): a cubic, the identity, the same
+    value returned twice, a gather by a constant index array, a static argument (a Python value closed over), a traced
+    function calling traced functions."""
+    _, (c,) = run(lambda a: a.mul(a).mul(a), f32(2).reshape(()))
+    assert c.tolist() == [8]
+    _, (i,) = run(lambda a: a, f32(3).reshape(()))
+    _, (d1, d2) = run(lambda a: [a, a], f32(3).reshape(()))
+    assert i.tolist() == [3] and d1.tolist() == [3] and d2.tolist() == [3]
+    idx = np.array([1, 3, 2, 0], np.int32)
+    _, (g,) = _run_typed(lambda a, ix: J.gather(a, [ix], [0], 0), [f32([10, 20, 30, 40]), idx], [F32, I32])
+    assert g.tolist() == [20, 40, 30, 10]
+    pick = lambda k: (lambda a: J.shrink(a, [(k, k + 1)]).reshape([]))
+    _, (s0,) = _run_typed(pick(0), [_i32(np.arange(20))], [I32])
+    _, (s3,) = _run_typed(pick(3), [_i32(np.arange(20))], [I32])
+    _, (s11,) = run(pick(3), f32([30, 1, 20, 11]))
+    assert s0.tolist() == [0] and s3.tolist() == [3] and s11.tolist() == [11]
+    f = lambda a: a.mul(a)
+    g2 = lambda a: f(f(a))
+    _, (q,) = run(g2, f32(3).reshape(()))
+    assert q.tolist() == [81]
