@@ -351,7 +351,12 @@ def _gen_sort(routine: Routine, numerics: str) -> Optional[KernelSource]:
     P = max(_next_pow2(n), 2)
     tile = min(P, SORT_TILE)
     kind, ctype = _SORT_KINDS[dtype]
+    # A thread moves eight words per pass (three strides at once, or its register group), so tile / 8 threads keep
+    # every lane busy and leave room for several blocks per CU, whose barriers then overlap; with few tiles in the
+    # launch the wider block (tile / 2) finishes its one tile sooner.
     threads = max(1, min(tile // 2, 1024))
+    if rows * (P // tile) >= 8 * 256 and tile >= 512:
+        threads = min(tile // 8, 1024)
     src = _prelude(numerics) + fill(template("sort.hip.inc"), dict(N=n, P=P, ROWS=rows, TILE=tile, ARGSORT=1 if argsort else 0,
                                                                    KIND=kind, T=ctype, THREADS=threads, GROUP=SORT_GROUP if P > 256 else 4))
     tiles = rows * (P // tile)
@@ -366,7 +371,7 @@ def _gen_sort(routine: Routine, numerics: str) -> Optional[KernelSource]:
             j //= 2
         steps.append(LaunchStep("jh_sort_merge", (tiles, 1, 1), (threads, 1, 1), 0, [("in", 0), ("scratch", 0)] + outs + [("const", k)]))
         k *= 2
-    scratch = [rows * P * 8] if P > tile else [8]
+    scratch = [rows * P * (8 if argsort else 4)] if P > tile else [8]
     need = {0: rows * n * byteWidth(dtype)}
     return KernelSource([src], steps, scratch, "sort", need, dict(n=n, rows=rows, P=P, tile=tile, argsort=argsort, launches=len(steps)))
 
