@@ -4,10 +4,10 @@ Every routine runs on the GPU; there is no host path.  A combination without a p
 kernels do not cover, an extent beyond a kernel's stated limit) raises `UnsupportedRoutineError` at prepare
 time, which is what the Backend interface prescribes for a routine a backend lacks (src/backend.ts:236-240).
 
-  Sort, Argsort                               `sort.hip.inc`     32-bit and float16 keys
-  Scatter                                     `scatter.hip.inc`  float32/float16/int32/uint32/bool updates
-  TriangularSolve, Cholesky, LU, JacobiEigh   `linalg.hip.inc`   float32
-  Fft                                         `fft.hip.inc`      float32
+  Sort, Argsort                               `sort.hip.inc`     32-bit, float16 and float64 keys
+  Scatter                                     `scatter.hip.inc`  float32/float16/float64/int32/uint32/bool updates
+  TriangularSolve, Cholesky, LU, JacobiEigh   `linalg.hip.inc`   float32/float64/float16 (arithmetic in double, as the reference)
+  Fft                                         `fft.hip.inc`      float32/float64/float16
   Attention (extension, not in the reference) `attention.hip.inc` float16, head size 64
 """
 
@@ -22,8 +22,8 @@ from .routine import Routine, Routines, ScatterOp
 from .shape import prod
 
 _SORT_KINDS = {DType.Float32: (0, "float"), DType.Float16: (1, "jh_f16"), DType.Int32: (2, "int"),
-               DType.Uint32: (3, "jh_u32"), DType.Bool: (2, "int")}
-SORT_TILE = 8192  # 64 KB of LDS: rows up to 8192 elements never leave the CU
+               DType.Uint32: (3, "jh_u32"), DType.Bool: (2, "int"), DType.Float64: (4, "double")}
+SORT_TILE = 8192  # 64 KB of LDS in 8-byte words: rows up to 8192 elements never leave the CU (4096 in 16-byte words)
 SORT_GROUP = 8    # elements a thread sorts in registers at the end of every stage (4 for rows of <= 256: more threads stay busy)
 CHOLESKY_PANEL_FROM = 192  # matrix order from which Cholesky runs panel by panel over the whole chip
 
@@ -53,15 +53,20 @@ def _round64(n: int, cap: int = 1024) -> int:
     return max(64, min(cap, (n + 63) // 64 * 64))
 
 
-_LINALG_DEFAULTS = dict(ROUTINE=0, N=1, M=1, THREADS=64, UNIT=0, IN_LDS=0, MAX_SWEEPS=0, TOL="0.0", BATCH=1, AHEAD=16, STAGED=0, RB=1)
+_LINALG_DEFAULTS = dict(ROUTINE=0, N=1, M=1, THREADS=64, UNIT=0, IN_LDS=0, MAX_SWEEPS=0, TOL="0.0", BATCH=1, AHEAD=16, STAGED=0, RB=1,
+                        ELEM="float", CMP="float")
+# Element types of the dense routines: C type, the type magnitudes are compared in, bytes per element.
+_FLOAT_ELEMS = {DType.Float32: ("float", "float", 4), DType.Float64: ("double", "double", 8), DType.Float16: ("jh_f16", "float", 2)}
 
 
 def _linalg_source(numerics: str, **params) -> str:
     return _prelude(numerics) + fill(template("linalg.hip.inc"), {**_LINALG_DEFAULTS, **params})
 
 
-def _all_f32(t) -> bool:
-    return all(d == DType.Float32 for d in t.inputDtypes)
+def _float_elem(t):
+    """(C type, comparison type, bytes) when every operand has one and the same floating-point type, else None."""
+    d = t.inputDtypes[0]
+    return _FLOAT_ELEMS.get(d) if all(x == d for x in t.inputDtypes) else None
 
 
 def _gen_cholesky(routine: Routine, numerics: str) -> Optional[KernelSource]:
@@ -72,15 +77,17 @@ def _gen_cholesky(routine: Routine, numerics: str) -> Optional[KernelSource]:
     n, m = shape[-2], shape[-1]
     if n != m:
         raise ValueError(f"cholesky: input must be square, got [{n}, {m}]")
-    if not _all_f32(t) or n > 8192:
+    el = _float_elem(t)
+    if el is None or n > 8192:
         return None
+    ctype, cmp_t, eb = el
     batch = prod(shape[:-2])
     if batch == 0 or n == 0:
         return _empty("cholesky", n=n, batch=batch)
     if n >= CHOLESKY_PANEL_FROM and batch * n * n * 8 <= CHOLESKY_RIGHT_LOOKING_MAX_BYTES:
         # Large matrices, right-looking: the running sums of the whole triangle in a double-precision scratch copy; per
         # 32-column panel one launch that finishes the panel and one that updates the trailing triangle (bit-identical).
-        src = _linalg_source(numerics, ROUTINE=5, N=n, M=batch)
+        src = _linalg_source(numerics, ROUTINE=5, N=n, M=batch, ELEM=ctype, CMP=cmp_t)
         grid1 = lambda count: (max(1, min((count + 255) // 256, 1 << 16)), 1, 1)  # noqa: E731
         steps = [LaunchStep("jh_chol_init", grid1(batch * n * n), (256, 1, 1), 0, [("in", 0), ("out", 0), ("scratch", 0)])]
         for j0 in range(0, n, 32):
@@ -90,12 +97,12 @@ def _gen_cholesky(routine: Routine, numerics: str) -> Optional[KernelSource]:
             if after > 0:
                 T = (after + 63) // 64
                 steps.append(LaunchStep("jh_chol_update", (batch * T * T, 1, 1), (256, 1, 1), 0, [("out", 0), ("scratch", 0), ("const", j0)]))
-        return KernelSource([src], steps, [batch * n * n * 8], "cholesky", {0: batch * n * n * 4},
+        return KernelSource([src], steps, [batch * n * n * 8], "cholesky", {0: batch * n * n * eb},
                             dict(n=n, batch=batch, panels=(n + 31) // 32, launches=len(steps), variant="right-looking"))
     if n >= CHOLESKY_PANEL_FROM and batch * n * n < (1 << 31):
         # Large matrices: 32-column panels, two launches each, every launch spread over the chip; the same sums in the
         # same order as the single-workgroup kernel (bit-identical results).
-        src = _linalg_source(numerics, ROUTINE=4, N=n, M=batch)
+        src = _linalg_source(numerics, ROUTINE=4, N=n, M=batch, ELEM=ctype, CMP=cmp_t)
         grid1 = lambda count: (max(1, min((count + 255) // 256, 1 << 16)), 1, 1)  # noqa: E731
         steps = [LaunchStep("jh_chol_zero", grid1(batch * n * n), (256, 1, 1), 0, [("out", 0)])]
         for j0 in range(0, n, 32):
@@ -104,12 +111,12 @@ def _gen_cholesky(routine: Routine, numerics: str) -> Optional[KernelSource]:
             after = max(0, n - j0 - 32)
             steps.append(LaunchStep("jh_chol_panel", (batch * max(1, (after + 63) // 64), 1, 1), (64, 1, 1), 0,
                                     [("scratch", 0), ("out", 0), ("const", j0)]))
-        return KernelSource([src], steps, [batch * n * 32 * 8], "cholesky", {0: batch * n * n * 4},
+        return KernelSource([src], steps, [batch * n * 32 * 8], "cholesky", {0: batch * n * n * eb},
                             dict(n=n, batch=batch, panels=(n + 31) // 32, launches=len(steps)))
     threads = _round64(n)
-    src = _linalg_source(numerics, ROUTINE=0, N=n, THREADS=threads)
+    src = _linalg_source(numerics, ROUTINE=0, N=n, THREADS=threads, ELEM=ctype, CMP=cmp_t)
     steps = [LaunchStep("jh_cholesky", (batch, 1, 1), (threads, 1, 1), 0, [("in", 0), ("out", 0), ("scratch", 0)])]
-    return KernelSource([src], steps, [batch * n * n * 4], "cholesky", {0: batch * n * n * 4}, dict(n=n, batch=batch, threads=threads))
+    return KernelSource([src], steps, [batch * n * n * eb], "cholesky", {0: batch * n * n * eb}, dict(n=n, batch=batch, threads=threads))
 
 
 def _gen_trisolve(routine: Routine, numerics: str) -> Optional[KernelSource]:
@@ -122,28 +129,31 @@ def _gen_trisolve(routine: Routine, numerics: str) -> Optional[KernelSource]:
     n = a_shape[-2]
     if n != a_shape[-1] or n != b_shape[-1]:
         raise ValueError(f"triangular_solve: incompatible shapes a={a_shape}, b={b_shape}")
-    if not _all_f32(t):
+    el = _float_elem(t)
+    if el is None:
         return None
+    ctype, cmp_t, eb = el
     mats, m = prod(a_shape[:-2]), b_shape[-2]
     if prod(b_shape[:-2]) != mats:
         raise ValueError(f"triangular_solve: incompatible shapes a={a_shape}, b={b_shape}")
     if mats == 0 or m == 0 or n == 0:
         return _empty("trisolve", n=n, m=m, batch=mats)
     unit = 1 if (routine.params or {}).get("unitDiagonal", False) else 0
-    need = {0: mats * n * n * 4, 1: mats * m * n * 4}
+    need = {0: mats * n * n * eb, 1: mats * m * n * eb}
     if TRISOLVE_STAGED_FROM <= n <= TRISOLVE_STAGED_MAX_N:
         # one wave of 64 right-hand sides + three waves staging blocks of rows in LDS as doubles (two buffers <= 128 KB)
         rb = max(1, min(8, TRISOLVE_STAGED_MAX_N // n))
-        src = _linalg_source(numerics, ROUTINE=1, N=n, M=m, THREADS=256, UNIT=unit, AHEAD=TRISOLVE_AHEAD, STAGED=1, RB=rb)
+        src = _linalg_source(numerics, ROUTINE=1, N=n, M=m, THREADS=256, UNIT=unit, AHEAD=TRISOLVE_AHEAD, STAGED=1, RB=rb,
+                             ELEM=ctype, CMP=cmp_t)
         steps = [LaunchStep("jh_trisolve_staged", (mats * ((m + 63) // 64), 1, 1), (256, 1, 1), 0,
                             [("in", 0), ("in", 1), ("out", 0), ("scratch", 0)])]
         return KernelSource([src], steps, [mats * m * n * 8], "trisolve", need,
                             dict(n=n, m=m, batch=mats, threads=256, staged=True, rows_per_block=rb))
     threads = 64 if m <= 64 else 256
-    src = _linalg_source(numerics, ROUTINE=1, N=n, M=m, THREADS=threads, UNIT=unit, AHEAD=TRISOLVE_AHEAD)
+    src = _linalg_source(numerics, ROUTINE=1, N=n, M=m, THREADS=threads, UNIT=unit, AHEAD=TRISOLVE_AHEAD, ELEM=ctype, CMP=cmp_t)
     blocks = mats * ((m + threads - 1) // threads)
     steps = [LaunchStep("jh_trisolve", (blocks, 1, 1), (threads, 1, 1), 0, [("in", 0), ("in", 1), ("out", 0), ("scratch", 0)])]
-    return KernelSource([src], steps, [mats * m * n * 4], "trisolve", need, dict(n=n, m=m, batch=mats, threads=threads, staged=False))
+    return KernelSource([src], steps, [mats * m * n * eb], "trisolve", need, dict(n=n, m=m, batch=mats, threads=threads, staged=False))
 
 
 def _gen_lu(routine: Routine, numerics: str) -> Optional[KernelSource]:
@@ -152,15 +162,17 @@ def _gen_lu(routine: Routine, numerics: str) -> Optional[KernelSource]:
     if len(shape) < 2:
         raise ValueError("lu: input must be at least 2D")
     m, n = shape[-2], shape[-1]
-    if not _all_f32(t):
+    el = _float_elem(t)
+    if el is None:
         return None
+    ctype, cmp_t, eb = el
     batch = prod(shape[:-2])
     if batch == 0 or m == 0:
         return _empty("lu", m=m, n=n, batch=batch)
     if min(m, n) >= LU_BY_COLUMNS_FROM and batch * m * n < (1 << 31):
         # Large matrices: two launches per column, the rank-1 update of the trailing block over the whole chip; the same
         # operations per element as the single-workgroup kernel (bit-identical).
-        src = _linalg_source(numerics, ROUTINE=6, N=n, M=m, THREADS=1024, BATCH=batch)
+        src = _linalg_source(numerics, ROUTINE=6, N=n, M=m, THREADS=1024, BATCH=batch, ELEM=ctype, CMP=cmp_t)
         grid1 = lambda count: (max(1, min((count + 255) // 256, 1 << 16)), 1, 1)  # noqa: E731
         steps = [LaunchStep("jh_lu_init", grid1(batch * m * n), (256, 1, 1), 0, [("in", 0), ("out", 0), ("out", 2)])]
         for j in range(min(m, n)):
@@ -170,14 +182,14 @@ def _gen_lu(routine: Routine, numerics: str) -> Optional[KernelSource]:
             if rows > 0 and cols > 0:
                 steps.append(LaunchStep("jh_lu_update", (batch * ((cols + 63) // 64) * ((rows + 31) // 32), 1, 1), (256, 1, 1), 0,
                                         [("out", 0), ("scratch", 0), ("scratch", 1), ("const", j)]))
-        return KernelSource([src], steps, [batch * m * 8, max(batch * 4, 16)], "lu", {0: batch * m * n * 4},
+        return KernelSource([src], steps, [batch * m * 8, max(batch * 4, 16)], "lu", {0: batch * m * n * eb},
                             dict(m=m, n=n, batch=batch, launches=len(steps), variant="by columns"))
     if m > 4096:  # single workgroup: the multipliers of one column live in LDS as doubles
         return None
     threads = _round64(max(m, n))
-    src = _linalg_source(numerics, ROUTINE=2, N=n, M=m, THREADS=threads)
+    src = _linalg_source(numerics, ROUTINE=2, N=n, M=m, THREADS=threads, ELEM=ctype, CMP=cmp_t)
     steps = [LaunchStep("jh_lu", (batch, 1, 1), (threads, 1, 1), 0, [("in", 0), ("out", 0), ("out", 1), ("out", 2)])]
-    return KernelSource([src], steps, [], "lu", {0: batch * m * n * 4}, dict(m=m, n=n, batch=batch, threads=threads))
+    return KernelSource([src], steps, [], "lu", {0: batch * m * n * eb}, dict(m=m, n=n, batch=batch, threads=threads))
 
 
 def _gen_jacobi(routine: Routine, numerics: str) -> Optional[KernelSource]:
@@ -190,18 +202,20 @@ def _gen_jacobi(routine: Routine, numerics: str) -> Optional[KernelSource]:
         raise ValueError(f"jacobi_eigh: input must be square, got {shape}")
     if t.inputDtypes[0] not in (DType.Float32, DType.Float16, DType.Float64):
         raise TypeError("jacobi_eigh: input must be floating-point")
-    if not _all_f32(t) or n > 16384:
+    el = _float_elem(t)
+    if el is None or n > 16384:
         return None
+    ctype, cmp_t, eb = el
     batch = prod(shape[:-2])
     if batch == 0 or n == 0:
         return _empty("jacobi", n=n, batch=batch)
     params = routine.params or {}
     threads = _round64(n)
-    in_lds = 1 if 2 * n * n * 4 <= 150 * 1024 else 0  # both matrices in the CU's 160 KB of LDS: n <= 138
+    in_lds = 1 if 2 * n * n * eb <= 150 * 1024 else 0  # both matrices in the CU's 160 KB of LDS: n <= 138 in float32
     src = _linalg_source(numerics, ROUTINE=3, N=n, THREADS=threads, IN_LDS=in_lds, MAX_SWEEPS=int(params["maxSweeps"]),
-                         TOL=repr(float(params["tolerance"])))
+                         TOL=repr(float(params["tolerance"])), ELEM=ctype, CMP=cmp_t)
     steps = [LaunchStep("jh_jacobi", (batch, 1, 1), (threads, 1, 1), 0, [("in", 0), ("out", 0), ("out", 1)])]
-    return KernelSource([src], steps, [], "jacobi", {0: batch * n * n * 4}, dict(n=n, batch=batch, threads=threads, in_lds=bool(in_lds)))
+    return KernelSource([src], steps, [], "jacobi", {0: batch * n * n * eb}, dict(n=n, batch=batch, threads=threads, in_lds=bool(in_lds)))
 
 
 TRISOLVE_STAGED_FROM = 128    # matrix size from which TriangularSolve stages the matrix in LDS with helper waves
@@ -226,17 +240,20 @@ def _gen_fft(routine: Routine, numerics: str) -> Optional[KernelSource]:
     factors = [int(f) for f in params["factors"]]
     if prod(factors) != n or any(f < 1 for f in factors):
         raise ValueError(f"fft: factors {factors} do not multiply to the axis length {n}")
-    if not _all_f32(t) or n >= (1 << 30):
+    el = _float_elem(t)
+    if el is None or n >= (1 << 30):
         return None
+    ctype, _, eb = el
     rows = prod(shape[:-1])
     if rows == 0:
         return _empty("fft", n=n, rows=rows)
     # Rows that fit the LDS twice over (16 bytes per point) run in one launch, one workgroup per row, unless there are
     # too few rows for that to use the chip (a single long row is quicker spread over many workgroups per stage).
     S = len(factors)
-    fused = S >= 1 and n <= FFT_FUSED_MAX_N and (n <= 2048 or rows >= 64)
+    fused_max = FFT_FUSED_MAX_N * 4 // max(eb, 4)  # four buffers of n elements: 128 KiB at most
+    fused = S >= 1 and n <= fused_max and (n <= 2048 or rows >= 64)
     if "singleLaunch" in params:  # tests pin either path
-        fused = bool(params["singleLaunch"]) and S >= 1 and n <= FFT_FUSED_MAX_N
+        fused = bool(params["singleLaunch"]) and S >= 1 and n <= fused_max
     threads = min(1024, max(64, _round64(n)))
     # Twiddle tables: stage s has span_s entries for (q, j) and radix_s^2 for (q, p), 16 bytes each.
     offsets, spans, prev = [0], [], 1
@@ -244,13 +261,13 @@ def _gen_fft(routine: Routine, numerics: str) -> Optional[KernelSource]:
         spans.append(prev * radix + radix * radix)
         offsets.append(offsets[-1] + spans[-1])
         prev *= radix
-    lds_entries = max(spans) if spans and 16 * n + 16 * max(spans) <= 150 * 1024 else 0
-    src = _prelude(numerics) + fill(template("fft.hip.inc"), dict(N=n, ROWS=rows, INVERSE=1 if params.get("inverse") else 0,
+    lds_entries = max(spans) if spans and 4 * eb * n + 16 * max(spans) <= 150 * 1024 else 0
+    src = _prelude(numerics) + fill(template("fft.hip.inc"), dict(N=n, ROWS=rows, ELEM=ctype, INVERSE=1 if params.get("inverse") else 0,
                                                                   NF=len(factors), FACTORS=", ".join(map(str, factors)) or "1",
                                                                   TW_OFFSETS=", ".join(map(str, offsets if S else [0, 0])),
                                                                   FUSED=1 if fused else 0, FUSED_THREADS=threads,
                                                                   FUSED_TABLE_ENTRIES=lds_entries))
-    need = {0: rows * n * 4, 1: rows * n * 4}
+    need = {0: rows * n * eb, 1: rows * n * eb}
     if fused:
         steps = [LaunchStep("jh_fft_rows", (min(rows, 1 << 16), 1, 1), (threads, 1, 1), 0, [("in", 0), ("in", 1), ("out", 0), ("out", 1)])]
         return KernelSource([src], steps, [], "fft", need, dict(n=n, rows=rows, factors=factors, launches=1, fused=True, lds_tables=bool(lds_entries)))
@@ -264,12 +281,12 @@ def _gen_fft(routine: Routine, numerics: str) -> Optional[KernelSource]:
                                 target(s_ - 1) + target(s_) + [("scratch", 2), ("const", prev), ("const", radix),
                                                                ("const", 1 if s_ == S - 1 else 0), ("const", s_)]))
         prev *= radix
-    scratch = [rows * n * 4, rows * n * 4, max(offsets[-1], 1) * 16] if S >= 1 else [8, 8, 16]
+    scratch = [rows * n * eb, rows * n * eb, max(offsets[-1], 1) * 16] if S >= 1 else [8, 8, 16]
     return KernelSource([src], steps, scratch, "fft", need, dict(n=n, rows=rows, factors=factors, launches=len(steps), fused=False))
 
 
 _SCATTER_KINDS = {DType.Float32: (0, "float"), DType.Float16: (1, "jh_f16"), DType.Int32: (2, "int"), DType.Uint32: (3, "jh_u32"),
-                  DType.Bool: (4, "int")}
+                  DType.Bool: (4, "int"), DType.Float64: (5, "double")}
 
 
 def _gen_scatter(routine: Routine, numerics: str) -> Optional[KernelSource]:
@@ -340,7 +357,7 @@ def _gen_sort(routine: Routine, numerics: str) -> Optional[KernelSource]:
     if len(shape) == 0:
         raise ValueError(f"{routine.name.value.lower()}: cannot sort a scalar")
     if dtype not in _SORT_KINDS:
-        return None  # float64 keys do not fit the 32-bit key
+        return None
     n = shape[-1]
     rows = prod(shape[:-1])
     argsort = routine.name == Routines.Argsort
@@ -349,8 +366,9 @@ def _gen_sort(routine: Routine, numerics: str) -> Optional[KernelSource]:
     if n >= (1 << 30):
         return None
     P = max(_next_pow2(n), 2)
-    tile = min(P, SORT_TILE)
     kind, ctype = _SORT_KINDS[dtype]
+    word = (8 if argsort else 4) * (2 if dtype == DType.Float64 else 1)  # bytes per keyed word
+    tile = min(P, SORT_TILE * 8 // max(word, 8))
     # A thread moves eight words per pass (three strides at once, or its register group), so tile / 8 threads keep
     # every lane busy and leave room for several blocks per CU, whose barriers then overlap; with few tiles in the
     # launch the wider block (tile / 2) finishes its one tile sooner.
@@ -371,7 +389,7 @@ def _gen_sort(routine: Routine, numerics: str) -> Optional[KernelSource]:
             j //= 2
         steps.append(LaunchStep("jh_sort_merge", (tiles, 1, 1), (threads, 1, 1), 0, [("in", 0), ("scratch", 0)] + outs + [("const", k)]))
         k *= 2
-    scratch = [rows * P * (8 if argsort else 4)] if P > tile else [8]
+    scratch = [rows * P * word] if P > tile else [16]
     need = {0: rows * n * byteWidth(dtype)}
     return KernelSource([src], steps, scratch, "sort", need, dict(n=n, rows=rows, P=P, tile=tile, argsort=argsort, launches=len(steps)))
 

@@ -4,7 +4,8 @@ run as GPU kernels or raise.
 
   Sort / Argsort      numpy (TypedArray.prototype.sort order: NaNs last; Argsort stable)   src/routine.ts:185-213
   Scatter             numpy, sequential semantics (later updates win, adds in order)        src/routine.ts:226-296
-  TriangularSolve, Cholesky, LU, JacobiEigh, Fft   C (`routines_oracle.c`), float32 only    src/routine.ts:298-640
+  TriangularSolve, Cholesky, LU, JacobiEigh, Fft   C (`routines_oracle.c` + `routines_body.h`), float32 / float64 /
+                      float16 elements, every scalar a double as in the reference                 src/routine.ts:298-640
   Attention           numpy float64 (the fused-attention extension)                        src/library/nn.ts:478-583
 
 Parity pinning: the linear-algebra and FFT functions are checked in `tests/test_routines_oracle.py` against what
@@ -29,7 +30,7 @@ _NP = {"float32": np.float32, "int32": np.int32, "uint32": np.uint32, "bool": np
 
 
 def build(force: bool = False) -> str:
-    srcs = [os.path.join(_HERE, f) for f in ("routines_oracle.c", "Makefile")]
+    srcs = [os.path.join(_HERE, f) for f in ("routines_oracle.c", "routines_body.h", "half.h", "Makefile")]
     stale = (not os.path.exists(_LIB_PATH)) or any(os.path.getmtime(s) > os.path.getmtime(_LIB_PATH) for s in srcs)
     if force or stale:
         subprocess.run(["make", "-C", _HERE, "-B" if force else "-s", "libroutines_oracle.so"], check=True, stdout=subprocess.DEVNULL)
@@ -42,12 +43,13 @@ def lib() -> ctypes.CDLL:
         build()
         _lib = ctypes.CDLL(_LIB_PATH)
         P, I64 = ctypes.c_void_p, ctypes.c_int64
-        _lib.ro_triangular_solve.argtypes = [P, P, P, I64, I64, I64, ctypes.c_int]
-        _lib.ro_cholesky.argtypes = [P, P, I64, I64]
-        _lib.ro_lu.argtypes = [P, P, P, P, I64, I64, I64]
-        _lib.ro_jacobi_eigh.argtypes = [P, P, P, I64, I64, I64, ctypes.c_double]
-        _lib.ro_fft.argtypes = [P, P, P, P, I64, I64, P, ctypes.c_int32, ctypes.c_int]
-        _lib.ro_fft.restype = ctypes.c_int
+        for sfx in ("", "_f64", "_f16"):
+            getattr(_lib, "ro_triangular_solve" + sfx).argtypes = [P, P, P, I64, I64, I64, ctypes.c_int]
+            getattr(_lib, "ro_cholesky" + sfx).argtypes = [P, P, I64, I64]
+            getattr(_lib, "ro_lu" + sfx).argtypes = [P, P, P, P, I64, I64, I64]
+            getattr(_lib, "ro_jacobi_eigh" + sfx).argtypes = [P, P, P, I64, I64, I64, ctypes.c_double]
+            getattr(_lib, "ro_fft" + sfx).argtypes = [P, P, P, P, I64, I64, P, ctypes.c_int32, ctypes.c_int]
+            getattr(_lib, "ro_fft" + sfx).restype = ctypes.c_int
     return _lib
 
 
@@ -73,9 +75,16 @@ def _typed(bufs: Sequence, dtypes, shapes, writable: bool, views=None) -> List[n
     return out
 
 
-def _f32_only(name, dtypes):
-    if any(str(d) != "float32" for d in dtypes):
-        raise NotImplementedError(f"{name}: the checker covers float32 operands")
+_DENSE = {"float32": ("", np.float32), "float64": ("_f64", np.float64), "float16": ("_f16", np.float16)}
+
+
+def _dense(name, fn, dtypes):
+    """The C function of `fn` for the operands' common floating-point type, and that type in numpy."""
+    kinds = {str(d) for d in dtypes}
+    if len(kinds) != 1 or next(iter(kinds)) not in _DENSE:
+        raise NotImplementedError(f"{name}: the checker covers operands of one floating-point type, got {sorted(kinds)}")
+    sfx, npt = _DENSE[next(iter(kinds))]
+    return getattr(lib(), fn + sfx), npt
 
 
 def runCpuRoutine(routine, inputs: Sequence, outputs: Sequence) -> None:
@@ -99,7 +108,7 @@ def runCpuRoutine(routine, inputs: Sequence, outputs: Sequence) -> None:
     elif name == "Scatter":
         scatter(t, ins, outs[0], params)
     elif name == "TriangularSolve":
-        _f32_only(name, t.inputDtypes)
+        fn, npt = _dense(name, "ro_triangular_solve", t.inputDtypes)
         a, b = np.ascontiguousarray(ins[0]), np.ascontiguousarray(ins[1])
         if a.ndim < 2 or b.ndim < 2:
             raise ValueError("triangular_solve: operands must be at least 2D")
@@ -107,46 +116,46 @@ def runCpuRoutine(routine, inputs: Sequence, outputs: Sequence) -> None:
         if n != a.shape[-1] or n != b.shape[-1]:
             raise ValueError(f"triangular_solve: incompatible shapes a={a.shape}, b={b.shape}")
         mats = a.size // (n * n) if n else 0
-        x = np.zeros(b.shape, np.float32)
-        lib().ro_triangular_solve(_ptr(a), _ptr(b), _ptr(x), mats, b.shape[-2], n, int(bool(params.get("unitDiagonal", False))))
+        x = np.zeros(b.shape, npt)
+        fn(_ptr(a), _ptr(b), _ptr(x), mats, b.shape[-2], n, int(bool(params.get("unitDiagonal", False))))
         outs[0][...] = x
     elif name == "Cholesky":
-        _f32_only(name, t.inputDtypes)
+        fn, npt = _dense(name, "ro_cholesky", t.inputDtypes)
         a = np.ascontiguousarray(ins[0])
         if a.ndim < 2:
             raise ValueError("cholesky: input must be at least 2D")
         n = a.shape[-2]
         if n != a.shape[-1]:
             raise ValueError(f"cholesky: input must be square, got [{n}, {a.shape[-1]}]")
-        y = np.zeros(a.shape, np.float32)
+        y = np.zeros(a.shape, npt)
         with np.errstate(all="ignore"):
-            lib().ro_cholesky(_ptr(a), _ptr(y), a.size // (n * n) if n else 0, n)
+            fn(_ptr(a), _ptr(y), a.size // (n * n) if n else 0, n)
         outs[0][...] = y
     elif name == "LU":
-        _f32_only(name, t.inputDtypes)
+        fn, npt = _dense(name, "ro_lu", t.inputDtypes)
         a = np.ascontiguousarray(ins[0])
         if a.ndim < 2:
             raise ValueError("lu: input must be at least 2D")
         m, n = a.shape[-2:]
         mats = int(np.prod(a.shape[:-2], dtype=np.int64))
-        lu = np.zeros(a.shape, np.float32)
+        lu = np.zeros(a.shape, npt)
         piv = np.zeros(a.shape[:-2] + (min(m, n),), np.int32)
         perm = np.zeros(a.shape[:-2] + (m,), np.int32)
-        lib().ro_lu(_ptr(a), _ptr(lu), _ptr(piv), _ptr(perm), mats, m, n)
+        fn(_ptr(a), _ptr(lu), _ptr(piv), _ptr(perm), mats, m, n)
         outs[0][...], outs[1][...], outs[2][...] = lu, piv, perm
     elif name == "JacobiEigh":
-        _f32_only(name, t.inputDtypes)
+        fn, npt = _dense(name, "ro_jacobi_eigh", t.inputDtypes)
         a = np.ascontiguousarray(ins[0])
         if a.ndim < 2:
             raise ValueError("jacobi_eigh: input must be at least 2D")
         n = a.shape[-1]
         if n != a.shape[-2]:
             raise ValueError(f"jacobi_eigh: input must be square, got {a.shape}")
-        d, v = np.zeros(a.shape, np.float32), np.zeros(a.shape, np.float32)
-        lib().ro_jacobi_eigh(_ptr(a), _ptr(d), _ptr(v), a.size // (n * n) if n else 0, n, int(params["maxSweeps"]), float(params["tolerance"]))
+        d, v = np.zeros(a.shape, npt), np.zeros(a.shape, npt)
+        fn(_ptr(a), _ptr(d), _ptr(v), a.size // (n * n) if n else 0, n, int(params["maxSweeps"]), float(params["tolerance"]))
         outs[0][...], outs[1][...] = d, v
     elif name == "Fft":
-        _f32_only(name, t.inputDtypes)
+        fn, npt = _dense(name, "ro_fft", t.inputDtypes)
         re, im = np.ascontiguousarray(ins[0]), np.ascontiguousarray(ins[1])
         if re.ndim < 1:
             raise ValueError("fft: input must be at least 1D")
@@ -154,8 +163,8 @@ def runCpuRoutine(routine, inputs: Sequence, outputs: Sequence) -> None:
         if n < 1:
             raise ValueError(f"fft: final axis must be non-empty, got {n}")
         factors = np.asarray(list(params["factors"]), np.int32)
-        o_re, o_im = np.zeros(re.shape, np.float32), np.zeros(re.shape, np.float32)
-        if lib().ro_fft(_ptr(re), _ptr(im), _ptr(o_re), _ptr(o_im), re.size // n, n, _ptr(factors), len(factors), int(bool(params["inverse"]))):
+        o_re, o_im = np.zeros(re.shape, npt), np.zeros(re.shape, npt)
+        if fn(_ptr(re), _ptr(im), _ptr(o_re), _ptr(o_im), re.size // n, n, _ptr(factors), len(factors), int(bool(params["inverse"]))):
             raise MemoryError("fft oracle: allocation failed")
         outs[0][...], outs[1][...] = o_re, o_im
     elif name == "Attention":

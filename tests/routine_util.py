@@ -69,21 +69,21 @@ def bits_equal(a, b):
 
 # Routine constructors in the shapes the reference's front-end hands a backend.
 def cholesky(a):
-    return routine_for(Routines.Cholesky, [a], [a.shape], [DType.Float32])
+    return routine_for(Routines.Cholesky, [a], [a.shape], [NP2DT[a.dtype]])
 
 
 def triangular_solve(a, b, unit_diagonal=False):
-    return routine_for(Routines.TriangularSolve, [a, b], [b.shape], [DType.Float32], dict(unitDiagonal=unit_diagonal))
+    return routine_for(Routines.TriangularSolve, [a, b], [b.shape], [NP2DT[b.dtype]], dict(unitDiagonal=unit_diagonal))
 
 
 def lu(a):
     m, n = a.shape[-2:]
     batch = list(a.shape[:-2])
-    return routine_for(Routines.LU, [a], [a.shape, batch + [min(m, n)], batch + [m]], [DType.Float32, DType.Int32, DType.Int32])
+    return routine_for(Routines.LU, [a], [a.shape, batch + [min(m, n)], batch + [m]], [NP2DT[a.dtype], DType.Int32, DType.Int32])
 
 
 def jacobi_eigh(a, max_sweeps=30, tolerance=1e-7):
-    return routine_for(Routines.JacobiEigh, [a], [a.shape, a.shape], [DType.Float32, DType.Float32], dict(maxSweeps=max_sweeps, tolerance=tolerance))
+    return routine_for(Routines.JacobiEigh, [a], [a.shape, a.shape], [NP2DT[a.dtype]] * 2, dict(maxSweeps=max_sweeps, tolerance=tolerance))
 
 
 def factor_fft_size(n):
@@ -106,7 +106,7 @@ def factor_fft_size(n):
 
 def fft(re, im, inverse=False, factors=None):
     factors = factor_fft_size(re.shape[-1]) if factors is None else factors
-    return routine_for(Routines.Fft, [re, im], [re.shape, re.shape], [DType.Float32, DType.Float32], dict(factors=factors, inverse=inverse))
+    return routine_for(Routines.Fft, [re, im], [re.shape, re.shape], [NP2DT[re.dtype]] * 2, dict(factors=factors, inverse=inverse))
 
 
 def scatter(updates, indices, op, shape, axis, out_dim, unique=False, dtype=None):

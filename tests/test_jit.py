@@ -1468,6 +1468,15 @@ def test_numpy_linalg_tables():
     np.testing.assert_array_equal(p0.reshape(2, 2), np.eye(2))
     np.testing.assert_allclose(p3.reshape(2, 2), np.linalg.matrix_power(sym.astype(np.float64), 3), rtol=1e-5)
     np.testing.assert_allclose(pm.reshape(2, 2), np.linalg.matrix_power(sym.astype(np.float64), -2), rtol=1e-4)
+    # "inv preserves input dtype" / "matrixPower(A, 0) preserves input dtype" (:270-283, :297-309): float64 on the CPU
+    # devices, float16 on the GPU device -- both element types run through the LU and triangular-solve routines here
+    for dt, npt in ((DType.Float64, np.float64), (DType.Float16, np.float16)):
+        seen = {}
+        _, (ident, p0) = run(lambda a: [L.matmul(a, seen.setdefault("inv", L.inv(a))), J._raise(seen.setdefault("p0", L.matrixPower(a, 0))).mul(1)],
+                             sym.astype(npt), dtype=dt)
+        assert seen["inv"].dtype == dt and seen["p0"].dtype == dt and ident.dtype == npt and p0.dtype == npt
+        np.testing.assert_allclose(ident.reshape(2, 2).astype(np.float64), np.eye(2), rtol=0, atol=1e-3)
+        np.testing.assert_allclose(p0.reshape(2, 2).astype(np.float64), np.eye(2), rtol=0, atol=1e-3)
     A, B, C = f32([[1, 2], [3, 4]]), f32([[5, 6, 7], [8, 9, 10]]), f32([[11, 12], [13, 14], [15, 16]])
     _, (m3, m2) = run(lambda a, b, c: [L.multiDot([a, b, c]), L.multiDot([a, b])], A, B, C)
     np.testing.assert_allclose(m3.reshape(2, 2), A @ B @ C, rtol=1e-6)

@@ -78,8 +78,10 @@ def test_argsort_tables_and_stability():
 
 
 def _data(shape, dtype):
-    if dtype == DType.Float32 or dtype == DType.Float16:
+    if dtype in (DType.Float32, DType.Float16, DType.Float64):
         x = RNG.normal(0, 10, shape).astype(numpyDtype(dtype))
+        if dtype == DType.Float64:  # keys that differ only below float32 resolution
+            x += RNG.integers(-3, 4, shape) * 2.0 ** -40
         flat = x.reshape(-1)
         n = flat.size
         if n >= 8:
@@ -101,7 +103,7 @@ SHAPES = [(1,), (2,), (7, 3), (5, 100), (3, 2048), (4, 4096), (2, 5000), (33, 81
 
 
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
-@pytest.mark.parametrize("dtype", [DType.Float32, DType.Int32, DType.Uint32, DType.Float16, DType.Bool], ids=lambda d: d.value)
+@pytest.mark.parametrize("dtype", [DType.Float32, DType.Int32, DType.Uint32, DType.Float16, DType.Bool, DType.Float64], ids=lambda d: d.value)
 def test_sort_matches_host_routine(shape, dtype):
     x = _data(shape, dtype)
     (y,), (want,) = run(Routines.Sort, x, dtype)
@@ -112,7 +114,7 @@ def test_sort_matches_host_routine(shape, dtype):
 
 
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
-@pytest.mark.parametrize("dtype", [DType.Float32, DType.Int32, DType.Float16], ids=lambda d: d.value)
+@pytest.mark.parametrize("dtype", [DType.Float32, DType.Int32, DType.Float16, DType.Float64], ids=lambda d: d.value)
 def test_argsort_matches_host_routine(shape, dtype):
     x = _data(shape, dtype)
     (v, i), (wv, wi) = run(Routines.Argsort, x, dtype)
@@ -131,6 +133,7 @@ def test_zero_sized_rows_and_unsupported_dtype_path():
     assert be.readSync(b) == b""
     be.decRef(a)
     be.decRef(b)
-    # float64 keys do not fit the 64-bit key|position words: refused at prepare time, never run on the host.
+    # An element type a routine's kernels do not cover is refused at prepare time, never run on the host.
+    import routine_util as R
     with pytest.raises(UnsupportedRoutineError):
-        be.prepareRoutineSync(make(Routines.Sort, (4, 50), DType.Float64))
+        be.prepareRoutineSync(R.routine_for(Routines.Cholesky, [np.zeros((4, 4), np.int32)], [(4, 4)], [DType.Int32]))

@@ -1,7 +1,7 @@
 """Scatter, TriangularSolve, Cholesky, LU, JacobiEigh and Fft as GPU kernels against the CPU checker.
 
-The linear-algebra kernels keep the reference's arithmetic (double scalars, float32 stores, the same order per stored
-element), so their results must be bit-identical to the checker's.  Scatter is bit-identical except float
+The linear-algebra kernels keep the reference's arithmetic (double scalars, stores rounded to the element type --
+float32, float64 or float16 --, the same order per stored element), so their results must be bit-identical to the checker's.  Scatter is bit-identical except float
 accumulation onto repeated destinations (atomic adds in any order: compared within a sum-scaled bound).  Fft takes
 its sines and cosines from the device math library, whose last-place differences from the host's can decide a
 float32 rounding tie in a butterfly (seen for radix-3 stages behind an even stride; power-of-two and prime sizes come
@@ -189,6 +189,93 @@ def test_fft_factor_orders_and_validation():
         R.run_gpu(R.fft(re, im, False, [4, 4]), [re, im])
 
 
+# ---- float64 and float16 elements: the same kernels with another stored type (every kernel variant once per type)
+ELEMS = [np.float64, np.float16]
+
+
+@pytest.mark.parametrize("dt", ELEMS, ids=lambda d: np.dtype(d).name)
+@pytest.mark.parametrize("shape", [(3, 3), (2, 3, 64, 64), (200, 200), (2, 333, 333)], ids=str)
+def test_cholesky_other_element_types(shape, dt, monkeypatch):
+    n = shape[-1]
+    x = (spd(tuple(shape[:-2]), n).astype(np.float64) / (1.0 if dt == np.float64 else n)).astype(dt)
+    got, want, ks = both(R.cholesky(x), [x])
+    assert got[0].dtype == dt and ("panels" in ks.info) == (n >= 192)
+    assert_bits(got, want, f"cholesky {shape} {np.dtype(dt).name} {ks.info}")
+    if n >= 192:  # and the left-looking panels
+        from jaxjs_hip import routinegen
+        from gpu_util import backend
+        monkeypatch.setattr(routinegen, "CHOLESKY_RIGHT_LOOKING_MAX_BYTES", 0)
+        backend().clearCache()
+        left, k2 = R.run_gpu(R.cholesky(x), [x])
+        backend().clearCache()
+        assert "variant" not in k2.info and "panels" in k2.info
+        assert_bits(left, want, f"cholesky left-looking {shape} {np.dtype(dt).name}")
+
+
+@pytest.mark.parametrize("dt", ELEMS, ids=lambda d: np.dtype(d).name)
+@pytest.mark.parametrize("case", [((9, 9), 4), ((2, 2, 16, 16), 100), ((2, 131, 131), 70), ((300, 300), 300)], ids=str)
+@pytest.mark.parametrize("unit", [False, True])
+def test_triangular_solve_other_element_types(case, unit, dt):
+    ashape, m = case
+    n = ashape[-1]
+    a = (np.triu(RNG.standard_normal(ashape)) * (0.3 if unit else 1.0) + (0 if unit else 1) * np.sqrt(n) * np.eye(n)
+         + np.tril(RNG.standard_normal(ashape), -1)).astype(dt)
+    b = RNG.standard_normal(ashape[:-2] + (m, n)).astype(dt)
+    got, want, ks = both(R.triangular_solve(a, b, unit), [a, b])
+    assert got[0].dtype == dt and ks.info["staged"] == (n >= 128)
+    assert_bits(got, want, f"triangular_solve {case} {np.dtype(dt).name} {ks.info}")
+
+
+@pytest.mark.parametrize("dt", ELEMS, ids=lambda d: np.dtype(d).name)
+@pytest.mark.parametrize("shape", [(2, 7, 5), (3, 12, 20), (150, 97), (260, 300), (2, 300, 256)], ids=str)
+def test_lu_other_element_types(shape, dt):
+    a = RNG.uniform(-1, 1, shape).astype(dt)
+    if shape == (260, 300):
+        a[:, 3] = 0       # a zero pivot column
+        a[10, 5] = np.nan  # a NaN that must not win the pivot search
+        a[20:23, 7] = [0.75, -0.75, 0.75]
+    got, want, ks = both(R.lu(a), [a])
+    assert got[0].dtype == dt and (ks.info.get("variant") == "by columns") == (min(shape[-2:]) >= 192)
+    assert_bits(got, want, f"lu {shape} {np.dtype(dt).name} {ks.info}")
+
+
+@pytest.mark.parametrize("dt", ELEMS, ids=lambda d: np.dtype(d).name)
+@pytest.mark.parametrize("shape", [(2, 2), (4, 20, 20), (2, 64, 64), (100, 100), (150, 150)], ids=str)
+def test_jacobi_eigh_other_element_types(shape, dt):
+    a = RNG.standard_normal(shape)
+    sym = (a + np.swapaxes(a, -1, -2)).astype(dt) + np.triu(RNG.standard_normal(shape), 1).astype(dt)
+    tol = 1e-14 if dt == np.float64 else 1e-3
+    got, want, ks = both(R.jacobi_eigh(sym, 30 if dt == np.float64 else 6, tol), [sym])
+    eb = np.dtype(dt).itemsize
+    assert got[0].dtype == dt and ks.info["in_lds"] == (2 * shape[-1] ** 2 * eb <= 150 * 1024)
+    assert_bits(got, want, f"jacobi_eigh {shape} {np.dtype(dt).name} {ks.info}")
+
+
+@pytest.mark.parametrize("dt", ELEMS, ids=lambda d: np.dtype(d).name)
+@pytest.mark.parametrize("n", [1, 4, 12, 49, 97, 210, 1024, 4096])
+def test_fft_other_element_types(n, dt):
+    """float64 results carry the device sine/cosine's last-place differences from the host's unrounded: compared within
+    1e-13 of the row's magnitude per stage; float16 within one unit of its last place of that magnitude."""
+    from jaxjs_hip.routine import Routine
+    rows = (2, 3) if n < 1000 else (70,)
+    re, im = RNG.standard_normal(rows + (n,)).astype(dt), RNG.standard_normal(rows + (n,)).astype(dt)
+    for inverse in (False, True):
+        base = R.fft(re, im, inverse)
+        got, want, ks = both(base, [re, im])
+        scale = float(max(np.abs(want[0].astype(np.float64)).max(), np.abs(want[1].astype(np.float64)).max()))
+        atol = (1e-13 * max(1, len(base.params["factors"])) if dt == np.float64 else 1e-3) * scale
+        for g, w in zip(got, want):
+            assert g.dtype == dt
+            np.testing.assert_allclose(g.astype(np.float64), w.astype(np.float64), rtol=0, atol=atol, err_msg=str(ks.info))
+        if n <= (4096 if dt == np.float64 else 8192) and n > 1:  # single launch and one launch per stage: the same bits
+            one = Routine(base.name, base.type, dict(base.params, singleLaunch=True))
+            many = Routine(base.name, base.type, dict(base.params, singleLaunch=False))
+            a, ka = R.run_gpu(one, [re, im])
+            b, kb = R.run_gpu(many, [re, im])
+            assert ka.info["launches"] == 1 and kb.info["launches"] == 1 + len(base.params["factors"])
+            assert_bits(a, b, f"fft paths n={n} {np.dtype(dt).name} inverse={inverse}")
+
+
 def _sc(updates, indices, op, shape, axis, out_dim, unique=False, dtype=None):
     return R.scatter(updates, indices, op, shape, axis, out_dim, unique, dtype), [updates] + list(indices)
 
@@ -228,10 +315,11 @@ SCATTER_CASES = [
 
 @pytest.mark.parametrize("case", SCATTER_CASES, ids=lambda c: "x".join(map(str, c[0])))
 @pytest.mark.parametrize("op", ["add", "update"])
-@pytest.mark.parametrize("dtype", [DType.Float32, DType.Int32, DType.Uint32, DType.Float16, DType.Bool], ids=lambda d: d.value)
+@pytest.mark.parametrize("dtype", [DType.Float32, DType.Int32, DType.Uint32, DType.Float16, DType.Bool, DType.Float64], ids=lambda d: d.value)
 def test_scatter_random(case, op, dtype):
     ushape, ishapes, oshape, axis, out_dim = case
-    npdt = {DType.Float32: F32, DType.Int32: np.int32, DType.Uint32: np.uint32, DType.Float16: np.float16, DType.Bool: np.int32}[dtype]
+    npdt = {DType.Float32: F32, DType.Int32: np.int32, DType.Uint32: np.uint32, DType.Float16: np.float16, DType.Bool: np.int32,
+            DType.Float64: np.float64}[dtype]
     if dtype == DType.Bool:
         upd = RNG.integers(0, 2, ushape).astype(npdt)
     elif dtype in (DType.Int32, DType.Uint32):
@@ -257,7 +345,7 @@ def test_scatter_float_accumulation_within_bound_and_unique_promise():
         assert ks.info["mode"] == 0
         assert_bits(got, want)
     with pytest.raises(UnsupportedRoutineError):
-        R.run_gpu(*_sc(np.zeros(3), [np.zeros(3, np.int32)], "add", [4], [0], 0))  # float64 updates
+        R.run_gpu(*_sc(np.zeros(3, F32), [np.zeros(3, F32)], "add", [4], [0], 0))  # index arrays must be integers
 
 
 def test_outputs_are_fully_initialised_without_updates():

@@ -209,6 +209,107 @@ def test_fft_reference_tables_and_any_factor_order():
         np.testing.assert_allclose(re + 1j * im, want, atol=2e-5)
 
 
+# ---- float64 and float16 elements (the reference's typed arrays: a Float64Array keeps every double, a Float16Array rounds it once)
+
+def test_dense_routines_in_float64_against_the_identities_and_libraries_at_double_precision():
+    x = spd((2,), 40).astype(np.float64)
+    (L,) = R.run_oracle(R.cholesky(x), [x])
+    assert L.dtype == np.float64 and np.all(np.triu(L, 1) == 0)
+    np.testing.assert_allclose(L, np.linalg.cholesky(x), rtol=1e-13, atol=1e-14)
+    a = np.triu(RNG.standard_normal((2, 30, 30))) + 6 * np.eye(30)
+    b = RNG.standard_normal((2, 7, 30))
+    for unit in (False, True):
+        (sol,) = R.run_oracle(R.triangular_solve(a, b, unit), [a, b])
+        for k in range(2):
+            want = scipy.linalg.solve_triangular(a[k], b[k].T, lower=False, unit_diagonal=unit).T
+            np.testing.assert_allclose(sol[k], want, rtol=1e-9, atol=1e-9 * np.abs(want).max())
+    m = RNG.uniform(0, 1, (2, 25, 25))
+    lu, piv, perm = R.run_oracle(R.lu(m), [m])
+    for k in range(2):
+        ref_lu, ref_piv = scipy.linalg.lu_factor(m[k])
+        assert piv[k].tolist() == ref_piv.tolist()
+        np.testing.assert_allclose(lu[k], ref_lu, rtol=1e-10, atol=1e-12)
+        np.testing.assert_allclose((np.tril(lu[k], -1) + np.eye(25)) @ np.triu(lu[k]), m[k][perm[k]], rtol=1e-13, atol=1e-14)
+    g = RNG.standard_normal((2, 20, 20))
+    sym = g + np.swapaxes(g, -1, -2)
+    d, v = R.run_oracle(R.jacobi_eigh(sym, 30, 1e-14), [sym])
+    for k in range(2):
+        w = np.diagonal(d[k])
+        np.testing.assert_allclose(np.sort(w), np.linalg.eigvalsh(sym[k]), rtol=1e-12, atol=1e-12)
+        np.testing.assert_allclose(v[k].T @ v[k], np.eye(20), atol=1e-13)
+        np.testing.assert_allclose((v[k] * w) @ v[k].T, sym[k], atol=1e-12)
+    for n in (12, 49, 64, 97):
+        re, im = RNG.standard_normal((2, n)), RNG.standard_normal((2, n))
+        o_re, o_im = R.run_oracle(R.fft(re, im), [re, im])
+        np.testing.assert_allclose(o_re + 1j * o_im, np.fft.fft(re + 1j * im), atol=1e-12 * n)
+        i_re, i_im = R.run_oracle(R.fft(re, im, True), [re, im])
+        np.testing.assert_allclose(i_re + 1j * i_im, np.fft.ifft(re + 1j * im), atol=1e-13)
+
+
+def _once(x):
+    """A float64 array rounded once to float16 (numpy's conversion from double is a single rounding)."""
+    return np.asarray(x, np.float64).astype(np.float16)
+
+
+def test_dense_routines_in_float16_round_each_store_once_from_the_double():
+    """Small cases worked by hand in Python floats (= the reference's JavaScript numbers) with every store rounded to
+    float16: a wrong rounding point (through float32, or keeping a double between stores) changes these bits."""
+    H = np.float16
+    x = np.array([[4, 2, 1], [2, 5, 3], [1, 3, 6]], H)
+    (L,) = R.run_oracle(R.cholesky(x), [x])
+    want = np.zeros((3, 3), H)
+    for i in range(3):
+        for j in range(i + 1):
+            s = float(x[i, j])
+            for k in range(j):
+                s -= float(want[i, k]) * float(want[j, k])
+            want[i, j] = _once(np.sqrt(s)) if i == j else _once(s / float(want[j, j]))
+    assert L.dtype == H and R.bits_equal(L, want)
+    a, b = np.array([[2, 1, 0.3], [0, 3, 0.7], [0, 0, 1.1]], H), np.array([[5, 3, 0.1], [1, 2, 3]], H)
+    (sol,) = R.run_oracle(R.triangular_solve(a, b), [a, b])
+    want = np.zeros((2, 3), H)
+    for t in range(2):
+        for i in (2, 1, 0):
+            s = float(b[t, i])
+            for j in range(i + 1, 3):
+                s -= float(a[i, j]) * float(want[t, j])
+            want[t, i] = _once(s / float(a[i, i]))
+    assert R.bits_equal(sol, want)
+    m = np.array([[0.3, 3, 1.7], [6, 3, 0.9], [1.1, -2, 5]], H)
+    lu, piv, perm = R.run_oracle(R.lu(m), [m])
+    w, pr, pv = m.copy(), [0, 1, 2], []
+    for j in range(3):
+        r = j + int(np.argmax(np.abs(w[j:, j].astype(np.float64))))
+        pv.append(r)
+        if r != j:
+            w[[j, r]] = w[[r, j]]
+            pr[j], pr[r] = pr[r], pr[j]
+        for i in range(j + 1, 3):
+            f = float(w[i, j]) / float(w[j, j])
+            w[i, j] = _once(f)
+            for c in range(j + 1, 3):
+                w[i, c] = _once(float(w[i, c]) - f * float(w[j, c]))  # the unrounded factor, as the reference keeps it
+    assert R.bits_equal(lu, w) and piv.tolist() == pv and perm.tolist() == pr
+    # One Jacobi sweep limit and the DFT of four points: identities within float16 resolution.
+    g = RNG.standard_normal((8, 8))
+    sym = (g + g.T).astype(H)
+    d, v = R.run_oracle(R.jacobi_eigh(sym, 30, 1e-3), [sym])
+    wv = np.diagonal(d).astype(np.float64)
+    np.testing.assert_allclose(np.sort(wv), np.linalg.eigvalsh(np.tril(sym.astype(np.float64)) + np.tril(sym.astype(np.float64), -1).T), atol=3e-2)
+    np.testing.assert_allclose(v.astype(np.float64).T @ v.astype(np.float64), np.eye(8), atol=2e-2)
+    re, im = np.array([0, 1, 2, 3], H), np.zeros(4, H)
+    o_re, o_im = R.run_oracle(R.fft(re, im), [re, im])
+    assert o_re.dtype == H and o_re.tolist() == [6, -2, -2, -2]
+    np.testing.assert_allclose(o_im.astype(np.float64), [0, 2, 0, -2], atol=1e-3)
+    # the float16 store itself: halfway cases straight from the double (1 + 2^-11 + 2^-30 rounds up; through float32 it would tie to even)
+    tie = np.array([[1.0 + 2.0 ** -11 + 2.0 ** -30]])
+    assert _once(tie)[0, 0] == np.float16(1.0 + 2.0 ** -10)
+    x = np.array([[4.0]], H)
+    bvec = np.array([[4.0 * (1.0 + 2.0 ** -11) + 2.0 ** -20]], np.float64)
+    (sol,) = R.run_oracle(R.triangular_solve(x, bvec.astype(H)), [x, bvec.astype(H)])
+    assert sol[0, 0] == _once(float(bvec.astype(H)[0, 0]) / 4.0)[()]
+
+
 def test_attention_checker_against_reference_tables_and_composition():
     """The fused-attention checker (not a reference routine): the reference's dotProductAttention tables
     (test/nn.test.ts:274-390) and, on random float16 operands, the unfused composition replayed kernel by kernel."""
