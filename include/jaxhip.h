@@ -73,7 +73,9 @@ int jh_memcpy_h2d(jh_devptr dst, const void *src, size_t bytes);
 
 /*
  * Device -> host read of `bytes` starting `offset` bytes into `src`.  Backs `Backend.readSync`
- * (src/backend.ts:189): returns after every previously issued kernel has finished.
+ * (src/backend.ts:189): returns after every previously issued kernel has finished.  Reads of
+ * 1 MiB and more are pipelined through two pinned 8 MiB buffers that the library allocates at the
+ * first such read and keeps until `jh_shutdown`.
  */
 int jh_memcpy_d2h(void *dst, jh_devptr src, size_t offset, size_t bytes);
 

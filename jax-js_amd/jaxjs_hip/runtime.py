@@ -9,6 +9,8 @@ from __future__ import annotations
 import ctypes
 import hashlib
 import os
+
+import numpy as np
 from typing import List, Optional, Sequence, Tuple
 
 from .errors import HipRuntimeError
@@ -207,8 +209,8 @@ class Device:
         mv = memoryview(data).cast("B")
         if len(mv) == 0:
             return
-        buf = (ctypes.c_char * len(mv)).from_buffer_copy(mv) if mv.readonly else (ctypes.c_char * len(mv)).from_buffer(mv)
-        check(self.lib.jh_memcpy_h2d(ctypes.c_void_p(dst), ctypes.cast(buf, ctypes.c_void_p), len(mv)), "jh_memcpy_h2d")
+        src = np.frombuffer(mv, dtype=np.uint8)  # the buffer's own address, read-only or not: no host-side copy
+        check(self.lib.jh_memcpy_h2d(ctypes.c_void_p(dst), ctypes.c_void_p(src.ctypes.data), len(mv)), "jh_memcpy_h2d")
 
     def d2h(self, src: int, offset: int, nbytes: int) -> bytearray:
         out = bytearray(nbytes)

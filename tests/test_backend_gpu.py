@@ -274,6 +274,33 @@ def test_dispatch_order_and_buffer_reuse(be):
     be.decRef(cur)
 
 
+def test_large_uploads_and_reads_through_the_pinned_staging_buffers(be):
+    """Reads of 1 MiB and more are pipelined through two pinned 8 MiB buffers; uploads take the source's own memory
+    (no host-side copy, read-only or not): sizes around the threshold and the chunk size, odd tails, partial reads at an
+    offset, the source overwritten right after the call returns, and a kernel queued between upload and read."""
+    rng = np.random.default_rng(5)
+    M = 1 << 20
+    sizes = [M - 4, M, M + 4, 8 * M - 4, 8 * M, 8 * M + 4, 16 * M, 20 * M + 12, 40 * M + 4]
+    slots, keep = [], []
+    for n in sizes:
+        data = bytearray(rng.integers(0, 256, n, dtype=np.uint8).tobytes())
+        keep.append(bytes(data))
+        slots.append(be.malloc(n, data))
+        data[:] = b"\x00" * n  # the call has returned: the library no longer reads the source
+    for n, slot, want in zip(sizes, slots, keep):
+        assert bytes(be.readSync(slot)) == want
+        for start, count in ((4, n - 8), (n // 2 + 4, min(9 * M + 4, n - n // 2 - 4)), (n - 4, 4), (8, 0)):
+            assert bytes(be.readSync(slot, start, count)) == want[start:start + count]
+    n = sizes[-1] // 4
+    st = ShapeTracker.fromShape([n])
+    inc = be.prepareKernelSync(Kernel(1, n, AluExp.add(AluExp.globalView(DType.Int32, 0, st, [AluVar.gidx]), AluExp.i32(1))))
+    out = be.malloc(n * 4)
+    be.dispatch(inc, [slots[-1]], [out])  # queued behind the upload's last chunk
+    np.testing.assert_array_equal(np.frombuffer(be.readSync(out), np.int32), np.frombuffer(keep[-1], np.int32) + 1)
+    for s_ in slots + [out]:
+        be.decRef(s_)
+
+
 def test_read_is_asynchronous(be):
     """`read` (src/backend.ts:182-186) queues its copy behind the pending dispatches and yields to the event loop until it
     has landed: another coroutine runs, and dispatches more work, while the read is still pending; the bytes are those
