@@ -5,7 +5,7 @@ of bench.py -- never by the package.  `run_kernel` serialises the expression *as
 built it* (`Kernel.exp_raw`, `Reduction.epilogue_raw`, GlobalView nodes untouched), so neither
 the host-side simplifier nor the view lowering the product uses is on the checking path.  One fold
 is applied while serialising, because the reference applies it before any of its backends runs: a
-float constant under a cast to another float type becomes that constant in the target type.
+subexpression of constants becomes one constant, evaluated in JavaScript doubles and left unrounded.
 """
 from __future__ import annotations
 
@@ -67,10 +67,25 @@ def lib() -> ctypes.CDLL:
     return _lib
 
 
+_LEAVES = (AluOp.Const, AluOp.Special, AluOp.Variable, AluOp.GlobalIndex, AluOp.GlobalView)
+_FLOATS = (DType.Float32, DType.Float16, DType.Float64)
+
+
+def _fold_constant(e: AluExp) -> Optional[AluExp]:
+    """`e` with all-constant operands as one constant holding the unrounded JavaScript number (None: leave `e`)."""
+    if e.op in _LEAVES or not e.src or any(x.op != AluOp.Const for x in e.src):
+        return None
+    probe = AluExp.cast(DType.Float64, e) if e.dtype in _FLOATS else e
+    (value,) = run_kernel(Kernel(0, 1, probe), [], MODE_CPU, fold_constants=False)
+    if e.dtype in _FLOATS:
+        return AluExp.const(e.dtype, float(value))
+    return AluExp.const(e.dtype, bool(value) if e.dtype == DType.Bool else int(value))
+
+
 class _Program:
     """Topologically ordered flat encoding of an expression DAG."""
 
-    def __init__(self, exp: Optional[AluExp], views: List[int]):
+    def __init__(self, exp: Optional[AluExp], views: List[int], fold_constants: bool = True):
         self.op: List[int] = []
         self.dt: List[int] = []
         self.soff: List[int] = [0]
@@ -126,12 +141,14 @@ class _Program:
             self.fa.append(f)
             return i
 
-        # A float constant under a cast to another float type is that constant in the target type, not first rounded to
-        # its own: the reference folds constants in JS doubles before any backend sees them (src/alu.ts:671-675, with
-        # `evaluate` returning a Const's number as it is, :1128-1137), so `x_f64 + 3.141592653589793` adds the double.
-        _fl = (DType.Float32, DType.Float16, DType.Float64)
-        exp = exp.rewrite(lambda e: AluExp.const(e.dtype, e.src[0].arg) if e.op == AluOp.Cast and e.dtype in _fl
-                          and e.src[0].op == AluOp.Const and e.src[0].dtype in _fl else None)
+        # The reference folds constant subexpressions before any backend sees the kernel: a node whose operands are all
+        # constants becomes `const(dtype, evaluate())` (src/alu.ts:670-675), evaluated in JavaScript doubles with the
+        # CPU backend's arithmetic and *not* rounded to the node's type (`evaluate` hands a Const's number on as it is,
+        # :1128-1137) -- so `x_f64 + 3.141592653589793` adds the double although the literal was typed float32, and
+        # `cos(1.0) * x` multiplies by the rounded double cosine, not by the Wasm polynomial's value.  The same fold,
+        # bottom-up, with the checker's own CPU-mode evaluator:
+        if fold_constants:
+            exp = exp.rewrite(_fold_constant)
         exp.fold(emit)
         # `fold` visits the root last, so the result is the last node.
         assert index[id(exp)] == len(self.op) - 1
@@ -152,7 +169,7 @@ def _ptr(a: np.ndarray):
 
 
 def run_kernel(kernel: Kernel, inputs: Sequence, mode: int = MODE_WASM, gidx: Optional[Sequence[int]] = None,
-               return_oob: bool = False):
+               return_oob: bool = False, fold_constants: bool = True):
     """Evaluate `kernel` over host arrays.  Returns the typed output (length `kernel.size`, or
     `len(gidx)` when only selected output positions are requested)."""
     L = lib()
@@ -164,7 +181,7 @@ def run_kernel(kernel: Kernel, inputs: Sequence, mode: int = MODE_WASM, gidx: Op
             exp = AluExp.cast(re.dtype, exp)
         epi = re.epilogue_raw
     views: List[int] = [0]
-    pe, pp = _Program(exp, views), _Program(epi, views)
+    pe, pp = _Program(exp, views, fold_constants), _Program(epi, views, fold_constants)
     ea, pa = pe.arrays(), pp.arrays()
     va = np.asarray(views, dtype=np.int64)
 

@@ -13,6 +13,8 @@ from jaxjs_hip.lowering import mapKernel, reduceKernel
 
 pytestmark = pytest.mark.gpu
 F32, I32, U32, BOOL = DType.Float32, DType.Int32, DType.Uint32, DType.Bool
+# JAXHIP_FUZZ_OFFSET=<n> shifts every seed below by n: the same tests over expressions, shapes and views not seen before.
+OFFSET = int(__import__("os").environ.get("JAXHIP_FUZZ_OFFSET", "0"))
 
 
 def rand_exp(rng, leaves, dtype, depth):
@@ -104,7 +106,7 @@ def leaves_for(views):
 
 @pytest.mark.parametrize("seed", range(150))
 def test_random_map_kernels(seed):
-    rng = random.Random(1000 + seed)
+    rng = random.Random(1000 + seed + OFFSET)
     n = rng.choice([1, 5, 64, 1000, 4099, 65536 + 3])
     inputs = make_inputs(rng, n)
     out_dt = rng.choice([F32, F32, I32, U32, BOOL])
@@ -121,7 +123,7 @@ def test_random_map_kernels(seed):
 
 @pytest.mark.parametrize("seed", range(100))
 def test_random_reductions(seed):
-    rng = random.Random(5000 + seed)
+    rng = random.Random(5000 + seed + OFFSET)
     rows, L = rng.choice([(1, 1000), (7, 129), (64, 64), (300, 33), (5, 4097), (1000, 8)])
     inputs = make_inputs(rng, rows * L)
     out_dt = rng.choice([F32, I32, U32, BOOL])
@@ -136,7 +138,20 @@ def test_random_reductions(seed):
     arrays = [a for _, a in inputs]
     if out_dt == F32:
         if op == AluOp.Add:
-            assert_parity(k, arrays, rtol=2e-5 * max(1.0, math.sqrt(L)), atol=1e-4 * L)
+            # plus a few float32 rounding units of sum |term| (far inside the K-scaled bound L * 2^-24 * sum |term|): the
+            # integer inputs hold +-2^31, which cancel in some rows and leave an error of that order whatever the order
+            from jaxjs_hip.alu import Kernel, Reduction
+            from oracle import oracle
+            e = k.exp_raw
+            mag = Kernel(k.nargs, k.size, AluExp.where(AluExp.cmplt(e, AluExp.f32(0.0)), AluExp.sub(AluExp.f32(0.0), e), e), Reduction(F32, AluOp.Add, L))
+            total = np.nan_to_num(oracle.run_kernel(mag, arrays, oracle.MODE_CPU).astype(np.float64), nan=0.0, posinf=0.0)
+            from gpu_util import device_run
+            got, ks = device_run(k, arrays)
+            want = oracle.run_kernel(k, arrays, oracle.MODE_WASM)
+            assert got.dtype == want.dtype and got.shape == want.shape and np.array_equal(np.isnan(got), np.isnan(want))
+            bound = 1e-4 * L + 8.0 * 2.0 ** -24 * total + 2e-5 * max(1.0, math.sqrt(L)) * np.abs(want.astype(np.float64))
+            ok = np.isnan(want) | (got == want) | (np.abs(got.astype(np.float64) - want.astype(np.float64)) <= bound)
+            assert ok.all(), f"class {ks.klass} {ks.info}: {np.flatnonzero(~ok)[:5]} {got[~ok][:5]} vs {want[~ok][:5]}"
         else:
             assert_parity(k, arrays, rtol=1e-5, atol=1e-6)
     else:
@@ -187,7 +202,7 @@ def _random_view(rng):
 def test_random_view_chains_in_maps_and_reductions(seed):
     """Movement ops are pure index arithmetic (multi-view trackers, masks, negative strides): the GPU result must
     equal numpy's on the same chain, bit for bit, as an elementwise kernel and under a row reduction."""
-    rng = random.Random(9000 + seed)
+    rng = random.Random(9000 + seed + OFFSET)
     st, base, ref = _random_view(rng)
     shape = list(st.shape)
     k = mapKernel(shape, [(I32, st)], lambda v: AluExp.add(AluExp.mul(v, AluExp.i32(3)), AluExp.i32(1)))
@@ -207,13 +222,13 @@ def test_random_contractions(seed):
     axis shared or broadcast, optional fused bias/cast epilogue) with small integer data: every class the tuner may
     pick (direct-LDS / general / f32 GEMM, swapped roles, or a plain reduction for thin shapes) must be exact."""
     from jaxjs_hip.lowering import reduceKernel as rk
-    rng = random.Random(7000 + seed)
+    rng = random.Random(7000 + seed + OFFSET)
     dim = lambda: rng.choice([1, 8, 31] if rng.random() < 0.15 else [64, 100, 128, 160, 256, 300, 512])  # noqa: E731
     M, N = dim(), dim()
     K = rng.choice([8, 32, 40, 64, 96, 128, 136, 512])
     batch = rng.choice([[], [], [3], [2, 2]])
     dt, npdt = rng.choice([(DType.Float16, np.float16), (DType.Float32, np.float32)])
-    npr = np.random.default_rng(seed)
+    npr = np.random.default_rng(seed + OFFSET)
     full = batch + [M, N, K]
     nb = len(batch)
     a_t, b_t = rng.random() < 0.3, rng.random() < 0.5
@@ -294,8 +309,8 @@ def rand_f16_exp(rng, leaves, depth):
 def test_random_f16_kernels(seed):
     """Maps and reductions over float16 buffers (packs of 8 halves, f32 accumulation of f16 sums, native half
     arithmetic) against the checker, within the float16 tolerance (rel 1e-2)."""
-    rng = random.Random(9000 + seed)
-    npr = np.random.default_rng(seed)
+    rng = random.Random(9000 + seed + OFFSET)
+    npr = np.random.default_rng(seed + OFFSET)
     reduce_ = seed % 3 == 2
     if reduce_:
         rows, L = rng.choice([(1, 1000), (7, 129), (64, 64), (300, 33), (5, 2049)])

@@ -349,3 +349,29 @@ def test_wasm_port_matmul_matvec_against_f64():
                                 y.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(M), ctypes.c_int64(K)) == 0
     ref = W.astype(np.float64) @ x.astype(np.float64)
     assert np.all(np.abs(y - ref) <= 2 * K * np.finfo(np.float32).eps * (np.abs(W).astype(np.float64) @ np.abs(x)))
+
+
+def test_constant_subexpressions_are_folded_in_doubles_before_either_mode_runs():
+    """src/alu.ts:670-675: a node whose operands are all constants becomes one constant, evaluated in JavaScript doubles
+    and not rounded to its type -- so the Wasm mode multiplies by Math.cos(1) rounded once to float32 (not by its own
+    cosine polynomial's value), a float64 consumer sees the whole double, and integer folds stay exact.  An expression
+    that reads a buffer or an index is left to the mode's own arithmetic."""
+    st = ShapeTracker.fromShape([3])
+    x = AluExp.globalView(DType.Float32, 0, st, [AluVar.gidx])
+    one = np.ones(3, np.float32)
+    cos1 = AluExp.cos(AluExp.f32(1.0))
+    for mode in (oracle.MODE_WASM, oracle.MODE_CPU):
+        got = oracle.run_kernel(Kernel(1, 3, AluExp.cast(DType.Float64, AluExp.mul(cos1, x))), [one], mode)
+        assert got.dtype == np.float64
+        assert got[0] == (float(np.float32(math.cos(1.0))) if mode == oracle.MODE_WASM else math.cos(1.0))
+        wide = oracle.run_kernel(Kernel(1, 3, AluExp.add(AluExp.cast(DType.Float64, x), AluExp.cast(DType.Float64, cos1))), [one], mode)
+        assert wide[0] == 1.0 + math.cos(1.0)  # the double, although the cosine node is typed float32
+    k = Kernel(1, 3, AluExp.cast(DType.Float64, AluExp.mul(AluExp.mul(AluExp.f32(2.0), AluExp.erf(AluExp.f32(0.5))), x)))
+    folded = 2.0 * oracle.lib().jo_js_erf(0.5)
+    assert oracle.run_kernel(k, [one], oracle.MODE_WASM)[0] == float(np.float32(folded))
+    i = AluExp.add(AluExp.mul(AluExp.i32(65537), AluExp.i32(65537)), AluExp.cast(DType.Int32, AluExp.f32(3e9)))
+    got = oracle.run_kernel(Kernel(0, 2, AluExp.add(i, AluExp.cast(DType.Int32, AluVar.gidx))), [], oracle.MODE_WASM)
+    assert got.tolist() == [(131073 + 2147483647 + 2 ** 32) % 2 ** 32 - 2 ** 32, (131073 + 2147483647 + 1 + 2 ** 32) % 2 ** 32 - 2 ** 32]
+    # not folded: the Wasm cosine of a loaded 1.0 is the polynomial's value
+    poly = oracle.run_kernel(Kernel(1, 3, AluExp.cos(x)), [one], oracle.MODE_WASM)[0]
+    assert poly == np.float32(oracle.wasm_builtin("cos", 1.0))
