@@ -278,6 +278,84 @@ class Tracer:
     def astype(self, dtype: DType):
         return self if self.dtype == dtype else bind1("Cast", [self], dict(dtype=dtype))
 
+    def view(self, dtype: Optional[DType] = None):
+        """Reinterpret the bits as another type of the same width (core.ts:937-940)."""
+        return self if dtype is None or dtype == self.dtype else bitcast(self, dtype)
+
+    def greater(self, o): return greater(self, o)
+    def greaterEqual(self, o): return greaterEqual(self, o)
+    def less(self, o): return less(self, o)
+    def lessEqual(self, o): return lessEqual(self, o)
+    def equal(self, o): return equal(self, o)
+    def notEqual(self, o): return notEqual(self, o)
+
+    def flatten(self):
+        return reshape(self, [-1])
+
+    def ravel(self):
+        return reshape(self, [-1])
+
+    def slice(self, *index):
+        """Indexing as the reference's `Tracer.slice` spells it (core.ts:1110-1231): an int picks one entry of an axis and
+        drops the axis (negative counts from the end), `[]` keeps the axis, `[i]` is `i:`, `[i, j]` is `i:j`, `None` adds
+        an axis, an integer array gathers along its axis.  Several arrays broadcast together; their dimensions stay in
+        place when the arrays and ints sit next to each other in the index and move to the front otherwise (numpy's
+        rule).  Strided slices are not part of it."""
+        def bound(n: int, i: int) -> int:
+            if i > n or i < -n:
+                raise IndexError(f"Index {i} out of bounds for axis of size {n}")
+            return n + i if i < 0 else i
+
+        is_array = lambda v: isinstance(v, (Tracer, ConstArray))  # noqa: E731
+        arrays = [v for v in index if is_array(v)]
+        gather_axes: List[int] = []
+        out_dim = -1
+        if arrays:
+            advanced, at = [], 0
+            for pos, v in enumerate(index):
+                if is_array(v):
+                    advanced.append(pos)
+                    gather_axes.append(at)
+                    at += 1
+                elif isinstance(v, int) and not isinstance(v, bool):
+                    advanced.append(pos)  # squeezed out: takes no axis of the sliced array
+                else:
+                    at += 1
+            out_dim = gather_axes[0] if advanced[-1] - advanced[0] == len(advanced) - 1 else 0
+        window, shape, reshaped, axis = [], [], False, 0
+        for v in index:
+            if v is None:
+                shape.append(1)
+                reshaped = True
+                continue
+            if axis >= self.ndim:
+                raise IndexError("Too many indices")
+            n = self.shape[axis]
+            axis += 1
+            if is_array(v):
+                shape.append(n)
+                window.append((0, n))
+            elif isinstance(v, int) and not isinstance(v, bool):
+                i = bound(n, v)
+                window.append((i, i + 1))
+                reshaped = True
+            elif isinstance(v, (list, tuple)) and len(v) <= 2:
+                lo = bound(n, v[0]) if len(v) >= 1 else 0
+                hi = bound(n, v[1]) if len(v) == 2 else n
+                if lo > hi:
+                    raise IndexError(f"Slice start at {lo} > end at {hi}")
+                shape.append(hi - lo)
+                window.append((lo, hi))
+            else:
+                raise TypeError(f"Invalid slice argument: {v!r}")
+        for n in self.shape[axis:]:
+            window.append((0, n))
+            shape.append(n)
+        out = shrink(self, window)
+        if reshaped:
+            out = reshape(out, shape)
+        return gather(out, arrays, gather_axes, out_dim) if arrays else out
+
     def reshape(self, shape):
         return reshape(self, shape)
 
@@ -337,7 +415,14 @@ def _out_aval(prim: str, avals: List[ShapedArray], params: Dict[str, Any]) -> Sh
     if prim == "Where":
         xy = promoteAvals(avals[1], avals[2])
         return ShapedArray(generalBroadcast(avals[0].shape, xy.shape), xy.dtype, xy.weak)
-    if prim in ("Cast", "Bitcast"):
+    if prim == "Bitcast":  # src/frontend/jaxpr.ts:838-848
+        src_dt, dtype = avals[0].dtype, params["dtype"]
+        if src_dt != dtype and DType.Bool in (src_dt, dtype):
+            raise TypeError("Bitcast to/from bool is not allowed")
+        if byteWidth(src_dt) != byteWidth(dtype):
+            raise TypeError(f"Bitcast from {src_dt.value} to {dtype.value} with different byte width")
+        return ShapedArray(avals[0].shape, dtype, False)
+    if prim == "Cast":
         return ShapedArray(avals[0].shape, params["dtype"], False)
     if prim in UNARY_FUSABLE:
         return avals[0]

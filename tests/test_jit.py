@@ -1980,3 +1980,103 @@ def test_jit_cases_of_the_tracing_suite():
     g2 = lambda a: f(f(a))
     _, (q,) = run(g2, f32(3).reshape(()))
     assert q.tolist() == [81]
+
+
+def test_array_suite_tables():
+    """src/frontend/array.test.ts: construction and elementwise product with a transposed read (:177-187), broadcasting
+    [2,1,2]*[2,3,1] (:189-216), flatten/ravel (:218-229), an array added to itself twice (:231-236), booleans and the six
+    comparisons (:248-281, incl. arange(5000)+1 < 2500), comparisons against NaN (:283-292), slicing with ints, negative
+    ints, ranges and new axes (:294-321), sums along negative axes (:323-330), means over several axes (:332-342), integer
+    array indexing as gather (:344-363), uint32 wrap-around (:390-400), casts (:402-413), saturating casts (:415-432),
+    bit views and their type rules (:434-482)."""
+    a, b = f32([1, 2, 3, 4]), f32([10, 5, 2, -8.5])
+    _, (c, ct) = run(lambda p, q: [p.mul(q), p.mul(q).reshape([2, 2]).transpose()], a, b)
+    assert c.tolist() == [10, 10, 6, -34] and ct.tolist() == [10, 6, 10, -34]
+    p, q = f32([[1, 22], [3, 9]]), f32([[10, 5, -2], [-8, 0, 3]])
+    seen = {}
+    _, (o,) = run(lambda u, v: seen.setdefault("o", u.reshape([2, 1, 2]).mul(v.reshape([2, 3, 1]))), p, q)
+    assert tuple(seen["o"].shape) == (2, 3, 2)
+    assert o.reshape(2, 3, 2).tolist() == [[[10, 220], [5, 110], [-2, -44]], [[-24, -72], [0, 0], [9, 27]]]
+    _, (fl, rv, sc) = run(lambda u, s: [u.flatten().mul(1), u.ravel().mul(1), s.flatten().mul(1)], f32([[[1, 2], [3, 4]]]), f32(3))
+    assert fl.tolist() == [1, 2, 3, 4] and rv.tolist() == [1, 2, 3, 4] and sc.tolist() == [3]
+    _, (tw,) = run(lambda u: u.add(u).add(u), f32([1, 2, 3]))
+    assert tw.tolist() == [3, 6, 9]
+    # booleans are int32 0/1 in memory; comparisons
+    x = f32([1, 3, 4])
+    _, (g2, e3, ne) = run(lambda u, v: [u.greater(2), u.equal(3), u.notEqual(v)], x, f32([2, 3, 4]))
+    assert g2.dtype == np.int32 and g2.tolist() == [0, 1, 1] and e3.tolist() == [0, 1, 0] and ne.tolist() == [1, 0, 0]
+    _, outs = run(lambda u: [u.greater(2), u.greaterEqual(2), u.less(2), u.lessEqual(2), u.equal(2), u.notEqual(2)], f32([1, 2, 3]))
+    assert [o_.tolist() for o_ in outs] == [[0, 0, 1], [0, 1, 1], [1, 0, 0], [1, 1, 0], [0, 1, 0], [1, 0, 1]]
+    (lt,) = run0(lambda: J._raise(L.arange(0, 5000, 1, F32)).add(1).less(2500))
+    assert lt.tolist() == [1 if i + 1 < 2500 else 0 for i in range(5000)]
+    nan = float("nan")
+    _, outs = run(lambda u: [u.greater(nan), u.less(nan), u.equal(nan), u.notEqual(nan), u.greaterEqual(nan), u.lessEqual(nan)], f32([nan, 0]))
+    assert [o_.tolist() for o_ in outs] == [[0, 0], [0, 0], [0, 0], [1, 1], [0, 0], [0, 0]]
+    # slicing
+    m = f32([[1, 2, 3], [4, 5, 6]])
+    shapes = []
+
+    def pick(u):
+        outs_ = [u.slice(0, 0), u.slice(0, 2), u.slice(1, 2), u.slice(1), u.slice(), u.slice(-1, -1), u.slice(-2, -1), u.slice(-1, -3),
+                 u.slice(0, 0, None), u.slice(0, None, 0), u.slice(None), u.slice([], [1]), u.slice([0, 1], [1, 3]), u.slice(None, 1, None, [0, 2])]
+        shapes.extend(tuple(o_.shape) for o_ in outs_)
+        return [o_.mul(1) for o_ in outs_]
+
+    _, outs = run(pick, m)
+    assert shapes == [(), (), (), (3,), (2, 3), (), (), (), (1,), (1,), (1, 2, 3), (2, 2), (1, 2), (1, 1, 2)]
+    assert [o_.tolist() for o_ in outs] == [[1], [3], [6], [4, 5, 6], [1, 2, 3, 4, 5, 6], [6], [3], [4], [1], [1], [1, 2, 3, 4, 5, 6],
+                                           [2, 3, 5, 6], [2, 3], [4, 5]]
+    for bad in ((3,), (0, 4), (-3,), (0, 0, 0), ([2, 1],), ("x",)):
+        with pytest.raises((IndexError, TypeError)):
+            J.jit(lambda u: u.slice(*bad), [ShapedArray((2, 3), F32)])
+    _, (s1, s2) = run(lambda u: [u.sum(-1), u.sum(-2)], m)
+    assert s1.tolist() == [6, 15] and s2.tolist() == [5, 7, 9]
+    _, (m0, m01, ma, mb) = run(lambda u: [u.mean(), u.mean([0, 1]), u.mean(0), u.mean(1)], m)
+    assert m0.tolist() == [3.5] and m01.tolist() == [3.5] and ma.tolist() == [2.5, 3.5, 4.5] and mb.tolist() == [2, 5]
+    # integer arrays as indices: np.eye(5)[[1,3,2]], np.eye(5)[[1,3,2], np.newaxis], np.eye(5)[1:4, [1,3,2]]
+    idx = np.array([1, 3, 2], np.int32)
+    shapes = []
+
+    def adv(i):
+        e = J._raise(L.eye(5))
+        outs_ = [e.slice(i), e.slice(i, None), e.slice([1, 4], i)]
+        shapes.extend(tuple(o_.shape) for o_ in outs_)
+        return outs_
+
+    _, (g0, g1, g2) = run_typed(adv, [idx], [I32])
+    assert shapes == [(3, 5), (3, 1, 5), (3, 3)]
+    assert g0.reshape(3, 5).tolist() == np.eye(5)[idx].tolist() and g1.reshape(3, 5).tolist() == np.eye(5)[idx].tolist()
+    assert g2.reshape(3, 3).tolist() == np.eye(5)[1:4, idx].tolist()
+    # numpy's placement rule when ints and arrays are apart: x[:, i, :, 1] puts the index dimensions first
+    t4 = np.arange(2 * 3 * 4 * 5, dtype=np.float32).reshape(2, 3, 4, 5)
+    shapes = []
+    _, (apart, together) = run_typed(lambda u, i: [shapes.append(tuple(u.slice([], i, [], 1).shape)) or u.slice([], i, [], 1),
+                                                    shapes.append(tuple(u.slice([], i, 2).shape)) or u.slice([], i, 2)], [t4, np.array([2, 0], np.int32)], [F32, I32])
+    assert shapes == [(2, 2, 4), (2, 2, 5)]
+    np.testing.assert_array_equal(apart.reshape(2, 2, 4), t4[:, [2, 0], :, 1])
+    np.testing.assert_array_equal(together.reshape(2, 2, 5), t4[:, [2, 0], 2])
+    # uint32 wraps, casts, saturation
+    _, (w,) = run_typed(lambda u, two: u.sub(two), [np.array([1, 2, 3], np.uint32), np.array(2, np.uint32)], [DType.Uint32, DType.Uint32])
+    assert w.dtype == np.uint32 and w.tolist() == [4294967295, 0, 1]
+    _, (cf,) = run_typed(lambda u: u.astype(F32), [np.array([1, 2, 3], np.int32)], [I32])
+    assert cf.dtype == np.float32 and cf.tolist() == [1, 2, 3]
+    big = f32([1e20, -1e20, 1e10, -1e10, 1e5, -1e5])
+    _, (si, su) = run(lambda u: [u.astype(I32), u.astype(DType.Uint32)], big)
+    assert si.tolist() == [2147483647, -2147483648, 2147483647, -2147483648, 100000, -100000]
+    assert su.tolist() == [4294967295, 0, 4294967295, 0, 100000, 0]
+    # bit views
+    _, (vi, back) = run(lambda u: [u.view(I32), u.view(I32).view(F32)], f32([1.0, 2.0]))
+    assert vi.dtype == np.int32 and vi.tolist() == [1065353216, 1073741824] and back.tolist() == [1.0, 2.0]
+    _, (vf,) = run_typed(lambda u: u.view(F32), [np.array([1065353216, 1073741824], np.int32)], [I32])
+    assert vf.dtype == np.float32 and vf.tolist() == [1.0, 2.0]
+    same = {}
+    _, (idn,) = run(lambda u: same.setdefault("v", u.view(F32)).mul(1), f32([1, 2, 3]))
+    assert idn.tolist() == [1, 2, 3]
+    with pytest.raises(TypeError):
+        J.jit(lambda u: u.view(I32), [ShapedArray((2,), DType.Bool)])
+    with pytest.raises(TypeError):
+        J.jit(lambda u: u.view(DType.Bool), [ShapedArray((2,), I32)])
+    with pytest.raises(TypeError):
+        J.jit(lambda u: u.view(DType.Float16), [ShapedArray((2,), I32)])
+    _, (sp,) = run(lambda u: u.view(I32).view(F32), f32([np.inf, -np.inf, np.nan]))
+    assert sp[0] == np.inf and sp[1] == -np.inf and np.isnan(sp[2])

@@ -30,7 +30,7 @@ TABLE_TESTS = [
     "test_polynomial_convolution_and_statistics_tables", "test_unwrap_tables", "test_reductions_views_dot_and_sort_tables",
     "test_activation_tables", "test_top_k_tables", "test_numpy_linalg_tables", "test_numpy_fft_tables", "test_random_distribution_tables",
     "test_einsum_tables", "test_dtype_promotion_and_half_double_tables", "test_cholesky_lu_eigvalsh_and_argreduce_tables",
-    "test_frexp_ldexp_and_flips", "test_jit_cases_of_the_tracing_suite",
+    "test_frexp_ldexp_and_flips", "test_jit_cases_of_the_tracing_suite", "test_array_suite_tables",
 ]
 
 
