@@ -65,6 +65,10 @@ def check_each_kernel(prog, bufs, f16_rtol=1e-2):
             np.testing.assert_array_equal(got, want, err_msg=msg)
         elif k.dtype == DType.Float16:
             np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64), rtol=f16_rtol, atol=2e-3, equal_nan=True, err_msg=msg)
+        elif k.exp.collect(lambda e: e.dtype == DType.Float16):
+            # float32 statistics of float16 data (sum of x*x): a float16 product feeding a wider accumulator is formed
+            # exactly on the GPU (as an MFMA forms it) where the checker rounds it to float16 first: float16 tolerance
+            np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64), rtol=2e-3, atol=2e-3, equal_nan=True, err_msg=msg)
         else:
             R = k.reduction.size if k.reduction is not None else 1
             np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64), rtol=1e-5 * max(1, math.sqrt(R)), atol=1e-6, equal_nan=True, err_msg=msg)
