@@ -246,3 +246,61 @@ def test_native_numerics_track_libm(name, fn, ref):
     nb.decRef(s)
     nb.decRef(o)
     np.testing.assert_allclose(got, ref(x.astype(np.float64)), rtol=3e-7, atol=1e-7)
+
+
+# ---- index arithmetic at the top of the int32 range ---------------------------------------------------------
+
+def test_two_billion_elements_through_map_row_and_column_reductions():
+    """The IR's indices are int32, so a buffer holds fewer than 2^31 elements; just under that -- float16
+    [32768, 65534], 4.3 GB -- a nullary fill, a map and both reduction orientations must still address every element.
+    Everything stays on the device; the small integer pattern ((flat index mod 251) - 125, then + 1) makes every
+    float32 partial sum an exact integer, so the results are compared with closed forms bit for bit."""
+    rows, L = 32768, 65534
+    n = rows * L
+    assert 2 ** 31 - 2 ** 17 < n < 2 ** 31
+    st = ShapeTracker.fromShape([rows, L])
+    fill = Kernel(0, n, AluExp.cast(F16, AluExp.sub(AluExp.mod(AluVar.gidx, AluExp.i32(251)), AluExp.i32(125))))
+    plus1 = mapKernel([n], [(F16, flat(n))], lambda v: AluExp.add(v, AluExp.const(F16, 1.0)))
+    row_sum = reduceKernel([rows, L], [(F16, st)], lambda v: AluExp.cast(F32, v), AluOp.Add)
+    col_sum = reduceKernel([L, rows], [(F16, st.permute([1, 0]))], lambda v: AluExp.cast(F32, v), AluOp.Add)
+    tail = Kernel(1, 64, AluExp.globalView(F16, 0, flat(n), [AluExp.add(AluVar.gidx, AluExp.i32(n - 64))]))
+    if WARM_ONLY:
+        from jaxjs_hip.kernelgen import generate
+        from jaxjs_hip.runtime import compile_source
+        for k in (fill, plus1, row_sum, col_sum, tail):
+            for src in generate(k, "wasm").sources:
+                compile_source(src)
+        pytest.skip("warm-up run: compiled only")
+    be = backend()
+    a, b = be.malloc(n * 2), be.malloc(n * 2)
+    r, c, t = be.malloc(rows * 4), be.malloc(L * 4), be.malloc(64 * 2)
+    try:
+        be.dispatch(be.prepareKernelSync(fill), [], [a])
+        be.dispatch(be.prepareKernelSync(plus1), [a], [b])
+        be.dispatch(be.prepareKernelSync(row_sum), [b], [r])
+        be.dispatch(be.prepareKernelSync(col_sum), [b], [c])
+        be.dispatch(be.prepareKernelSync(tail), [b], [t])
+        got_r = np.frombuffer(be.readSync(r), np.float32)
+        got_c = np.frombuffer(be.readSync(c), np.float32)
+        got_t = np.frombuffer(be.readSync(t), np.float16)
+    finally:
+        for s_ in (a, b, r, c, t):
+            be.decRef(s_)
+    # closed forms: value(i) = i % 251 - 124
+    period = np.arange(251, dtype=np.int64) - 124
+    pre = np.concatenate([[0], np.cumsum(period)])  # pre[m] = sum of the first m values of a period
+
+    def span(lo, count):  # sum of value(i) for i in [lo, lo + count), vectorised over lo
+        lo = np.asarray(lo, dtype=np.int64)
+        first = lo % 251
+        whole, rest = np.divmod(first + count, 251)
+        return whole * pre[251] + pre[rest] - pre[first]
+
+    want_r = span(np.arange(rows, dtype=np.int64) * L, L)
+    np.testing.assert_array_equal(got_r.astype(np.int64), want_r)
+    # column j: rows r contribute value(r * L + j); L % 251 = 23, so the residues walk with step 23: count them
+    j = np.arange(L, dtype=np.int64)
+    counts = np.bincount((np.arange(rows, dtype=np.int64) * L) % 251, minlength=251)  # residue of r * L
+    table = np.array([sum(int(counts[q]) * int(period[(q + s) % 251]) for q in range(251)) for s in range(251)], dtype=np.int64)
+    np.testing.assert_array_equal(got_c.astype(np.int64), table[j % 251])
+    np.testing.assert_array_equal(got_t.astype(np.int64), (np.arange(n - 64, n, dtype=np.int64) % 251) - 124)

@@ -209,6 +209,41 @@ def test_gemm_8192_cubed_every_element_exact():
     np.testing.assert_array_equal(got.reshape(n, n), ref)
 
 
+def test_gemm_output_just_under_two_to_the_31_elements():
+    """46336 x 46336 outputs (2,147,024,896 float16 values, 4.3 GB) over a short k axis: tile origins, the tile walk and the
+    store addresses near the end of the int32 index range.  Integer entries keep every value exact; rows from the first, a
+    middle and the last two block-tile rows are read back by range and compared bit for bit, in both layouts of B."""
+    from gpu_util import WARM_ONLY, backend
+    n, K = 46336, 64
+    assert 2 ** 31 - 2 ** 20 < n * n < 2 ** 31
+    A = RNG.integers(-2, 3, (n, K)).astype(np.float16)
+    B = RNG.integers(-2, 3, (K, n)).astype(np.float16)
+    rows = [0, 1, 255, 256, 23167, 23168, 46079, 46080, 46081, 46207, 46334, 46335]
+    for bt in (False, True):
+        k = matmulKernel(n, n, K, DType.Float16, b_transposed=bt)
+        if WARM_ONLY:
+            from jaxjs_hip.kernelgen import generate
+            from jaxjs_hip.runtime import compile_source
+            for src in generate(k).sources:
+                compile_source(src)
+            if bt:
+                pytest.skip("warm-up run: compiled only")
+            continue
+        be = backend()
+        exe = be.prepareKernelSync(k)
+        assert exe.data.ks.klass.startswith("gemm"), exe.data.ks.info
+        Bh = np.ascontiguousarray(B.T) if bt else B
+        a, b, out = be.malloc(A.nbytes, A.tobytes()), be.malloc(Bh.nbytes, Bh.tobytes()), be.malloc(k.bytes)
+        try:
+            be.dispatch(exe, [a, b], [out])
+            for r in rows:
+                got = np.frombuffer(be.readSync(out, r * n * 2, n * 2), np.float16)
+                np.testing.assert_array_equal(got.astype(np.float32), A[r].astype(np.float32) @ B.astype(np.float32), err_msg=f"row {r} {exe.data.ks.info}")
+        finally:
+            for s_ in (a, b, out):
+                be.decRef(s_)
+
+
 # The dense-GEMM sweep of the benchmark configuration: square 2048 / 4096 / 8192 and the skinny 128 x 14336 x 4096,
 # in f16 and f32.  Each case pins the launch shape the tuner picks for it (block tile, k split, workgroups) and is
 # checked against f64 dot products under the K-scaled bound on a row sample that meets every block-tile row.
