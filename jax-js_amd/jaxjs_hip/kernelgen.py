@@ -130,9 +130,10 @@ class _Body:
             idx = strip_parens(cg.run(n.src[0]))
             st = STORAGE_CTYPE[n.dtype]
             ptr = self.args[n.arg[0]]
-            if self.classes[id(n)] == "vector":
+            if self.classes[id(n)] in ("vector", "vector_u"):
                 var = f"v{self.tag}{k}"
-                cg.emit(f"const jh_pack<{st}, {self.V}> {var} = jh_vload<{st}, {self.V}>({ptr} + ({idx}));")
+                load = "jh_vload" if self.classes[id(n)] == "vector" else "jh_vload_u"
+                cg.emit(f"const jh_pack<{st}, {self.V}> {var} = {load}<{st}, {self.V}>({ptr} + ({idx}));")
                 loads[id(n)] = f"{var}.v[lane]"
             else:
                 var = f"u{self.tag}{k}"
