@@ -364,3 +364,45 @@ def test_matvec_f16(M, K, transposed):
     if M * K <= 1 << 16:
         want = oracle.run_kernel(k, [Wbuf, x], oracle.MODE_CPU)
         np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64), rtol=1e-2, atol=1e-4)
+
+
+# ---- rows and views off the vector grid: wide loads from addresses aligned to one element only ----------------
+
+def _sum_kernel(dt, rows, L, over_rows):
+    st = ShapeTracker.fromShape([rows, L])
+    if over_rows:  # reduce axis 0: outputs are the L columns
+        return reduceKernel([L, rows], [(dt, st.permute([1, 0]))], lambda v: AluExp.cast(DType.Float32 if dt != DType.Int32 else dt, v), AluOp.Add)
+    return reduceKernel([rows, L], [(dt, st)], lambda v: AluExp.cast(DType.Float32 if dt != DType.Int32 else dt, v), AluOp.Add)
+
+
+@pytest.mark.parametrize("dt,rows,L,over_rows", [
+    (DType.Float16, 257, 4095, False), (DType.Float32, 300, 1001, False), (DType.Int32, 64, 4099, False),
+    (DType.Float16, 1000, 1007, True), (DType.Float16, 4096, 1003, True), (DType.Int32, 4096, 1003, True), (DType.Float32, 33, 70001, True),
+], ids=str)
+def test_sums_over_rows_of_odd_length_use_wide_loads_and_stay_exact(dt, rows, L, over_rows):
+    """Small integer data (every partial sum exact in float32): the results must equal numpy's bit for bit whatever
+    lane layout the tuner picks; the plan must show the wide (`V` > 1) loads, which used to need aligned rows, and a
+    column sum whose width is not a multiple of V runs its leftover columns through the shared tail."""
+    from jaxjs_hip.tuner import tuneHip
+    k = _sum_kernel(dt, rows, L, over_rows)
+    t = tuneHip(k)
+    assert t.params["V"] > 1 and "vector_u" in t.vector_loads.values(), (t.klass, t.params)
+    npdt = {DType.Float16: np.float16, DType.Float32: np.float32, DType.Int32: np.int32}[dt]
+    x = RNG.integers(-3, 4, (rows, L)).astype(npdt)
+    got, ks = device_run(k, [x])
+    want = x.astype(np.int64).sum(0 if over_rows else 1)
+    np.testing.assert_array_equal(got.astype(np.int64), want, err_msg=f"{ks.klass} {ks.info}")
+    if over_rows:
+        assert L % t.params["V"] != 0  # leftover columns exist
+
+
+def test_shifted_views_in_a_map_use_wide_loads():
+    """x[1:] - x[:-1] and x[3:] * x[:-3] over float16 and float32: the shifted operand starts off the vector grid."""
+    from jaxjs_hip.tuner import tuneHip
+    for dt, npdt, n, shift in ((DType.Float16, np.float16, 100001, 1), (DType.Float32, np.float32, 65539, 3)):
+        st = ShapeTracker.fromShape([n + shift])
+        k = mapKernel([n], [(dt, st.shrink([(shift, n + shift)])), (dt, st.shrink([(0, n)]))], lambda a, b: AluExp.sub(AluExp.mul(a, b), b))
+        assert "vector_u" in tuneHip(k).vector_loads.values()
+        x = RNG.integers(-5, 6, n + shift).astype(npdt)
+        got, _ = device_run(k, [x, x])
+        np.testing.assert_array_equal(got, x[shift:] * x[:-shift] - x[:-shift])
