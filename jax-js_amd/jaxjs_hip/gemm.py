@@ -542,7 +542,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         raise ValueError(f"direct-to-LDS slab depth must be 32 or 64, got {dBK}")
     full = g["M"] % BM == 0 and g["N"] % BN == 0 and g["K"] % dBK == 0 and BM >= 128 and BN >= 128
     any_gather = bool(g.get("a_gather") or g.get("b_gather"))
-    dlds = g["dtype"] == DType.Float16 and full and tile.get("DLDS", 1) and not any_gather
+    loose = {tag: 1 if g.get(tag + "_loose") and not g.get(tag + "_gather") else 0 for tag in ("a", "b")}
+    dlds = g["dtype"] == DType.Float16 and full and tile.get("DLDS", 1) and not any_gather and not (loose["a"] or loose["b"])
     if dlds:
         tmpl = "gemm_f16_dlds.hip.inc"
     if dlds:
@@ -581,9 +582,10 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
             sched.update(VEC_EPI=0, VEPI_LOADS="", VEPI_BODY="", VEPI_VALUE="0", OUT_T=out_t)
     elif g["dtype"] == DType.Float16:
         sched = dict(COMMIT_A=tile.get("CA", 2), COMMIT_B=tile.get("CB", 3), FETCH_A=tile.get("FA", 0),
-                     FETCH_B=tile.get("FB", 1), IGLP=tile.get("IGLP", -1), SCHED_FENCE=tile.get("FENCE", 0))
+                     FETCH_B=tile.get("FB", 1), IGLP=tile.get("IGLP", -1), SCHED_FENCE=tile.get("FENCE", 0),
+                     A_LOOSE=loose["a"], B_LOOSE=loose["b"])
     else:
-        sched = dict(BK=fBK, FRAG_FENCE=int(tile.get("FENCE", 1)), FUSEK=fusek)
+        sched = dict(BK=fBK, FRAG_FENCE=int(tile.get("FENCE", 1)), FUSEK=fusek, A_LOOSE=loose["a"], B_LOOSE=loose["b"])
     if not dlds:
         sched.update(GATHER_FNS="\n".join(gather_fns), A_GATHER=gather_flags["a"], B_GATHER=gather_flags["b"],
                      GATHER_A_CALL=gather_calls["a"], GATHER_B_CALL=gather_calls["b"],

@@ -519,21 +519,27 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
 
 def _gemm_worthwhile(g: dict) -> bool:
     """MFMA tiles only pay off for a real dense contraction; thin shapes stream better through the
-    row-reduce template (matvec and friends).  The tile loaders move 128-bit vectors, so every
-    address they form must be a multiple of the vector: unit stride on k or on the row axis, all
-    other strides and offsets divisible by the vector length."""
+    row-reduce template (matvec and friends).  The tile loaders move 128-bit vectors along an operand's unit-stride
+    axis (k or the row axis); the direct-to-LDS template needs every such vector whole and on the 16-byte grid, the
+    general float16 template and the float32 template also take operands where they are not (see `operand_ok`)."""
     if g["M"] < 32 or g["N"] < 32 or g["K"] < 32:
         return False
     vec = 8 if g["dtype"] == DType.Float16 else 4
     bstr_a = [b[1] for b in g["batch"]]
     bstr_b = [b[2] for b in g["batch"]]
 
-    def operand_ok(sk, srow, rows, off, bstr):
+    def operand_ok(tag, sk, srow, rows, off, bstr, k0):
+        """An operand with a unit-stride axis.  `g[tag + "_loose"]` records whether its 128-bit groups are all whole and
+        on the 16-byte grid; if not, the general float16 template and the float32 template load them loosely (under-aligned
+        addresses, the group across the end of the axis element by element) -- a two-level k axis has no such path."""
         if sk == 1:
-            return g["K"] % vec == 0 and srow % vec == 0 and off % vec == 0 and all(x % vec == 0 for x in bstr)
-        if srow == 1:
-            return rows % vec == 0 and sk % vec == 0 and off % vec == 0 and all(x % vec == 0 for x in bstr)
-        return False
+            tight = g["K"] % vec == 0 and srow % vec == 0 and off % vec == 0 and all(x % vec == 0 for x in bstr)
+        elif srow == 1:
+            tight = rows % vec == 0 and sk % vec == 0 and off % vec == 0 and all(x % vec == 0 for x in bstr)
+        else:
+            return False
+        g[tag + "_loose"] = not tight
+        return tight or k0 == g["K"]
 
     def split_ok(k0, sk, sk1):
         # A two-level k axis is only loaded along unit-stride runs, and no k-slab may straddle two runs.
@@ -543,6 +549,6 @@ def _gemm_worthwhile(g: dict) -> bool:
         # The gather loader packs 8 (f16) / 4 (f32) consecutive k per store and has no ragged-k path.
         if g["K"] % vec != 0:
             return False
-    return ((g.get("a_gather") or operand_ok(g["a_sk"], g["a_sm"], g["M"], g["a_off"], bstr_a))
-            and (g.get("b_gather") or operand_ok(g["b_sk"], g["b_sn"], g["N"], g["b_off"], bstr_b))
+    return ((g.get("a_gather") or operand_ok("a", g["a_sk"], g["a_sm"], g["M"], g["a_off"], bstr_a, g["a_k0"]))
+            and (g.get("b_gather") or operand_ok("b", g["b_sk"], g["b_sn"], g["N"], g["b_off"], bstr_b, g["b_k0"]))
             and split_ok(g["a_k0"], g["a_sk"], g["a_sk1"]) and split_ok(g["b_k0"], g["b_sk"], g["b_sk1"]))

@@ -244,6 +244,54 @@ def test_gemm_output_just_under_two_to_the_31_elements():
                 be.decRef(s_)
 
 
+# ---- operands off the 16-byte grid: extents that are not multiples of the 128-bit groups, odd row pitches, shifted starts
+
+LOOSE_CASES = [
+    # dtype, M, N, K, B stored [N,K], batch
+    (DType.Float16, 130, 257, 100, False, ()), (DType.Float16, 130, 257, 100, True, ()), (DType.Float16, 333, 1001, 515, False, ()),
+    (DType.Float16, 333, 1001, 515, True, ()), (DType.Float16, 64, 50257 // 16, 768, False, ()), (DType.Float16, 257, 129, 66, False, (3,)),
+    (DType.Float16, 1025, 1027, 1029, False, ()), (DType.Float16, 200, 72, 4100, True, ()),
+    (DType.Float32, 130, 257, 101, False, ()), (DType.Float32, 130, 257, 101, True, ()), (DType.Float32, 333, 1001, 515, False, ()),
+    (DType.Float32, 129, 66, 257, True, (2,)), (DType.Float32, 1025, 1027, 1029, False, ()),
+]
+
+
+@pytest.mark.parametrize("dt,M,N,K,bt,batch", LOOSE_CASES, ids=lambda v: v.value if isinstance(v, DType) else str(v))
+def test_gemm_operands_off_the_vector_grid_are_exact(dt, M, N, K, bt, batch):
+    """np.matmul with extents like 1001 or 50257 (row pitches that are not multiples of 16 bytes, a last 128-bit group
+    that crosses the end of the axis): still the matrix-core class -- the loaders take whole groups from under-aligned
+    addresses and the crossing group element by element -- and, with small integer entries, exact in every element."""
+    npdt = np.float16 if dt == DType.Float16 else np.float32
+    A = RNG.integers(-2, 3, batch + (M, K)).astype(npdt)
+    B = RNG.integers(-2, 3, batch + (K, N)).astype(npdt)
+    k = matmulKernel(M, N, K, dt, b_transposed=bt, batch=batch)
+    if dt == DType.Float16:
+        k = _f32_out(k, K)
+    got, ks = device_run(k, [A, np.ascontiguousarray(np.swapaxes(B, -1, -2)) if bt else B])
+    assert ks.klass.startswith("gemm") and not ks.info.get("direct_lds"), (ks.klass, ks.info)
+    np.testing.assert_array_equal(got.reshape(batch + (M, N)).astype(np.float32), A.astype(np.float32) @ B.astype(np.float32), err_msg=str(ks.info))
+
+
+@pytest.mark.parametrize("dt", [DType.Float16, DType.Float32], ids=lambda d: d.value)
+def test_gemm_operands_that_start_off_the_vector_grid(dt):
+    """Full tiles (256 x 256 x 128) but both operands are views that start one and three elements into their buffers:
+    nothing is ragged, every 128-bit group is misaligned, and the direct-to-LDS template must not be picked."""
+    M, N, K = 256, 256, 128
+    npdt = np.float16 if dt == DType.Float16 else np.float32
+    abuf = RNG.integers(-2, 3, M * K + 1).astype(npdt)
+    bbuf = RNG.integers(-2, 3, K * N + 3).astype(npdt)
+    full = [M, N, K]
+    stA = ShapeTracker.fromShape([M * K + 1]).shrink([(1, M * K + 1)]).reshape([M, 1, K]).expand(full)
+    stB = ShapeTracker.fromShape([K * N + 3]).shrink([(3, K * N + 3)]).reshape([K, N]).permute([1, 0]).reshape([1, N, K]).expand(full)
+    k = reduceKernel(full, [(dt, stA), (dt, stB)], lambda a, b: AluExp.mul(a, b), AluOp.Add)
+    if dt == DType.Float16:
+        k = _f32_out(k, K)
+    got, ks = device_run(k, [abuf, bbuf])
+    assert ks.klass.startswith("gemm") and not ks.info.get("direct_lds"), (ks.klass, ks.info)
+    want = abuf[1:].reshape(M, K).astype(np.float32) @ bbuf[3:].reshape(K, N).astype(np.float32)
+    np.testing.assert_array_equal(got.reshape(M, N).astype(np.float32), want)
+
+
 # The dense-GEMM sweep of the benchmark configuration: square 2048 / 4096 / 8192 and the skinny 128 x 14336 x 4096,
 # in f16 and f32.  Each case pins the launch shape the tuner picks for it (block tile, k split, workgroups) and is
 # checked against f64 dot products under the K-scaled bound on a row sample that meets every block-tile row.
