@@ -570,6 +570,16 @@ def main():
             Am = hostrand.uniform(1004, (mm, kk), dtype=npdt)
             Bm = hostrand.uniform(1005, (kk, nn), dtype=npdt, stream=1)
             run(tag, matmulKernel(mm, nn, kk, dt), [Am, Bm], 2.0 * mm * nn * kk, "TFLOP/s", peak)
+        # A linear layer on a few tokens and matmul against a vocabulary of 50257 columns: HBM-bound on B / rows and row
+        # pitches off the 16-byte grid; reported in GB/s of algorithmic bytes and TFLOP/s respectively.
+        for mm in (4, 16, 64):
+            Am = hostrand.uniform(1004, (mm, 4096), dtype=np.float16)
+            Bm = hostrand.uniform(1005, (4096, 14336), dtype=np.float16, stream=1)
+            run(f"gemm_f16_{mm}x14336x4096", matmulKernel(mm, 14336, 4096, DType.Float16), [Am, Bm],
+                2.0 * (mm * 4096 + 4096 * 14336 + mm * 14336), "GB/s", PEAK_HBM_GBS)
+        Am = hostrand.uniform(1004, (8192, 768), dtype=np.float16)
+        Bm = hostrand.uniform(1005, (768, 50257), dtype=np.float16, stream=1)
+        run("gemm_f16_8192x50257x768", matmulKernel(8192, 50257, 768, DType.Float16), [Am, Bm], 2.0 * 8192 * 50257 * 768, "TFLOP/s", PEAK_F16_TFLOPS)
         Am = hostrand.uniform(1004, (8192, 8192), dtype=np.float16)
         Bm = hostrand.uniform(1005, (8192, 8192), dtype=np.float16, stream=1)
         run("gemm_f16_8192_NT(B stored [N,K])", matmulKernel(8192, 8192, 8192, DType.Float16, b_transposed=True), [Am, Bm],

@@ -47,19 +47,35 @@ def choose_tile(g: dict) -> Dict[str, int]:
             # The slices are folded inside the launch (1024^3: 30.2 -> 27.8 us, 128x14336x4096: 169 -> 166, same bits);
             # four waves stacked along m then measure another 1 % better than 2x2.
             return dict(BM=128, BN=64, BK=bk, SPLITK=split, **(dict(FUSEK=1, WM=4, WN=1) if split > 1 else {}))
-        return dict(BM=64, BN=64, BK=bk)
+        # Fewer than 128 rows or 64 columns: 64x64 tiles, the k axis cut the same way when they are few.
+        split = 1
+        while plain_k and tiles(64, 64) * split < 1.5 * CU and split < 8 and g["K"] % (split * 2 * bk) == 0 and g["K"] // (split * 2) >= 256:
+            split *= 2
+        return dict(BM=64, BN=64, BK=bk, **(dict(SPLITK=split, FUSEK=1) if split > 1 else {}))
     # f16: estimated time = (tiles the busiest CU runs) x (tile area) x (K + fixed per-tile overhead) / efficiency.
     # Efficiencies are measured rates of each tile shape relative to 256x256 on large problems (MI355X):
     # 128x256 0.84, 256x128 0.79, 128x128 0.72 with two workgroups resident per CU (0.64 alone).  The fixed
     # overhead (pipeline fill + epilogue) is about 100 k-steps.  This picks big tiles for big problems and
     # smaller ones when 256x256 would leave the last round of CUs nearly empty (e.g. 288 tiles on 256 CUs).
-    if g["M"] <= 64 and g["N"] >= 256:
-        # Few rows (e.g. 64 output channels of a convolution against thousands of positions): a 64-row tile.
-        return dict(BM=64, BN=256, WM=1, WN=4)
+    def k_split(count):
+        # Fewer workgroups than 1.5 per CU: cut the k axis (partial sums in scratch, fold kernel) while slices stay >= 512 deep.
+        split = 1
+        while plain_k and count * split < 1.5 * CU and split < 8 and g["K"] % (split * 2 * 64) == 0 and g["K"] // (split * 2) >= 512:
+            split *= 2
+        return dict(SPLITK=split) if split > 1 else {}
+
+    if g["M"] <= 64 and g["N"] >= 128:
+        # Few rows.  Many tiles (64 output channels of a convolution against thousands of positions): 64 x 256.
+        if g["N"] >= 256 and tiles(64, 256) >= CU:
+            return dict(BM=64, BN=256, WM=1, WN=4)
+        # Few tiles (a linear layer on 2..64 tokens): bound by streaming B once, so what matters is enough workgroups
+        # in flight -- 64 x 128 tiles and a k split (64 x 14336 x 4096: 65.7 us with 56 tiles of 64 x 256, 26.6 us with
+        # 112 x 4 slices; 16 rows 24.6 us, 4 rows 23.5 us; B alone takes 20 us at the HBM rate).
+        return dict(BM=64, BN=128, WM=1, WN=4, **k_split(tiles(64, 128)))
     if g["N"] <= 64 and g["M"] >= 128:
         # A 128-wide tile would compute and store a half-empty block (attention's probabilities x V, N = head
         # size 64): measured 30 % faster with 128x64 tiles, which is then bound by reading A.
-        return dict(BM=128, BN=64, WM=2, WN=2)
+        return dict(BM=128, BN=64, WM=2, WN=2, **k_split(tiles(128, 64)))
     best = None
     for bm, bn, eff, extra in ((256, 256, 1.00, dict()), (128, 256, 0.84, dict(WM=1, WN=4)), (256, 128, 0.79, dict()),
                                 (128, 128, 0.72, dict())):

@@ -517,13 +517,21 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
     return t
 
 
+GEMM_MIN_ROWS = 32  # fewer rows (or columns) than this only against a large operand (see _gemm_worthwhile)
+
+
 def _gemm_worthwhile(g: dict) -> bool:
     """MFMA tiles only pay off for a real dense contraction; thin shapes stream better through the
     row-reduce template (matvec and friends).  The tile loaders move 128-bit vectors along an operand's unit-stride
     axis (k or the row axis); the direct-to-LDS template needs every such vector whole and on the 16-byte grid, the
     general float16 template and the float32 template also take operands where they are not (see `operand_ok`)."""
-    if g["M"] < 32 or g["N"] < 32 or g["K"] < 32:
+    thin = min(g["M"], g["N"])
+    if g["K"] < 32 or thin < 2:
+        return False  # one row or column is a matvec: the reduction classes stream it at the HBM rate
+    if thin < GEMM_MIN_ROWS and (max(g["M"], g["N"]) < 128 or g["K"] < 256 or max(g["M"], g["N"]) * g["K"] < (1 << 20)):
         return False
+    # (2..31 rows against a large operand -- a linear layer on a handful of tokens -- do go to the matrix cores: as
+    # separate dot products the large operand is read once per row, 202 us for 16 x 14336 x 4096 against 25 us.)
     vec = 8 if g["dtype"] == DType.Float16 else 4
     bstr_a = [b[1] for b in g["batch"]]
     bstr_b = [b[2] for b in g["batch"]]

@@ -292,6 +292,37 @@ def test_gemm_operands_that_start_off_the_vector_grid(dt):
     np.testing.assert_array_equal(got.reshape(M, N).astype(np.float32), want)
 
 
+# ---- a handful of rows (or columns) against a large operand: a linear layer on a few tokens
+
+THIN_CASES = [
+    # dtype, M, N, K, B stored [N,K], expected tile and k split
+    (DType.Float16, 2, 14336, 4096, False, dict(BM=64, BN=128, splitk=4)), (DType.Float16, 16, 14336, 4096, True, dict(BM=64, BN=128, splitk=4)),
+    (DType.Float16, 31, 4096, 4096, False, dict(BM=64, BN=128, splitk=8)), (DType.Float16, 64, 14336, 4096, False, dict(BM=64, BN=128, splitk=4)),
+    (DType.Float16, 14336, 16, 4096, False, dict(BM=128, BN=64, splitk=4)), (DType.Float16, 7, 1000, 4100, True, dict(BM=64, BN=128)),
+    (DType.Float32, 4, 14336, 4096, False, dict(BM=64, BN=64, splitk=2)), (DType.Float32, 14336, 16, 4096, False, dict(BM=64, BN=64, splitk=2)),
+]
+
+
+@pytest.mark.parametrize("dt,M,N,K,bt,want", THIN_CASES, ids=lambda v: v.value if isinstance(v, DType) else str(v) if not isinstance(v, dict) else "")
+def test_gemm_with_a_handful_of_rows_runs_on_the_matrix_cores(dt, M, N, K, bt, want):
+    """2..64 rows against a large B (or columns against a large A): as separate dot products the large operand would be
+    read once per row; as one GEMM with 64-row tiles and the k axis cut over several workgroups it is read once.  The
+    plan is pinned, the result (small integers) exact."""
+    npdt = np.float16 if dt == DType.Float16 else np.float32
+    A = RNG.integers(-1, 2, (M, K)).astype(npdt)
+    B = RNG.integers(-1, 2, (K, N)).astype(npdt)
+    k = matmulKernel(M, N, K, dt, b_transposed=bt)
+    got, ks = device_run(k, [A, np.ascontiguousarray(B.T) if bt else B])
+    assert ks.klass.startswith("gemm") and all(ks.info.get(a) == b for a, b in want.items()), (ks.klass, ks.info)
+    np.testing.assert_array_equal(got.reshape(M, N).astype(np.float32), A.astype(np.float32) @ B.astype(np.float32), err_msg=str(ks.info))
+
+
+def test_single_rows_and_small_operands_stay_with_the_reduction_classes():
+    from jaxjs_hip.tuner import tuneHip
+    for M, N, K in ((1, 14336, 4096), (14336, 1, 4096), (5, 300, 700), (16, 64, 64), (8, 100, 2048)):
+        assert tuneHip(matmulKernel(M, N, K, DType.Float16)).klass.startswith("reduce"), (M, N, K)
+
+
 # The dense-GEMM sweep of the benchmark configuration: square 2048 / 4096 / 8192 and the skinny 128 x 14336 x 4096,
 # in f16 and f32.  Each case pins the launch shape the tuner picks for it (block tile, k split, workgroups) and is
 # checked against f64 dot products under the K-scaled bound on a row sample that meets every block-tile row.
