@@ -99,7 +99,11 @@ def choose_tile(g: dict) -> Dict[str, int]:
         # launch, 24.7 folded in the launch; 128x4096x4096: 16.1 us in two slices, 13.9 in four; with 112 tiles four
         # slices cost more in partial sums than they gain).
         if tiles(128, 128) * 2 <= CU and g["K"] >= 2048 and g["K"] % 128 == 0:
-            tile.update(SPLITK=4 if tiles(128, 128) * 4 <= CU and g["K"] >= 4096 and g["K"] % 256 == 0 else 2, FUSEK=1)
+            tile.update(SPLITK=4 if tiles(128, 128) * 4 <= CU and g["K"] >= 4096 and g["K"] % 256 == 0 else 2)
+            # Folding inside the launch is the direct-to-LDS template's: whole tiles, operands on the 16-byte grid.  Ragged
+            # or loose shapes (100 x 14336 x 4096) keep the split and fold in a second launch.
+            if g["M"] % 128 == 0 and g["N"] % 128 == 0 and not (g.get("a_loose") or g.get("b_loose")):
+                tile.update(FUSEK=1)
     return tile
 
 
