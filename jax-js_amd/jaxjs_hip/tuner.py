@@ -517,6 +517,7 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
     return t
 
 
+GEMM_MIN_K = 32     # a shorter reduce axis than this: the reduction classes
 GEMM_MIN_ROWS = 32  # fewer rows (or columns) than this only against a large operand (see _gemm_worthwhile)
 
 
@@ -526,7 +527,9 @@ def _gemm_worthwhile(g: dict) -> bool:
     axis (k or the row axis); the direct-to-LDS template needs every such vector whole and on the 16-byte grid, the
     general float16 template and the float32 template also take operands where they are not (see `operand_ok`)."""
     thin = min(g["M"], g["N"])
-    if g["K"] < 32 or thin < 2:
+    # (A convolution's gathered operand makes the reduction classes walk its window arithmetic once per output; it
+    # pays to pad even a 27-long k axis -- 3 channels x 3 x 3 -- to one slab: 83 -> 14 us.)
+    if g["K"] < (GEMM_MIN_K // 2 if g.get("a_gather") or g.get("b_gather") else GEMM_MIN_K) or thin < 2:
         return False  # one row or column is a matvec: the reduction classes stream it at the HBM rate
     if thin < GEMM_MIN_ROWS and (max(g["M"], g["N"]) < 128 or g["K"] < 256 or max(g["M"], g["N"]) * g["K"] < (1 << 20)):
         return False
@@ -553,10 +556,8 @@ def _gemm_worthwhile(g: dict) -> bool:
         # A two-level k axis is only loaded along unit-stride runs, and no k-slab may straddle two runs.
         return k0 == g["K"] or (sk == 1 and k0 % 64 == 0 and sk1 % vec == 0 and sk1 > 0)
 
-    if g.get("a_gather") or g.get("b_gather"):
-        # The gather loader packs 8 (f16) / 4 (f32) consecutive k per store and has no ragged-k path.
-        if g["K"] % vec != 0:
-            return False
+    # (Gather operands take any k extent: the element loader and the row-vector loader check every k, and the block
+    # loaders of the tap-major order are only chosen when k is a multiple of 8.)
     return ((g.get("a_gather") or operand_ok("a", g["a_sk"], g["a_sm"], g["M"], g["a_off"], bstr_a, g["a_k0"]))
             and (g.get("b_gather") or operand_ok("b", g["b_sk"], g["b_sn"], g["N"], g["b_off"], bstr_b, g["b_k0"]))
             and split_ok(g["a_k0"], g["a_sk"], g["a_sk1"]) and split_ok(g["b_k0"], g["b_sk"], g["b_sk1"]))

@@ -179,6 +179,10 @@ CONV_CASES = [
     dict(x=(1, 4, 9, 9), w=(2, 4, 3, 3), strides=[2, 2], padding=[(1, 1), (1, 1)], rd=[2, 1]),
     dict(x=(1, 2, 5, 4, 3), w=(2, 2, 2, 2, 2), strides=[1, 1, 1], padding=[(0, 0), (1, 0), (0, 1)]),
     dict(x=(3, 8, 6, 6), w=(16, 8, 1, 1), strides=[1, 1], padding=[(0, 0), (0, 0)]),
+    # k = C * kh * kw is not a multiple of the loaders' groups (147, 27, 900): still implicit GEMMs on the GPU
+    dict(x=(2, 3, 30, 30), w=(32, 3, 7, 7), strides=[2, 2], padding=[(2, 3), (2, 3)]),
+    dict(x=(2, 3, 16, 16), w=(32, 3, 3, 3), strides=[1, 1], padding=[(1, 1), (1, 1)]),
+    dict(x=(1, 100, 12, 12), w=(40, 100, 3, 3), strides=[1, 1], padding=[(1, 1), (1, 1)]),
 ]
 
 
@@ -249,6 +253,25 @@ def test_convolution_on_gpu(case):
                 compile_source(src)
         pytest.skip("warm-up run: compiled only")
     _conv_case(case, backend())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [DType.Float16, F32], ids=lambda d: d.value)
+@pytest.mark.parametrize("case", CONV_CASES[-3:], ids=lambda c: "x".join(map(str, c["x"])) + "*" + "x".join(map(str, c["w"])))
+def test_convolutions_with_a_ragged_k_axis_are_implicit_gemms(case, dt):
+    """3 input channels under a 7x7 or 3x3 window, 100 channels under 3x3: C * kh * kw = 147, 27, 900.  The kernel class
+    must be the matrix-core one (the gathered operand's loaders check every k) and small integers come out exact."""
+    from gpu_util import device_run
+    from jaxjs_hip.alu import numpyDtype
+    prog = J.jit(lambda a, b: L.convGeneralDilated(a, b, case["strides"], case["padding"]), [ShapedArray(case["x"], dt), ShapedArray(case["w"], dt)])
+    assert len(prog.kernels) == 1
+    rng = np.random.default_rng(5)
+    x = rng.integers(-2, 3, case["x"]).astype(numpyDtype(dt))
+    w = rng.integers(-1, 2, case["w"]).astype(numpyDtype(dt))
+    got, ks = device_run(prog.kernels[0], [x, w])
+    assert ks.klass.startswith("gemm"), (ks.klass, ks.info)
+    want = conv_reference(x.astype(np.float32), w.astype(np.float32), case["strides"], case["padding"], None, None)
+    np.testing.assert_array_equal(got.astype(np.float32).reshape(want.shape), want, err_msg=str(ks.info))
 
 
 @pytest.mark.gpu
