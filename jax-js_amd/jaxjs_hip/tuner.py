@@ -512,7 +512,10 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
     t.klass = "reduce_col"
     t.vector_loads = along_g if V > 1 else {}
     t.params = dict(V=V, T=T, lx=lx, block=lx * T, split=split, unroll=unroll, interleave=interleave)
-    t.params["grid"] = _grid_for((groups + lx - 1) // lx)
+    # The cap on the grid is meant for 256-thread blocks; blocks of one wave (no split of the fold over row slots) get
+    # proportionally more of them, or a short fold over many outputs (a depthwise convolution: 6.4 M outputs of 9 terms)
+    # runs four waves per SIMD where it wants sixteen.
+    t.params["grid"] = max(1, min((groups + lx - 1) // lx, MAX_GRID_BLOCKS * max(1, 256 // (lx * T))))
     t.epi_vector_loads = classify_loads(t.epilogue, "gidx", V) if V > 1 else {}
     return t
 
