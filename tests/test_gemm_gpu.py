@@ -301,8 +301,8 @@ THIN_CASES = [
     (DType.Float16, 14336, 16, 4096, False, dict(BM=128, BN=64, splitk=4)), (DType.Float16, 7, 1000, 4100, True, dict(BM=64, BN=128)),
     (DType.Float32, 4, 14336, 4096, False, dict(BM=64, BN=64, splitk=2)), (DType.Float32, 14336, 16, 4096, False, dict(BM=64, BN=64, splitk=2)),
     # 65..127 rows, few 128x128 tiles, long k: the tile is not whole, so the k split folds in a second launch
-    (DType.Float16, 100, 14336, 4096, False, dict(BM=128, BN=128, splitk=2, direct_lds=False)), (DType.Float16, 65, 4096, 4096, True, dict(BM=128, BN=128, splitk=4)),
-    (DType.Float16, 300, 300, 8192, False, dict(BM=128, BN=128, splitk=4)), (DType.Float16, 8192, 100, 4096, False, dict(BM=128, BN=128, splitk=4)),
+    (DType.Float16, 100, 14336, 4096, False, dict(BM=128, BN=128, splitk=4, direct_lds=False)), (DType.Float16, 65, 4096, 4096, True, dict(BM=128, BN=128, splitk=8)),
+    (DType.Float16, 300, 300, 8192, False, dict(BM=128, BN=128, splitk=8)), (DType.Float16, 8192, 100, 4096, False, dict(BM=128, BN=128, splitk=8)),
 ]
 
 
