@@ -15,6 +15,7 @@ from typing import Dict, List, Optional, Tuple
 from .alu import AluExp, AluOp, AluVar, DType, Kernel, Reduction, byteWidth
 from .codegen import CTYPE, STORAGE_CTYPE, HipExpCodegen, const_literal, strip_parens
 from .errors import UnsupportedOpError
+from .shape import prod
 from .tuner import TuneResult, tuneHip
 
 _TEMPLATE_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc", "templates")
@@ -180,6 +181,8 @@ def generate(kernel: Kernel, numerics: str = "wasm", tune: Optional[TuneResult] 
     t = tune or tuneHip(kernel, **tune_opts)
     if t.klass == "map":
         return _gen_map(kernel, t, numerics, name)
+    if t.klass == "map_t":
+        return _gen_map_transposed(kernel, t, numerics, name)
     if t.klass == "reduce_row":
         return _gen_reduce(kernel, t, numerics, name, row=True)
     if t.klass == "reduce_col":
@@ -207,6 +210,35 @@ def _gen_map(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     step = LaunchStep(name, (grid, 1, 1), (block, 1, 1), 0,
                       [("in", i) for i in range(kernel.nargs)] + [("out", 0)])
     return KernelSource([src], [step], [], "map", _min_bytes(t.exp), dict(t.params))
+
+
+def _gen_map_transposed(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelSource:
+    """64 x 64 tiles through LDS for a map whose operand runs along another axis than its output (map_t.hip.inc)."""
+    p = t.params
+    shape, strides, j = p["shape"], p["strides"], p["j"]
+    n = len(shape)
+    ostr = [1] * n
+    for i in range(n - 2, -1, -1):
+        ostr[i] = ostr[i + 1] * shape[i + 1]
+    used = _used_args(kernel.nargs, t.exp)
+    out_t = STORAGE_CTYPE[kernel.dtype]
+    params, args = _params(used, out_t)
+    (load,) = t.exp.collect(lambda x: x.op == AluOp.GlobalIndex)
+    cg = HipExpCodegen(args, IDENT, "        ", prefix="m", numerics=numerics)
+    cg.loads = {id(load): "jh_x"}
+    cg.countReferences(t.exp)
+    value = strip_parens(cg.run(t.exp))
+    body = "\n".join(cg.take_lines())
+    outer = [i for i in range(n - 1) if i != j]
+    decode = []
+    for i in reversed(outer):
+        decode.append(f"  {{ const long long d = rem % {shape[i]}ll; rem /= {shape[i]}ll; in_base += d * {strides[i]}ll; out_base += d * {ostr[i]}ll; }}")
+    blocks = prod([shape[i] for i in outer]) * -(-shape[j] // 64) * -(-shape[-1] // 64)
+    src = _prelude(numerics) + fill(template("map_t.hip.inc"), dict(
+        NJ=shape[j], NC=shape[-1], SC=strides[-1], OSJ=ostr[j], NAME=name, PARAMS=params, OUT_T=out_t,
+        IN_T=STORAGE_CTYPE[load.dtype], IN_PTR=args[p["gid"]], IN_OFF=p["offset"], OUTER_DECODE="\n".join(decode), BODY=body, VALUE=value))
+    step = LaunchStep(name, (blocks, 1, 1), (256, 1, 1), 0, [("in", i) for i in range(kernel.nargs)] + [("out", 0)])
+    return KernelSource([src], [step], [], "map_t", _min_bytes(t.exp), dict(tile=64, blocks=blocks, j=j, shape=shape))
 
 
 def _partial_pitch(size: int, V: int) -> int:

@@ -403,6 +403,36 @@ def _grid_for(blocks_needed: int) -> int:
     return max(1, min(int(blocks_needed), MAX_GRID_BLOCKS))
 
 
+def match_transposed_map(kernel: Kernel) -> Optional[dict]:
+    """A map over exactly one operand, read through one unmasked strided view whose unit-stride axis is not the output's
+    fastest axis (a transpose or axis permutation written out): {gid, shape, strides, offset, j} with j the operand's
+    unit-stride axis.  Anything else (several operands, masks, position-dependent expressions, small arrays) is None."""
+    if kernel.reduction is not None or kernel.size < (1 << 16):
+        return None
+    exp = kernel.exp
+    views = exp.collect(lambda n: n.op == AluOp.GlobalView)
+    if len(views) != 1 or exp.collect(lambda n: n.op == AluOp.GlobalIndex):
+        return None
+    node = views[0]
+    gid, st = node.arg
+    if len(st.views) != 1 or st.views[0].mask is not None or node.dtype not in (DType.Float16, DType.Float32, DType.Int32, DType.Uint32):
+        return None
+    v = st.views[0]
+    shape, strides = list(v.shape), list(v.strides)
+    if len(shape) < 2 or math.prod(shape) != kernel.size or strides[-1] in (0, 1) or any(x < 0 for x in strides):
+        return None
+    expected = [u.simplify() for u in unravelAlu(shape, AluVar.gidx)]
+    if len(node.src) != len(expected) or any(x.simplify() is not y for x, y in zip(node.src, expected)):
+        return None
+    rest = exp.rewrite(lambda n: AluExp.const(n.dtype, 0) if n is node else None)
+    if references(rest, "gidx"):
+        return None  # the expression also depends on the position itself
+    js = [i for i in range(len(shape) - 1) if strides[i] == 1 and shape[i] >= 32]
+    if not js or shape[-1] < 32:
+        return None
+    return dict(gid=gid, shape=shape, strides=strides, offset=v.offset, j=js[-1])
+
+
 def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True,
             gemm_tile: Optional[tuple] = None, col_strip: Optional[tuple] = None,
             row_lanes: Optional[int] = None) -> TuneResult:
@@ -412,6 +442,11 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
     size = kernel.size
 
     if re is None:
+        tm = match_transposed_map(kernel)
+        if tm is not None:
+            t.klass = "map_t"
+            t.params = dict(tm)
+            return t
         V = _pick_vector_width(kernel, t, size)
         t.klass = "map"
         t.vector_loads = classify_loads(t.exp, "gidx", V)

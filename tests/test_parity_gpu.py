@@ -406,3 +406,50 @@ def test_shifted_views_in_a_map_use_wide_loads():
         x = RNG.integers(-5, 6, n + shift).astype(npdt)
         got, _ = device_run(k, [x, x])
         np.testing.assert_array_equal(got, x[shift:] * x[:-shift] - x[:-shift])
+
+
+# ---- materialised transposes / axis permutations: 64 x 64 tiles through LDS -------------------------------------
+
+TRANSPOSED_MAPS = [
+    # buffer shape, permutation, dtype
+    ((1000, 4096), (1, 0), DType.Float16), ((777, 333), (1, 0), DType.Float32), ((4096, 1000), (1, 0), DType.Int32),
+    ((5, 300, 200), (0, 2, 1), DType.Float16), ((300, 7, 200), (2, 1, 0), DType.Float32), ((64, 3, 5, 100), (3, 1, 2, 0), DType.Uint32),
+]
+
+
+@pytest.mark.parametrize("shape,perm,dt", TRANSPOSED_MAPS, ids=str)
+def test_materialised_permutations_go_through_lds_tiles_and_are_exact(shape, perm, dt):
+    """`x.transpose(perm)` written out, bare and under an elementwise expression with a cast: the tile class must be
+    picked, every element must land where numpy puts it, ragged tile edges and the remaining axes included."""
+    from jaxjs_hip.tuner import tuneHip
+    npdt = {DType.Float16: np.float16, DType.Float32: np.float32, DType.Int32: np.int32, DType.Uint32: np.uint32}[dt]
+    st = ShapeTracker.fromShape(list(shape)).permute(list(perm))
+    x = RNG.integers(0, 100, shape).astype(npdt)
+    want = np.ascontiguousarray(x.transpose(perm))
+    k = mapKernel(list(st.shape), [(dt, st)], lambda v: v)
+    assert tuneHip(k).klass == "map_t"
+    got, ks = device_run(k, [x])
+    assert ks.klass == "map_t"
+    np.testing.assert_array_equal(got.reshape(want.shape), want)
+    if dt in (DType.Float16, DType.Float32):
+        k2 = mapKernel(list(st.shape), [(dt, st)], lambda v: AluExp.cast(DType.Float32, AluExp.add(AluExp.mul(v, AluExp.const(dt, 2.0)), AluExp.const(dt, 1.0))))
+        got, ks = device_run(k2, [x])
+        assert ks.klass == "map_t" and got.dtype == np.float32
+        np.testing.assert_array_equal(got.reshape(want.shape), want.astype(np.float32) * 2 + 1)
+
+
+def test_transposed_view_with_an_offset_and_the_cases_that_stay_plain_maps():
+    from jaxjs_hip.tuner import tuneHip
+    R, C = 300, 500
+    buf = RNG.integers(0, 100, R * C + 7).astype(np.float32)
+    st = ShapeTracker.fromShape([R * C + 7]).shrink([(7, R * C + 7)]).reshape([R, C]).permute([1, 0])
+    k = mapKernel([C, R], [(DType.Float32, st)], lambda v: v)
+    got, ks = device_run(k, [buf])
+    assert ks.klass == "map_t"
+    np.testing.assert_array_equal(got.reshape(C, R), buf[7:].reshape(R, C).T)
+    # two operands, a position-dependent expression, an innermost axis kept in place, a small array: the plain map
+    t2 = ShapeTracker.fromShape([512, 512]).permute([1, 0])
+    assert tuneHip(mapKernel([512, 512], [(DType.Float32, t2), (DType.Float32, ShapeTracker.fromShape([512, 512]))], lambda a, b: AluExp.add(a, b))).klass == "map"
+    assert tuneHip(mapKernel([512, 512], [(DType.Float32, t2)], lambda a: AluExp.add(a, AluExp.cast(DType.Float32, AluVar.gidx)))).klass == "map"
+    assert tuneHip(mapKernel([8, 64, 12, 64], [(DType.Float16, ShapeTracker.fromShape([8, 12, 64, 64]).permute([0, 2, 1, 3]))], lambda a: a)).klass == "map"
+    assert tuneHip(mapKernel([100, 100], [(DType.Float32, ShapeTracker.fromShape([100, 100]).permute([1, 0]))], lambda a: a)).klass == "map"
