@@ -75,7 +75,8 @@ int jh_memcpy_h2d(jh_devptr dst, const void *src, size_t bytes);
  * Device -> host read of `bytes` starting `offset` bytes into `src`.  Backs `Backend.readSync`
  * (src/backend.ts:189): returns after every previously issued kernel has finished.  Reads of
  * 1 MiB and more are pipelined through two pinned 8 MiB buffers that the library allocates at the
- * first such read and keeps until `jh_shutdown`.
+ * first such read and keeps until `jh_shutdown`.  Those two buffers are shared by every call: the
+ * function is not reentrant, call it from one thread at a time (as every other entry point).
  */
 int jh_memcpy_d2h(void *dst, jh_devptr src, size_t offset, size_t bytes);
 
@@ -90,7 +91,8 @@ int jh_memcpy_d2h_async(void *dst, jh_devptr src, size_t offset, size_t bytes, j
 /* Device -> device copy on the stream (used when a routine result is moved into an output slot). */
 int jh_memcpy_d2d(jh_devptr dst, jh_devptr src, size_t bytes);
 
-/* Pinned host memory for asynchronous reads. */
+/* Pinned host memory for asynchronous reads.  `jh_host_free` also works after `jh_shutdown` (a garbage collector
+ * may return a staging buffer late). */
 int jh_host_alloc(size_t bytes, void **out);
 int jh_host_free(void *ptr);
 

@@ -244,7 +244,7 @@ int jh_host_alloc(size_t bytes, void **out) {
 }
 
 int jh_host_free(void *ptr) {
-  JH_NEED_INIT();
+  // No JH_NEED_INIT: a garbage collector may hand pinned memory back after jh_shutdown; hipHostFree needs no stream.
   if (!ptr) return 0;
   JH_HIP(hipHostFree(ptr));
   return 0;

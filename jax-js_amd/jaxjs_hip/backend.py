@@ -69,12 +69,23 @@ class _Prepared:
         # jh_launch's leading arguments per step, converted once
         self.launch_head = [(ctypes.c_void_p(fn), *step.grid, *step.block, step.shared) for step, fn in zip(ks.steps, functions)]
         self.released = False
+        self.pins = 0               # holders that replay this executable without going through dispatch (HIP graphs)
+
+    def rezero(self, dev) -> None:
+        """Put the scratch buffers that every launch must find zero (the ticket counters of an in-launch fold) back to
+        zero.  A launch that fails part-way may leave tickets drawn; without this every later launch of the executable
+        would wait for a last ticket that never comes and leave its output unwritten."""
+        for i in self.ks.zeroed_scratch:
+            dev.sync()
+            dev.h2d(self.scratch[i], bytes(self.ks.scratch_bytes[i]))
 
     def release(self, dev) -> None:
         """Give back what the executable owns on the device: its scratch buffers and its loaded code objects.  Waits for
         the stream first, so launches of it that are still queued finish on live code and memory."""
         if self.released:
             return
+        if self.pins:
+            raise ValueError("executable is pinned by a captured graph that still replays it")
         self.released = True
         dev.sync()
         for ptr in self.scratch:
@@ -136,6 +147,7 @@ class HipBackend:
         self._trace_base = None                 # (event, host ms) pair fixing the profiler hook's time base
         self._trace_pending: list = []          # (TraceInfo, start event, stop event) per traced dispatch
         self._trace_registered = False
+        self.capturing = False                  # a HIP graph is being recorded: no events, no synchronisation
 
     # -- memory -----------------------------------------------------------------------------------
     @staticmethod
@@ -283,16 +295,27 @@ class HipBackend:
         """Keep at most `cacheLimit` prepared executables; the least recently prepared one is released (scratch freed,
         code objects unloaded) when the limit is passed.  Dispatching a released executable raises."""
         self._exes[key] = exe
-        while len(self._exes) > self.cacheLimit:
-            _, old = self._exes.popitem(last=False)
-            old.data.release(self.dev)
+        if len(self._exes) > self.cacheLimit:
+            # oldest first; an executable that a captured graph replays is passed over (the graph launches its code
+            # objects and writes its scratch without coming through dispatch)
+            for k in [k for k, e in self._exes.items() if not e.data.pins and e is not exe][:len(self._exes) - self.cacheLimit]:
+                self._exes.pop(k).data.release(self.dev)
         return exe
 
     def clearCache(self) -> None:
-        """Release every prepared executable (device scratch and loaded code objects)."""
-        while self._exes:
-            _, old = self._exes.popitem(last=False)
-            old.data.release(self.dev)
+        """Release every prepared executable (device scratch and loaded code objects) except those pinned by a captured
+        graph, which stay prepared until the graph is closed."""
+        for k in [k for k, e in self._exes.items() if not e.data.pins]:
+            self._exes.pop(k).data.release(self.dev)
+
+    def pin(self, exe: Executable) -> None:
+        """Keep `exe` prepared until `unpin`: for holders that launch it outside `dispatch` (a captured graph)."""
+        if exe.data.released:
+            raise ValueError("executable was released (evicted from the backend's cache): prepare it again")
+        exe.data.pins += 1
+
+    def unpin(self, exe: Executable) -> None:
+        exe.data.pins -= 1
 
     def prepareKernelSync(self, kernel: Kernel, **tune_opts) -> Executable:
         key = (kernel.key(), self.numerics, tuple(sorted(tune_opts.items())))
@@ -425,7 +448,7 @@ class HipBackend:
         self._trace_pending, self._trace_base = [], None
 
     def dispatch(self, exe: Executable, inputs: Sequence[int], outputs: Sequence[int], repeat: int = 1) -> None:
-        if tracing.isTracing():
+        if tracing.isTracing() and not self.capturing:
             e0 = self._trace_begin()
             try:
                 self._dispatch(exe, inputs, outputs, repeat)
@@ -464,6 +487,8 @@ class HipBackend:
             if self.trace is None and repeat == 1:
                 rc = self.dev.lib.jh_launch(*head, argv)
                 if rc:
+                    if prep.ks.zeroed_scratch and not self.capturing:
+                        prep.rezero(self.dev)
                     check(rc, "jh_launch")
             elif self.trace is not None:
                 e0, e1 = self.dev.event(), self.dev.event()

@@ -107,8 +107,11 @@ def choose_tile(g: dict) -> Dict[str, int]:
             tile.update(SPLITK=4 if tiles(128, 128) * 4 <= CU and g["K"] >= 4096 and g["K"] % 256 == 0 else 2)
             # Folding inside the launch is the direct-to-LDS template's: whole tiles, operands on the 16-byte grid.  Ragged
             # or loose shapes (100 x 14336 x 4096) keep the split and fold in a second launch.
+            # Two slices only: with four, the last workgroup's read-back of four slices behind the acknowledged stores
+            # costs more than a fold launch (128x4096x4096: 16.0 us folded in the launch, 14.4 us with the fold kernel).
             if g["M"] % 128 == 0 and g["N"] % 128 == 0 and not (g.get("a_loose") or g.get("b_loose")):
-                tile.update(FUSEK=1)
+                if tile["SPLITK"] == 2:
+                    tile.update(FUSEK=1)
             else:  # the general template gains from more slices (100 x 14336 x 4096: 41.1 us in two, 34.6 us in four)
                 tile.update(k_split(tiles(128, 128)) or dict(SPLITK=tile["SPLITK"]))
     return tile

@@ -27,6 +27,12 @@ class GraphedProgram:
         steps = [s for s in prog.steps if s.kind == "execute"]
         # compile + load before any capture; a routine step is several launches and outputs, recorded the same way
         exes = [backend.prepareRoutineSync(s.routine) if s.routine is not None else backend.prepareKernelSync(s.kernel) for s in steps]
+        # The graph launches these executables' code objects and writes their scratch buffers without going through
+        # dispatch: pin them so that neither cache eviction nor clearCache() can release them under a replay.
+        self._exes = []
+        for exe in exes:
+            backend.pin(exe)
+            self._exes.append(exe)
         sizes = {s.output: s.size for s in prog.steps if s.kind == "malloc"}
         for s in steps:
             for o in (s.outputs if s.routine is not None else [s.output]):
@@ -41,7 +47,9 @@ class GraphedProgram:
 
         issue()  # one eager pass: every code object is resident before the capture starts
         backend.dev.sync()
+        self._graph = None
         trace, backend.trace = backend.trace, None  # event records are not part of the graph
+        backend.capturing = True                    # nor is the profiler hook's event pair (it synchronises)
         try:
             backend.dev.graph_begin()
             try:
@@ -49,12 +57,16 @@ class GraphedProgram:
             finally:
                 self._graph = backend.dev.graph_end()
         finally:
-            backend.trace = trace
+            backend.trace, backend.capturing = trace, False
         self.outputs = [self._slots[o] for o in prog.outputs]
         self.kernels = len(steps)
 
     def launch(self) -> None:
         """Queue one replay of the whole program (asynchronous, in order with everything else)."""
+        if self._graph is None:
+            raise ValueError("the graphed program was closed")
+        if any(exe.data.released for exe in self._exes):
+            raise ValueError("an executable of this graph was released: capture the program again")
         self.backend.dev.graph_launch(self._graph)
 
     def close(self) -> None:
@@ -62,6 +74,9 @@ class GraphedProgram:
             self.backend.dev.sync()
             self.backend.dev.graph_destroy(self._graph)
             self._graph = None
+            for exe in self._exes:
+                self.backend.unpin(exe)
+            self._exes = []
             for s in self._owned:
                 self.backend.decRef(s)
             self._owned = []

@@ -9,6 +9,7 @@ from __future__ import annotations
 import ctypes
 import hashlib
 import os
+import threading
 
 import numpy as np
 from typing import List, Optional, Sequence, Tuple
@@ -166,7 +167,7 @@ def compile_source(source: str, name: str = "kernel.hip", options: Optional[Sequ
     if use_cache:
         try:
             os.makedirs(CACHE_DIR, exist_ok=True)
-            tmp = path + f".tmp{os.getpid()}"
+            tmp = path + f".tmp{os.getpid()}.{threading.get_ident()}"  # compilations run on several threads
             with open(tmp, "wb") as f:
                 f.write(blob)
             os.replace(tmp, path)

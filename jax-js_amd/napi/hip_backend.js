@@ -116,8 +116,13 @@ class HipBackend {
             return;
           }
           addon.eventDestroy(pending.event);
+          pending.event = undefined;
           resolve(pending.data);
         } catch (e) {
+          if (pending.event !== undefined) {
+            try { addon.eventDestroy(pending.event); } catch (_) { /* the first error is the one to report */ }
+            pending.event = undefined;
+          }
           reject(e);
         }
       };

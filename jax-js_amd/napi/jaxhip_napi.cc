@@ -163,6 +163,18 @@ napi_value D2H(napi_env env, napi_callback_info info) {  // d2h(src, offset, byt
   return out;
 }
 
+napi_value D2D(napi_env env, napi_callback_info info) {  // d2d(dst, src, bytes): copy on the stream, in dispatch order
+  Args a(env, info);
+  uint64_t dst, src, bytes;
+  if (a.argc < 3 || !get_u64(env, a.argv[0], &dst) || !get_u64(env, a.argv[1], &src) || !get_u64(env, a.argv[2], &bytes)) {
+    napi_throw_type_error(env, nullptr, "d2d(dst, src, bytes)"); return nullptr;
+  }
+  if (bytes) JH_OK(jh_memcpy_d2d((jh_devptr)(uintptr_t)dst, (jh_devptr)(uintptr_t)src, (size_t)bytes));
+  return nullptr;
+}
+
+// Runs when the collector drops the buffer, possibly after shutdown() or at process exit: jh_host_free needs no
+// initialised runtime and its status is ignored here (there is nobody to report it to).
 void free_pinned(napi_env, void* data, void*) {  // finalizer of the array buffers d2hAsync hands out
   if (data) (void)jh_host_free(data);
 }
@@ -393,6 +405,7 @@ NAPI_MODULE_INIT() {
       {"eventRecord", EventRecord}, {"eventQuery", EventQuery}, {"eventElapsedMs", EventElapsed},
       {"eventDestroy", EventDestroy}, {"graphBegin", GraphBegin}, {"graphEnd", GraphEnd}, {"graphLaunch", GraphLaunch},
       {"graphDestroy", GraphDestroy}, {"abiVersion", AbiVersion}, {"d2hAsync", D2HAsync}, {"compilerVersion", CompilerVersion},
+      {"d2d", D2D},
   };
   for (const auto& e : table) {
     napi_value fn;

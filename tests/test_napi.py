@@ -24,7 +24,7 @@ needs_node = pytest.mark.skipif(NODE is None or not os.path.exists(os.path.join(
 
 EXPORTS = ["init", "shutdown", "deviceInfo", "malloc", "free", "h2d", "d2h", "compile", "moduleLoad", "moduleUnload",
            "moduleFunction", "launch", "sync", "eventCreate", "eventRecord", "eventQuery", "eventElapsedMs", "eventDestroy",
-           "graphBegin", "graphEnd", "graphLaunch", "graphDestroy", "abiVersion", "d2hAsync", "compilerVersion"]
+           "graphBegin", "graphEnd", "graphLaunch", "graphDestroy", "abiVersion", "d2hAsync", "compilerVersion", "d2d"]
 
 
 @needs_node
