@@ -92,6 +92,13 @@ def _params(used: List[Optional[DType]], out_t: str, out_name: str = "out") -> T
     return ", ".join(parts), names
 
 
+def _in_params(used: List[Optional[DType]]) -> Tuple[str, str]:
+    """The input pointers as a parameter list and as the matching argument list (for a generated loader function)."""
+    names = [f"in{i}" for i in range(len(used))]
+    return ("".join(f"const {STORAGE_CTYPE[d or DType.Float32]}* __restrict__ {n}, " for d, n in zip(used, names)),
+            "".join(f"{n}, " for n in names))
+
+
 def _reduce_text(op: AluOp, dtype: DType) -> str:
     ct = CTYPE[dtype]
     if dtype == DType.Bool:
@@ -131,9 +138,9 @@ class _Body:
             idx = strip_parens(cg.run(n.src[0]))
             st = STORAGE_CTYPE[n.dtype]
             ptr = self.args[n.arg[0]]
-            if self.classes[id(n)] in ("vector", "vector_u"):
+            if self.classes[id(n)] in ("vector", "vector_u", "vector_nt"):
                 var = f"v{self.tag}{k}"
-                load = "jh_vload" if self.classes[id(n)] == "vector" else "jh_vload_u"
+                load = {"vector": "jh_vload", "vector_u": "jh_vload_u", "vector_nt": "jh_vload_nt"}[self.classes[id(n)]]
                 cg.emit(f"const jh_pack<{st}, {self.V}> {var} = {load}<{st}, {self.V}>({ptr} + ({idx}));")
                 loads[id(n)] = f"{var}.v[lane]"
             else:
@@ -142,12 +149,42 @@ class _Body:
                 loads[id(n)] = var
         return "\n".join(cg.take_lines()), loads
 
+    def batched(self, holder: str = "Lc") -> Tuple[str, str, Dict[int, str]]:
+        """The hoisted loads as a value type: (field declarations of a struct, body of a function that performs the
+        loads at `lane_base` and returns the struct, the names under which the per-lane body finds them in an instance
+        called `holder`).  A template fills an array of such structs first and consumes it afterwards, which is what
+        puts several loads per lane in flight: left to itself the compiler issues a load, waits for it and folds it into
+        the accumulator chain before it issues the next."""
+        text, loads = self.hoisted()
+        fields, names = [], []
+        nodes = [n for n in self.exp.collect(lambda x: x.op == AluOp.GlobalIndex) if id(n) in self.classes]
+        out: Dict[int, str] = {}
+        for n in nodes:
+            ref = loads[id(n)]
+            var = ref.split(".")[0]
+            st = STORAGE_CTYPE[n.dtype]
+            if var not in names:
+                names.append(var)
+                fields.append(f"jh_pack<{st}, {self.V}> {var};" if ref.endswith(".v[lane]") else f"{st} {var};")
+            out[id(n)] = f"{holder}.{ref}"
+        body = text + ("\n" if text else "") + self.indent + "return jh_loads{" + ", ".join(names) + "};"
+        return " ".join(fields), body, out
+
     def lanes(self, loads: Dict[int, str]) -> Tuple[str, str]:
         cg = HipExpCodegen(self.args, self.names, self.indent + "  ", prefix=f"l{self.tag}", numerics=self.numerics)
         cg.loads = loads
         cg.countReferences(self.exp)
         value = strip_parens(cg.run(self.exp))
         return "\n".join(cg.take_lines()), value
+
+    def lanes_of(self, loads: Dict[int, str], exps: List[AluExp]) -> Tuple[str, List[str]]:
+        """`lanes` for several expressions that share one statement list (the two factors of a product)."""
+        cg = HipExpCodegen(self.args, self.names, self.indent + "  ", prefix=f"l{self.tag}", numerics=self.numerics)
+        cg.loads = loads
+        for e in exps:
+            cg.countReferences(e)
+        values = [strip_parens(cg.run(e)) for e in exps]
+        return "\n".join(cg.take_lines()), values
 
     def scalar(self, indent: Optional[str] = None, prefix: str = "s") -> Tuple[str, str]:
         cg = HipExpCodegen(self.args, self.names, indent or self.indent, prefix=f"{prefix}{self.tag}",
@@ -241,6 +278,36 @@ def _gen_map_transposed(kernel: Kernel, t: TuneResult, numerics: str, name: str)
     return KernelSource([src], [step], [], "map_t", _min_bytes(t.exp), dict(tile=64, blocks=blocks, j=j, shape=shape))
 
 
+def _exact_product(exp: AluExp, re: Reduction) -> Optional[Tuple[AluExp, AluExp]]:
+    """The two float16 factors when a float32 sum adds up products of float16 values widened to float32.  Such a
+    product is exact in float32 (11-bit significands, exponents far inside the range), so `fma(a, b, acc)` rounds once,
+    exactly where `acc + a * b` rounds: the same bits from one instruction (v_fma_mix_f32 converts both halves on the
+    way in) instead of two conversions, a multiply and an add."""
+    if re.op != AluOp.Add or re.dtype != DType.Float32 or exp.dtype != DType.Float32:
+        return None
+
+    def widened(e: AluExp) -> Optional[AluExp]:
+        return e.src[0] if e.op == AluOp.Cast and e.dtype == DType.Float32 and e.src[0].dtype == DType.Float16 else None
+
+    if exp.op == AluOp.Mul:
+        a, b = widened(exp.src[0]), widened(exp.src[1])
+        if a is not None and b is not None:
+            return a, b
+    if exp.op == AluOp.Cast and exp.src[0].op == AluOp.Mul and exp.src[0].dtype == DType.Float16:
+        return exp.src[0].src[0], exp.src[0].src[1]  # multiplied in float32 by convention (see codegen, Cast of a product)
+    return None
+
+
+def _lane_accumulate(body: "_Body", loads: Dict[int, str], exp: AluExp, re: Reduction, acc_t: str, acc: str) -> Tuple[str, str]:
+    """(statements, expression for the accumulator's new value) of one lane's step of the fold."""
+    pair = _exact_product(exp, re)
+    if pair is not None:
+        text, (a, b) = body.lanes_of(loads, list(pair))
+        return text, f"__builtin_fmaf((float)({a}), (float)({b}), {acc})"
+    text, value = body.lanes(loads)
+    return text, f"JH_REDUCE({acc}, ({acc_t})({value}))"
+
+
 def _partial_pitch(size: int, V: int) -> int:
     """Row pitch of the slice-major partial buffer: the vector stores of each slice must stay aligned."""
     return -(-size // max(V, 1)) * max(V, 1)
@@ -260,7 +327,7 @@ def _gen_reduce(kernel: Kernel, t: TuneResult, numerics: str, name: str, row: bo
     ident = const_literal(re.dtype, re.identity)
 
     if split > 1:
-        unit = T * V if row else T
+        unit = T * V if row else T * p.get("unroll", 1)  # column class: whole batches of loads per row slot
         slice_len = -(-R // split)
         slice_len = -(-slice_len // unit) * unit
         split = -(-R // slice_len)
@@ -271,23 +338,26 @@ def _gen_reduce(kernel: Kernel, t: TuneResult, numerics: str, name: str, row: bo
     params, args = _params(used, acc_t if split > 1 else out_t, "partial" if split > 1 else "out")
 
     if row:
-        body = _Body(t.exp, args, IDENT, "ridx", "r0", V, t.vector_loads, numerics, "        ")
-        hoisted, loads = body.hoisted()
-        lane_body, lane_value = body.lanes(loads)
+        body = _Body(t.exp, args, IDENT, "ridx", "r0", V, t.vector_loads, numerics, "  ")
+        load_fields, hoisted, loads = body.batched()
+        body.indent = "          "
+        lane_body, lane_value = _lane_accumulate(body, loads, t.exp, re, acc_t, "acc")
         scalar_body, scalar_value = body.scalar("        ")
         epi = _Body(t.epilogue, args, {"gidx": "gidx", "acc": "acc"}, "gidx", "gidx", 1, {}, numerics, "      ", "e")
         epi_body, epi_value = epi.scalar("      ", "e") if split == 1 else ("", "0")
         src = _prelude(numerics) + fill(template("reduce_row.hip.inc"), dict(
             SIZE=size, R=R, V=V, T=T, BLOCK=p["block"], ROWS=p["rows"], SPLIT=split, SLICE=slice_len,
-            REDUCE=_reduce_text(re.op, re.dtype), NAME=name, PARAMS=params, ACC_T=acc_t, OUT_T=out_t,
-            IDENTITY=ident, VECTOR_LOADS=hoisted, LANE_BODY=lane_body, LANE_VALUE=lane_value,
+            UNROLL=p.get("unroll", 4), REDUCE=_reduce_text(re.op, re.dtype), NAME=name, PARAMS=params, ACC_T=acc_t, OUT_T=out_t,
+            LOAD_FIELDS=load_fields, LOAD_PARAMS=_in_params(used)[0], LOAD_ARGS=_in_params(used)[1],
+            IDENTITY=ident, VECTOR_LOADS=hoisted, LANE_BODY=lane_body, LANE_ACCUM=lane_value,
             SCALAR_BODY=scalar_body, SCALAR_VALUE=scalar_value, EPILOGUE_BODY=epi_body, EPILOGUE_VALUE=epi_value))
         grid_x = p["grid"]
         block = p["block"]
     else:
-        body = _Body(t.exp, args, IDENT, "gidx", "g0", V, t.vector_loads, numerics, "        ")
-        hoisted, loads = body.hoisted()
-        lane_body, lane_value = body.lanes(loads)
+        body = _Body(t.exp, args, IDENT, "gidx", "g0", V, t.vector_loads, numerics, "  ")
+        load_fields, hoisted, loads = body.batched()
+        body.indent = "          "
+        lane_body, lane_value = _lane_accumulate(body, loads, t.exp, re, acc_t, "acc[lane]")
         scalar_body, scalar_value = body.scalar("      ")
         epi = _Body(t.epilogue, args, {"gidx": "gidx", "acc": "accv"}, "gidx", "g0", V, t.epi_vector_loads,
                     numerics, "      ", "e")
@@ -301,8 +371,9 @@ def _gen_reduce(kernel: Kernel, t: TuneResult, numerics: str, name: str, row: bo
         src = _prelude(numerics) + fill(template("reduce_col.hip.inc"), dict(
             SIZE=size, R=R, V=V, T=T, LX=p["lx"], SPLIT=split, SLICE=slice_len, PITCH=_partial_pitch(size, V),
             UNROLL=p.get("unroll", 4), INTERLEAVE=p.get("interleave", 0),
+            LOAD_FIELDS=load_fields, LOAD_PARAMS=_in_params(used)[0], LOAD_ARGS=_in_params(used)[1],
             REDUCE=_reduce_text(re.op, re.dtype), NAME=name, PARAMS=params, ACC_T=acc_t, OUT_T=out_t,
-            IDENTITY=ident, VECTOR_LOADS=hoisted, LANE_BODY=lane_body, LANE_VALUE=lane_value,
+            IDENTITY=ident, VECTOR_LOADS=hoisted, LANE_BODY=lane_body, LANE_ACCUM=lane_value,
             SCALAR_BODY=scalar_body, SCALAR_VALUE=scalar_value,
             EPI_VECTOR_LOADS=epi_hoisted, EPILOGUE_BODY=epi_body, EPILOGUE_VALUE=epi_value,
             TAIL_EPILOGUE_BODY=tail_body, TAIL_EPILOGUE_VALUE=tail_value))

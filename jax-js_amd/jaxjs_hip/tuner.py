@@ -435,7 +435,7 @@ def match_transposed_map(kernel: Kernel) -> Optional[dict]:
 
 def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True,
             gemm_tile: Optional[tuple] = None, col_strip: Optional[tuple] = None,
-            row_lanes: Optional[int] = None) -> TuneResult:
+            row_lanes: Optional[int] = None, row_unroll: Optional[int] = None, row_nt: Optional[int] = None, col_nt: Optional[int] = None) -> TuneResult:
     """Pick the kernel class and its parameters for one Kernel on MI355X."""
     t = tuneNullopt(kernel)
     re = kernel.reduction
@@ -507,8 +507,23 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
                 want = (CU_COUNT * 1024) // max(lanes_busy, 1)
                 split = max(1, min(want, R // (T * V * 8), 1024))
         t.klass = "reduce_row"
-        t.vector_loads = along_r if V > 1 else {}
-        t.params = dict(V=V, T=T, block=block, rows=rows, split=split)
+        t.vector_loads = dict(along_r) if V > 1 else {}
+        # A stream that this launch reads once (about one element per (output, reduce index) pair: the matrix of a
+        # matvec, the rows of a row reduction) is loaded with the nontemporal hint, so that it does not displace the
+        # operands every row reuses from L2.
+        if row_nt is None or row_nt:
+            for node in loads:
+                if t.vector_loads.get(id(node)) == "vector" and node.arg[1] * 2 >= size * R and size * R >= (1 << 22):
+                    t.vector_loads[id(node)] = "vector_nt"
+        # All of a lane's vector loads of a row are issued before the first is consumed when the row is short enough
+        # (at most 16 per lane); longer rows go four at a time.
+        trips = R // (T * V) if split == 1 else 0
+        nvec = max(1, len(t.vector_loads))
+        unroll = trips if 1 <= trips <= 16 else 4
+        unroll = max(1, min(unroll, 32 // nvec))  # a batch holds unroll x nvec x 4 registers per lane
+        if row_unroll:
+            unroll = int(row_unroll)
+        t.params = dict(V=V, T=T, block=block, rows=rows, split=split, unroll=unroll)
         nrb = (size + rows - 1) // rows
         t.params["grid"] = _grid_for(nrb)
         return t
@@ -527,13 +542,18 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
     if allow_split and groups * T < CU_COUNT * 512 and R // T >= 64:
         want = (CU_COUNT * 1024) // max(groups * T, 1)
         split = max(1, min(want, R // (T * 16), 1024))
-    unroll, interleave = 4, 0
-    # Few column groups but a long fold: instead of two launches (slices + fold), give each block a strip
-    # only one 128-byte line wide and ALL of the reduce axis -- 1024 lanes as 8 column lanes x 128 row slots,
-    # 8 independent vector loads in flight per lane.  Enough strips for half the CUs already saturates HBM.
-    # (Not when the rows start off the vector grid: a strip then straddles two lines in every row, and the neighbouring
-    # strip, on another CU, fetches both of them again -- 35 us against 17 for the aligned [4096, 11008] float16 sum.)
-    if split > 1 and V > 1 and (col_strip or "vector_u" not in along_g.values()):
+    # Row loads a lane issues before it consumes the first (reduce_col.hip.inc fills a batch, then folds it).
+    nvec_g = max(1, sum(1 for c in along_g.values() if c.startswith("vector")))
+    unroll, interleave = (8 if nvec_g <= 2 else 4), 0
+    if split > 1 and V > 1:
+        # Slices over blocks: a lane keeps 16 of its row loads in flight (8 when the expression reads more than two
+        # vector streams), and slices are whole batches long (kernelgen rounds them), so no batch is ragged.
+        unroll = 16 if nvec_g <= 2 else 8
+    if split > 1 and V > 1 and col_strip:
+        # Tuning override, kept for measurements: strips of `lanes` x 16 bytes handled by blocks of `block` threads.  The
+        # default above -- 1 KiB strips, 4 row slots per block, the rows cut until the launch has about three blocks per
+        # CU, partial sums folded by a second launch -- measured 16.0-16.3 us on the transposed float16 matvec
+        # [4096, 11008] against 16.9 us for one launch of 172 blocks that each own a 128-byte strip and all rows.
         lx_line = 8  # 8 lanes x 16 bytes = one 128-byte line per row
         blk = 1024
         rows_split = 1
@@ -542,10 +562,14 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
             rows_split = col_strip[3] if len(col_strip) > 3 else 1
             interleave = col_strip[4] if len(col_strip) > 4 else 0
         strips = -(-groups // lx_line)
-        if strips >= CU_COUNT // 2 and R // (blk // lx_line) >= 8:
+        if (strips >= CU_COUNT // 2 or (col_strip and strips * rows_split >= CU_COUNT // 2)) and R // (blk // lx_line) >= 8:
             lx, T, split, unroll = lx_line, blk // lx_line, rows_split, (unroll if col_strip else 8)
     t.klass = "reduce_col"
-    t.vector_loads = along_g if V > 1 else {}
+    t.vector_loads = dict(along_g) if V > 1 else {}
+    if col_nt is None or col_nt:  # a stream read once by this launch: nontemporal, as in the row class
+        for node in loads:
+            if t.vector_loads.get(id(node)) == "vector" and node.arg[1] * 2 >= size * R and size * R >= (1 << 22):
+                t.vector_loads[id(node)] = "vector_nt"
     t.params = dict(V=V, T=T, lx=lx, block=lx * T, split=split, unroll=unroll, interleave=interleave)
     # The cap on the grid is meant for 256-thread blocks; blocks of one wave (no split of the fold over row slots) get
     # proportionally more of them, or a short fold over many outputs (a depthwise convolution: 6.4 M outputs of 9 terms)
