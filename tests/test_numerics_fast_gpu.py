@@ -124,7 +124,7 @@ CASES = [
     ("reduce_col", "reduce_col", reduceKernel([4096, 64], [(DType.Int32, ShapeTracker.fromShape([64, 4096]).permute([1, 0]))], lambda x: x, AluOp.Add), DType.Int32, 0),
     ("fold", "reduce_row+fold", reduceKernel([1, 1 << 22], [(F32, ShapeTracker.fromShape([1, 1 << 22]))], lambda x: x, AluOp.Add), F32, 1e-4),
     ("matvec", "reduce_row", matvecKernel(1024, 512, DType.Float16), DType.Float16, 1e-2),
-    ("matvec_t", "reduce_col", matvecKernel(11008, 2048, DType.Float16, w_transposed=True), DType.Float16, 1e-2),
+    ("matvec_t", "reduce_col+fold", matvecKernel(11008, 2048, DType.Float16, w_transposed=True), DType.Float16, 1e-2),
     ("gemm_dlds", "gemm", matmulKernel(256, 256, 128, DType.Float16), DType.Float16, 1e-2),
     ("gemm_dlds_ring", "gemm", matmulKernel(256, 256, 256, DType.Float16, b_transposed=True), DType.Float16, 1e-2),
     ("gemm_ragged", "gemm", matmulKernel(100, 72, 40, DType.Float16), DType.Float16, 1e-2),
