@@ -9,34 +9,41 @@ from oracle import oracle
 
 WARM_ONLY = os.environ.get("JAXHIP_WARM") == "1"  # compile every kernel into the on-disk cache, run nothing
 
-_backend = None
+_backends = {}
+NUMERICS = "wasm"  # the mode `backend()` hands out; the `numerics_mode` fixture of a test module switches it
+
+
+def set_numerics(mode):
+    global NUMERICS
+    NUMERICS = mode
 
 
 def backend():
-    """The backend the parity tests run on: Wasm-faithful numerics, so that f32 maps can be held to 2 ulp of the
-    checker.  (The backend's default, "fast", is covered by `fast_backend()` under the rel 1e-5 bar.)"""
-    global _backend
-    if _backend is None:
+    """The backend the parity tests run on.  By default Wasm-faithful numerics, so that f32 maps can be held to 2 ulp of
+    the checker; test modules that carry the `numerics_mode` fixture run a second time on the backend's own default,
+    "fast" (exp and reciprocal on hardware instructions, within rel 1e-5 of the checker)."""
+    if "wasm" not in _backends:
         from jaxjs_hip import getBackend, init
 
         init("hip", numerics="wasm")
-        _backend = getBackend("hip")
-    return _backend
+        _backends["wasm"] = getBackend("hip")
+    if NUMERICS not in _backends:
+        from jaxjs_hip.backend import HipBackend
 
-
-_fast = None
+        _backends[NUMERICS] = HipBackend(numerics=NUMERICS)
+        assert _backends[NUMERICS].numerics == NUMERICS
+    return _backends[NUMERICS]
 
 
 def fast_backend():
     """A second backend object on the same device with the default ("fast") numerics."""
-    global _fast
-    if _fast is None:
-        from jaxjs_hip.backend import HipBackend
+    from jaxjs_hip.backend import HipBackend
 
-        backend()
-        _fast = HipBackend()
-        assert _fast.numerics == "fast"
-    return _fast
+    backend()
+    if "fast" not in _backends:
+        _backends["fast"] = HipBackend()
+        assert _backends["fast"].numerics == "fast"
+    return _backends["fast"]
 
 
 def device_run(kernel, inputs, **tune_opts):
@@ -45,7 +52,7 @@ def device_run(kernel, inputs, **tune_opts):
         from jaxjs_hip.kernelgen import generate
         from jaxjs_hip.runtime import compile_source
 
-        for src in generate(kernel, **tune_opts).sources:
+        for src in generate(kernel, NUMERICS, **tune_opts).sources:
             compile_source(src)
         pytest.skip("warm-up run: compiled only")
     be = backend()
