@@ -121,6 +121,47 @@ def pool(st: ShapeTracker, ks: Sequence[int], strides=1, dilation=1) -> ShapeTra
     return st.permute(list(range(nn)) + [nn + 2 * j + 1 for j in range(nk)] + [nn + 2 * j for j in range(nk)])
 
 
+def poolTranspose(st: ShapeTracker, inShape: Sequence[int], ks: Sequence[int], strides=1, dilation=1) -> ShapeTracker:
+    """The adjoint view of `pool` (src/frontend/convolution.ts:274-378): re-view a pooled array `[..., *out, *ks]` as
+    `[*inShape, *repeats]` so that summing the trailing axes adds up, for every input position, the pooled elements
+    that were read from it (masked where there is none).  This is the Kernel a transform emits for the cotangent of a
+    window reduction or convolution input; nothing in the forward library traces it."""
+    ks = list(ks)
+    if not ks:
+        return st
+    nk = len(ks)
+    s_ = [strides] * nk if isinstance(strides, int) else list(strides)
+    d_ = [dilation] * nk if isinstance(dilation, int) else list(dilation)
+    noop = list(inShape[:-nk])
+    nn = len(noop)
+    i_ = list(inShape[-nk:])
+    o_ = [-(-(i - d * (k - 1)) // s) for i, d, k, s in zip(i_, d_, ks, s_)]
+
+    if all(d == 1 for d in d_) and all(k <= s for k, s in zip(ks, s_)):
+        # Non-overlapping windows: interleave (o, k) again, pad each k up to its stride, merge, fit to the input extent.
+        st = st.permute(list(range(nn)) + [x for j in range(nk) for x in (nn + j, nn + nk + j)])
+        st = st.pad([(0, 0)] * nn + [pr for s, k in zip(s_, ks) for pr in ((0, 0), (0, s - k))])
+        st = st.reshape(noop + [o * s for o, s in zip(o_, s_)])
+        st = st.padOrShrink([(0, 0)] * nn + [(0, i - o * s) for i, o, s in zip(i_, o_, s_)])
+        return st.reshape(list(st.shape) + [1] * nk)  # the repeat axes the general form has, of extent 1
+
+    if o_ != list(st.shape[nn:nn + nk]):
+        raise ValueError("poolTranspose() called with mismatched output shape")
+    f_ = [1 + int(o * s > i - d * (k - 1)) for o, s, i, d, k in zip(o_, s_, i_, d_, ks)]
+    kidf = list(zip(ks, i_, d_, f_))
+    kos = list(zip(ks, o_, s_))
+    # every step of pool()'s general form, undone in reverse order
+    st = st.permute(list(range(nn)) + [x for j in range(nk) for x in (nn + nk + j, nn + j)])
+    st = st.reshape(noop + [x for k, o, s in kos for x in (k, o, 1)])
+    st = st.pad([(0, 0)] * nn + [pr for s in s_ for pr in ((0, 0), (0, 0), (0, s - 1))])
+    st = st.reshape(noop + [x for k, o, s in kos for x in (k, o * s)])
+    st = st.pad([(0, 0)] * nn + [pr for (k, i, d, f), o, s in zip(kidf, o_, s_) for pr in ((0, 0), (0, i * f + d - o * s))])
+    st = st.reshape(noop + [k * (i * f + d) for k, i, d, f in kidf])
+    st = st.pad([(0, 0)] * nn + [(0, -(-(k * (i * f + d)) // i) * i - k * (i * f + d)) for k, i, d, f in kidf])
+    st = st.reshape(noop + [x for k, i, d, f in kidf for x in (-(-(k * (i * f + d)) // i), i)])
+    return st.permute(list(range(nn)) + [nn + 2 * j + 1 for j in range(nk)] + [nn + 2 * j for j in range(nk)])
+
+
 def applyDilation(st: ShapeTracker, dilation: Sequence[int]) -> ShapeTracker:
     """Insert `s-1` zeros between the elements of the last axes (transposed convolution)."""
     if all(s == 1 for s in dilation):

@@ -28,7 +28,15 @@ def choose_tile(g: dict) -> Dict[str, int]:
         return -(-g["M"] // bm) * -(-g["N"] // bn) * nb
 
     CU = tuner.CU_COUNT
+    # Slices of the k axis at most: 8, or 64 when the axis is very long (k = batch x positions of a filter cotangent:
+    # 100352 against 9 output tiles), where the partial sums stay tiny next to the operands.
+    max_split = 64 if g["K"] >= 32768 else 8
     plain_k = not (g.get("a_gather") or g.get("b_gather")) and g["a_k0"] == g["K"] and g["b_k0"] == g["K"]
+    # A k axis that may be cut over workgroups: one stride per plain operand (a slice is a pointer offset), any gather
+    # operand (a slice is an offset on the k its loader is asked for).
+    # With exactly one gather operand and a short k axis the kernel is a forward convolution, whose stride-1 form has
+    # its own template (image patch in LDS) that takes the whole k axis: those keep one slice.
+    cut_k = g["a_k0"] == g["K"] and g["b_k0"] == g["K"] and (bool(g.get("a_gather")) == bool(g.get("b_gather")) or g["K"] >= 8192)
     if g["dtype"] == DType.Float32:
         # The f32 matrix pipe is 16x slower than the f16 one, so LDS traffic matters little and filling
         # every CU matters most: take the largest tile that still yields two workgroups per CU (the
@@ -49,9 +57,9 @@ def choose_tile(g: dict) -> Dict[str, int]:
             return dict(BM=128, BN=64, BK=bk, SPLITK=split, **(dict(FUSEK=1, WM=4, WN=1) if split > 1 else {}))
         # Fewer than 128 rows or 64 columns: 64x64 tiles, the k axis cut the same way when they are few.
         split = 1
-        while plain_k and tiles(64, 64) * split < 1.5 * CU and split < 8 and g["K"] % (split * 2 * bk) == 0 and g["K"] // (split * 2) >= 256:
+        while cut_k and tiles(64, 64) * split < 1.5 * CU and split < max_split and g["K"] % (split * 2 * bk) == 0 and g["K"] // (split * 2) >= 256:
             split *= 2
-        return dict(BM=64, BN=64, BK=bk, **(dict(SPLITK=split, FUSEK=1) if split > 1 else {}))
+        return dict(BM=64, BN=64, BK=bk, **(dict(SPLITK=split, FUSEK=1 if plain_k else 0) if split > 1 else {}))
     # f16: estimated time = (tiles the busiest CU runs) x (tile area) x (K + fixed per-tile overhead) / efficiency.
     # Efficiencies are measured rates of each tile shape relative to 256x256 on large problems (MI355X):
     # 128x256 0.84, 256x128 0.79, 128x128 0.72 with two workgroups resident per CU (0.64 alone).  The fixed
@@ -60,7 +68,7 @@ def choose_tile(g: dict) -> Dict[str, int]:
     def k_split(count):
         # Fewer workgroups than 1.5 per CU: cut the k axis (partial sums in scratch, fold kernel) while slices stay >= 512 deep.
         split = 1
-        while plain_k and count * split < 1.5 * CU and split < 8 and g["K"] % (split * 2 * 64) == 0 and g["K"] // (split * 2) >= 512:
+        while cut_k and count * split < 1.5 * CU and split < max_split and g["K"] % (split * 2 * 64) == 0 and g["K"] // (split * 2) >= 512:
             split *= 2
         return dict(SPLITK=split) if split > 1 else {}
 
@@ -76,6 +84,13 @@ def choose_tile(g: dict) -> Dict[str, int]:
         # A 128-wide tile would compute and store a half-empty block (attention's probabilities x V, N = head
         # size 64): measured 30 % faster with 128x64 tiles, which is then bound by reading A.
         return dict(BM=128, BN=64, WM=2, WN=2, **k_split(tiles(128, 64)))
+    if (g["K"] <= 128 and g["K"] % 32 == 0 and plain_k and g["M"] % 128 == 0 and g["N"] % 128 == 0 and tiles(128, 128) >= 4 * CU
+            and not (g.get("a_loose") or g.get("b_loose"))):
+        # A k axis of one to four slabs (attention scores: q.k^T over a head size of 64): the launch is bound by writing
+        # C, and a workgroup spends its life in prologue and epilogue.  128x128 tiles with two shallow stages leave
+        # room for four workgroups per CU, so that one's stores overlap another's loads and MFMAs
+        # (96 x 1024 x 1024 x 64: 47.5 us with 256x256 tiles in the deep pipeline, 41.3 us = 5.5 TB/s this way).
+        return dict(BM=128, BN=128, BK=32, STAGES=2, PIPE=0)
     best = None
     for bm, bn, eff, extra in ((256, 256, 1.00, dict()), (128, 256, 0.84, dict(WM=1, WN=4)), (256, 128, 0.79, dict()),
                                 (128, 128, 0.72, dict())):
@@ -114,6 +129,10 @@ def choose_tile(g: dict) -> Dict[str, int]:
                     tile.update(FUSEK=1)
             else:  # the general template gains from more slices (100 x 14336 x 4096: 41.1 us in two, 34.6 us in four)
                 tile.update(k_split(tiles(128, 128)) or dict(SPLITK=tile["SPLITK"]))
+    elif not plain_k and cut_k and per_cu == 1 and tiles(tile["BM"], tile["BN"]) * 2 <= CU:
+        # Gather operands on both sides and a handful of tiles over a long k axis (the filter cotangent of a
+        # convolution: 9 taps x one tile, k = batch x positions): slices over workgroups, folded by a second launch.
+        tile.update(k_split(tiles(tile["BM"], tile["BN"])))
     return tile
 
 
@@ -332,8 +351,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     K_full = g["K"]
     if split > 1:
         vec_k = 8 if g["dtype"] == DType.Float16 else 4
-        if (g.get("a_gather") or g.get("b_gather") or g["a_k0"] != K_full or g["b_k0"] != K_full
-                or K_full % split or (K_full // split) % vec_k):
+        if g["a_k0"] != K_full or g["b_k0"] != K_full or K_full % split or (K_full // split) % vec_k:
             split = 1
     # ... or, with FUSEK (f32 template), folded inside the same launch by the slice that arrives last at the tile's
     # counter: one launch instead of two.
@@ -402,7 +420,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         flat = AluExp.mul(AluExp.special(I32, "row", max(extent, 1)), AluExp.i32(c_stride))
         for k, (size, _sa, _sb, sc) in enumerate(g["batch"]):
             flat = AluExp.add(AluExp.mul(AluExp.special(I32, f"b{k}", size), AluExp.i32(sc)), flat)
-        kvar = AluExp.special(I32, "k", max(g["K"], 1))
+        kvar = AluExp.special(I32, "k", max(K_full, 1))  # the whole axis: a slice's loader is asked for k + its offset
 
         def _retarget_operand(node, flat=flat, kvar=kvar):
             if node.op == AluOp.Special and node.arg[0] == "gidx":
@@ -556,6 +574,10 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     if split > 1:
         lines.append(f"  a_base += (long long)blockIdx.y * {g['K'] * g['a_sk']}ll; b_base += (long long)blockIdx.y * {g['K'] * g['b_sk']}ll;"
                      + ("" if fusek else f" c_base += (long long)blockIdx.y * {pitch}ll;"))
+        lines.append(f"  const int jh_k_off = (int)blockIdx.y * {g['K']};  // a gather loader is asked for k of the whole axis")
+        for d in (gather_calls, gather_slow):
+            for tag in list(d):
+                d[tag] = d[tag].replace("(row, k, ", "(row, k + jh_k_off, ")
 
     tmpl = "gemm_f16.hip.inc" if g["dtype"] == DType.Float16 else "gemm_f32.hip.inc"
     fBK = int(tile.get("BK", 16)) if g["dtype"] == DType.Float32 else 0  # slab depth of the f32 template

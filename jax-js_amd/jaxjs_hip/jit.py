@@ -13,7 +13,7 @@ Kernel sequence to the `hip` backend that `jit()` would:
 
 Only the primitives whose lowering is a fused Kernel are covered (elementwise, Compare, Where,
 Reduce, Dot, Conv, Pool, Transpose/Reshape/Broadcast/Flip/Shrink/Pad); routines, Gather, RandomBits,
-PoolTranspose and Concatenate/Split are not traced here.
+Concatenate/Split are not traced here; PoolTranspose, which only transforms emit, can be bound by hand.
 """
 
 from __future__ import annotations
@@ -23,7 +23,7 @@ from dataclasses import dataclass, field
 from typing import Any, Callable, Dict, List, Optional, Sequence, Set, Tuple, Union
 
 from .alu import AluExp, AluOp, AluVar, DType, Kernel, Reduction, byteWidth, isFloatDtype
-from .convolution import ConvParams, checkConvShape, checkPoolShape, pool, prepareConv
+from .convolution import ConvParams, checkConvShape, checkPoolShape, pool, poolTranspose, prepareConv
 from .shape import ShapeTracker, prod, unravelAlu
 
 # ---- abstract values ------------------------------------------------------------------------------
@@ -115,7 +115,7 @@ class JaxprEqn:
 
 
 VIEW_PRIMITIVES = ("Transpose", "Broadcast", "Reshape", "Flip", "Shrink", "Pad")  # src/frontend/jit.ts:905-912
-REDUCE_PRIMITIVES = ("Reduce", "Dot", "Conv")
+REDUCE_PRIMITIVES = ("Reduce", "Dot", "Conv", "PoolTranspose")
 UNARY_FUSABLE = ("Neg", "Reciprocal", "Floor", "Ceil", "StopGradient", "Cast", "Bitcast", "Sin", "Cos", "Asin", "Atan",
                  "Exp", "Log", "Erf", "Erfc", "Sqrt")
 BINARY_FUSABLE = ("Add", "Mul", "Idiv", "Mod", "Min", "Max", "BitCombine", "BitShift")
@@ -437,6 +437,11 @@ def _out_aval(prim: str, avals: List[ShapedArray], params: Dict[str, Any]) -> Sh
         return ShapedArray(tuple(checkConvShape(avals[0].shape, avals[1].shape, params["conv"])), c.dtype, c.weak)
     if prim == "Pool":
         return ShapedArray(tuple(checkPoolShape(avals[0].shape, params["window"], params["strides"])), avals[0].dtype, avals[0].weak)
+    if prim == "PoolTranspose":  # src/frontend/jaxpr.ts:867-882
+        want = checkPoolShape(params["inShape"], params["window"], params["strides"])
+        if list(avals[0].shape) != list(want):
+            raise ValueError(f"poolTranspose() of shape {list(avals[0].shape)}: a pool of {list(params['inShape'])} has shape {want}")
+        return ShapedArray(tuple(params["inShape"]), avals[0].dtype, avals[0].weak)
     if prim == "Transpose":
         return ShapedArray(tuple(avals[0].shape[p] for p in params["perm"]), avals[0].dtype, avals[0].weak)
     if prim in ("Reshape", "Broadcast"):
@@ -846,6 +851,22 @@ def _conv_rule(exps, avals, params):
     return _dot_rule([a, b], [as_, bs_], {})
 
 
+def _pool_transpose_rule(exps, avals, params):
+    """src/frontend/jit.ts:623-638: the adjoint pool view with its repeat axes merged, summed over them."""
+    inShape = list(params["inShape"])
+    stX = poolTranspose(ShapeTracker.fromShape(list(avals[0].shape)), inShape, list(params["window"]), list(params["strides"]))
+    stX = stX.reshape(inShape + [prod(list(stX.shape[len(inShape):]))])
+    a = reshapeViews(exps[0], lambda st: st.compose(stX), True)
+    return [a], Reduction(a.dtype, AluOp.Add, stX.shape[-1])
+
+
+def poolTransposeWindows(ct, inShape, window, strides):
+    """The PoolTranspose primitive (src/frontend/core.ts:112-116): `[..., *out, *window] -> inShape`, every pooled element
+    added back onto the input position it was read from.  Only transforms bind it in the reference (the transpose rule
+    of Pool, src/frontend/linearize.ts:755-762); it is here so that those Kernels can be presented to the backend."""
+    return bind1("PoolTranspose", [ct], dict(inShape=tuple(inShape), window=tuple(window), strides=tuple(strides)))
+
+
 def _flip_rule(st, params):
     arg = [False] * len(st.shape)
     for ax in params["axis"]:
@@ -959,6 +980,7 @@ JIT_RULES: Dict[str, Callable] = {
     "Dot": _dot_rule,
     "Conv": _conv_rule,
     "Pool": _reshape_rule(lambda st, p: pool(st, list(p["window"]), list(p["strides"]))),
+    "PoolTranspose": _pool_transpose_rule,
     "Compare": _broadcasted(lambda e, p: aluCompare(e[0], e[1], p["op"])),
     "Where": _broadcasted(lambda e, p: AluExp.where(e[0], e[1], e[2]), skipCastIdx=(0,)),
     "Transpose": _reshape_rule(lambda st, p: st.permute(p["perm"])),

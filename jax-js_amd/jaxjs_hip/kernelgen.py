@@ -236,12 +236,14 @@ def _gen_map(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     used = _used_args(kernel.nargs, t.exp)
     out_t = STORAGE_CTYPE[kernel.dtype]
     params, args = _params(used, out_t)
-    body = _Body(t.exp, args, IDENT, "gidx", "g0", V, t.vector_loads, numerics, "    ")
-    hoisted, loads = body.hoisted()
+    body = _Body(t.exp, args, IDENT, "gidx", "g0", V, t.vector_loads, numerics, "  ")
+    load_fields, hoisted, loads = body.batched()
+    body.indent = "        "
     lane_body, lane_value = body.lanes(loads)
     scalar_body, scalar_value = body.scalar("    ")
     src = _prelude(numerics) + fill(template("map.hip.inc"), dict(
-        SIZE=kernel.size, V=V, BLOCK=block, NAME=name, PARAMS=params, OUT_T=out_t,
+        SIZE=kernel.size, V=V, BLOCK=block, UNROLL=t.params.get("unroll", 1), NT_STORE=t.params.get("nt_store", 0), NAME=name, PARAMS=params, OUT_T=out_t,
+        LOAD_FIELDS=load_fields, LOAD_PARAMS=_in_params(used)[0], LOAD_ARGS=_in_params(used)[1],
         VECTOR_LOADS=hoisted, LANE_BODY=lane_body, LANE_VALUE=lane_value,
         SCALAR_BODY=scalar_body, SCALAR_VALUE=scalar_value))
     step = LaunchStep(name, (grid, 1, 1), (block, 1, 1), 0,

@@ -46,6 +46,7 @@ def set_compute_units(n: int) -> None:
 # and more (measured: copy, a+b, exp(x)/2 in f16 and f32; unrolling the strided loop made it slower).
 MAP_GRID_BLOCKS = 1 << 22
 MAP_BLOCK = 256
+MAP_NT_BYTES = 320 << 20  # streams of a map beyond this: nontemporal loads and stores
 GEMM_ENABLED = True
 
 
@@ -307,8 +308,9 @@ def match_gemm(kernel: Kernel) -> Optional[dict]:
     if da is None or db is None:
         return None
     (va, ka0, ka1, ga), (vb, kb0, kb1, gb) = da, db
-    if ga and gb:
-        return None  # at least one operand streams through vector loads
+    # (Both operands may be gather operands: the cotangent of a convolution's activations contracts a patch view of the
+    # output cotangent with the filter read through a flip and a transpose.  Both tiles are then built by element
+    # loaders -- slower to fill than vector loads, but the products still run on the matrix cores.)
     if va.shape != vb.shape or len(va.shape) < 1:
         return None
     shape = list(va.shape)
@@ -345,10 +347,17 @@ def match_gemm(kernel: Kernel) -> Optional[dict]:
         merged.append(ax)
     # Several M (or N) axes that do not nest (rows of a transposed activation): keep the innermost as
     # the tile axis and walk the outer ones like batch axes (the other operand's stride there is 0).
-    for role in ("m", "n"):
+    # (For a gather operand, whose strides play no part, the tile axis is the largest of them when the innermost is
+    # short: the filter cotangent of a convolution has rows (channels, ky, kx) with the output channels between the two
+    # -- 64 rows by channel and 9 taps as batch fill an MFMA tile, 9 rows per channel do not.)
+    for role, gathered in (("m", ga), ("n", gb)):
         idx = [i for i, x in enumerate(merged) if x[0] == role]
-        for i in idx[:-1]:
-            merged[i][0] = "batch"
+        keep = idx[-1] if idx else None
+        if gathered and len(idx) > 1 and merged[idx[-1]][1] < 32:
+            keep = max(idx, key=lambda i: (merged[i][1], i))
+        for i in idx:
+            if i != keep:
+                merged[i][0] = "batch"
     ms = [x for x in merged if x[0] == "m"]
     ns = [x for x in merged if x[0] == "n"]
     bs = [x for x in merged if x[0] == "batch"]
@@ -435,7 +444,8 @@ def match_transposed_map(kernel: Kernel) -> Optional[dict]:
 
 def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True,
             gemm_tile: Optional[tuple] = None, col_strip: Optional[tuple] = None,
-            row_lanes: Optional[int] = None, row_unroll: Optional[int] = None, row_nt: Optional[int] = None, col_nt: Optional[int] = None) -> TuneResult:
+            row_lanes: Optional[int] = None, row_unroll: Optional[int] = None, row_nt: Optional[int] = None, col_nt: Optional[int] = None,
+            map_unroll: Optional[int] = None, map_nt: Optional[int] = None) -> TuneResult:
     """Pick the kernel class and its parameters for one Kernel on MI355X."""
     t = tuneNullopt(kernel)
     re = kernel.reduction
@@ -451,8 +461,26 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
         t.klass = "map"
         t.vector_loads = classify_loads(t.exp, "gidx", V)
         groups = max(size // V, 1)
-        blocks = (groups + MAP_BLOCK - 1) // MAP_BLOCK
-        t.params = dict(V=V, block=MAP_BLOCK, grid=max(1, min(blocks, MAP_GRID_BLOCKS)))
+        # Groups per lane (their loads all issued before the first is consumed).  One by default: with a block per 256
+        # groups the resident waves already keep enough loads in flight, and 2-8 groups per lane measured 1-15 % slower
+        # on 50-400 MB streams; the option stays for measurements.
+        unroll = int(map_unroll) if map_unroll else 1
+        blocks = (groups + MAP_BLOCK * unroll - 1) // (MAP_BLOCK * unroll)
+        nt_store = 0
+        # Streams that together exceed the 256 MB memory-side cache are read with the nontemporal hint (float16 copy of
+        # 201 MB: 67 -> 58 us, the softmax maps of a 96 x 1024 x 1024 score tensor 67 -> 56 us; the hint on the stores
+        # adds nothing, and plain stores leave the result in that cache for the next kernel); smaller streams keep
+        # ordinary loads (268 MB of float32 in and out: 37 us against 41 with the hint).
+        if map_nt is None:
+            streamed = kernel.bytes + sum(n.arg[1] * byteWidth(n.dtype) for n in _load_nodes(t.exp) if t.vector_loads.get(id(n)) == "vector")
+            map_nt = 2 if streamed >= MAP_NT_BYTES else 0  # the loads carry the gain; plain stores leave the result cached
+        if map_nt:  # 1: loads and stores, 2: loads only, 3: stores only
+            t.vector_loads = dict(t.vector_loads)
+            for node in _load_nodes(t.exp):
+                if map_nt != 3 and t.vector_loads.get(id(node)) == "vector" and node.arg[1] * 2 >= size and size >= (1 << 22):
+                    t.vector_loads[id(node)] = "vector_nt"
+            nt_store = 1 if size >= (1 << 22) and map_nt != 2 else 0
+        t.params = dict(V=V, block=MAP_BLOCK, unroll=unroll, nt_store=nt_store, grid=max(1, min(blocks, MAP_GRID_BLOCKS)))
         return t
 
     R = re.size

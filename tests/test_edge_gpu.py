@@ -219,6 +219,33 @@ def test_f16_elementwise():
     assert_parity(k, [a], rtol=1e-2, atol=1e-3)
 
 
+@pytest.mark.parametrize("op", [AluOp.Max, AluOp.Min])
+def test_f16_min_max_propagate_nan_and_order_signed_zeros(op):
+    """float16 min / max run on v_min_f16 / v_max_f16 with an unordered select: a NaN on either side gives NaN, -0 sorts
+    below +0, infinities behave -- elementwise, and as a row reduction whose rows hold those values at every lane and
+    batch position (bit patterns compared, so the sign of a zero counts)."""
+    special = np.array([np.nan, 0.0, -0.0, np.inf, -np.inf, 1.5, -1.5, 65504.0, 6e-8], np.float16)
+    a, b = [x.ravel() for x in np.meshgrid(special, special)]
+    pad = 8 * 13 - len(a) % 8
+    a, b = np.concatenate([a, special[:pad]]), np.concatenate([b, special[pad - 1::-1][:pad]])
+    n = len(a)
+    fn = AluExp.max if op == AluOp.Max else AluExp.min
+    got, want, _ = assert_parity(mapKernel([n], [(F16, flat(n)), (F16, flat(n))], lambda x, y: fn(x, y)), [a, b], rtol=0, atol=0)
+    np.testing.assert_array_equal(got.view(np.uint16)[~np.isnan(want)], want.view(np.uint16)[~np.isnan(want)])
+    rows, L = 64, 2048
+    x = RNG.normal(0, 1, (rows, L)).astype(np.float16)
+    x[::2] = np.abs(x[::2]) * (1 if op == AluOp.Min else -1)      # every other row has one sign only ...
+    for r in range(0, rows, 2):
+        x[r, (r * 37) % L] = 0.0 if op == AluOp.Min else -0.0      # ... and one zero of the sign that loses ...
+        x[r, (r * 91 + 5) % L] = -0.0 if op == AluOp.Min else 0.0  # ... and one of the sign that wins
+    x[7, 1000] = np.nan
+    x[9, 3] = np.inf if op == AluOp.Max else -np.inf
+    got, want, _ = assert_parity(reduceKernel([rows, L], [(F16, ShapeTracker.fromShape([rows, L]))], lambda v: v, op), [x], rtol=0, atol=0)
+    assert np.isnan(got[7]) and np.isnan(want[7])
+    np.testing.assert_array_equal(np.delete(got, 7).view(np.uint16), np.delete(want, 7).view(np.uint16))
+    assert got[0].view(np.uint16) == (0x8000 if op == AluOp.Min else 0x0000)
+
+
 @pytest.mark.parametrize("name,fn,ref", [("exp", AluExp.exp, np.exp), ("log", AluExp.log, np.log), ("sin", AluExp.sin, np.sin),
                                          ("cos", AluExp.cos, np.cos), ("atan", AluExp.atan, np.arctan)])
 def test_native_numerics_track_libm(name, fn, ref):
