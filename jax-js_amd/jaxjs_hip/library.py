@@ -382,16 +382,14 @@ def logsumexp(x: Tracer, axis=None, keepdims: bool = False):
 def dotProductAttention(query: Tracer, key: Tracer, value: Tracer, isCausal: bool = False, scale: Optional[float] = None,
                         fused: bool = False):
     """[B,L,N,H] attention with equal query and key/value head counts (nn.ts:478-583).  `fused=True` hands the whole
-    chain to the backend as one `Attention` routine when the shapes fit its kernel (float16, head size 64, L a multiple
-    of 128, S of 64) -- a front-end switch the reference does not have; otherwise the reference's composition is
-    traced."""
+    chain to the backend as one `Attention` routine when the operands fit its kernel (float16, head size 32, 64 or 128;
+    any L and S) -- a front-end switch the reference does not have; otherwise the reference's composition is traced."""
     B, L, N, H = query.shape
     S = key.shape[1]
     if key.shape != value.shape or key.shape[0] != B or key.shape[3] != H or key.shape[2] != N:
         raise ValueError("dotProductAttention: shape mismatch")
     scale = 1 / math.sqrt(H) if scale is None else scale
-    if (fused and H == 64 and L % 128 == 0 and S % 64 == 0
-            and all(t.dtype == DType.Float16 for t in (query, key, value))):
+    if fused and H in (32, 64, 128) and L >= 1 and S >= 1 and all(t.dtype == DType.Float16 for t in (query, key, value)):
         return J.attention(query, key, value, scale, isCausal)
     scores = einsum("BLNH,BSNH->BNLS", query, key).mul(scale)
     if isCausal:

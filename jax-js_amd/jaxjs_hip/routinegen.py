@@ -8,7 +8,7 @@ time, which is what the Backend interface prescribes for a routine a backend lac
   Scatter                                     `scatter.hip.inc`  float32/float16/float64/int32/uint32/bool updates
   TriangularSolve, Cholesky, LU, JacobiEigh   `linalg.hip.inc`   float32/float64/float16 (arithmetic in double, as the reference)
   Fft                                         `fft.hip.inc`      float32/float64/float16
-  Attention (extension, not in the reference) `attention.hip.inc` float16, head size 64
+  Attention (extension, not in the reference) `attention.hip.inc` float16, head size 32 / 64 / 128, any L and S
 """
 
 from __future__ import annotations
@@ -395,8 +395,8 @@ def _gen_sort(routine: Routine, numerics: str) -> Optional[KernelSource]:
 
 
 def _gen_attention(routine: Routine, numerics: str) -> Optional[KernelSource]:
-    """Fused attention over [B, L, N, 64] / [B, S, N, 64] float16 operands (contiguous, or strided views with unit
-    stride along the head dimension)."""
+    """Fused attention over [B, L, N, H] / [B, S, N, H] float16 operands with H = 32, 64 or 128 and any L and S >= 1
+    (contiguous, or strided views with unit stride along the head dimension)."""
     import math
 
     t = routine.type
@@ -407,11 +407,11 @@ def _gen_attention(routine: Routine, numerics: str) -> Optional[KernelSource]:
     if list(ks) != list(vs) or ks[0] != B or ks[2] != N or ks[3] != H:
         raise ValueError(f"attention: shape mismatch q={t.inputShapes[0]} k={ks} v={vs}")
     S = ks[1]
-    if any(d != DType.Float16 for d in t.inputDtypes) or H != 64 or L % 128 != 0 or S % 64 != 0:
-        return None
+    if any(d != DType.Float16 for d in t.inputDtypes) or H not in (32, 64, 128):
+        return None  # the kernel takes float16 and head sizes of one, two or four 32-row MFMA tiles
     if B * N * L == 0:
         return _empty("attention", B=B, L=L, S=S, N=N)
-    if B * N * (L // 128) >= (1 << 31) or max(B * L * N * H, B * S * N * H) >= (1 << 31):
+    if B * N * -(-L // 128) >= (1 << 31) or max(B * L * N * H, B * S * N * H) >= (1 << 31):
         return None
     scale = float(params.get("scale", 1 / math.sqrt(H)))
     # Each operand is a base buffer read through (batch, position, head) strides and an offset: contiguous
@@ -431,9 +431,9 @@ def _gen_attention(routine: Routine, numerics: str) -> Optional[KernelSource]:
             need[i] = v["elements"] * 2
     (qb, ql, qn, qo), (kb, ksp, kn, ko), (vb, vsp, vn, vo) = lay
     src = _prelude(numerics) + fill(template("attention.hip.inc"), dict(
-        B=B, NH=N, L=L, S=S, CAUSAL=1 if params.get("isCausal") else 0, SCALE_LOG2E=repr(scale * math.log2(math.e)),
+        B=B, NH=N, L=L, S=S, H=H, CAUSAL=1 if params.get("isCausal") else 0, SCALE_LOG2E=repr(scale * math.log2(math.e)),
         QB=qb, QL=ql, QN=qn, QOFF=qo, KB=kb, KS=ksp, KN=kn, KOFF=ko, VB=vb, VS=vsp, VN=vn, VOFF=vo,
         OB=L * N * H, OL=N * H, ON=H))
-    blocks = B * N * (L // 128)
+    blocks = B * N * -(-L // 128)
     steps = [LaunchStep("jh_attention", (blocks, 1, 1), (256, 1, 1), 0, [("in", 0), ("in", 1), ("in", 2), ("out", 0)])]
     return KernelSource([src], steps, [], "attention", need, dict(B=B, L=L, S=S, N=N, H=H, causal=bool(params.get("isCausal")), blocks=blocks))

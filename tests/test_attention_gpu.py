@@ -24,16 +24,20 @@ def attention_routine(B, L, S, N, causal, scale=None, H=64):
     return Routine(Routines.Attention, t, dict(scale=1 / math.sqrt(H) if scale is None else scale, isCausal=causal))
 
 
-CASES = [(1, 128, 64, 1), (1, 128, 128, 1), (2, 256, 256, 3), (1, 384, 192, 2), (1, 128, 320, 2), (2, 1024, 1024, 4)]
+CASES = [(1, 128, 64, 1, 64), (1, 128, 128, 1, 64), (2, 256, 256, 3, 64), (1, 384, 192, 2, 64), (1, 128, 320, 2, 64), (2, 1024, 1024, 4, 64),
+         # other head sizes, and lengths that are not whole tiles (a last query block and a last key tile that are partly
+         # empty, fewer queries than a wave holds, one key)
+         (2, 256, 256, 2, 32), (1, 256, 192, 3, 128), (1, 100, 128, 1, 64), (1, 128, 100, 1, 64), (2, 77, 333, 3, 32), (1, 130, 65, 2, 128),
+         (1, 1, 1, 1, 64), (3, 5, 700, 2, 64), (1, 1000, 1000, 2, 128), (2, 513, 511, 1, 32)]
 
 
 @pytest.mark.parametrize("causal", [False, True], ids=["full", "causal"])
-@pytest.mark.parametrize("case", CASES, ids=lambda c: "B%d_L%d_S%d_N%d" % c)
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "B%d_L%d_S%d_N%d_H%d" % c)
 def test_attention_matches_float64(case, causal):
-    B, L, S, N = case
-    rng = np.random.default_rng(B * 1000 + L + S + N)
-    q, k, v = [rng.standard_normal((B, T, N, 64)).astype(np.float16) for T in (L, S, S)]
-    routine = attention_routine(B, L, S, N, causal)
+    B, L, S, N, H = case
+    rng = np.random.default_rng(B * 1000 + L + S + N + H)
+    q, k, v = [rng.standard_normal((B, T, N, H)).astype(np.float16) for T in (L, S, S)]
+    routine = attention_routine(B, L, S, N, causal, H=H)
     got, ks = R.run_gpu(routine, [q, k, v])
     want = R.run_oracle(routine, [q, k, v])
     np.testing.assert_allclose(got[0].astype(np.float64), want[0].astype(np.float64), rtol=1e-2, atol=3e-3, err_msg=str(ks.info))
@@ -95,9 +99,36 @@ def test_shapes_outside_the_kernel_are_refused_not_faked():
     if WARM_ONLY:
         pytest.skip("nothing to compile")
     be = backend()
-    for routine in (attention_routine(1, 100, 128, 1, False), attention_routine(1, 128, 100, 1, False), attention_routine(1, 128, 128, 1, False, H=32)):
+    t32 = RoutineType([[1, 128, 1, 64]] * 3, [DType.Float32] * 3, [[1, 128, 1, 64]], [DType.Float32])
+    for routine in (attention_routine(1, 128, 128, 1, False, H=16), attention_routine(1, 128, 128, 1, False, H=96),
+                    Routine(Routines.Attention, t32, dict(scale=0.125, isCausal=False))):
         with pytest.raises(UnsupportedRoutineError):
             be.prepareRoutineSync(routine)
+
+
+def test_reference_attention_tables_on_the_fused_kernel():
+    """test/nn.test.ts:275-390 on the fused kernel.  The tables use head sizes of 2 and 4; the operands are padded with
+    zeros to 32 (dot products and the meaningful output columns are unchanged) and the scale is the table's own
+    1/sqrt(H).  Two or three queries and keys: every tile is ragged."""
+    def run(q, k, v, scale, causal):
+        H0 = np.asarray(q).shape[-1]
+        pad = lambda a: np.pad(np.asarray(a, np.float16), [(0, 0)] * 3 + [(0, 32 - H0)])  # noqa: E731
+        q, k, v = pad(q), pad(k), pad(v)
+        routine = attention_routine(q.shape[0], q.shape[1], k.shape[1], q.shape[2], causal, scale=scale, H=32)
+        got, _ = R.run_gpu(routine, [q, k, v])
+        out = got[0].astype(np.float64).reshape(q.shape)
+        assert not out[..., H0:].any()
+        return out[..., :H0]
+    q = [[[[1, 0, 0, 0]], [[0, 1, 0, 0]]]]
+    out = run(q, q, [[[[1, 2, 3, 4]], [[5, 6, 7, 8]]]], 0.5, False)
+    np.testing.assert_allclose(out[0, 0, 0], [0.62245935 * a + 0.37754068 * b for a, b in zip((1, 2, 3, 4), (5, 6, 7, 8))], rtol=2e-3)
+    e = [[[[1, 0]], [[0, 1]]]]
+    out = run(e, e, e, 1.0, False)
+    np.testing.assert_allclose(out[0, 0, 0], [0.7310586, 0.26894143], rtol=2e-3)
+    out = run([[[[1, 0]], [[0.2, 0.2]], [[1, 1]]]], [[[[1, 0]], [[0, 1]], [[1, 1]]]], [[[[1, 0]], [[0, 1]], [[0, 0]]]], 1 / math.sqrt(2), True)
+    np.testing.assert_allclose(out[0, 0, 0], [1, 0], atol=1e-3)
+    np.testing.assert_allclose(out[0, 1, 0], [0.5, 0.5], rtol=2e-3)
+    np.testing.assert_allclose(out[0, 2, 0], [1 / (2 + math.exp(math.sqrt(0.5)))] * 2, rtol=2e-3)
 
 
 def test_gpt2_block_with_fused_attention():
@@ -109,7 +140,8 @@ def test_gpt2_block_with_fused_attention():
     assert [r.name for r in fused.routines] == [Routines.Attention] and not plain.routines
     assert len(fused.kernels) == len(plain.kernels) - 7  # seven attention kernels out; q, k, v are views of the QKV output
     assert all(v is not None for v in fused.routines[0].params["views"])
-    assert not W.gpt2BlockProgram(batch, 64, d, heads, d_ff, fusedAttention=True).routines  # L = 64: composition kept
+    assert not W.gpt2BlockProgram(batch, seq, d, 8, d_ff, fusedAttention=True).routines  # heads of 16: composition kept
+    assert W.gpt2BlockProgram(batch, 100, d, 4, d_ff, fusedAttention=True).routines     # heads of 32, a ragged length: fused
     if WARM_ONLY:
         from test_programs_gpu import warm
         warm(fused)
