@@ -441,9 +441,11 @@ def main():
     ap.add_argument("--no-settle", action="store_true", help="skip the clock-settling launches before the warm-up steps")
     ap.add_argument("--no-graphs", action="store_true", help="skip the HIP-graph replays of the C5 programs (for runs under a profiler "
                                                              "whose graph-launch tracing is not to be relied on)")
-    ap.add_argument("--only", choices=["all", "gemm", "copy", "hbm"], default="all",
+    ap.add_argument("--only", choices=["all", "gemm", "copy", "hbm", "matvec"], default="all",
                     help="gemm: headline kernel only; copy: a plain f32 copy kernel of known size (counter calibration); "
-                         "hbm: headline + the HBM-bound secondary workloads only (matvecs, row kernels, map)")
+                         "hbm: headline + the HBM-bound secondary workloads only (matvecs, row kernels, map); "
+                         "matvec: the two f16 matvec layouts under the launch plans compared in profiles/ (each as its own "
+                         "named kernel, cache-resident and cold), nothing else")
     args = ap.parse_args()
     global USE_GRAPHS
     USE_GRAPHS = not args.no_graphs
@@ -469,6 +471,38 @@ def main():
         w_ms, e_ms = timed(be, ex, [src], dst, args.steps, args.warmup)
         print(json.dumps({"workload": "copy f32 [8192,4096]", "bytes_read": rows * L * 4, "bytes_written": rows * L * 4,
                           "ms": e_ms, "GBps": 2 * rows * L * 4 / (e_ms * 1e-3) / 1e9}))
+        return
+
+    if args.only == "matvec":
+        # The decode matvec W[11008,4096] . x and its transposed layout, each under the default plan and under the plan
+        # it replaced, so that a profiler's per-kernel rows (durations, counters) can be compared.  "cold": four copies
+        # of W taken in turn (360 MB > the 256 MB memory-side cache), "warm": one W re-read by every launch.
+        M, K = 11008, 4096
+        W = hostrand.normal(1003, (M, K), 0.02, np.float16)
+        x = hostrand.normal(1003, (K,), 1.0, np.float16, stream=1)
+        mv_bytes = M * K * 2 + K * 2 + M * 2
+        rows = {}
+        for layout, kern, w_host in (("W", matvecKernel(M, K, DType.Float16), W),
+                                     ("WT", matvecKernel(M, K, DType.Float16, w_transposed=True), np.ascontiguousarray(W.T))):
+            plans = ([("batched_nt", {}), ("one_load_in_flight", dict(row_unroll=1, row_nt=0))] if layout == "W" else
+                     [("wide_strips_two_launches", {}), ("line_strips_one_launch", dict(col_strip=(8, 1024, 8), col_nt=0))])
+            xs = upload(be, x)
+            ws = [upload(be, w_host) for _ in range(4)]
+            o = be.malloc(kern.bytes)
+            for plan, opts in plans:
+                for temp, use in (("warm", ws[:1]), ("cold", ws)):
+                    name = f"jh_mv_{layout}_{plan}_{temp}"
+                    ex = be.prepareKernelSync(kern, name=name, **opts)
+                    sets = [[w, xs] for w in use]
+                    n_launch = max(args.steps, 1) * 20  # 400 by default; fewer under a profiler that serialises dispatches
+                    _, e1 = timed_rotating(be, ex, sets, o, n_launch, n_launch)
+                    _, e2 = timed_rotating(be, ex, sets, o, n_launch, 0)
+                    ms = min(e1, e2)
+                    rows[name] = {"class": ex.data.ks.klass, "plan": {k_: v for k_, v in ex.data.ks.info.items() if k_ != "stage2"}, "us": round(ms * 1e3, 2),
+                                  "GB/s": round(mv_bytes / (ms * 1e-3) / 1e9, 1), "frac_of_peak": round(mv_bytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+            for s_ in ws + [xs, o]:
+                be.decRef(s_)
+        print(json.dumps({"workload": "f16 matvec [11008,4096], both layouts, plans compared", "bytes_per_launch": mv_bytes, "rows": rows}))
         return
 
     # ---- headline: f16 GEMM n^3 -----------------------------------------------------------------

@@ -592,6 +592,12 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
         strips = -(-groups // lx_line)
         if (strips >= CU_COUNT // 2 or (col_strip and strips * rows_split >= CU_COUNT // 2)) and R // (blk // lx_line) >= 8:
             lx, T, split, unroll = lx_line, blk // lx_line, rows_split, (unroll if col_strip else 8)
+    if split == 1 and T % 4 == 0 and V > 1 and lx == 64 and 64 <= groups < 64 * (CU_COUNT // 2) and not col_strip:
+        # Few column groups and no cut over blocks (the fold launch behind a cut reduction is the typical case: 11008
+        # outputs x 32 slices): 64-lane strips would give a handful of workgroups that each walk their rows alone.
+        # Strips of 16 lanes (256 bytes per row) put four times as many CUs on the same bytes, the row slots sharing a
+        # wave and meeting through lane exchanges instead of LDS (whole waves only: four row slots or a multiple).
+        lx = 16
     t.klass = "reduce_col"
     t.vector_loads = dict(along_g) if V > 1 else {}
     if col_nt is None or col_nt:  # a stream read once by this launch: nontemporal, as in the row class
