@@ -352,6 +352,62 @@ def test_layer_sized_convolution_cotangents_run_on_the_matrix_cores(dt, npdt):
     assert any(c.startswith("gemm") for c in cls_x) and any(c.startswith("gemm") for c in cls_w), (cls_x, cls_w)
 
 
+def conv_vjp_by_taps(x, w, ct, strides, padding, rhs_dil):
+    """Adjoints of y[n,o,oy,ox] = sum x[n,c,oy*s+ky*d-p, ox*s+kx*d-p] w[o,c,ky,kx] (2-d, no input dilation), one filter tap
+    at a time in float64: dx gets ct x w scattered back, dw gets x windows contracted with ct."""
+    N, C, H, W = x.shape
+    O, _, KH, KW = w.shape
+    (sy, sx), (dy, dx_) = strides, rhs_dil
+    (pt, pb), (pl, pr) = padding
+    xp = np.pad(x.astype(np.float64), [(0, 0), (0, 0), (pt, pb), (pl, pr)])
+    OH, OW = ct.shape[2:]
+    gx = np.zeros_like(xp)
+    gw = np.zeros(w.shape)
+    c64, w64 = ct.astype(np.float64), w.astype(np.float64)
+    for ky in range(KH):
+        for kx in range(KW):
+            ys = slice(ky * dy, ky * dy + (OH - 1) * sy + 1, sy)
+            xs = slice(kx * dx_, kx * dx_ + (OW - 1) * sx + 1, sx)
+            gw[:, :, ky, kx] = np.einsum("nchw,nohw->oc", xp[:, :, ys, xs], c64)
+            gx[:, :, ys, xs] += np.einsum("nohw,oc->nchw", c64, w64[:, :, ky, kx])
+    return gx[:, :, pt:pt + H, pl:pl + W], gw
+
+
+RANDOM_CONVS = [
+    # N, C, O, H, W, KH, KW, strides, padding, filter dilation
+    (4, 32, 32, 12, 12, 3, 3, (1, 1), ((1, 1), (1, 1)), (1, 1)),
+    (2, 32, 64, 16, 14, 3, 3, (2, 2), ((1, 1), (1, 1)), (1, 1)),
+    (3, 48, 32, 13, 15, 3, 2, (1, 2), ((0, 0), (1, 0)), (1, 1)),
+    (2, 32, 32, 17, 17, 3, 3, (1, 1), ((2, 2), (2, 2)), (2, 2)),
+    (2, 64, 32, 9, 20, 1, 5, (1, 1), ((0, 0), (2, 2)), (1, 1)),
+    (1, 32, 96, 20, 20, 5, 5, (2, 2), ((2, 2), (2, 2)), (1, 1)),
+    (5, 40, 40, 8, 8, 2, 2, (2, 2), ((0, 0), (0, 0)), (1, 1)),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt,npdt", [(F32, np.float32), (F16, np.float16)])
+@pytest.mark.parametrize("cfg", RANDOM_CONVS, ids=lambda c: "x".join(map(str, c[:7])) + "_s%d%d_d%d%d" % (c[7] + c[9]))
+def test_convolution_cotangents_over_strides_paddings_and_dilations(cfg, dt, npdt):
+    """Both cotangent convolutions for strided, padded, dilated and asymmetric windows, sized so that the matcher hands
+    them to the matrix-core templates (gather loaders on both operands, input dilation by the forward stride): exact on
+    small-integer data against tap-by-tap adjoints."""
+    N, C, O, H, W, KH, KW, strides, padding, rd = cfg
+    rng = np.random.default_rng(sum(cfg[:7]))
+    x = rng.integers(-2, 3, (N, C, H, W)).astype(npdt)
+    w = rng.integers(-1, 2, (O, C, KH, KW)).astype(npdt)
+    p = ConvParams(0, list(strides), [tuple(q) for q in padding], [1, 1], list(rd))
+    from jaxjs_hip.convolution import checkConvShape
+    out_shape = checkConvShape(list(x.shape), list(w.shape), p)
+    ct = rng.integers(-1, 2, out_shape).astype(npdt)
+    dx_want, dw_want = conv_vjp_by_taps(x, w, ct, strides, padding, rd)
+    _, (dx,), cls_x = on_gpu(lambda c, f: conv_transposed_to_lhs(c, f, list(x.shape), p), [ct, w], dt)
+    _, (dw,), cls_w = on_gpu(lambda a, c: conv_transposed_to_rhs(a, c, list(w.shape), p), [x, ct], dt)
+    assert np.abs(dx_want).max() < 2048 and np.abs(dw_want).max() < 2048  # exact in float16 too
+    np.testing.assert_array_equal(dx.astype(np.float64).reshape(dx_want.shape), dx_want, err_msg=str(cls_x))
+    np.testing.assert_array_equal(dw.astype(np.float64).reshape(dw_want.shape), dw_want, err_msg=str(cls_w))
+
+
 @pytest.mark.gpu
 def test_transposed_dot_and_gather_cotangents_on_the_gpu():
     """`transposeDot` (src/frontend/linearize.ts:767-774): for c = a @ b the cotangents are ct @ b^T and a^T @ ct -- the
