@@ -36,7 +36,14 @@ def choose_tile(g: dict) -> Dict[str, int]:
     # operand (a slice is an offset on the k its loader is asked for).
     # With exactly one gather operand and a short k axis the kernel is a forward convolution, whose stride-1 form has
     # its own template (image patch in LDS) that takes the whole k axis: those keep one slice.
-    cut_k = g["a_k0"] == g["K"] and g["b_k0"] == g["K"] and (bool(g.get("a_gather")) == bool(g.get("b_gather")) or g["K"] >= 8192)
+    # A plain operand whose k axis has two strides (runs of k0 elements) can be cut where a slice is whole runs.
+    two_level = [g[t + "_k0"] for t in ("a", "b") if g[t + "_k0"] != g["K"]]
+
+    def runs_ok(slices):
+        return all((g["K"] // slices) % k0 == 0 for k0 in two_level)
+
+    cut_k = (all(g["K"] % k0 == 0 for k0 in two_level)
+             and (bool(g.get("a_gather")) == bool(g.get("b_gather")) or g["K"] >= 8192))
     if g["dtype"] == DType.Float32:
         # The f32 matrix pipe is 16x slower than the f16 one, so LDS traffic matters little and filling
         # every CU matters most: take the largest tile that still yields two workgroups per CU (the
@@ -57,7 +64,7 @@ def choose_tile(g: dict) -> Dict[str, int]:
             return dict(BM=128, BN=64, BK=bk, SPLITK=split, **(dict(FUSEK=1, WM=4, WN=1) if split > 1 else {}))
         # Fewer than 128 rows or 64 columns: 64x64 tiles, the k axis cut the same way when they are few.
         split = 1
-        while cut_k and tiles(64, 64) * split < 1.5 * CU and split < max_split and g["K"] % (split * 2 * bk) == 0 and g["K"] // (split * 2) >= 256:
+        while cut_k and tiles(64, 64) * split < 1.5 * CU and split < max_split and g["K"] % (split * 2 * bk) == 0 and g["K"] // (split * 2) >= 256 and runs_ok(split * 2):
             split *= 2
         return dict(BM=64, BN=64, BK=bk, **(dict(SPLITK=split, FUSEK=1 if plain_k else 0) if split > 1 else {}))
     # f16: estimated time = (tiles the busiest CU runs) x (tile area) x (K + fixed per-tile overhead) / efficiency.
@@ -68,7 +75,7 @@ def choose_tile(g: dict) -> Dict[str, int]:
     def k_split(count):
         # Fewer workgroups than 1.5 per CU: cut the k axis (partial sums in scratch, fold kernel) while slices stay >= 512 deep.
         split = 1
-        while cut_k and count * split < 1.5 * CU and split < max_split and g["K"] % (split * 2 * 64) == 0 and g["K"] // (split * 2) >= 512:
+        while cut_k and count * split < 1.5 * CU and split < max_split and g["K"] % (split * 2 * 64) == 0 and g["K"] // (split * 2) >= 512 and runs_ok(split * 2):
             split *= 2
         return dict(SPLITK=split) if split > 1 else {}
 
@@ -351,14 +358,16 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     K_full = g["K"]
     if split > 1:
         vec_k = 8 if g["dtype"] == DType.Float16 else 4
-        if g["a_k0"] != K_full or g["b_k0"] != K_full or K_full % split or (K_full // split) % vec_k:
+        # a two-stride k axis is cut between runs only
+        if (K_full % split or (K_full // split) % vec_k
+                or any(g[t + "_k0"] != K_full and (K_full // split) % g[t + "_k0"] for t in ("a", "b"))):
             split = 1
     # ... or, with FUSEK (f32 template), folded inside the same launch by the slice that arrives last at the tile's
     # counter: one launch instead of two.
     fusek = 0
     if split > 1:
         KS = K_full // split
-        g = dict(g, K=KS, a_k0=KS, b_k0=KS)
+        g = dict(g, K=KS, a_k0=KS if g["a_k0"] == K_full else g["a_k0"], b_k0=KS if g["b_k0"] == K_full else g["b_k0"])
         fusek = split if tile.get("FUSEK", 0) else 0
         if not fusek:
             out_t = "float"
@@ -572,7 +581,10 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         nbatch *= b[0]
     pitch = -(-kernel.size // 8) * 8  # elements between two slices' partial outputs
     if split > 1:
-        lines.append(f"  a_base += (long long)blockIdx.y * {g['K'] * g['a_sk']}ll; b_base += (long long)blockIdx.y * {g['K'] * g['b_sk']}ll;"
+        # a slice starts K elements further along k: K * sk for one stride, (K / k0) runs of sk1 for two
+        a_step = g["K"] * g["a_sk"] if g["a_k0"] == g["K"] else (g["K"] // g["a_k0"]) * g["a_sk1"]
+        b_step = g["K"] * g["b_sk"] if g["b_k0"] == g["K"] else (g["K"] // g["b_k0"]) * g["b_sk1"]
+        lines.append(f"  a_base += (long long)blockIdx.y * {a_step}ll; b_base += (long long)blockIdx.y * {b_step}ll;"
                      + ("" if fusek else f" c_base += (long long)blockIdx.y * {pitch}ll;"))
         lines.append(f"  const int jh_k_off = (int)blockIdx.y * {g['K']};  // a gather loader is asked for k of the whole axis")
         for d in (gather_calls, gather_slow):

@@ -245,6 +245,15 @@ def _flatten_k_split(st) -> Optional[tuple]:
             return None
         expect *= n
     lead = live[:-1]
+    # Trailing axes of the inner view that are contiguous with each other count as one (the cotangent of a convolution
+    # read as [O, N, H, W] -> [O, N*H*W]: H and W merge, N stays a second stride).
+    ishape, istrides = list(inner.shape), list(inner.strides)
+    while len(ishape) > len(lead) + 2 and istrides[-2] == istrides[-1] * ishape[-1]:
+        ishape[-2:] = [ishape[-2] * ishape[-1]]
+        istrides[-2:] = [istrides[-1]]
+    if len(ishape) != len(inner.shape):
+        from .shape import View
+        inner = View(tuple(ishape), tuple(istrides), inner.offset, None)
     if len(lead) != len(inner.shape) - 2 or any(n != inner.shape[j] for j, (_, n) in enumerate(lead)):
         return None
     K1, K0 = inner.shape[-2], inner.shape[-1]
@@ -298,7 +307,10 @@ def match_gemm(kernel: Kernel) -> Optional[dict]:
     def describe(gv):
         f = _flatten_k_split(gv.arg[1])
         if f is not None and f[0].mask is None:
-            return f[0], f[1], f[2], False
+            vec = 8 if gv.dtype == DType.Float16 else 4
+            # a two-stride k axis is only loadable in runs that hold whole 64-deep slabs; otherwise: element loader
+            if not f[1] or (f[0].strides[-1] == 1 and f[1] % 64 == 0 and f[2] % vec == 0 and f[2] > 0):
+                return f[0], f[1], f[2], False
         outer = gv.arg[1].views[-1]
         if outer.mask is not None:
             return None
