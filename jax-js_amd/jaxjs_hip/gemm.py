@@ -44,6 +44,13 @@ def choose_tile(g: dict) -> Dict[str, int]:
 
     cut_k = (all(g["K"] % k0 == 0 for k0 in two_level)
              and (bool(g.get("a_gather")) == bool(g.get("b_gather")) or g["K"] >= 8192))
+    repack = _repack_operand(g)  # that operand is read from an aligned copy (rows padded to whole groups)
+    loose_ops = bool(g.get("a_loose") or g.get("b_loose")) and repack is None
+
+    def edge_ok(bm, bn):
+        return ((repack == "a" or _edge_ok(g["M"], bm, g["a_sk"] == 1))
+                and (repack == "b" or _edge_ok(g["N"], bn, g["b_sk"] == 1)))
+
     if g["dtype"] == DType.Float32:
         # The f32 matrix pipe is 16x slower than the f16 one, so LDS traffic matters little and filling
         # every CU matters most: take the largest tile that still yields two workgroups per CU (the
@@ -69,7 +76,8 @@ def choose_tile(g: dict) -> Dict[str, int]:
         return dict(BM=64, BN=64, BK=bk, **(dict(SPLITK=split, FUSEK=1 if plain_k else 0) if split > 1 else {}))
     # f16: estimated time = (tiles the busiest CU runs) x (tile area) x (K + fixed per-tile overhead) / efficiency.
     # Efficiencies are measured rates of each tile shape relative to 256x256 on large problems (MI355X):
-    # 128x256 0.84, 256x128 0.79, 128x128 0.72 with two workgroups resident per CU (0.64 alone).  The fixed
+    # 128x256 0.84, 256x128 0.79, 128x128 0.62 with two workgroups resident per CU (8000^3: 0.63; 4100 x 4100 x 4096:
+    # 218 us against 180 us with 128x256), 0.64 alone with its deeper slabs.  The fixed
     # overhead (pipeline fill + epilogue) is about 100 k-steps.  This picks big tiles for big problems and
     # smaller ones when 256x256 would leave the last round of CUs nearly empty (e.g. 288 tiles on 256 CUs).
     def k_split(count):
@@ -92,23 +100,32 @@ def choose_tile(g: dict) -> Dict[str, int]:
         # size 64): measured 30 % faster with 128x64 tiles, which is then bound by reading A.
         return dict(BM=128, BN=64, WM=2, WN=2, **k_split(tiles(128, 64)))
     if (g["K"] <= 128 and g["K"] % 32 == 0 and plain_k and g["M"] % 128 == 0 and g["N"] % 128 == 0 and tiles(128, 128) >= 4 * CU
-            and not (g.get("a_loose") or g.get("b_loose"))):
+            and not loose_ops and repack is None):
         # A k axis of one to four slabs (attention scores: q.k^T over a head size of 64): the launch is bound by writing
         # C, and a workgroup spends its life in prologue and epilogue.  128x128 tiles with two shallow stages leave
         # room for four workgroups per CU, so that one's stores overlap another's loads and MFMAs
         # (96 x 1024 x 1024 x 64: 47.5 us with 256x256 tiles in the deep pipeline, 41.3 us = 5.5 TB/s this way).
         return dict(BM=128, BN=128, BK=32, STAGES=2, PIPE=0)
+    if (g["K"] <= 1024 and g["K"] % 32 == 0 and plain_k and g["M"] % 128 == 0 and g["N"] % 256 == 0 and tiles(128, 256) >= 2 * CU
+            and not loose_ops and repack is None and not (g["a_sk"] == 1 and g["b_sk"] == 1)):
+        # A short k axis under many tiles (the projections of a transformer block: 8192 x 2304 x 768, 8192 x 3072 x 768):
+        # a workgroup's prologue and its C stores weigh as much as its MFMAs.  128x256 tiles in two shallow stages
+        # (48 KiB, 164 registers) put three workgroups on a CU, whose phases overlap: 39.5 -> 36.3 us and 43.4 -> 40.7 us;
+        # the same as the deep pipeline at 4096 x 4096 x 1024 and 2048 x 8192 x 512; slower from k = 3072 (65.9 against
+        # 41.9 us) and with fewer than two tiles per CU (8192 x 768 x 768: 17.0 against 14.9 us).
+        return dict(BM=128, BN=256, WM=1, WN=4, BK=32, STAGES=2, PIPE=0)
     best = None
     for bm, bn, eff, extra in ((256, 256, 1.00, dict()), (128, 256, 0.84, dict(WM=1, WN=4)), (256, 128, 0.79, dict()),
-                                (128, 128, 0.72, dict())):
+                                (128, 128, 0.62, dict())):
         if (bm > 128 and g["M"] < bm) or (bn > 128 and g["N"] < bn):
             continue
         per_cu = -(-tiles(bm, bn) // tuner.CU_COUNT)
         if (bm, bn) == (128, 128) and per_cu < 2:
             eff = 0.64
-        whole = g["M"] % bm == 0 and g["N"] % bn == 0 and g["K"] % 32 == 0 and plain_k and not (g.get("a_loose") or g.get("b_loose"))
+        whole = edge_ok(bm, bn) and g["K"] % 32 == 0 and plain_k and not loose_ops
         if not whole:
-            # Ragged extents or operands off the 16-byte grid run the general template, whose small tiles lose more
+            # A ragged k axis, operands off the 16-byte grid or an edge the direct loads cannot clamp run the general
+            # template, whose small tiles lose more
             # (8000^3: 838 / 597 / 691 / 512 TFLOP/s for the four shapes, against 1340 for whole 256x256 tiles).
             eff = {(256, 256): 0.63, (128, 256): 0.45, (256, 128): 0.52, (128, 128): 0.38}[(bm, bn)]
         cost = per_cu * bm * bn * (g["K"] + 100) / eff
@@ -127,11 +144,12 @@ def choose_tile(g: dict) -> Dict[str, int]:
         # slices cost more in partial sums than they gain).
         if tiles(128, 128) * 2 <= CU and g["K"] >= 2048 and g["K"] % 128 == 0:
             tile.update(SPLITK=4 if tiles(128, 128) * 4 <= CU and g["K"] >= 4096 and g["K"] % 256 == 0 else 2)
-            # Folding inside the launch is the direct-to-LDS template's: whole tiles, operands on the 16-byte grid.  Ragged
-            # or loose shapes (100 x 14336 x 4096) keep the split and fold in a second launch.
+            # Folding inside the launch is the direct-to-LDS template's: operands on the 16-byte grid, edges it can clamp.
+            # Other shapes keep the split and fold in a second launch.
             # Two slices only: with four, the last workgroup's read-back of four slices behind the acknowledged stores
             # costs more than a fold launch (128x4096x4096: 16.0 us folded in the launch, 14.4 us with the fold kernel).
-            if g["M"] % 128 == 0 and g["N"] % 128 == 0 and not (g.get("a_loose") or g.get("b_loose")):
+            # Edge tiles fold the same way (100 x 14336 x 4096: 31.1 us in four slices with a fold launch, 25.5 us in two).
+            if edge_ok(128, 128) and not (g.get("a_loose") or g.get("b_loose")):  # (a repacked operand takes no k split)
                 if tile["SPLITK"] == 2:
                     tile.update(FUSEK=1)
             else:  # the general template gains from more slices (100 x 14336 x 4096: 41.1 us in two, 34.6 us in four)
@@ -141,6 +159,34 @@ def choose_tile(g: dict) -> Dict[str, int]:
         # convolution: 9 taps x one tile, k = batch x positions): slices over workgroups, folded by a second launch.
         tile.update(k_split(tiles(tile["BM"], tile["BN"])))
     return tile
+
+
+def _repack_operand(g: dict):
+    """The operand ("a" or "b") that a pre-pass copies onto the 16-byte grid before the direct-to-LDS template reads it,
+    or None.  An f16 operand that runs along its rows in memory with rows off the grid (np.matmul against a [K, N]
+    matrix with N = 50257: every row starts at an odd element) would otherwise send the whole GEMM to the general
+    template (8192 x 50257 x 768: 1.19 ms); copied once into scratch as [K][rows rounded up to 8] (K x rows x 4 bytes of
+    traffic) the GEMM runs on the fast path.  Worth it when the other operand has enough rows to amortise the copy."""
+    if g["dtype"] != DType.Float16 or g["batch"] or g.get("a_gather") or g.get("b_gather"):
+        return None
+    if g["K"] % 32 or g["a_k0"] != g["K"] or g["b_k0"] != g["K"]:
+        return None
+    loose = [t for t in ("a", "b") if g.get(t + "_loose")]
+    if len(loose) != 1:
+        return None
+    tag = loose[0]
+    srow = g["a_sm"] if tag == "a" else g["b_sn"]
+    rows, other = (g["M"], g["N"]) if tag == "a" else (g["N"], g["M"])
+    if srow != 1 or rows < 128 or other < 512:
+        return None
+    return tag
+
+
+def _edge_ok(extent: int, tile: int, k_contiguous: bool) -> bool:
+    """Whether the direct-to-LDS template can take an operand whose row count is `extent` in tiles of `tile` rows: whole
+    tiles, or an edge tile whose loads can be clamped -- to the last row when the operand runs along k in memory, to
+    the last whole 16-byte group of rows when it runs along its rows (the count must then be whole groups)."""
+    return extent % tile == 0 or k_contiguous or (extent % 8 == 0 and extent >= 8)
 
 
 def _strip_casts(e: AluExp) -> AluExp:
@@ -372,13 +418,26 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         if not fusek:
             out_t = "float"
 
+    # An operand off the 16-byte grid that a pre-pass copies into scratch (see `_repack_operand`): from here on it is a
+    # dense [K][rows_pad] operand named `jh_repack`.
+    repack = _repack_operand(g) if split == 1 and tile.get("REPACK", 1) else None
+    load_rows = dict(a=g["M"], b=g["N"])
+    repack_src = None
+    if repack:
+        rows = load_rows[repack]
+        rows_pad = -(-rows // 8) * 8
+        repack_src = dict(gid=g["gid_" + repack], off=g[repack + "_off"], sk=g[repack + "_sk"], rows=rows, rows_pad=rows_pad)
+        load_rows[repack] = rows_pad
+        g = dict(g, **{repack + "_off": 0, repack + "_sk": rows_pad, repack + "_loose": False})
+
     used = _used_args(kernel.nargs, t.epilogue)
     used[g["gid_a"]] = g["dtype"]
     used[g["gid_b"]] = g["dtype"]
     names = [f"in{i}" for i in range(kernel.nargs)]
     params = ", ".join(
         [f"const {STORAGE_CTYPE[d or DType.Float32]}* __restrict__ {n}" for d, n in zip(used, names)]
-        + [f"{out_t}* __restrict__ out"] + (["float* __restrict__ jh_part", "unsigned* __restrict__ jh_count"] if fusek else []))
+        + [f"{out_t}* __restrict__ out"] + (["float* __restrict__ jh_part", "unsigned* __restrict__ jh_count"] if fusek else [])
+        + (["const jh_f16* __restrict__ jh_repack"] if repack else []))
 
     # Fused epilogue as a device function of (acc, row, col, batch coordinates, buffers...).  The kernel's
     # epilogue is written over the flat output index; here that index is re-expressed through the tile's own
@@ -604,10 +663,18 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     dBK = tile.get("BK", 64 if both_k and tile.get("PIPE", 1) else 32) if g["dtype"] == DType.Float16 else 32
     if dBK not in (32, 64):
         raise ValueError(f"direct-to-LDS slab depth must be 32 or 64, got {dBK}")
-    full = g["M"] % BM == 0 and g["N"] % BN == 0 and g["K"] % dBK == 0 and BM >= 128 and BN >= 128
+    a_kc, b_kc = g["a_sk"] == 1 or g["K"] == 1, g["b_sk"] == 1 or g["K"] == 1
+    full = (_edge_ok(load_rows["a"], BM, a_kc) and _edge_ok(load_rows["b"], BN, b_kc) and g["K"] % dBK == 0 and BM >= 128 and BN >= 128
+            and tile.get("EDGE", 1) | (g["M"] % BM == 0 and g["N"] % BN == 0))
     any_gather = bool(g.get("a_gather") or g.get("b_gather"))
     loose = {tag: 1 if g.get(tag + "_loose") and not g.get(tag + "_gather") else 0 for tag in ("a", "b")}
     dlds = g["dtype"] == DType.Float16 and full and tile.get("DLDS", 1) and not any_gather and not (loose["a"] or loose["b"])
+    if repack and not dlds:  # the copy only serves the direct loads: plan again without it
+        import copy
+
+        t2 = copy.copy(t)
+        t2.params = dict(t.params, gemm_tile=tuple(sorted(dict(override, REPACK=0).items())))
+        return gen_gemm(kernel, t2, numerics, name)
     if dlds:
         tmpl = "gemm_f16_dlds.hip.inc"
     if dlds:
@@ -655,12 +722,12 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                      GATHER_A_CALL=gather_calls["a"], GATHER_B_CALL=gather_calls["b"],
                      GATHER_A_SLOW=gather_slow.get("a", "jh_half8{0, 0, 0, 0, 0, 0, 0, 0}"), GATHER_B_SLOW=gather_slow.get("b", "jh_half8{0, 0, 0, 0, 0, 0, 0, 0}"))
     src = _prelude(numerics) + fill(template(tmpl), dict(sched, 
-        M=g["M"], N=g["N"], K=g["K"], BM=BM, BN=BN, WM=WM, WN=WN,
+        M=g["M"], N=g["N"], K=g["K"], M_LOAD=load_rows["a"], N_LOAD=load_rows["b"], BM=BM, BN=BN, WM=WM, WN=WN,
         A_KCONTIG=0 if gather_flags["a"] in (2, 3) else (1 if g["a_sk"] == 1 or g["K"] == 1 or gather_flags["a"] in (1, 4) else 0),
         B_KCONTIG=0 if gather_flags["b"] in (2, 3) else (1 if g["b_sk"] == 1 or g["K"] == 1 or gather_flags["b"] in (1, 4) else 0),
         NBATCH=nbatch, EPILOGUE_FN=epi_fn, NAME=name, PARAMS=params,
         A_OFF=g["a_off"], B_OFF=g["b_off"], BATCH_DECODE="\n".join(lines),
-        A_PTR=names[g["gid_a"]], B_PTR=names[g["gid_b"]],
+        A_PTR="jh_repack" if repack == "a" else names[g["gid_a"]], B_PTR="jh_repack" if repack == "b" else names[g["gid_b"]],
         A_SM=g["a_sm"], A_SK=g["a_sk"], B_SN=g["b_sn"], B_SK=g["b_sk"],
         A_K0=g["a_k0"], A_SK1=g["a_sk1"], B_K0=g["b_k0"], B_SK1=g["b_sk1"],
         C_SM=g["c_sm"], C_SN=g["c_sn"], EPILOGUE_ARGS=epi_args))
@@ -685,6 +752,32 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                                 4: "tap-major strided"}[gather_flags[tag]] for tag in ("a", "b")}
         if tap_major is not None:
             info["tap_major"] = tap_major
+    if repack:
+        rs = repack_src
+        groups = rs["rows_pad"] // 8
+        src += (f"""
+// Operand [K][{rs['rows']} rows] (k stride {rs['sk']} elements, first element {rs['off']}: rows off the 16-byte grid) -> jh_repack [K][{rs['rows_pad']}],
+// eight rows per thread: one under-aligned 16-byte load, one aligned store; the rows past the end are zeros.
+struct __attribute__((packed, aligned(2))) jh_half8_u {{ jh_half8 v; }};
+extern "C" __global__ __launch_bounds__(256) void {name}_repack(const jh_f16* __restrict__ src, jh_f16* __restrict__ dst) {{
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= {g['K']}ll * {groups}) return;
+  const int k = (int)(i / {groups}), r0 = (int)(i % {groups}) * 8;
+  const jh_f16* __restrict__ p = src + {rs['off']}ll + (long long)k * {rs['sk']}ll + r0;
+  jh_half8 v;
+  if (r0 + 8 <= {rs['rows']}) {{
+    v = reinterpret_cast<const jh_half8_u*>(p)->v;
+  }} else {{
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = r0 + e < {rs['rows']} ? p[e] : (jh_f16)0.0f;
+  }}
+  *reinterpret_cast<jh_half8*>(dst + (long long)k * {rs['rows_pad']} + r0) = v;
+}}
+""")
+        prep = LaunchStep(name + "_repack", (-(-g["K"] * groups // 256), 1, 1), (256, 1, 1), 0, [("in", rs["gid"]), ("scratch", 0)])
+        step.args.append(("scratch", 0))
+        info["repack"] = repack
+        return KernelSource([src], [prep, step], [g["K"] * rs["rows_pad"] * 2], "gemm", need, info)
     if split == 1:
         return KernelSource([src], [step], [], "gemm", need, info)
     if fusek:

@@ -292,6 +292,42 @@ def test_gemm_operands_that_start_off_the_vector_grid(dt):
     np.testing.assert_array_equal(got.reshape(M, N).astype(np.float32), want)
 
 
+# ---- an operand that runs along its rows with rows off the grid, against >= 512 rows of the other: copied once into scratch
+
+REPACK_CASES = [
+    # M, N, K, layout, element offset of the off-grid operand's view, tile options
+    (520, 1001, 512, "NN", 0, dict()), (1024, 50257 // 16, 768, "NN", 0, dict()), (1001, 520, 256, "TN", 0, dict()),
+    (512, 256, 128, "NN", 3, dict()), (640, 777, 96, "NN", 1, dict(BM=256, BN=256)), (513, 1001, 64, "NN", 0, dict(BM=256, BN=128, SADDR=0)),
+]
+
+
+@pytest.mark.parametrize("M,N,K,layout,off,tile", REPACK_CASES, ids=lambda v: "-".join(f"{k}{x}" for k, x in v.items()) or "default" if isinstance(v, dict) else str(v))
+def test_gemm_f16_rows_off_the_grid_are_repacked(M, N, K, layout, off, tile):
+    """np.matmul against a [K, 1001] matrix: every row of B starts at an odd element.  With enough rows on the other side a
+    pre-pass copies B into scratch as [K][1008] and the direct-to-LDS template runs on the copy (edge tiles clamped, the
+    padding never stored).  Small integer entries: exact in every element."""
+    A = RNG.integers(-2, 3, (M, K)).astype(np.float16)
+    B = RNG.integers(-2, 3, (K, N)).astype(np.float16)
+    full = [M, N, K]
+    if layout == "TN":  # A stored [K, M], M off the grid
+        abuf = np.concatenate([np.zeros(off, np.float16), np.ascontiguousarray(A.T).ravel()])
+        stA = ShapeTracker.fromShape([K * M + off]).shrink([(off, K * M + off)]).reshape([K, M]).permute([1, 0]).reshape([M, 1, K]).expand(full)
+        bbuf = B
+        stB = ShapeTracker.fromShape([K, N]).permute([1, 0]).reshape([1, N, K]).expand(full)
+        want = "a"
+    else:
+        abuf = A
+        stA = ShapeTracker.fromShape([M, K]).reshape([M, 1, K]).expand(full)
+        bbuf = np.concatenate([np.zeros(off, np.float16), B.ravel()])
+        stB = ShapeTracker.fromShape([K * N + off]).shrink([(off, K * N + off)]).reshape([K, N]).permute([1, 0]).reshape([1, N, K]).expand(full)
+        want = "b"
+    k = _f32_out(reduceKernel(full, [(DType.Float16, stA), (DType.Float16, stB)], lambda a, b: AluExp.mul(a, b), AluOp.Add), K)
+    opts = dict(gemm_tile=tuple(sorted(tile.items()))) if tile else {}
+    got, ks = device_run(k, [abuf, bbuf], **opts)
+    assert ks.klass == "gemm" and ks.info["direct_lds"] and ks.info.get("repack") == want, (ks.klass, ks.info)
+    np.testing.assert_array_equal(got.reshape(M, N).astype(np.float32), A.astype(np.float32) @ B.astype(np.float32), err_msg=str(ks.info))
+
+
 # ---- a handful of rows (or columns) against a large operand: a linear layer on a few tokens
 
 THIN_CASES = [
@@ -300,8 +336,8 @@ THIN_CASES = [
     (DType.Float16, 31, 4096, 4096, False, dict(BM=64, BN=128, splitk=8)), (DType.Float16, 64, 14336, 4096, False, dict(BM=64, BN=128, splitk=4)),
     (DType.Float16, 14336, 16, 4096, False, dict(BM=128, BN=64, splitk=4)), (DType.Float16, 7, 1000, 4100, True, dict(BM=64, BN=128)),
     (DType.Float32, 4, 14336, 4096, False, dict(BM=64, BN=64, splitk=2)), (DType.Float32, 14336, 16, 4096, False, dict(BM=64, BN=64, splitk=2)),
-    # 65..127 rows, few 128x128 tiles, long k: the tile is not whole, so the k split folds in a second launch
-    (DType.Float16, 100, 14336, 4096, False, dict(BM=128, BN=128, splitk=4, direct_lds=False)), (DType.Float16, 65, 4096, 4096, True, dict(BM=128, BN=128, splitk=8)),
+    # 65..127 rows, few 128x128 tiles, long k: the tile is not whole (edge loads clamp); two slices folded inside the launch
+    (DType.Float16, 100, 14336, 4096, False, dict(BM=128, BN=128, splitk=2, direct_lds=True, fused_fold=True)), (DType.Float16, 65, 4096, 4096, True, dict(BM=128, BN=128, splitk=4, direct_lds=True)),
     (DType.Float16, 300, 300, 8192, False, dict(BM=128, BN=128, splitk=8)), (DType.Float16, 8192, 100, 4096, False, dict(BM=128, BN=128, splitk=8)),
 ]
 
@@ -362,9 +398,11 @@ def test_gemm_sweep_shapes(dt, M, N, K, want):
     _check(got.reshape(M, N)[rows], A[rows], B, K, out_f16=(dt == DType.Float16))
 
 
-@pytest.mark.parametrize("M,N,K,split,bt", [(384, 640, 1024, 4, False), (128, 1792, 2048, 2, False), (256, 256, 4096, 8, True), (640, 128, 512, 2, True)])
+@pytest.mark.parametrize("M,N,K,split,bt", [(384, 640, 1024, 4, False), (128, 1792, 2048, 2, False), (256, 256, 4096, 8, True), (640, 128, 512, 2, True),
+                                            (200, 392, 2048, 2, False), (100, 1001, 1024, 2, True)])
 def test_gemm_f16_in_launch_fold_matches_the_fold_kernel_bit_for_bit(M, N, K, split, bt):
-    """The same check for the direct-to-LDS f16 template (15, 14, 4 and 5 tiles; B stored [K,N] and [N,K])."""
+    """The same check for the direct-to-LDS f16 template (15, 14, 4 and 5 tiles; B stored [K,N] and [N,K]; the last two
+    shapes have edge tiles along both axes)."""
     from gpu_util import WARM_ONLY, backend
     k = matmulKernel(M, N, K, DType.Float16, b_transposed=bt)
     tiles = dict(BM=128, BN=128, SPLITK=split)
@@ -464,6 +502,54 @@ def test_gemm_f16_direct_lds_variants(M, N, K, bt, tile):
     if bt and "BK" not in tile and K % 64 == 0 and K >= 128:
         assert ks.info["BK"] == 64, ks.info
     _check(got, A, B, K)
+
+
+# Edge tiles of the direct-to-LDS template: extents that are not whole block tiles.  An operand that runs along k is
+# clamped to its last row (any extent), one that runs along its rows to its last whole group of eight (extent % 8 == 0);
+# what lies past the edge is computed on repeated data and never stored.  (M, N, K, layout, tile options, row bias + ReLU)
+EDGE_CASES = [
+    (1000, 1000, 1024, "NN", dict(), False), (300, 520, 256, "NN", dict(), False), (1000, 1001, 512, "NT", dict(), False),
+    (1000, 336, 512, "TN", dict(), False), (104, 1000, 256, "TN", dict(), False), (2050, 2056, 384, "NN", dict(), False),
+    (520, 392, 320, "NT", dict(BM=256, BN=256, BK=64, RING=5), False), (520, 392, 320, "NN", dict(BM=256, BN=256), False),
+    (520, 392, 320, "NN", dict(BM=256, BN=128, PIN=0, SADDR=0), False), (520, 392, 320, "NT", dict(BM=128, BN=256, WM=1, WN=4, SADDR=0), False),
+    (1000, 1000, 512, "NN", dict(), True), (777, 520, 512, "NN", dict(BM=256, BN=256), True), (333, 136, 256, "NT", dict(), True),
+    (129, 136, 64, "NN", dict(BM=128, BN=128), False), (130, 129, 64, "NT", dict(BM=128, BN=128), False),
+    (200, 392, 2048, "NN", dict(BM=128, BN=128, SPLITK=4), True), (100, 14336, 4096, "NN", dict(), False),
+]
+
+
+@pytest.mark.parametrize("M,N,K,layout,tile,bias", EDGE_CASES, ids=lambda v: "-".join(f"{k}{x}" for k, x in v.items()) or "default" if isinstance(v, dict) else str(v))
+def test_gemm_f16_direct_lds_edge_tiles(M, N, K, layout, tile, bias):
+    A = RNG.uniform(-1, 1, (M, K)).astype(np.float16)
+    B = RNG.uniform(-1, 1, (K, N)).astype(np.float16)
+    full = [M, N, K]
+    stA = (ShapeTracker.fromShape([K, M]).permute([1, 0]) if layout == "TN" else ShapeTracker.fromShape([M, K])).reshape([M, 1, K]).expand(full)
+    stB = (ShapeTracker.fromShape([N, K]) if layout == "NT" else ShapeTracker.fromShape([K, N]).permute([1, 0])).reshape([1, N, K]).expand(full)
+    base = reduceKernel(full, [(DType.Float16, stA), (DType.Float16, stB)], lambda a, b: AluExp.mul(a, b), AluOp.Add)
+    bufs = [np.ascontiguousarray(A.T) if layout == "TN" else A, np.ascontiguousarray(B.T) if layout == "NT" else B]
+    if bias:
+        bv = RNG.uniform(-1, 1, N).astype(np.float32)
+        acc = AluVar.acc(DType.Float32)
+        n_idx = unravelAlu([M, N], AluVar.gidx)[1]
+        b = AluExp.globalView(DType.Float32, 2, ShapeTracker.fromShape([N]), [n_idx])
+        k = Kernel(3, M * N, base.exp_raw, Reduction(DType.Float32, AluOp.Add, K, AluExp.max(AluExp.add(acc, b), AluExp.f32(0))))
+        bufs.append(bv)
+    else:
+        k = base
+    opts = dict(gemm_tile=tuple(sorted(tile.items()))) if tile else {}
+    got, ks = device_run(k, bufs, **opts)
+    assert ks.klass.startswith("gemm") and ks.info["direct_lds"], (ks.klass, ks.info)
+    assert M % ks.info["BM"] or N % ks.info["BN"], ks.info  # an edge tile exists
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    mag = np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)
+    bound = 2 * K * np.finfo(np.float32).eps * mag
+    if bias:
+        ref = np.maximum(ref + bv, 0)
+        bound = bound + 4 * np.finfo(np.float32).eps * (np.abs(ref) + 1)
+    else:
+        bound = bound + np.abs(ref) * 2.0**-11 + 2.0**-24
+    err = np.abs(got.astype(np.float64).reshape(ref.shape) - ref)
+    assert np.all(err <= bound), f"max excess {np.max(err - bound)} with {ks.info}"
 
 
 F32_SHAPES = [(64, 64, 64), (128, 128, 64), (200, 264, 136), (1024, 1024, 1024), (96, 1028, 72), (512, 384, 100)]
