@@ -93,9 +93,15 @@ def choose_tile(g: dict) -> Dict[str, int]:
             return dict(BM=64, BN=256, WM=1, WN=4)
         # Few tiles (a linear layer on 2..64 tokens): bound by streaming B once, so what matters is enough workgroups
         # in flight -- 64 x 128 tiles and a k split (64 x 14336 x 4096: 65.7 us with 56 tiles of 64 x 256, 26.6 us with
-        # 112 x 4 slices; 16 rows 24.6 us, 4 rows 23.5 us; B alone takes 20 us at the HBM rate).
-        return dict(BM=64, BN=128, WM=1, WN=4, **k_split(tiles(64, 128)))
-    if g["N"] <= 64 and g["M"] >= 128:
+        # 112 x 4 slices; 16 rows 24.6 us, 4 rows 23.5 us; B alone takes 15 us at the HBM rate).
+        # When the direct-to-LDS template can take the shape (its A loads clamp to the last row that exists) its
+        # 128x128 tiles in two or four slices stream B faster than the register-staged loaders, the empty rows of the
+        # tile costing nothing that matters here: 4 / 16 / 64 x 14336 x 4096 25.2 / 25.9 / 28.2 -> 20.7 / 21.2 / 23.5 us,
+        # 31 x 4096 x 4096 15.5 -> 13.0 us.  Those fall through to the plan below.
+        if not (edge_ok(128, 128) and plain_k and not loose_ops and repack is None and g["K"] >= 2048 and g["K"] % 128 == 0
+                and tiles(128, 128) * 2 <= CU):
+            return dict(BM=64, BN=128, WM=1, WN=4, **k_split(tiles(64, 128)))
+    elif g["N"] <= 64 and g["M"] >= 128:
         # A 128-wide tile would compute and store a half-empty block (attention's probabilities x V, N = head
         # size 64): measured 30 % faster with 128x64 tiles, which is then bound by reading A.
         return dict(BM=128, BN=64, WM=2, WN=2, **k_split(tiles(128, 64)))
@@ -149,8 +155,10 @@ def choose_tile(g: dict) -> Dict[str, int]:
             # Two slices only: with four, the last workgroup's read-back of four slices behind the acknowledged stores
             # costs more than a fold launch (128x4096x4096: 16.0 us folded in the launch, 14.4 us with the fold kernel).
             # Edge tiles fold the same way (100 x 14336 x 4096: 31.1 us in four slices with a fold launch, 25.5 us in two).
+            # Up to 64 rows the fold launch is the cheaper one: it touches the rows that exist, the fold inside the launch
+            # whole tiles of partial sums (64 x 14336 x 4096: 23.5 against 23.7 us, 4 rows: 20.7 against 22.4 us).
             if edge_ok(128, 128) and not (g.get("a_loose") or g.get("b_loose")):  # (a repacked operand takes no k split)
-                if tile["SPLITK"] == 2:
+                if tile["SPLITK"] == 2 and g["M"] > 64:
                     tile.update(FUSEK=1)
             else:  # the general template gains from more slices (100 x 14336 x 4096: 41.1 us in two, 34.6 us in four)
                 tile.update(k_split(tiles(128, 128)) or dict(SPLITK=tile["SPLITK"]))

@@ -332,8 +332,10 @@ def test_gemm_f16_rows_off_the_grid_are_repacked(M, N, K, layout, off, tile):
 
 THIN_CASES = [
     # dtype, M, N, K, B stored [N,K], expected tile and k split
-    (DType.Float16, 2, 14336, 4096, False, dict(BM=64, BN=128, splitk=4)), (DType.Float16, 16, 14336, 4096, True, dict(BM=64, BN=128, splitk=4)),
-    (DType.Float16, 31, 4096, 4096, False, dict(BM=64, BN=128, splitk=8)), (DType.Float16, 64, 14336, 4096, False, dict(BM=64, BN=128, splitk=4)),
+    # (f16 rows that the direct-to-LDS loads can clamp take its 128x128 tiles; a k axis that is not whole slabs keeps 64x128)
+    (DType.Float16, 2, 14336, 4096, False, dict(BM=128, BN=128, splitk=2, direct_lds=True)), (DType.Float16, 16, 14336, 4096, True, dict(BM=128, BN=128, splitk=2, direct_lds=True)),
+    (DType.Float16, 31, 4096, 4096, False, dict(BM=128, BN=128, splitk=4, direct_lds=True)), (DType.Float16, 64, 14336, 4096, False, dict(BM=128, BN=128, splitk=2, direct_lds=True)),
+    (DType.Float16, 16, 14336, 4000, False, dict(BM=64, BN=128, splitk=1, direct_lds=False)),
     (DType.Float16, 14336, 16, 4096, False, dict(BM=128, BN=64, splitk=4)), (DType.Float16, 7, 1000, 4100, True, dict(BM=64, BN=128)),
     (DType.Float32, 4, 14336, 4096, False, dict(BM=64, BN=64, splitk=2)), (DType.Float32, 14336, 16, 4096, False, dict(BM=64, BN=64, splitk=2)),
     # 65..127 rows, few 128x128 tiles, long k: the tile is not whole (edge loads clamp); two slices folded inside the launch
