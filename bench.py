@@ -639,6 +639,7 @@ def main():
             (1024, 1024, 1024, DType.Float32, "c1_matmul_f32_1024", PEAK_F32_MATRIX_TFLOPS),
             (2048, 2048, 2048, DType.Float16, "gemm_f16_2048", PEAK_F16_TFLOPS),
             (4096, 4096, 4096, DType.Float16, "gemm_f16_4096", PEAK_F16_TFLOPS),
+            (8000, 8000, 8000, DType.Float16, "gemm_f16_8000 (edge tiles)", PEAK_F16_TFLOPS),
             (128, 14336, 4096, DType.Float16, "gemm_f16_skinny_128x14336x4096", PEAK_F16_TFLOPS),
             (4096, 4096, 4096, DType.Float32, "gemm_f32_4096", PEAK_F32_MATRIX_TFLOPS),
         ]:
