@@ -348,6 +348,54 @@ def bench_program_gpt2_fused(be, hostrand, timed):
                                 "TFLOP/s_causal_half": round(full / 2 / (attn_ms * 1e-3) / 1e12, 1)}}
 
 
+def bench_reference_matmul_matvec_cases(be, timed):
+    """The cases of the reference's own matmul and matvec benches on this backend (bench/matmul-wasm.bench.ts:5-46,
+    bench/matmul-webgpu.bench.ts:11, bench/matvec-wasm.bench.ts:5-53, bench/matvec-webgpu.bench.ts:11): f32 n x n against
+    n x n (and against the transpose), n x n (and its transpose) against a vector, with the operand values of the Wasm
+    benches.  `ms_sync` is one dispatch + fence per iteration as there (best of 5); `ms` is the kernel back to back."""
+    from jaxjs_hip import DType
+    from jaxjs_hip.lowering import matmulKernel, matvecKernel
+
+    out = {}
+
+    def one(kernel, arrays):
+        exe = be.prepareKernelSync(kernel)
+        ins = [upload(be, a) for a in arrays]
+        o = be.malloc(kernel.bytes)
+        be.dispatch(exe, ins, [o])
+        be.dev.sync()
+        best = float("inf")
+        for _ in range(5):
+            t0 = time.perf_counter()
+            be.dispatch(exe, ins, [o])
+            be.dev.sync()
+            best = min(best, (time.perf_counter() - t0) * 1e3)
+        _, est = timed(be, exe, ins, o, 5, 3)
+        n_steps = int(min(max(5.0 / max(est, 1e-4), 20), 2000))
+        _, ms = timed(be, exe, ins, o, n_steps, max(n_steps // 4, 3))
+        for s_ in ins + [o]:
+            be.decRef(s_)
+        return {"class": exe.data.ks.klass, "ms_sync": round(best, 4), "ms": round(ms, 5)}
+
+    def matrix(n):
+        return ((np.arange(n * n, dtype=np.int64) % 7) - 3).astype(np.float32).reshape(n, n)
+
+    for n in (64, 128, 256, 512, 1024, 2048, 4096):
+        a = matrix(n)
+        for tag, bt in ((f"matmul {n}x{n}", False), (f"matmul {n}x{n} @ transpose", True)):
+            row = one(matmulKernel(n, n, n, DType.Float32, b_transposed=bt), [a, a])
+            row["TFLOP/s"] = round(2.0 * n ** 3 / (row["ms"] * 1e-3) / 1e12, 2)
+            out[tag] = row
+    for n in (512, 1024, 2048, 4096):
+        a = matrix(n)
+        x = ((np.arange(n, dtype=np.int64) % 5) - 2).astype(np.float32)
+        for tag, wt in ((f"matvec {n}x{n} @ vector", False), (f"matvec {n}x{n}.T @ vector", True)):
+            row = one(matvecKernel(n, n, DType.Float32, w_transposed=wt), [a, x])
+            row["GB/s"] = round((n * n + 2 * n) * 4 / (row["ms"] * 1e-3) / 1e9, 1)
+            out[tag] = row
+    return out
+
+
 def bench_reference_routine_cases(be):
     """The cases of the reference's own routine benches on this backend (bench/fft.bench.ts:6-13, sort.bench.ts:15-16,
     cholesky-webgpu.bench.ts:16): one dispatch + fence per iteration as there, best of 5; operands resident."""
@@ -718,6 +766,7 @@ def main():
         be.decRef(xs)
         del X
         extra["reference_routine_benches"] = bench_reference_routine_cases(be)
+        extra["reference_matmul_matvec_benches"] = bench_reference_matmul_matvec_cases(be, timed)
         result["extra"] = extra
 
     if not args.no_cpu:

@@ -203,7 +203,7 @@ def gen_conv(kernel, g: dict, oexp: AluExp, numerics: str, name: str, params: st
     BN = int(tile.get("CBN", 256 if NV >= 256 else 128))
     wide = O % 128 == 0 and O >= 256 and -(-NV // BN) * (O // 128) * cv["NB"] >= tuner.CU_COUNT
     BM = int(tile.get("CBM", 128 if wide else 64))
-    WM, WN = 2, 2
+    WM, WN = int(tile.get("CWM", 2)), int(tile.get("CWN", 2))
     if O % BM or BM % (32 * WM) or BN % (32 * WN) or BN % 4:
         return None
     # output rows a tile's BN consecutive positions span; the image rows behind them live in SY planes (by row % SY) of
