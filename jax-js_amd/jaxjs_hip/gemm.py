@@ -718,7 +718,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         # cast-and-store epilogue measures the same either way and keeps the simpler path.
         has_loads = bool(epilogue.collect(lambda x: x.op == AluOp.GlobalIndex)) and split == 1
         vec = (split == 1 and tile.get("VEPI", 1 if has_loads else 0) and g["c_sn"] == 1 and g["c_sm"] % 8 == 0 and all(b[3] % 8 == 0 for b in g["batch"])
-               and kernel.dtype != DType.Bool)
+               and kernel.dtype != DType.Bool and (g["N"] % BN == 0 or g["N"] % 8 == 0))  # an edge tile ends on a whole group of 8
         if vec:
             vnames = {"acc": "acc", "row": "row", "col": "col", "b0": "b0", "b1": "b1", "b2": "b2"}
             body = _Body(epilogue, names, vnames, "col", "c0", 8, classify_loads(epilogue, "col", 8), numerics, "      ", "e")
