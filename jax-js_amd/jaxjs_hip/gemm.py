@@ -158,6 +158,10 @@ def choose_tile(g: dict) -> Dict[str, int]:
         # slices cost more in partial sums than they gain).
         if tiles(128, 128) * 2 <= CU and g["K"] >= 2048 and g["K"] % 128 == 0:
             tile.update(SPLITK=4 if tiles(128, 128) * 4 <= CU and g["K"] >= 4096 and g["K"] % 256 == 0 else 2)
+            # The slices take 32-deep slabs in four stages (64 KiB, so two workgroups fit a CU): as fast as the 64-deep
+            # ones at their best and steady, where those swing between 21 and 28 us from launch to launch
+            # (16 x 14336 x 4096: 20.2-20.7 us against 24-27; 128 rows: 26.0-26.6 against 29.6-32.9).
+            tile.update(BK=32, STAGES=4)
             # Folding inside the launch is the direct-to-LDS template's: operands on the 16-byte grid, edges it can clamp.
             # Other shapes keep the split and fold in a second launch.
             # Two slices only: with four, the last workgroup's read-back of four slices behind the acknowledged stores

@@ -371,7 +371,7 @@ SWEEP = [
     (DType.Float16, 2048, 2048, 2048, dict(BM=128, BN=128, BK=64, stages=4, tiles=256, splitk=1, direct_lds=True)),
     (DType.Float16, 4096, 4096, 4096, dict(BM=256, BN=256, BK=32, tiles=256, splitk=1, direct_lds=True)),
     # fewer tiles than CUs: the k axis is cut over blockIdx.y, f32 partials in scratch, folded inside the launch
-    (DType.Float16, 128, 14336, 4096, dict(BM=128, BN=128, BK=64, stages=4, tiles=112, splitk=2, direct_lds=True, fused_fold=True)),
+    (DType.Float16, 128, 14336, 4096, dict(BM=128, BN=128, BK=32, stages=4, tiles=112, splitk=2, direct_lds=True, fused_fold=True)),
     # f32 k splits are folded inside the launch by the last slice to arrive at the tile's counter
     (DType.Float32, 1024, 1024, 1024, dict(BM=128, BN=64, BK=32, tiles=128, splitk=4, fused_fold=True)),
     (DType.Float32, 2048, 2048, 2048, dict(BM=128, BN=64, BK=32, tiles=512, splitk=1)),
