@@ -19,3 +19,93 @@ def test_every_contraction_shape_gets_a_plan():
             for bt in (False, True):
                 ks = generate(matmulKernel(*shape, dt, b_transposed=bt), "fast")
                 assert ks.steps and ks.sources, (dt, shape, bt)
+
+
+PINNED_PLANS = [
+    # dtype, M, N, K, B stored [N,K] -> what the plan must say
+    # whole tiles
+    (DType.Float16, 8192, 8192, 8192, False, dict(BM=256, BN=256, direct_lds=True, splitk=1)),
+    (DType.Float16, 2048, 2048, 2048, False, dict(BM=128, BN=128, BK=64, stages=4, direct_lds=True, splitk=1)),
+    # edge tiles on the direct-to-LDS template: clamped loads
+    (DType.Float16, 8000, 8000, 8000, False, dict(BM=256, BN=256, direct_lds=True, splitk=1)),
+    (DType.Float16, 1000, 1001, 512, True, dict(BM=128, BN=128, direct_lds=True)),
+    (DType.Float16, 100, 14336, 4096, False, dict(BM=128, BN=128, BK=32, direct_lds=True, splitk=2, fused_fold=True)),
+    # rows of B off the 16-byte grid: repack pre-pass when the other side has >= 512 rows, the general template below
+    (DType.Float16, 8192, 50257, 768, False, dict(BM=256, BN=256, direct_lds=True, repack="b")),
+    (DType.Float16, 300, 1001, 512, False, dict(direct_lds=False)),
+    # a k axis that is not whole slabs stays on the general template
+    (DType.Float16, 4100, 4100, 4100, False, dict(direct_lds=False)),
+    # a few rows against a large matrix: clamped rows on 128x128 tiles, k in slices, fold launch
+    (DType.Float16, 4, 14336, 4096, False, dict(BM=128, BN=128, BK=32, stages=4, direct_lds=True, splitk=2)),
+    (DType.Float16, 31, 4096, 4096, True, dict(BM=128, BN=128, direct_lds=True, splitk=4)),
+    (DType.Float16, 16, 14336, 4000, False, dict(BM=64, BN=128, direct_lds=False)),
+    # short k under many tiles: shallow stages, several workgroups per CU
+    (DType.Float16, 8192, 3072, 768, False, dict(BM=128, BN=256, BK=32, stages=2, direct_lds=True)),
+    (DType.Float16, 8192, 768, 3072, False, dict(BM=128, BN=256, stages=4, direct_lds=True)),
+    # f32: small shapes in 64x64 tiles with in-launch k slices, the rest unchanged
+    (DType.Float32, 256, 256, 256, False, dict(BM=64, BN=64, splitk=4, fused_fold=True)),
+    (DType.Float32, 512, 512, 512, True, dict(BM=64, BN=64, splitk=4, fused_fold=True)),
+    (DType.Float32, 1024, 1024, 1024, False, dict(BM=128, BN=64, splitk=4, fused_fold=True)),
+    (DType.Float32, 4096, 4096, 4096, False, dict(BM=128, BN=128, splitk=1)),
+]
+
+
+def test_gemm_plans_are_pinned():
+    """The launch plan the tile chooser picks for the shapes its rules were measured on."""
+    from jaxjs_hip.lowering import matmulKernel
+    for dt, M, N, K, bt, want in PINNED_PLANS:
+        ks = generate(matmulKernel(M, N, K, dt, b_transposed=bt), "fast")
+        assert ks.klass.startswith("gemm"), (M, N, K, ks.klass)
+        got = {key: ks.info.get(key) for key in want}
+        assert got == want, ((dt.value, M, N, K, bt), got, want)
+        if want.get("repack"):
+            assert [s.name.rsplit("_", 1)[-1] for s in ks.steps][0] == "repack" and len(ks.scratch_bytes) == 1
+            assert ks.scratch_bytes[0] == K * (-(-N // 8) * 8) * 2
+
+
+def _direct_lds_load_offsets(rows, bk, nwaves, k_contiguous, row_stride, k_stride, last):
+    """Element offsets (from the tile's first row and the slab's first k) of every 16-byte load of one operand slab, as the
+    direct-to-LDS template computes them: (tile row or first row of the group, k or first k of the chunk, offset)."""
+    out = []
+    for q in range(rows * bk * 2 // 1024 // nwaves):
+        for wave in range(nwaves):
+            inst = q * nwaves + wave
+            for lane in range(64):
+                if k_contiguous:
+                    lpr = bk // 8
+                    row = inst * (64 // lpr) + lane // lpr
+                    swz = (row >> 2) & 3 if bk == 32 else (row >> 1) & 7
+                    lc = (lane % lpr) ^ swz
+                    out.append((row, lc * 8, min(row, last) * row_stride + lc * 8))
+                else:
+                    row_bytes = rows * 2
+                    off = lane * 16
+                    k = inst * (1024 // row_bytes) + off // row_bytes
+                    pc = (off % row_bytes) >> 4
+                    lchunk = (((pc >> 2) ^ (k & 3)) << 2) | (pc & 3)
+                    lastc = (last + 1) // 8 - 1
+                    out.append((lchunk * 8, k, k * k_stride + min(lchunk, lastc) * 8))
+    return out
+
+
+def test_clamped_edge_loads_stay_inside_the_operand():
+    """A model of the direct-to-LDS loaders' source addresses (the arithmetic of `jh_lane_offset` with its clamp to the
+    last row, or last whole group of eight rows, that exists): for operands whose extent is not whole tiles every
+    16-byte load lies inside the operand, and the rows that exist read their own elements."""
+    cases = [(8000, 64, 256, 32, 4, True), (8000, 128, 256, 64, 4, True), (8000, 64, 256, 32, 4, False), (136, 64, 128, 32, 4, False),
+             (100, 64, 128, 32, 4, True), (50257, 64, 256, 32, 4, True), (50264, 64, 128, 64, 4, False), (8, 64, 128, 32, 4, False),
+             (1, 64, 128, 32, 4, True), (4104, 96, 256, 32, 8, False)]
+    for extent, K, tile, bk, nwaves, k_contiguous in cases:
+        row_stride, k_stride = (K, 1) if k_contiguous else (1, extent)
+        for t in range(-(-extent // tile)):
+            r0 = t * tile
+            last = min(extent - 1 - r0, tile - 1)
+            for slab in range(K // bk):
+                base = r0 * row_stride + slab * bk * k_stride
+                for r, kk, src in _direct_lds_load_offsets(tile, bk, nwaves, k_contiguous, row_stride, k_stride, last):
+                    a = base + src
+                    assert 0 <= a and a + 8 <= extent * K, (extent, K, tile, t, slab, r, kk)
+                    if k_contiguous and r <= last:
+                        assert a == (r0 + r) * K + slab * bk + kk
+                    if not k_contiguous and r + 7 <= last:
+                        assert a == (slab * bk + kk) * extent + r0 + r
