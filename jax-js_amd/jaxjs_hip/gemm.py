@@ -48,8 +48,8 @@ def choose_tile(g: dict) -> Dict[str, int]:
     loose_ops = bool(g.get("a_loose") or g.get("b_loose")) and repack is None
 
     def edge_ok(bm, bn):
-        return ((repack == "a" or _edge_ok(g["M"], bm, g["a_sk"] == 1))
-                and (repack == "b" or _edge_ok(g["N"], bn, g["b_sk"] == 1)))
+        return (("a" in (repack or "") or _edge_ok(g["M"], bm, g["a_sk"] == 1))
+                and ("b" in (repack or "") or _edge_ok(g["N"], bn, g["b_sk"] == 1)))
 
     if g["dtype"] == DType.Float32:
         # The f32 matrix pipe is 16x slower than the f16 one, so LDS traffic matters little and filling
@@ -136,7 +136,7 @@ def choose_tile(g: dict) -> Dict[str, int]:
         per_cu = -(-tiles(bm, bn) // tuner.CU_COUNT)
         if (bm, bn) == (128, 128) and per_cu < 2:
             eff = 0.64
-        whole = edge_ok(bm, bn) and g["K"] % 32 == 0 and plain_k and not loose_ops
+        whole = edge_ok(bm, bn) and (g["K"] % 32 == 0 or repack is not None) and plain_k and not loose_ops
         if not whole:
             # A ragged k axis, operands off the 16-byte grid or an edge the direct loads cannot clamp run the general
             # template, whose small tiles lose more
@@ -182,24 +182,29 @@ def choose_tile(g: dict) -> Dict[str, int]:
 
 
 def _repack_operand(g: dict):
-    """The operand ("a" or "b") that a pre-pass copies onto the 16-byte grid before the direct-to-LDS template reads it,
-    or None.  An f16 operand that runs along its rows in memory with rows off the grid (np.matmul against a [K, N]
-    matrix with N = 50257: every row starts at an odd element) would otherwise send the whole GEMM to the general
-    template (8192 x 50257 x 768: 1.19 ms); copied once into scratch as [K][rows rounded up to 8] (K x rows x 4 bytes of
-    traffic) the GEMM runs on the fast path.  Worth it when the other operand has enough rows to amortise the copy."""
+    """The operands ("a", "b" or "ab") that a pre-pass copies into scratch before the direct-to-LDS template reads them,
+    or None.  That template loads whole 16-byte groups from the 16-byte grid and walks k in whole 32-deep slabs; an
+    f16 operand off the grid (np.matmul against a [K, N] matrix with N = 50257: every row starts at an odd element) or a
+    k axis that is not whole slabs (k = 50257, 4100, 1000) would otherwise send the whole GEMM to the general template
+    (8192 x 50257 x 768: 1.19 ms against 0.80 ms).  The copy keeps the operand's orientation -- [rows][k] or [k][rows] --
+    with rows rounded up to 8 and k to 32, zeros in the padding (2 x 2 bytes of traffic per element); a ragged k axis
+    takes both operands.  Worth it when the other operand has enough rows to amortise the copy."""
     if g["dtype"] != DType.Float16 or g["batch"] or g.get("a_gather") or g.get("b_gather"):
         return None
-    if g["K"] % 32 or g["a_k0"] != g["K"] or g["b_k0"] != g["K"]:
+    if g["a_k0"] != g["K"] or g["b_k0"] != g["K"] or g["K"] < 64:
         return None
-    loose = [t for t in ("a", "b") if g.get(t + "_loose")]
-    if len(loose) != 1:
+    ragged_k = g["K"] % 32 != 0
+    tags = "".join(t for t in ("a", "b") if g.get(t + "_loose") or ragged_k)
+    if not tags:
         return None
-    tag = loose[0]
-    srow = g["a_sm"] if tag == "a" else g["b_sn"]
-    rows, other = (g["M"], g["N"]) if tag == "a" else (g["N"], g["M"])
-    if srow != 1 or rows < 128 or other < 512:
-        return None
-    return tag
+    for t in tags:
+        rows, other = (g["M"], g["N"]) if t == "a" else (g["N"], g["M"])
+        srow, sk = (g["a_sm"], g["a_sk"]) if t == "a" else (g["b_sn"], g["b_sk"])
+        if (srow != 1 and sk != 1) or rows < 128 or other < 512:
+            return None
+    if sum((g["M"] if t == "a" else g["N"]) for t in tags) * (g["K"] + 32) * 2 > (1 << 30):
+        return None  # more than 1 GiB of copies: not at the price of that much scratch
+    return tags
 
 
 def _edge_ok(extent: int, tile: int, k_contiguous: bool) -> bool:
@@ -442,13 +447,20 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     # dense [K][rows_pad] operand named `jh_repack`.
     repack = _repack_operand(g) if split == 1 and tile.get("REPACK", 1) else None
     load_rows = dict(a=g["M"], b=g["N"])
-    repack_src = None
+    repack_src = {}
     if repack:
-        rows = load_rows[repack]
-        rows_pad = -(-rows // 8) * 8
-        repack_src = dict(gid=g["gid_" + repack], off=g[repack + "_off"], sk=g[repack + "_sk"], rows=rows, rows_pad=rows_pad)
-        load_rows[repack] = rows_pad
-        g = dict(g, **{repack + "_off": 0, repack + "_sk": rows_pad, repack + "_loose": False})
+        k_pad = -(-g["K"] // 32) * 32
+        for tg in repack:
+            rows = load_rows[tg]
+            srow = g["a_sm"] if tg == "a" else g["b_sn"]
+            rkey = "a_sm" if tg == "a" else "b_sn"
+            kc = g[tg + "_sk"] == 1  # runs along k: copied as [rows][k_pad]; else along its rows: [k_pad][rows_pad]
+            rows_pad = rows if kc else -(-rows // 8) * 8
+            repack_src[tg] = dict(gid=g["gid_" + tg], off=g[tg + "_off"], sk=g[tg + "_sk"], srow=srow, rows=rows, rows_pad=rows_pad,
+                                  k=g["K"], k_pad=k_pad, kc=kc)
+            load_rows[tg] = rows_pad
+            g = dict(g, **{tg + "_off": 0, tg + "_sk": 1 if kc else rows_pad, rkey: k_pad if kc else 1, tg + "_loose": False})
+        g = dict(g, K=k_pad, a_k0=k_pad, b_k0=k_pad)
 
     used = _used_args(kernel.nargs, t.epilogue)
     used[g["gid_a"]] = g["dtype"]
@@ -457,7 +469,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     params = ", ".join(
         [f"const {STORAGE_CTYPE[d or DType.Float32]}* __restrict__ {n}" for d, n in zip(used, names)]
         + [f"{out_t}* __restrict__ out"] + (["float* __restrict__ jh_part", "unsigned* __restrict__ jh_count"] if fusek else [])
-        + (["const jh_f16* __restrict__ jh_repack"] if repack else []))
+        + [f"const jh_f16* __restrict__ jh_repack_{tg}" for tg in (repack or "")])
 
     # Fused epilogue as a device function of (acc, row, col, batch coordinates, buffers...).  The kernel's
     # epilogue is written over the flat output index; here that index is re-expressed through the tile's own
@@ -747,7 +759,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         B_KCONTIG=0 if gather_flags["b"] in (2, 3) else (1 if g["b_sk"] == 1 or g["K"] == 1 or gather_flags["b"] in (1, 4) else 0),
         NBATCH=nbatch, EPILOGUE_FN=epi_fn, NAME=name, PARAMS=params,
         A_OFF=g["a_off"], B_OFF=g["b_off"], BATCH_DECODE="\n".join(lines),
-        A_PTR="jh_repack" if repack == "a" else names[g["gid_a"]], B_PTR="jh_repack" if repack == "b" else names[g["gid_b"]],
+        A_PTR="jh_repack_a" if "a" in (repack or "") else names[g["gid_a"]], B_PTR="jh_repack_b" if "b" in (repack or "") else names[g["gid_b"]],
         A_SM=g["a_sm"], A_SK=g["a_sk"], B_SN=g["b_sn"], B_SK=g["b_sk"],
         A_K0=g["a_k0"], A_SK1=g["a_sk1"], B_K0=g["b_k0"], B_SK1=g["b_sk1"],
         C_SM=g["c_sm"], C_SN=g["c_sn"], EPILOGUE_ARGS=epi_args))
@@ -773,31 +785,45 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         if tap_major is not None:
             info["tap_major"] = tap_major
     if repack:
-        rs = repack_src
-        groups = rs["rows_pad"] // 8
-        src += (f"""
-// Operand [K][{rs['rows']} rows] (k stride {rs['sk']} elements, first element {rs['off']}: rows off the 16-byte grid) -> jh_repack [K][{rs['rows_pad']}],
-// eight rows per thread: one under-aligned 16-byte load, one aligned store; the rows past the end are zeros.
-struct __attribute__((packed, aligned(2))) jh_half8_u {{ jh_half8 v; }};
-extern "C" __global__ __launch_bounds__(256) void {name}_repack(const jh_f16* __restrict__ src, jh_f16* __restrict__ dst) {{
+        src += "\nstruct __attribute__((packed, aligned(2))) jh_half8_u { jh_half8 v; };\n"
+        preps, scratch = [], []
+        for si, tg in enumerate(repack):
+            rs = repack_src[tg]
+            if rs["kc"]:
+                groups, outer, total = rs["k_pad"] // 8, rs["rows"], rs["rows"] * (rs["k_pad"] // 8)
+                body = (f"  const int r = (int)(i / {groups}), k0 = (int)(i % {groups}) * 8;\n"
+                        f"  const jh_f16* __restrict__ p = src + {rs['off']}ll + (long long)r * {rs['srow']}ll + k0;\n"
+                        f"  const int valid = {rs['k']} - k0;\n"
+                        f"  jh_f16* const q = dst + (long long)r * {rs['k_pad']} + k0;\n")
+                what = f"[{rs['rows']} rows][{rs['k']} k] (row stride {rs['srow']}) -> [{rs['rows']}][{rs['k_pad']}]"
+            else:
+                groups, total = rs["rows_pad"] // 8, rs["k_pad"] * (rs["rows_pad"] // 8)
+                body = (f"  const int k = (int)(i / {groups}), r0 = (int)(i % {groups}) * 8;\n"
+                        f"  const jh_f16* __restrict__ p = src + {rs['off']}ll + (long long)k * {rs['sk']}ll + r0;\n"
+                        f"  const int valid = k < {rs['k']} ? {rs['rows']} - r0 : 0;\n"
+                        f"  jh_f16* const q = dst + (long long)k * {rs['rows_pad']} + r0;\n")
+                what = f"[{rs['k']} k][{rs['rows']} rows] (k stride {rs['sk']}) -> [{rs['k_pad']}][{rs['rows_pad']}]"
+            src += (f"""
+// Operand {tg.upper()} {what}, first element {rs['off']}: eight elements per thread, one under-aligned 16-byte load and one
+// aligned store; what lies past the operand's extents is zeros.
+extern "C" __global__ __launch_bounds__(256) void {name}_repack_{tg}(const jh_f16* __restrict__ src, jh_f16* __restrict__ dst) {{
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
-  if (i >= {g['K']}ll * {groups}) return;
-  const int k = (int)(i / {groups}), r0 = (int)(i % {groups}) * 8;
-  const jh_f16* __restrict__ p = src + {rs['off']}ll + (long long)k * {rs['sk']}ll + r0;
-  jh_half8 v;
-  if (r0 + 8 <= {rs['rows']}) {{
+  if (i >= {total}ll) return;
+{body}  jh_half8 v;
+  if (valid >= 8) {{
     v = reinterpret_cast<const jh_half8_u*>(p)->v;
   }} else {{
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = r0 + e < {rs['rows']} ? p[e] : (jh_f16)0.0f;
+    for (int e = 0; e < 8; ++e) v[e] = e < valid ? p[e] : (jh_f16)0.0f;
   }}
-  *reinterpret_cast<jh_half8*>(dst + (long long)k * {rs['rows_pad']} + r0) = v;
+  *reinterpret_cast<jh_half8*>(q) = v;
 }}
 """)
-        prep = LaunchStep(name + "_repack", (-(-g["K"] * groups // 256), 1, 1), (256, 1, 1), 0, [("in", rs["gid"]), ("scratch", 0)])
-        step.args.append(("scratch", 0))
+            preps.append(LaunchStep(f"{name}_repack_{tg}", (-(-total // 256), 1, 1), (256, 1, 1), 0, [("in", rs["gid"]), ("scratch", si)]))
+            step.args.append(("scratch", si))
+            scratch.append(rs["k_pad"] * rs["rows_pad"] * 2)
         info["repack"] = repack
-        return KernelSource([src], [prep, step], [g["K"] * rs["rows_pad"] * 2], "gemm", need, info)
+        return KernelSource([src], preps + [step], scratch, "gemm", need, info)
     if split == 1:
         return KernelSource([src], [step], [], "gemm", need, info)
     if fusek:

@@ -250,7 +250,7 @@ LOOSE_CASES = [
     # dtype, M, N, K, B stored [N,K], batch
     (DType.Float16, 130, 257, 100, False, ()), (DType.Float16, 130, 257, 100, True, ()), (DType.Float16, 333, 1001, 515, False, ()),
     (DType.Float16, 333, 1001, 515, True, ()), (DType.Float16, 64, 50257 // 16, 768, False, ()), (DType.Float16, 257, 129, 66, False, (3,)),
-    (DType.Float16, 1025, 1027, 1029, False, ()), (DType.Float16, 200, 72, 4100, True, ()),
+    (DType.Float16, 400, 1027, 1029, False, ()), (DType.Float16, 200, 72, 4100, True, ()),
     (DType.Float32, 130, 257, 101, False, ()), (DType.Float32, 130, 257, 101, True, ()), (DType.Float32, 333, 1001, 515, False, ()),
     (DType.Float32, 129, 66, 257, True, (2,)), (DType.Float32, 1025, 1027, 1029, False, ()),
 ]
@@ -298,6 +298,9 @@ REPACK_CASES = [
     # M, N, K, layout, element offset of the off-grid operand's view, tile options
     (520, 1001, 512, "NN", 0, dict()), (1024, 50257 // 16, 768, "NN", 0, dict()), (1001, 520, 256, "TN", 0, dict()),
     (512, 256, 128, "NN", 3, dict()), (640, 777, 96, "NN", 1, dict(BM=256, BN=256)), (513, 1001, 64, "NN", 0, dict(BM=256, BN=128, SADDR=0)),
+    # a k axis that is not whole slabs: both operands copied, k padded with zeros
+    (520, 600, 1000, "NN", 0, dict()), (1000, 1000, 1000, "NT", 0, dict()), (515, 1001, 333, "NT", 0, dict()), (1001, 520, 100, "TN", 0, dict()),
+    (600, 520, 72, "NN", 1, dict(BM=256, BN=256)), (1027, 1025, 1029, "NN", 0, dict()),
 ]
 
 
@@ -305,7 +308,8 @@ REPACK_CASES = [
 def test_gemm_f16_rows_off_the_grid_are_repacked(M, N, K, layout, off, tile):
     """np.matmul against a [K, 1001] matrix: every row of B starts at an odd element.  With enough rows on the other side a
     pre-pass copies B into scratch as [K][1008] and the direct-to-LDS template runs on the copy (edge tiles clamped, the
-    padding never stored).  Small integer entries: exact in every element."""
+    padding never stored); a k axis that is not whole 32-deep slabs takes copies of both operands with k padded by
+    zeros.  Small integer entries: exact in every element."""
     A = RNG.integers(-2, 3, (M, K)).astype(np.float16)
     B = RNG.integers(-2, 3, (K, N)).astype(np.float16)
     full = [M, N, K]
@@ -315,12 +319,20 @@ def test_gemm_f16_rows_off_the_grid_are_repacked(M, N, K, layout, off, tile):
         bbuf = B
         stB = ShapeTracker.fromShape([K, N]).permute([1, 0]).reshape([1, N, K]).expand(full)
         want = "a"
+    elif layout == "NT":  # B stored [N, K]
+        abuf = A
+        stA = ShapeTracker.fromShape([M, K]).reshape([M, 1, K]).expand(full)
+        bbuf = np.concatenate([np.zeros(off, np.float16), np.ascontiguousarray(B.T).ravel()])
+        stB = ShapeTracker.fromShape([N * K + off]).shrink([(off, N * K + off)]).reshape([1, N, K]).expand(full)
+        want = "b"
     else:
         abuf = A
         stA = ShapeTracker.fromShape([M, K]).reshape([M, 1, K]).expand(full)
         bbuf = np.concatenate([np.zeros(off, np.float16), B.ravel()])
         stB = ShapeTracker.fromShape([K * N + off]).shrink([(off, K * N + off)]).reshape([K, N]).permute([1, 0]).reshape([1, N, K]).expand(full)
         want = "b"
+    if K % 32:
+        want = "ab"
     k = _f32_out(reduceKernel(full, [(DType.Float16, stA), (DType.Float16, stB)], lambda a, b: AluExp.mul(a, b), AluOp.Add), K)
     opts = dict(gemm_tile=tuple(sorted(tile.items()))) if tile else {}
     got, ks = device_run(k, [abuf, bbuf], **opts)

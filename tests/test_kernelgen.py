@@ -33,8 +33,13 @@ PINNED_PLANS = [
     # rows of B off the 16-byte grid: repack pre-pass when the other side has >= 512 rows, the general template below
     (DType.Float16, 8192, 50257, 768, False, dict(BM=256, BN=256, direct_lds=True, repack="b")),
     (DType.Float16, 300, 1001, 512, False, dict(direct_lds=False)),
-    # a k axis that is not whole slabs stays on the general template
-    (DType.Float16, 4100, 4100, 4100, False, dict(direct_lds=False)),
+    # a k axis that is not whole slabs: both operands copied with k padded to 32 (zeros), unless the copies are huge or the
+    # shape is small
+    (DType.Float16, 4100, 4100, 4100, False, dict(BM=128, BN=256, direct_lds=True, repack="ab")),
+    (DType.Float16, 1000, 1000, 1000, True, dict(BM=128, BN=128, direct_lds=True, repack="ab")),
+    (DType.Float16, 8192, 768, 50257, False, dict(direct_lds=True, repack="ab")),
+    (DType.Float16, 16384, 16384, 16400, False, dict(direct_lds=False, repack=None)),
+    (DType.Float16, 300, 300, 1000, False, dict(direct_lds=False, repack=None)),
     # a few rows against a large matrix: clamped rows on 128x128 tiles, k in slices, fold launch
     (DType.Float16, 4, 14336, 4096, False, dict(BM=128, BN=128, BK=32, stages=4, direct_lds=True, splitk=2)),
     (DType.Float16, 31, 4096, 4096, True, dict(BM=128, BN=128, direct_lds=True, splitk=4)),
@@ -59,7 +64,9 @@ def test_gemm_plans_are_pinned():
         got = {key: ks.info.get(key) for key in want}
         assert got == want, ((dt.value, M, N, K, bt), got, want)
         if want.get("repack"):
-            assert [s.name.rsplit("_", 1)[-1] for s in ks.steps][0] == "repack" and len(ks.scratch_bytes) == 1
+            assert [s.name.rsplit("_", 2)[-2] for s in ks.steps][:len(want["repack"])] == ["repack"] * len(want["repack"])
+            assert len(ks.scratch_bytes) == len(want["repack"])
+        if want.get("repack") == "b" and not bt:
             assert ks.scratch_bytes[0] == K * (-(-N // 8) * 8) * 2
 
 
