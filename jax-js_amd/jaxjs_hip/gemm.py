@@ -593,6 +593,37 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
             gather_flags[tag] = 2
             gather_group[tag] = G
 
+        # float32: four consecutive rows of an aligned group as one 128-bit load (the image of a stride-1 convolution),
+        # the operand staged like one that runs along its rows.  Groups whose bytes would leave the buffer take the
+        # element loader, which applies the mask itself.
+        if g["dtype"] == DType.Float32 and tile.get("ROWS4", 1) and extent % 4 == 0 and g["K"] % 8 == 0:
+            r4 = rows8_form(oexp, extent, 4)
+            if r4 is not None:
+                idx0, cond_e, gnode = r4
+                vnames = {"row": "row", "e": "e", "k": "k", "b0": "b0", "b1": "b1", "b2": "b2"}
+                icg = HipExpCodegen(names, vnames, "  ", prefix=f"i{tag}", numerics=numerics)
+                icg.countReferences(idx0)
+                ival = strip_parens(icg.run(idx0))
+                gather_fns.append(f"static __device__ __forceinline__ int jh_gindex_{tag}(int row, int k, int b0, int b1, int b2) {{\n"
+                                  + "\n".join(icg.take_lines()) + f"\n  return {ival};\n}}")
+                maskbit = "true"
+                if cond_e is not None:
+                    mcg = HipExpCodegen(names, vnames, "  ", prefix=f"m{tag}", numerics=numerics)
+                    mcg.countReferences(cond_e)
+                    mval = strip_parens(mcg.run(cond_e))
+                    gather_fns.append(f"static __device__ __forceinline__ bool jh_gmask_{tag}(int row, int e, int k, int b0, int b1, int b2) {{\n"
+                                      + "\n".join(mcg.take_lines()) + f"\n  return {mval};\n}}")
+                    maskbit = f"jh_gmask_{tag}(row, e, k, b0, b1, b2)"
+                buf = names[gnode.arg[0]]
+                gather_fns.append(
+                    f"static __device__ __forceinline__ jh_float4 jh_gather4_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
+                    f"  const int i0 = jh_gindex_{tag}(row, k, b0, b1, b2);\n  jh_float4 v;\n"
+                    f"  if ((unsigned)i0 <= (unsigned)({gnode.arg[1]} - 4)) {{\n    __builtin_memcpy(&v, {buf} + i0, 16);\n"
+                    f"#pragma unroll\n    for (int e = 0; e < 4; ++e) v[e] = {maskbit} ? v[e] : 0.0f;\n  }} else {{\n"
+                    f"#pragma unroll\n    for (int e = 0; e < 4; ++e) v[e] = jh_gather_{tag}(row + e, k, b0, b1, b2{epi_args});\n  }}\n  return v;\n}}")
+                gather_calls[tag] = f"jh_gather4_{tag}(row, k, jh_b0, jh_b1, jh_b2{epi_args})"
+                gather_flags[tag], gather_group[tag] = 5, 4
+
     # Tap-major k order (see `tap_major_form`): one gather operand whose k splits into (channel, tap), the other a plain
     # strided operand.  Both are then loaded through block/chunk loaders that take the first k' of eight consecutive
     # ones: k' = tap * C + c, original k = c * T + tap.
@@ -755,8 +786,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                      GATHER_A_SLOW=gather_slow.get("a", "jh_half8{0, 0, 0, 0, 0, 0, 0, 0}"), GATHER_B_SLOW=gather_slow.get("b", "jh_half8{0, 0, 0, 0, 0, 0, 0, 0}"))
     src = _prelude(numerics) + fill(template(tmpl), dict(sched, 
         M=g["M"], N=g["N"], K=g["K"], M_LOAD=load_rows["a"], N_LOAD=load_rows["b"], BM=BM, BN=BN, WM=WM, WN=WN,
-        A_KCONTIG=0 if gather_flags["a"] in (2, 3) else (1 if g["a_sk"] == 1 or g["K"] == 1 or gather_flags["a"] in (1, 4) else 0),
-        B_KCONTIG=0 if gather_flags["b"] in (2, 3) else (1 if g["b_sk"] == 1 or g["K"] == 1 or gather_flags["b"] in (1, 4) else 0),
+        A_KCONTIG=0 if gather_flags["a"] in (2, 3, 5) else (1 if g["a_sk"] == 1 or g["K"] == 1 or gather_flags["a"] in (1, 4) else 0),
+        B_KCONTIG=0 if gather_flags["b"] in (2, 3, 5) else (1 if g["b_sk"] == 1 or g["K"] == 1 or gather_flags["b"] in (1, 4) else 0),
         NBATCH=nbatch, EPILOGUE_FN=epi_fn, NAME=name, PARAMS=params,
         A_OFF=g["a_off"], B_OFF=g["b_off"], BATCH_DECODE="\n".join(lines),
         A_PTR="jh_repack_a" if "a" in (repack or "") else names[g["gid_a"]], B_PTR="jh_repack_b" if "b" in (repack or "") else names[g["gid_b"]],
@@ -781,7 +812,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         info.update(stages=sched["STAGES"], ring=sched["RING"])
     if any_gather:
         info["gather"] = {tag: {0: "none", 1: "element", 2: f"rows{gather_group.get(tag, 8)}", 3: f"tap-major rows{gather_group.get(tag, 8)}",
-                                4: "tap-major strided"}[gather_flags[tag]] for tag in ("a", "b")}
+                                4: "tap-major strided", 5: "rows4"}[gather_flags[tag]] for tag in ("a", "b")}
         if tap_major is not None:
             info["tap_major"] = tap_major
     if repack:

@@ -401,6 +401,60 @@ def test_f16_convolution_loader_choice(case):
         assert tm.info["tap_major"]["T"] == int(np.prod(case["w"][2:])) and any(v.startswith("tap-major rows") for v in tm.info["gather"].values())
 
 
+# float32 convolutions on the gather loaders: stride-1 windows whose output width is a multiple of 4 read four consecutive
+# output positions with one 128-bit load (masked lanes zeroed), everything else element by element.
+F32_CONV_CASES = [
+    dict(x=(2, 8, 16, 16), w=(32, 8, 3, 3), strides=[1, 1], padding="SAME", loader="rows4"),
+    dict(x=(2, 8, 30, 30), w=(32, 8, 3, 3), strides=[1, 1], padding="VALID", loader="rows4"),
+    dict(x=(1, 8, 20, 40), w=(32, 8, 5, 5), strides=[1, 1], padding=[(3, 1), (0, 4)], loader="rows4"),
+    dict(x=(2, 8, 24, 24), w=(32, 8, 3, 3), strides=[1, 1], padding="SAME", rd=[2, 2], loader="rows4"),
+    dict(x=(2, 16, 64), w=(32, 16, 3), strides=[1], padding="SAME", loader="rows4"),
+    dict(x=(2, 8, 14, 14), w=(32, 8, 3, 3), strides=[1, 1], padding="SAME", loader="element"),
+    dict(x=(2, 8, 32, 32), w=(32, 8, 3, 3), strides=[2, 2], padding="SAME", loader="element"),
+    dict(x=(4, 16, 28, 28), w=(64, 16, 3, 3), strides=[1, 1], padding="SAME", loader="rows4"),
+]
+
+
+def _f32_conv_program(c):
+    return J.jit(lambda a, b: L.convGeneralDilated(a, b, c["strides"], c["padding"], rhsDilation=c.get("rd")),
+                 [ShapedArray(c["x"], DType.Float32), ShapedArray(c["w"], DType.Float32)])
+
+
+@pytest.mark.parametrize("case", F32_CONV_CASES, ids=lambda c: "x".join(map(str, c["x"])) + "*" + "x".join(map(str, c["w"])))
+def test_f32_convolution_loader_choice(case):
+    from jaxjs_hip.kernelgen import generate
+    ks = generate(_f32_conv_program(case).kernels[0])
+    assert ks.klass.startswith("gemm") and case["loader"] in ks.info["gather"].values(), ks.info
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", F32_CONV_CASES, ids=lambda c: "x".join(map(str, c["x"])) + "*" + "x".join(map(str, c["w"])))
+def test_f32_convolution_on_gpu_is_exact_on_small_integers(case):
+    from gpu_util import WARM_ONLY, backend
+    prog = _f32_conv_program(case)
+    if WARM_ONLY:
+        from jaxjs_hip.kernelgen import generate
+        from jaxjs_hip.runtime import compile_source
+        for src in generate(prog.kernels[0]).sources:
+            compile_source(src)
+        pytest.skip("warm-up run: compiled only")
+    rng = np.random.default_rng(13)
+    x = rng.integers(-2, 3, case["x"]).astype(np.float32)
+    w = rng.integers(-2, 3, case["w"]).astype(np.float32)
+    be = backend()
+    exe = be.prepareKernelSync(prog.kernels[0])
+    sx, sw, so = be.malloc(x.nbytes, x.tobytes()), be.malloc(w.nbytes, w.tobytes()), be.malloc(prog.kernels[0].bytes)
+    be.dispatch(exe, [sx, sw], [so])
+    r = np.frombuffer(be.readSync(so), np.float32).copy()
+    for s_ in (sx, sw, so):
+        be.decRef(s_)
+    pads = case["padding"]
+    if isinstance(pads, str):
+        pads = L.padtypeToPads(case["x"][2:], case["w"][2:], case["strides"], case.get("rd") or [1] * len(case["strides"]), pads)
+    want = conv_reference(x, w, case["strides"], pads, None, case.get("rd"))
+    np.testing.assert_array_equal(r.reshape(want.shape).astype(np.float64), want)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("tap_major", [0, 1], ids=["k-order", "tap-major"])
 @pytest.mark.parametrize("case", F16_CONV_CASES, ids=lambda c: "x".join(map(str, c["x"])) + "*" + "x".join(map(str, c["w"])))
