@@ -624,6 +624,69 @@ class AluExp:
 
         return self.rewrite(visit)
 
+    def _pureNonNegativeIndex(self) -> bool:
+        """Index arithmetic only (symbols, non-negative constants, +, *, % and / by positive constants): non-negative in
+        exact arithmetic by structure.  Nothing that reads a buffer qualifies."""
+        if self.dtype != DType.Int32:
+            return False
+        if self.op in (AluOp.Special, AluOp.Variable):
+            return True
+        if self.op == AluOp.Const:
+            return int(self.arg) >= 0
+        if self.op in (AluOp.Add, AluOp.Mul):
+            return self.src[0]._pureNonNegativeIndex() and self.src[1]._pureNonNegativeIndex()
+        if self.op in (AluOp.Mod, AluOp.Idiv):
+            return self.src[1].op == AluOp.Const and int(self.src[1].arg) > 0 and self.src[0]._pureNonNegativeIndex()
+        return False
+
+    def reduceExactIndex(self) -> "AluExp":
+        """`(sum of index terms) % D` and `/ D` with every term's constant multiplier reduced modulo D, in exact arithmetic.
+
+        The index expression of a chain of views unravels a flat index into conceptual arrays whose extents can pass
+        2^31 (output channels x batch x padded image: `(o * 349748352 + ... + x * 59) % 58` for the operands of a
+        layer-sized filter cotangent).  The reference's simplifier removes such terms because its range analysis never
+        wraps (src/alu.ts:425-571 with the rule "(x + A*y) % B => x % B when B | A"), so the kernels its backends compile
+        never evaluate them; the range analysis here gives up where a bound leaves 32 bits, so the same reduction is
+        done explicitly, and only on pure index arithmetic (symbols and constants: values read from buffers keep their
+        wrap-around semantics)."""
+
+        def visit(n: AluExp):
+            if n.op not in (AluOp.Mod, AluOp.Idiv) or n.dtype != DType.Int32 or n.src[1].op != AluOp.Const:
+                return None
+            D = int(n.src[1].arg)
+            if D <= 1 or not n.src[0]._pureNonNegativeIndex():
+                return None
+            terms = list(n.src[0].splitOp(AluOp.Add))
+            if len(terms) < 2:
+                return None
+            rest, quot, changed = [], [], False
+            for t in terms:
+                f = t.constFactor()
+                q = t.divides(f) if f > 1 else None
+                if q is None or f < D:
+                    rest.append(t)
+                    continue
+                changed = True
+                if f // D:
+                    quot.append(q if f // D == 1 else AluExp.mul(q, AluExp.i32(f // D)))
+                if f % D:
+                    rest.append(q if f % D == 1 else AluExp.mul(q, AluExp.i32(f % D)))
+            if not changed:
+                return None
+
+            def total(parts):
+                acc = parts[0]
+                for x in parts[1:]:
+                    acc = AluExp.add(acc, x)
+                return acc
+
+            low = total(rest) if rest else AluExp.i32(0)
+            if n.op == AluOp.Mod:
+                return AluExp.mod(low, n.src[1])
+            return total(quot + [AluExp.idiv(low, n.src[1])]) if quot else AluExp.idiv(low, n.src[1])
+
+        return self.rewrite(visit)
+
     def splitOp(self, sep: AluOp) -> Iterator["AluExp"]:
         """Flatten nested applications of an associative op (src/alu.ts:630-636)."""
         if self.op == sep:

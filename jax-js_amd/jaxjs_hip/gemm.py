@@ -343,6 +343,28 @@ def rows8_form(oexp: AluExp, extent: int, group: int = 8):
 
 
 
+def _swap_row_k(e: AluExp) -> AluExp:
+    """The same expression with the roles of the Specials `row` and `k` exchanged."""
+    def sw(n):
+        if n.op == AluOp.Special and n.arg[0] == "row":
+            return AluExp.special(n.dtype, "k", n.arg[1])
+        if n.op == AluOp.Special and n.arg[0] == "k":
+            return AluExp.special(n.dtype, "row", n.arg[1])
+        return None
+    return e.rewrite(sw)
+
+
+def kvec_form(oexp: AluExp, K: int, group: int = 8):
+    """`rows8_form` along the other axis: (index at the group's first k, mask as a function of `e`, the GlobalIndex node) if
+    `group` consecutive k of every aligned group read `group` consecutive elements of one row (the image operand of a
+    filter cotangent: k runs over batch x positions, and consecutive positions are consecutive pixels); else None."""
+    form = rows8_form(_swap_row_k(oexp), K, group)
+    if form is None:
+        return None
+    idx0, cond_e, node = form
+    return _swap_row_k(idx0).simplify(), (None if cond_e is None else _swap_row_k(cond_e).simplify()), node
+
+
 # ---- tap-major k order for convolution-like gather operands -----------------------------------------------------------
 #
 # The patch operand of a convolution reads element k = c * T + tap (T filter taps, tap fastest) of channel plane c:
@@ -427,6 +449,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     # (deterministic: no float atomics).  For launches that would otherwise leave most CUs without a workgroup.
     split = int(tile.get("SPLITK", 1))
     K_full = g["K"]
+    two_stride = dict(a=g["a_k0"] != K_full, b=g["b_k0"] != K_full)  # of the whole k axis, before any slicing
     if split > 1:
         vec_k = 8 if g["dtype"] == DType.Float16 else 4
         # a two-stride k axis is cut between runs only
@@ -528,7 +551,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
             if node.op == AluOp.Special and node.arg[0] == "ridx":
                 return kvar
             return None
-        oexp = operand_exps[gid].rewrite(_retarget_operand).simplify()
+        oexp = operand_exps[gid].rewrite(_retarget_operand).reduceExactIndex().simplify()
         gather_oexp[tag] = oexp
         if tag == "b" and g["dtype"] == DType.Float16 and not g.get("a_gather") and split == 1 and tile.get("CONV", 1) and not tile.get("TAPMAJOR", 0):
             # A stride-1 window walk over an image (verified on the operand's own index expression): the patch-in-LDS
@@ -624,6 +647,50 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                 gather_calls[tag] = f"jh_gather4_{tag}(row, k, jh_b0, jh_b1, jh_b2{epi_args})"
                 gather_flags[tag], gather_group[tag] = 5, 4
 
+        # k-vector loader: when neither row form applies but G consecutive k of an aligned group read G consecutive elements
+        # of one row (the activations under a filter cotangent: k = batch x positions), one G-element load per group feeds
+        # the k-contiguous staging path; masked lanes are zeroed, groups that would leave the buffer go element by element.
+        if gather_flags[tag] == 1 and tile.get("KVEC", 1) and g["K"] % 8 == 0:
+            kv, G = None, 0
+            for G in ((8, 4) if g["dtype"] == DType.Float16 else (4,)):
+                kv = kvec_form(oexp, K_full, G)
+                if kv is not None:
+                    break
+            if kv is not None:
+                idx0, cond_e, gnode = kv
+                vnames = {"row": "row", "e": "e", "k": "k", "b0": "b0", "b1": "b1", "b2": "b2"}
+                icg = HipExpCodegen(names, vnames, "  ", prefix=f"ki{tag}", numerics=numerics)
+                icg.countReferences(idx0)
+                ival = strip_parens(icg.run(idx0))
+                gather_fns.append(f"static __device__ __forceinline__ int jh_kindex_{tag}(int row, int k, int b0, int b1, int b2) {{\n"
+                                  + "\n".join(icg.take_lines()) + f"\n  return {ival};\n}}")
+                maskbit = "true"
+                if cond_e is not None:
+                    mcg = HipExpCodegen(names, vnames, "  ", prefix=f"km{tag}", numerics=numerics)
+                    mcg.countReferences(cond_e)
+                    mval = strip_parens(mcg.run(cond_e))
+                    gather_fns.append(f"static __device__ __forceinline__ bool jh_kmask_{tag}(int row, int e, int k, int b0, int b1, int b2) {{\n"
+                                      + "\n".join(mcg.take_lines()) + f"\n  return {mval};\n}}")
+                    maskbit = f"jh_kmask_{tag}(row, e, kk, b0, b1, b2)"
+                buf = names[gnode.arg[0]]
+                W = 8 if g["dtype"] == DType.Float16 else 4  # elements per chunk of the staging path
+                vec_t = "jh_half8" if g["dtype"] == DType.Float16 else "jh_float4"
+                zero = "(jh_f16)0.0f" if g["dtype"] == DType.Float16 else "0.0f"
+                gather_fns.append(
+                    f"typedef {in_t} jh_kpart_{tag} __attribute__((ext_vector_type({G})));\n"
+                    f"struct __attribute__((packed, aligned({2 if g['dtype'] == DType.Float16 else 4}))) jh_kpart_u_{tag} {{ jh_kpart_{tag} v; }};\n"
+                    f"static __device__ __forceinline__ {vec_t} jh_gatherk_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
+                    f"  {vec_t} out;\n#pragma unroll\n  for (int j = 0; j < {W // G}; ++j) {{\n    const int kk = k + j * {G};\n"
+                    f"    const int i0 = jh_kindex_{tag}(row, kk, b0, b1, b2);\n"
+                    f"    if ((unsigned)i0 <= (unsigned)({gnode.arg[1]} - {G})) {{\n"
+                    f"      const jh_kpart_{tag} part = reinterpret_cast<const jh_kpart_u_{tag}*>({buf} + i0)->v;\n"
+                    f"#pragma unroll\n      for (int e = 0; e < {G}; ++e) out[j * {G} + e] = {maskbit} ? part[e] : {zero};\n    }} else {{\n"
+                    f"#pragma unroll\n      for (int e = 0; e < {G}; ++e) out[j * {G} + e] = jh_gather_{tag}(row, kk + e, b0, b1, b2{epi_args});\n    }}\n  }}\n"
+                    f"  return out;\n}}")
+                gather_calls[tag] = f"jh_gatherk_{tag}(row, k, jh_b0, jh_b1, jh_b2{epi_args})"
+                gather_flags[tag] = 4 if g["dtype"] == DType.Float16 else 6
+                gather_group[tag] = G
+
     # Tap-major k order (see `tap_major_form`): one gather operand whose k splits into (channel, tap), the other a plain
     # strided operand.  Both are then loaded through block/chunk loaders that take the first k' of eight consecutive
     # ones: k' = tap * C + c, original k = c * T + tap.
@@ -704,8 +771,9 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     pitch = -(-kernel.size // 8) * 8  # elements between two slices' partial outputs
     if split > 1:
         # a slice starts K elements further along k: K * sk for one stride, (K / k0) runs of sk1 for two
-        a_step = g["K"] * g["a_sk"] if g["a_k0"] == g["K"] else (g["K"] // g["a_k0"]) * g["a_sk1"]
-        b_step = g["K"] * g["b_sk"] if g["b_k0"] == g["K"] else (g["K"] // g["b_k0"]) * g["b_sk1"]
+        # (whether the axis has two strides is the whole axis's property: a slice of exactly one run has k0 == K too)
+        a_step = g["K"] * g["a_sk"] if not two_stride["a"] else (g["K"] // g["a_k0"]) * g["a_sk1"]
+        b_step = g["K"] * g["b_sk"] if not two_stride["b"] else (g["K"] // g["b_k0"]) * g["b_sk1"]
         lines.append(f"  a_base += (long long)blockIdx.y * {a_step}ll; b_base += (long long)blockIdx.y * {b_step}ll;"
                      + ("" if fusek else f" c_base += (long long)blockIdx.y * {pitch}ll;"))
         lines.append(f"  const int jh_k_off = (int)blockIdx.y * {g['K']};  // a gather loader is asked for k of the whole axis")
@@ -786,8 +854,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                      GATHER_A_SLOW=gather_slow.get("a", "jh_half8{0, 0, 0, 0, 0, 0, 0, 0}"), GATHER_B_SLOW=gather_slow.get("b", "jh_half8{0, 0, 0, 0, 0, 0, 0, 0}"))
     src = _prelude(numerics) + fill(template(tmpl), dict(sched, 
         M=g["M"], N=g["N"], K=g["K"], M_LOAD=load_rows["a"], N_LOAD=load_rows["b"], BM=BM, BN=BN, WM=WM, WN=WN,
-        A_KCONTIG=0 if gather_flags["a"] in (2, 3, 5) else (1 if g["a_sk"] == 1 or g["K"] == 1 or gather_flags["a"] in (1, 4) else 0),
-        B_KCONTIG=0 if gather_flags["b"] in (2, 3, 5) else (1 if g["b_sk"] == 1 or g["K"] == 1 or gather_flags["b"] in (1, 4) else 0),
+        A_KCONTIG=0 if gather_flags["a"] in (2, 3, 5) else (1 if g["a_sk"] == 1 or g["K"] == 1 or gather_flags["a"] in (1, 4, 6) else 0),
+        B_KCONTIG=0 if gather_flags["b"] in (2, 3, 5) else (1 if g["b_sk"] == 1 or g["K"] == 1 or gather_flags["b"] in (1, 4, 6) else 0),
         NBATCH=nbatch, EPILOGUE_FN=epi_fn, NAME=name, PARAMS=params,
         A_OFF=g["a_off"], B_OFF=g["b_off"], BATCH_DECODE="\n".join(lines),
         A_PTR="jh_repack_a" if "a" in (repack or "") else names[g["gid_a"]], B_PTR="jh_repack_b" if "b" in (repack or "") else names[g["gid_b"]],
@@ -812,7 +880,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         info.update(stages=sched["STAGES"], ring=sched["RING"])
     if any_gather:
         info["gather"] = {tag: {0: "none", 1: "element", 2: f"rows{gather_group.get(tag, 8)}", 3: f"tap-major rows{gather_group.get(tag, 8)}",
-                                4: "tap-major strided", 5: "rows4"}[gather_flags[tag]] for tag in ("a", "b")}
+                                4: "tap-major strided" if tap_major is not None else f"k{gather_group.get(tag, 8)}", 5: "rows4", 6: "k4"}[gather_flags[tag]] for tag in ("a", "b")}
         if tap_major is not None:
             info["tap_major"] = tap_major
     if repack:

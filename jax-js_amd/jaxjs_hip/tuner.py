@@ -75,8 +75,8 @@ def tuneNullopt(kernel: Kernel) -> TuneResult:
             exp = AluExp.cast(re.dtype, exp)
     epilogue = None
     if re is not None:
-        epilogue = re.epilogue.substitute({"gidx": vars_["gidx"]}).rewriteGlobalViews().simplify()
-    return TuneResult(exp=exp.substitute(vars_).rewriteGlobalViews().simplify(), epilogue=epilogue)
+        epilogue = re.epilogue.substitute({"gidx": vars_["gidx"]}).rewriteGlobalViews().reduceExactIndex().simplify()
+    return TuneResult(exp=exp.substitute(vars_).rewriteGlobalViews().reduceExactIndex().simplify(), epilogue=epilogue)
 
 
 # ------------------------------------------------------------------------------------------------

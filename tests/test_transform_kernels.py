@@ -382,6 +382,10 @@ RANDOM_CONVS = [
     (2, 64, 32, 9, 20, 1, 5, (1, 1), ((0, 0), (2, 2)), (1, 1)),
     (1, 32, 96, 20, 20, 5, 5, (2, 2), ((2, 2), (2, 2)), (1, 1)),
     (5, 40, 40, 8, 8, 2, 2, (2, 2), ((0, 0), (0, 0)), (1, 1)),
+    # layer-sized: the filter cotangent's k axis (batch x 56 x 56 positions) is cut into slices of one image each, the
+    # cotangent operand read as a plain two-stride view (runs of 3136), the activations through the k-vector loader
+    (8, 32, 32, 56, 56, 3, 3, (1, 1), ((1, 1), (1, 1)), (1, 1)),
+    (4, 64, 64, 56, 56, 3, 3, (1, 1), ((1, 1), (1, 1)), (1, 1)),
 ]
 
 
