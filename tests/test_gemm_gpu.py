@@ -209,6 +209,26 @@ def test_gemm_8192_cubed_every_element_exact():
     np.testing.assert_array_equal(got.reshape(n, n), ref)
 
 
+def test_gemm_full_size_edge_tiles_and_repacked_operands_are_exact():
+    """The shapes the edge-tile and repack paths were measured on, at full size with entries in {-1, 0, 1} (every sum an
+    integer below 2^24: exact in the f32 accumulator, stored as f32): 8000^3 (edge tiles along both axes of the
+    direct-to-LDS template), 8192 x 50257 x 768 (B's rows off the 16-byte grid: repack pre-pass, 197 tile columns the last
+    one 81 wide) and 4100 x 4100 x 4100 (ragged k: both operands copied with k padded).  Rows from every tile row, the
+    last rows and the last columns included, against exact host products."""
+    for (M, N, K, want_repack) in ((8000, 8000, 8000, None), (8192, 50257, 768, "b"), (4100, 4100, 4100, "ab")):
+        A = RNG.integers(-1, 2, (M, K)).astype(np.float16)
+        B = RNG.integers(-1, 2, (K, N)).astype(np.float16)
+        got, ks = device_run(_f32_out(matmulKernel(M, N, K, DType.Float16), K), [A, B])
+        assert ks.klass == "gemm" and ks.info["direct_lds"] and ks.info.get("repack") == want_repack, ks.info
+        bm = ks.info["BM"]
+        rows = sorted({min(t * bm + r, M - 1) for t in range(-(-M // bm)) for r in (0, bm // 2 + 3, bm - 1)} | {M - 1, M - 2})
+        if len(rows) > 200:
+            rows = rows[::len(rows) // 150] + [M - 2, M - 1]
+        ref = A[rows].astype(np.float32) @ B.astype(np.float32)
+        np.testing.assert_array_equal(got.reshape(M, N)[rows], ref, err_msg=str((M, N, K)))
+        del got
+
+
 def test_gemm_output_just_under_two_to_the_31_elements():
     """46336 x 46336 outputs (2,147,024,896 float16 values, 4.3 GB) over a short k axis: tile origins, the tile walk and the
     store addresses near the end of the int32 index range.  Integer entries keep every value exact; rows from the first, a
