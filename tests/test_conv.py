@@ -401,6 +401,49 @@ def test_f16_convolution_loader_choice(case):
         assert tm.info["tap_major"]["T"] == int(np.prod(case["w"][2:])) and any(v.startswith("tap-major rows") for v in tm.info["gather"].values())
 
 
+# ---- the layer shapes the bench measures, at full size --------------------------------------------------------------
+
+LAYER_CONVS = [((32, 64, 56, 56), (64, 64, 3, 3), 1), ((32, 256, 28, 28), (256, 256, 3, 3), 1), ((32, 256, 14, 14), (256, 256, 3, 3), 1),
+               ((32, 64, 56, 56), (128, 64, 3, 3), 2)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt,npdt", [(DType.Float16, np.float16), (DType.Float32, np.float32)], ids=["f16", "f32"])
+@pytest.mark.parametrize("cx,cw,st", LAYER_CONVS, ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else f"s{v}")
+def test_layer_sized_convolutions_are_exact(cx, cw, st, dt, npdt):
+    """3x3 SAME convolutions of ResNet-sized layers (batch 32), stride 1 and 2, with entries in {-1, 0, 1}: every output is
+    an integer below 2048, exact in float16 and float32, and must equal a tap-by-tap host convolution everywhere."""
+    from gpu_util import WARM_ONLY, backend
+    prog = J.jit(lambda a, b: L.convGeneralDilated(a, b, [st, st], "SAME"), [ShapedArray(cx, dt), ShapedArray(cw, dt)])
+    if WARM_ONLY:
+        from jaxjs_hip.kernelgen import generate
+        from jaxjs_hip.runtime import compile_source
+        for src in generate(prog.kernels[0]).sources:
+            compile_source(src)
+        pytest.skip("warm-up run: compiled only")
+    rng = np.random.default_rng(21)
+    x = rng.integers(-1, 2, cx).astype(npdt)
+    w = rng.integers(-1, 2, cw).astype(npdt)
+    be = backend()
+    exe = be.prepareKernelSync(prog.kernels[0])
+    assert exe.data.ks.klass.startswith("gemm"), exe.data.ks.klass
+    sx, sw, so = be.malloc(x.nbytes, x.tobytes()), be.malloc(w.nbytes, w.tobytes()), be.malloc(prog.kernels[0].bytes)
+    be.dispatch(exe, [sx, sw], [so])
+    r = np.frombuffer(be.readSync(so), npdt).astype(np.float32)
+    for s_ in (sx, sw, so):
+        be.decRef(s_)
+    (pt, pb), (pl, pr) = L.padtypeToPads(cx[2:], cw[2:], [st, st], [1, 1], "SAME")
+    xp = np.pad(x.astype(np.float32), [(0, 0), (0, 0), (pt, pb), (pl, pr)])
+    OH, OW = -(-cx[2] // st), -(-cx[3] // st)
+    want = np.zeros((cx[0], cw[0], OH, OW), np.float32)
+    for ky in range(3):
+        for kx in range(3):
+            win = xp[:, :, ky:ky + (OH - 1) * st + 1:st, kx:kx + (OW - 1) * st + 1:st]
+            want += np.einsum("nchw,oc->nohw", win, w[:, :, ky, kx].astype(np.float32), optimize=True)
+    assert np.abs(want).max() < 2048
+    np.testing.assert_array_equal(r.reshape(want.shape), want, err_msg=str(exe.data.ks.info))
+
+
 # float32 convolutions on the gather loaders: stride-1 windows whose output width is a multiple of 4 read four consecutive
 # output positions with one 128-bit load (masked lanes zeroed), everything else element by element.
 F32_CONV_CASES = [
