@@ -156,6 +156,57 @@ def test_gemm_random_shapes_with_and_without_epilogue(dt, M, N, K, bt, bias):
     assert np.all(err <= bound), f"max excess {np.max(err - bound)} with {ks.info}"
 
 
+def _fuzz_gemm_cases(count=72, seed=5):
+    """Seeded random contractions over everything the tile chooser branches on: extents from 2 to 5000 (few rows or
+    columns against a long k included), k whole slabs or not, all four storage layouts of A and B, views that start a
+    few elements into their buffer, float16 and float32."""
+    rng = np.random.default_rng(seed)
+
+    def pick():
+        return int(rng.choice([rng.integers(2, 40), rng.integers(40, 300), rng.integers(300, 1500), rng.choice([64, 128, 256, 512, 1024, 2048]),
+                               rng.integers(1500, 5000)]))
+
+    cases = []
+    while len(cases) < count:
+        r = rng.integers(0, 6)
+        M, N = pick(), pick()
+        K = int(rng.choice([rng.integers(32, 200), rng.integers(200, 3000), rng.choice([64, 128, 256, 768, 1024, 2048, 4096, 8192]), rng.integers(3000, 9000),
+                            8 * rng.integers(4, 600), 32 * rng.integers(1, 200)]))
+        if r == 0:
+            M, N, K = int(rng.integers(2, 65)), int(rng.choice([4096, 14336, 1000, 2048])), int(rng.choice([1024, 2048, 4096, 4104, 8192]))
+        if r == 1:
+            N, M, K = int(rng.integers(2, 65)), int(rng.choice([4096, 2048, 1001])), int(rng.choice([1024, 2048, 4096]))
+        if M * N * K > 3e10 or M * N > 2e7:
+            continue
+        layout = str(rng.choice(["NN", "NT", "TN", "TT"]))
+        dt = DType.Float16 if rng.random() < 0.75 else DType.Float32
+        offs = tuple((int(rng.integers(1, 9)) if rng.random() < 0.25 else 0) for _ in range(2))
+        cases.append((M, N, K, layout, dt, offs))
+    return cases
+
+
+@pytest.mark.parametrize("M,N,K,layout,dt,offs", _fuzz_gemm_cases(), ids=lambda v: v.value if isinstance(v, DType) else "o%d%d" % v if isinstance(v, tuple) else str(v))
+def test_gemm_random_shapes_layouts_and_offsets_are_exact(M, N, K, layout, dt, offs):
+    """Whatever plan a shape gets (direct-to-LDS with edge tiles, repacked operands, k slices folded in or after the launch,
+    few-row tiles, the general templates, or a reduction class for thin shapes): entries in {-1, 0, 1}, the f32
+    accumulator stored as it is, every element equal to the host product."""
+    npdt = np.float16 if dt == DType.Float16 else np.float32
+    A = RNG.integers(-1, 2, (M, K)).astype(npdt)
+    B = RNG.integers(-1, 2, (K, N)).astype(npdt)
+    full = [M, N, K]
+    va = ShapeTracker.fromShape([M * K + offs[0]]).shrink([(offs[0], M * K + offs[0])])
+    vb = ShapeTracker.fromShape([K * N + offs[1]]).shrink([(offs[1], K * N + offs[1])])
+    stA = (va.reshape([K, M]).permute([1, 0]) if layout[0] == "T" else va.reshape([M, K])).reshape([M, 1, K]).expand(full)
+    stB = (vb.reshape([N, K]) if layout[1] == "T" else vb.reshape([K, N]).permute([1, 0])).reshape([1, N, K]).expand(full)
+    k = reduceKernel(full, [(dt, stA), (dt, stB)], lambda a, b: AluExp.mul(a, b), AluOp.Add)
+    if dt == DType.Float16:
+        k = _f32_out(k, K)
+    abuf = np.concatenate([np.zeros(offs[0], npdt), (A.T if layout[0] == "T" else A).ravel()])
+    bbuf = np.concatenate([np.zeros(offs[1], npdt), (B.T if layout[1] == "T" else B).ravel()])
+    got, ks = device_run(k, [abuf, bbuf])
+    np.testing.assert_array_equal(got.reshape(M, N), A.astype(np.float32) @ B.astype(np.float32), err_msg=f"{ks.klass} {ks.info}")
+
+
 def _tile_row_sample(n, bm=256):
     """Three rows of every block-tile row: the first, one in the second 128-row wave half, the last."""
     return sorted({t * bm + r for t in range(n // bm) for r in (0, bm // 2 + 3, bm - 1)})
