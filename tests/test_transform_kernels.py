@@ -412,6 +412,57 @@ def test_convolution_cotangents_over_strides_paddings_and_dilations(cfg, dt, npd
     np.testing.assert_array_equal(dw.astype(np.float64).reshape(dw_want.shape), dw_want, err_msg=str(cls_w))
 
 
+def _fuzz_conv_cases(count=24, seed=3):
+    """Seeded random 2-d convolutions: batch 1..16, 8..64 input and 16..128 output channels, images 7..56 wide, windows up
+    to 5x5, strides and filter dilations 1 or 2, asymmetric paddings 0..2."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        N, C, O = int(rng.choice([1, 2, 3, 4, 8, 16])), int(rng.choice([8, 16, 24, 32, 48, 64])), int(rng.choice([16, 32, 64, 96, 128]))
+        H, W = int(rng.choice([7, 8, 12, 14, 16, 20, 28, 30, 32, 56])), int(rng.choice([7, 8, 12, 14, 16, 20, 24, 28, 32, 40, 56]))
+        KH, KW = int(rng.choice([1, 2, 3, 5])), int(rng.choice([1, 2, 3, 5]))
+        st = (int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 2])))
+        rd = (int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 2])))
+        pad = ((int(rng.integers(0, 3)), int(rng.integers(0, 3))), (int(rng.integers(0, 3)), int(rng.integers(0, 3))))
+        if (KH - 1) * rd[0] + 1 > H + sum(pad[0]) or (KW - 1) * rd[1] + 1 > W + sum(pad[1]) or N * C * O * H * W * KH * KW > 2e9:
+            continue
+        cases.append((N, C, O, H, W, KH, KW, st, pad, rd, F16 if rng.random() < 0.5 else F32))
+    return cases
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("cfg", _fuzz_conv_cases(), ids=lambda c: "x".join(map(str, c[:7])) + "_s%d%d_d%d%d_" % (c[7] + c[9]) + c[10].value)
+def test_random_convolutions_forward_and_both_cotangents(cfg):
+    """Whatever class and loader each of the three kernels of a convolution layer gets (patch-in-LDS template, row-vector,
+    k-vector or element gather loaders, k slices with a fold, reduction classes for thin shapes): forward output, activation
+    cotangent and filter cotangent on small-integer data against tap-by-tap host convolutions, exact where the values
+    fit the dtype."""
+    N, C, O, H, W, KH, KW, st, pad, rd, dt = cfg
+    npdt = np.float16 if dt == F16 else np.float32
+    rng = np.random.default_rng(N * 1000 + C * 10 + H)
+    x = rng.integers(-2, 3, (N, C, H, W)).astype(npdt)
+    w = rng.integers(-1, 2, (O, C, KH, KW)).astype(npdt)
+    p = ConvParams(0, list(st), [tuple(q) for q in pad], [1, 1], list(rd))
+    from jaxjs_hip.convolution import checkConvShape
+    ct = rng.integers(-1, 2, checkConvShape(list(x.shape), list(w.shape), p)).astype(npdt)
+    _, (y,), _c = on_gpu(lambda a, b: L.convGeneralDilated(a, b, list(st), [tuple(q) for q in pad], rhsDilation=list(rd)), [x, w], dt)
+    _, (dx,), _c = on_gpu(lambda c, f: conv_transposed_to_lhs(c, f, list(x.shape), p), [ct, w], dt)
+    _, (dw,), cls_w = on_gpu(lambda a, c: conv_transposed_to_rhs(a, c, list(w.shape), p), [x, ct], dt)
+    dx_want, dw_want = conv_vjp_by_taps(x, w, ct, st, pad, rd)
+    xp = np.pad(x.astype(np.float64), [(0, 0), (0, 0), pad[0], pad[1]])
+    OH, OW = ct.shape[2:]
+    y_want = np.zeros(ct.shape)
+    for ky in range(KH):
+        for kx in range(KW):
+            win = xp[:, :, ky * rd[0]:ky * rd[0] + (OH - 1) * st[0] + 1:st[0], kx * rd[1]:kx * rd[1] + (OW - 1) * st[1] + 1:st[1]]
+            y_want += np.einsum("nchw,oc->nohw", win, w[:, :, ky, kx].astype(np.float64))
+    for got, want, what in ((y, y_want, "forward"), (dx, dx_want, "activation cotangent"), (dw, dw_want, "filter cotangent")):
+        if dt == F32 or np.abs(want).max() < 2048:
+            np.testing.assert_array_equal(got.astype(np.float64).reshape(want.shape), want, err_msg=f"{what} {cls_w}")
+        else:  # float16 cannot hold the sums exactly: half an ulp of the result
+            np.testing.assert_allclose(got.astype(np.float64).reshape(want.shape), want, rtol=2.0 ** -10, atol=0, err_msg=what)
+
+
 @pytest.mark.gpu
 def test_transposed_dot_and_gather_cotangents_on_the_gpu():
     """`transposeDot` (src/frontend/linearize.ts:767-774): for c = a @ b the cotangents are ct @ b^T and a^T @ ct -- the
