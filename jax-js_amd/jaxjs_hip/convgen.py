@@ -179,12 +179,12 @@ def _pitch(elems: int) -> int:
 
 
 def gen_conv(kernel, g: dict, oexp: AluExp, numerics: str, name: str, params: str, names: list, epi_fn: str, epi_args: str,
-             need: dict, tile: dict):
+             need: dict, tile: dict, a_gather_fns: Optional[str] = None):
     """KernelSource of the patch-in-LDS convolution for a GEMM whose B operand `oexp` is a stride-1 window walk, or None
     when the shape is outside what the template covers (it then stays on the generic gather loaders)."""
     from .kernelgen import KernelSource, LaunchStep, _prelude, fill, template
 
-    if g.get("b_k0") != g["K"] or g["a_k0"] != g["K"] or len(g["batch"]) > 1:
+    if g.get("b_k0") != g["K"] or (a_gather_fns is None and g["a_k0"] != g["K"]) or len(g["batch"]) > 1:
         return None
     cv = match_conv(oexp, g["N"], g["K"], g["batch"])
     if cv is None:
@@ -237,17 +237,23 @@ def gen_conv(kernel, g: dict, oexp: AluExp, numerics: str, name: str, params: st
         SC=cv["SC"], SB=cv["SB"], NB=cv["NB"], BM=BM, BN=BN, WM=WM, WN=WN, CS=CS, R=R, P=P, G=G, SMAX=smax,
         SX=SX, SY=SY, RP=RP, QMIN=qmin, XCH=int(xch),
         EPILOGUE_FN=epi_fn, EPILOGUE_ARGS=epi_args, NAME=name, PARAMS=params, IMG_PTR=names[cv["gid"]],
+        A_GATHER=0 if a_gather_fns is None else 1, A_GATHER_FNS=a_gather_fns or "",
         A_OFF=g["a_off"], A_SM=g["a_sm"], A_SK=g["a_sk"], C_SM=g["c_sm"], C_SN=g["c_sn"], C_SB=sb_c))
     T = cv["T"]
     total_w = T * O * C
     nargs = kernel.nargs
-    prep = LaunchStep(name + "_wprep", (-(-total_w // 256), 1, 1), (256, 1, 1), 0, [("in", g["gid_a"]), ("scratch", 0)])
+    if a_gather_fns is None:
+        prep_args = [("in", g["gid_a"]), ("scratch", 0)]
+    else:  # the element loader of a gathered filter takes every buffer of the kernel
+        prep_args = [("in", i) for i in range(nargs)] + [("out", 0), ("scratch", 0)]
+    prep = LaunchStep(name + "_wprep", (-(-total_w // 256), 1, 1), (256, 1, 1), 0, prep_args)
     tiles = n_tiles * (O // BM) * cv["NB"]
     main = LaunchStep(name, (tiles, 1, 1), (64 * WM * WN, 1, 1), 0,
                       [("in", i) for i in range(nargs)] + [("out", 0), ("scratch", 0)])
     need = dict(need)
-    need[g["gid_a"]] = max(need.get(g["gid_a"], 0), g["a_len"] * 2)
+    if a_gather_fns is None:
+        need[g["gid_a"]] = max(need.get(g["gid_a"], 0), g["a_len"] * 2)
     need[cv["gid"]] = max(need.get(cv["gid"], 0), ((cv["NB"] - 1) * cv["SB"] + (C - 1) * cv["SC"] + cv["H"] * cv["W"]) * 2)
     info = dict(BM=BM, BN=BN, WM=WM, WN=WN, BK=16, direct_lds=False, tiles=tiles, M=O, N=g["N"], K=g["K"], nbatch=cv["NB"], splitk=1,
-                conv=dict(cv, CS=CS, R=R, P=P, G=G, OWP=OWP, exchange=bool(xch)), gather=dict(a="none", b="patch"))
+                conv=dict(cv, CS=CS, R=R, P=P, G=G, OWP=OWP, exchange=bool(xch)), gather=dict(a="none" if a_gather_fns is None else "element (pre-pass)", b="patch"))
     return KernelSource([src], [prep, main], [total_w * 2], "gemm", need, info)

@@ -524,7 +524,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
 
     # Element loaders for gather operands: the operand's lowered expression (masked load through its view
     # chain) with the flat output index rebuilt from (tile row, batch coordinates) and ridx = k.
-    gather_fns, gather_calls, gather_flags, gather_group, gather_oexp, gather_slow = [], {}, {}, {}, {}, {}
+    gather_fns, gather_calls, gather_flags, gather_group, gather_oexp, gather_slow, element_fn = [], {}, {}, {}, {}, {}, {}
     lowered = _strip_casts(t.exp)
     operand_exps = {g["gid_a"]: None, g["gid_b"]: None}
     if g.get("a_gather") or g.get("b_gather"):
@@ -553,19 +553,27 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
             return None
         oexp = operand_exps[gid].rewrite(_retarget_operand).reduceExactIndex().simplify()
         gather_oexp[tag] = oexp
-        if tag == "b" and g["dtype"] == DType.Float16 and not g.get("a_gather") and split == 1 and tile.get("CONV", 1) and not tile.get("TAPMAJOR", 0):
+        if tag == "b" and g["dtype"] == DType.Float16 and split == 1 and tile.get("CONV", 1) and not tile.get("TAPMAJOR", 0):
             # A stride-1 window walk over an image (verified on the operand's own index expression): the patch-in-LDS
-            # convolution template instead of an im2col tile built element by element.
+            # convolution template instead of an im2col tile built element by element.  The other operand -- the filter --
+            # may itself be a gather operand (the flipped, transposed filter of the cotangent towards the activations): the
+            # template's weight pre-pass then reads it through its element loader.
             from .convgen import gen_conv
 
-            conv = gen_conv(kernel, g, oexp, numerics, name, params, names, epi_fn, epi_args, _min_bytes(t.epilogue), tile)
+            conv_need = _min_bytes(t.epilogue)
+            if g.get("a_gather"):
+                for gid_, b_ in _min_bytes(t.exp).items():
+                    conv_need[gid_] = max(conv_need.get(gid_, 0), b_)
+            conv = gen_conv(kernel, g, oexp, numerics, name, params, names, epi_fn, epi_args, conv_need, tile,
+                            a_gather_fns=element_fn["a"] if g.get("a_gather") else None)
             if conv is not None:
                 return conv
         gcg = HipExpCodegen(names, {"row": "row", "k": "k", "b0": "b0", "b1": "b1", "b2": "b2"}, "  ", prefix=f"g{tag}", numerics=numerics)
         gcg.countReferences(oexp)
         gval = strip_parens(gcg.run(oexp))
-        gather_fns.append(f"static __device__ __forceinline__ {in_t} jh_gather_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
-                          + "\n".join(gcg.take_lines()) + f"\n  return ({in_t})({gval});\n}}")
+        element_fn[tag] = (f"static __device__ __forceinline__ {in_t} jh_gather_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
+                           + "\n".join(gcg.take_lines()) + f"\n  return ({in_t})({gval});\n}}")
+        gather_fns.append(element_fn[tag])
         gather_calls[tag] = f"jh_gather_{tag}(row, k, jh_b0, jh_b1, jh_b2{epi_args})"
         # Row-vector loader: when G = 8 or 4 consecutive rows of an aligned group read G consecutive elements, one
         # unaligned G-element load replaces G element loads and their index arithmetic; masked lanes are zeroed

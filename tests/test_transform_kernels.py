@@ -463,6 +463,27 @@ def test_random_convolutions_forward_and_both_cotangents(cfg):
             np.testing.assert_allclose(got.astype(np.float64).reshape(want.shape), want, rtol=2.0 ** -10, atol=0, err_msg=what)
 
 
+def test_layer_sized_cotangent_plans():
+    """Which templates and loaders the two cotangent convolutions of a 3x3 layer [8,64,56,56] -> 64 channels get (decided
+    on the host): towards the activations the patch-in-LDS convolution template, its flipped and transposed filter read
+    through the element loader by the weight pre-pass; towards the filter a GEMM over k = batch x positions in slices of
+    one image, the activations through the k-vector loader, the cotangent as a plain two-stride view."""
+    from jaxjs_hip.kernelgen import generate
+    N, C, O, H = 8, 64, 64, 56
+    p = ConvParams(0, [1, 1], [(1, 1), (1, 1)], [1, 1], [1, 1])
+    for dt in (F16, F32):
+        pl = J.jit(lambda c, f: conv_transposed_to_lhs(c, f, [N, C, H, H], p), [ShapedArray((N, O, H, H), dt), ShapedArray((O, C, 3, 3), dt)])
+        pr = J.jit(lambda a, c: conv_transposed_to_rhs(a, c, [O, C, 3, 3], p), [ShapedArray((N, C, H, H), dt), ShapedArray((N, O, H, H), dt)])
+        kl, kr = generate(pl.kernels[0]), generate(pr.kernels[0])
+        assert kl.klass == "gemm" and kr.klass == "gemm+fold" and kr.info["splitk"] == N, (kl.klass, kr.klass, kr.info)
+        if dt == F16:
+            assert kl.info["gather"] == {"a": "element (pre-pass)", "b": "patch"} and len(kl.steps) == 2, kl.info
+            assert kr.info["gather"] == {"a": "k8", "b": "none"}, kr.info
+        else:
+            assert kl.info["gather"] == {"a": "element", "b": "rows4"}, kl.info
+            assert kr.info["gather"] == {"a": "k4", "b": "none"}, kr.info
+
+
 @pytest.mark.gpu
 def test_transposed_dot_and_gather_cotangents_on_the_gpu():
     """`transposeDot` (src/frontend/linearize.ts:767-774): for c = a @ b the cotangents are ct @ b^T and a^T @ ct -- the
