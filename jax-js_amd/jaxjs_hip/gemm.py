@@ -30,7 +30,7 @@ def choose_tile(g: dict) -> Dict[str, int]:
     CU = tuner.CU_COUNT
     # Slices of the k axis at most: 8, or 64 when the axis is very long (k = batch x positions of a filter cotangent:
     # 100352 against 9 output tiles), where the partial sums stay tiny next to the operands.
-    max_split = 64 if g["K"] >= 32768 else 8
+    max_split = 64 if g["K"] >= 16384 else 8
     plain_k = not (g.get("a_gather") or g.get("b_gather")) and g["a_k0"] == g["K"] and g["b_k0"] == g["K"]
     # A k axis that may be cut over workgroups: one stride per plain operand (a slice is a pointer offset), any gather
     # operand (a slice is an offset on the k its loader is asked for).
@@ -91,7 +91,8 @@ def choose_tile(g: dict) -> Dict[str, int]:
     def k_split(count):
         # Fewer workgroups than 1.5 per CU: cut the k axis (partial sums in scratch, fold kernel) while slices stay >= 512 deep.
         split = 1
-        while cut_k and count * split < 1.5 * CU and split < max_split and g["K"] % (split * 2 * 64) == 0 and g["K"] // (split * 2) >= 512 and runs_ok(split * 2):
+        gran = 64 if plain_k else 8  # whole slabs for the direct loads; the gather loaders take a ragged last slab
+        while cut_k and count * split < 1.5 * CU and split < max_split and g["K"] % (split * 2 * gran) == 0 and g["K"] // (split * 2) >= 512 and runs_ok(split * 2):
             split *= 2
         return dict(SPLITK=split) if split > 1 else {}
 
@@ -128,6 +129,11 @@ def choose_tile(g: dict) -> Dict[str, int]:
         # the same as the deep pipeline at 4096 x 4096 x 1024 and 2048 x 8192 x 512; slower from k = 3072 (65.9 against
         # 41.9 us) and with fewer than two tiles per CU (8192 x 768 x 768: 17.0 against 14.9 us).
         return dict(BM=128, BN=256, WM=1, WN=4, BK=32, STAGES=2, PIPE=0)
+    if not plain_k and cut_k and g["K"] >= 8192 and tiles(128, 128) * 8 <= CU:
+        # A handful of tiles over a very long k axis read through gather loaders (the filter cotangent of a convolution:
+        # 9 taps x 64 x 64 or 128 x 128 outputs, k = batch x positions): 64x64 tiles waste no half-empty MFMA tile and
+        # give the k slices four times as many workgroups ([32,64,56,56] 93 -> 72 us, [32,128,28,28] 187 -> 64 us).
+        return dict(BM=64, BN=64, **k_split(tiles(64, 64)))
     best = None
     for bm, bn, eff, extra in ((256, 256, 1.00, dict()), (128, 256, 0.84, dict(WM=1, WN=4)), (256, 128, 0.79, dict()),
                                 (128, 128, 0.62, dict())):
