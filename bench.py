@@ -740,6 +740,52 @@ def main():
                 [hostrand.normal(1007, cx, 1.0, np.float16), hostrand.normal(1007, cw, 0.05, np.float16, stream=1)],
                 2.0 * cx[0] * cw[0] * (cx[2] // st) * (cx[3] // st) * cw[1] * 9, "TFLOP/s", PEAK_F16_TFLOPS)
 
+        # The two cotangent convolutions of the 56x56x64 layer (what the transpose rule of Conv binds,
+        # src/frontend/linearize.ts:783-837): towards the activations and towards the filter (the latter followed by a
+        # small transposing map kernel, timed with it).
+        from jaxjs_hip.convolution import ConvParams
+        cx, cw = (32, 64, 56, 56), (64, 64, 3, 3)
+        cp = ConvParams(0, [1, 1], [(1, 1), (1, 1)], [1, 1], [1, 1])
+        for cdt, npdt, tag in ((DType.Float16, np.float16, "f16"), (DType.Float32, np.float32, "f32")):
+            xs_, ws_, cts_ = (hostrand.normal(1008, cx, 1.0, npdt), hostrand.normal(1008, cw, 0.05, npdt, stream=1),
+                              hostrand.normal(1008, (cx[0], cw[0]) + cx[2:], 1.0, npdt, stream=2))
+            for what, fn, arrs in (("activations", lambda c, f: J.convTransposeLhs(c, f, list(cx), cp), [cts_, ws_]),
+                                   ("filter", lambda a, c: J.convTransposeRhs(a, c, list(cw), cp), [xs_, cts_])):
+                cprog = J.jit(fn, [ShapedArray(tuple(a.shape), cdt) for a in arrs])
+                ins = []
+                for c_ in cprog.consts:  # closed-over constants come first
+                    kc = c_.kernel()
+                    ins.append(be.malloc(kc.bytes))
+                    be.dispatch(be.prepareKernelSync(kc), [], [ins[-1]])
+                ins += [upload(be, a) for a in arrs]
+                prepared = cprog.prepare(be)
+
+                def once():
+                    for o_ in cprog.execute(be, ins, prepared):
+                        be.decRef(o_)
+
+                for _ in range(5):
+                    once()
+                be.dev.sync()
+                e0, e1 = be.dev.event(), be.dev.event()
+                reps = 50
+                be.dev.record(e0)
+                for _ in range(reps):
+                    once()
+                be.dev.record(e1)
+                be.dev.sync()
+                ms = be.dev.elapsed_ms(e0, e1) / reps
+                be.dev.destroy_event(e0)
+                be.dev.destroy_event(e1)
+                for sl in ins:
+                    be.decRef(sl)
+                flops = 2.0 * 32 * 64 * 56 * 56 * 64 * 9
+                peak = PEAK_F16_TFLOPS if cdt == DType.Float16 else PEAK_F32_MATRIX_TFLOPS
+                extra[f"conv3x3_cotangent_{what}_{tag}[32,64,56,56]x[64,64,3,3]"] = {
+                    "class": "+".join(be.prepareKernelSync(k_).data.ks.klass for k_ in cprog.kernels), "ms": round(ms, 5),
+                    "achieved": round(flops / (ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "frac_of_peak": round(flops / (ms * 1e-3) / 1e12 / peak, 4),
+                    "timing": f"{reps} executions of the traced program back to back"}
+
         # Routines: sort / argsort of f32 [8192, 4096] rows (native bitonic network in LDS).
         from jaxjs_hip.routine import Routine, Routines, RoutineType
         rows, L = 8192, 4096

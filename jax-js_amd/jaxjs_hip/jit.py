@@ -867,6 +867,38 @@ def poolTransposeWindows(ct, inShape, window, strides):
     return bind1("PoolTranspose", [ct], dict(inShape=tuple(inShape), window=tuple(window), strides=tuple(strides)))
 
 
+def convTransposeLhs(ct, rhs, lhsShape, p):
+    """What the transpose rule of Conv binds for the cotangent of the activations (src/frontend/linearize.ts:783-812):
+    a convolution of the cotangent with the flipped filter whose channel axes are exchanged.  Only transforms bind it in
+    the reference; it is here, like `poolTransposeWindows`, so that those Kernels can be presented to the backend."""
+    v = p.vmapDims
+    rev01 = list(range(v)) + [v + 1, v] + list(range(v + 2, ct.ndim))
+    kernel = flip(transpose(rhs, rev01), list(range(v + 2, rhs.ndim)))
+    padding = []
+    for i, (pl, _pr) in enumerate(p.padding):
+        dil_k = (kernel.shape[i + v + 2] - 1) * p.rhsDilation[i] + 1
+        dil_ct = (ct.shape[i + v + 2] - 1) * p.strides[i] + 1
+        before = dil_k - 1 - pl
+        dil_lhs = (lhsShape[i + v + 2] - 1) * p.lhsDilation[i] + 1
+        padding.append((before, dil_lhs + dil_k - 1 - dil_ct - before))
+    return conv(ct, kernel, ConvParams(v, list(p.lhsDilation), padding, list(p.strides), list(p.rhsDilation)))
+
+
+def convTransposeRhs(lhs, ct, rhsShape, p):
+    """The cotangent of the filter (src/frontend/linearize.ts:813-837): the activations convolved with the cotangent, batch
+    and channel axes exchanged on both, window strides and filter dilations exchanged."""
+    v = p.vmapDims
+    rev01 = list(range(v)) + [v + 1, v] + list(range(v + 2, ct.ndim))
+    padding = []
+    for i, (pl, _pr) in enumerate(p.padding):
+        dil_lhs = (lhs.shape[i + v + 2] - 1) * p.lhsDilation[i] + 1
+        dil_k = (rhsShape[i + v + 2] - 1) * p.rhsDilation[i] + 1
+        dil_ct = (ct.shape[i + v + 2] - 1) * p.strides[i] + 1
+        padding.append((pl, dil_ct - dil_lhs + dil_k - pl - 1))
+    out = conv(transpose(lhs, rev01), transpose(ct, rev01), ConvParams(v, list(p.rhsDilation), padding, list(p.lhsDilation), list(p.strides)))
+    return transpose(out, rev01)
+
+
 def _flip_rule(st, params):
     arg = [False] * len(st.shape)
     for ax in params["axis"]:

@@ -32,33 +32,9 @@ F32, F16 = DType.Float32, DType.Float16
 
 # ---- what the transpose rules bind -----------------------------------------------------------------------------------
 
-def conv_transposed_to_lhs(ct, rhs, lhs_shape, p: ConvParams):
-    """Cotangent of the activations (src/frontend/linearize.ts:783-812)."""
-    v = p.vmapDims
-    rev01 = list(range(v)) + [v + 1, v] + list(range(v + 2, ct.ndim))
-    kernel = J.flip(J.transpose(rhs, rev01), list(range(v + 2, rhs.ndim)))
-    padding = []
-    for i, (pl, _pr) in enumerate(p.padding):
-        dil_k = (kernel.shape[i + v + 2] - 1) * p.rhsDilation[i] + 1
-        dil_ct = (ct.shape[i + v + 2] - 1) * p.strides[i] + 1
-        before = dil_k - 1 - pl
-        dil_lhs = (lhs_shape[i + v + 2] - 1) * p.lhsDilation[i] + 1
-        padding.append((before, dil_lhs + dil_k - 1 - dil_ct - before))
-    return J.conv(ct, kernel, ConvParams(v, list(p.lhsDilation), padding, list(p.strides), list(p.rhsDilation)))
-
-
-def conv_transposed_to_rhs(lhs, ct, rhs_shape, p: ConvParams):
-    """Cotangent of the filter (src/frontend/linearize.ts:813-837)."""
-    v = p.vmapDims
-    rev01 = list(range(v)) + [v + 1, v] + list(range(v + 2, ct.ndim))
-    padding = []
-    for i, (pl, _pr) in enumerate(p.padding):
-        dil_lhs = (lhs.shape[i + v + 2] - 1) * p.lhsDilation[i] + 1
-        dil_k = (rhs_shape[i + v + 2] - 1) * p.rhsDilation[i] + 1
-        dil_ct = (ct.shape[i + v + 2] - 1) * p.strides[i] + 1
-        padding.append((pl, dil_ct - dil_lhs + dil_k - pl - 1))
-    out = J.conv(J.transpose(lhs, rev01), J.transpose(ct, rev01), ConvParams(v, list(p.rhsDilation), padding, list(p.lhsDilation), list(p.strides)))
-    return J.transpose(out, rev01)
+# (restated in the package beside the other primitives that only transforms bind: src/frontend/linearize.ts:783-837)
+conv_transposed_to_lhs = J.convTransposeLhs
+conv_transposed_to_rhs = J.convTransposeRhs
 
 
 # ---- numpy references ------------------------------------------------------------------------------------------------
