@@ -432,6 +432,7 @@ def _gen_attention(routine: Routine, numerics: str) -> Optional[KernelSource]:
     (qb, ql, qn, qo), (kb, ksp, kn, ko), (vb, vsp, vn, vo) = lay
     src = _prelude(numerics) + fill(template("attention.hip.inc"), dict(
         B=B, NH=N, L=L, S=S, H=H, CAUSAL=1 if params.get("isCausal") else 0, SCALE_LOG2E=repr(scale * math.log2(math.e)),
+        FOLD_SCALE=1 if 0 < scale < float("inf") else 0,
         QB=qb, QL=ql, QN=qn, QOFF=qo, KB=kb, KS=ksp, KN=kn, KOFF=ko, VB=vb, VS=vsp, VN=vn, VOFF=vo,
         OB=L * N * H, OL=N * H, ON=H))
     blocks = B * N * -(-L // 128)

@@ -56,6 +56,20 @@ def test_attention_is_stable_for_large_scores_and_peaked_rows():
         np.testing.assert_allclose(got[0].astype(np.float64), want[0].astype(np.float64), rtol=1e-2, atol=4e-3)
 
 
+@pytest.mark.parametrize("scale", [-0.125, 0.0, 1e-3, 3.0], ids=lambda s: "scale%g" % s)
+def test_attention_takes_any_scale(scale):
+    """A scale that is zero or negative does not commute with the row maximum (the kernel then scales the scores before
+    taking it); ragged lengths so the masked key tile and the diagonal are covered under both forms."""
+    rng = np.random.default_rng(11)
+    q, k, v = [rng.standard_normal((2, T, 2, 64)).astype(np.float16) for T in (200, 200, 200)]
+    for causal in (False, True):
+        routine = attention_routine(2, 200, 200, 2, causal, scale=scale)
+        got, _ = R.run_gpu(routine, [q, k, v])
+        want = R.run_oracle(routine, [q, k, v])
+        assert np.isfinite(got[0]).all()
+        np.testing.assert_allclose(got[0].astype(np.float64), want[0].astype(np.float64), rtol=1e-2, atol=4e-3)
+
+
 def _view(strides, offset, shape):
     return dict(strides=list(strides), offset=offset, elements=offset + sum((d - 1) * s for d, s in zip(shape, strides)) + 1)
 
