@@ -39,8 +39,8 @@ def choose_tile(g: dict) -> Dict[str, int]:
     # A plain operand whose k axis has two strides (runs of k0 elements) can be cut where a slice is whole runs.
     two_level = [g[t + "_k0"] for t in ("a", "b") if g[t + "_k0"] != g["K"]]
 
-    def runs_ok(slices):
-        return all((g["K"] // slices) % k0 == 0 for k0 in two_level)
+    def runs_ok(slices):  # whole runs, or a whole fraction of one
+        return all((g["K"] // slices) % k0 == 0 or k0 % (g["K"] // slices) == 0 for k0 in two_level)
 
     cut_k = (all(g["K"] % k0 == 0 for k0 in two_level)
              and (bool(g.get("a_gather")) == bool(g.get("b_gather")) or g["K"] >= 8192))
@@ -132,7 +132,8 @@ def choose_tile(g: dict) -> Dict[str, int]:
     if not plain_k and cut_k and g["K"] >= 8192 and tiles(128, 128) * 8 <= CU:
         # A handful of tiles over a very long k axis read through gather loaders (the filter cotangent of a convolution:
         # 9 taps x 64 x 64 or 128 x 128 outputs, k = batch x positions): 64x64 tiles waste no half-empty MFMA tile and
-        # give the k slices four times as many workgroups ([32,64,56,56] 93 -> 72 us, [32,128,28,28] 187 -> 64 us).
+        # give the k slices four times as many workgroups ([32,64,56,56] 93 -> 72 us, [32,128,28,28] 187 -> 64 us); slices
+        # of half an image (a run of the cotangent's k axis cut in two) double them again: 72 -> 57 us.
         return dict(BM=64, BN=64, **k_split(tiles(64, 64)))
     best = None
     for bm, bn, eff, extra in ((256, 256, 1.00, dict()), (128, 256, 0.84, dict(WM=1, WN=4)), (256, 128, 0.79, dict()),
@@ -458,16 +459,19 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     two_stride = dict(a=g["a_k0"] != K_full, b=g["b_k0"] != K_full)  # of the whole k axis, before any slicing
     if split > 1:
         vec_k = 8 if g["dtype"] == DType.Float16 else 4
-        # a two-stride k axis is cut between runs only
+        # a two-stride k axis is cut into whole runs, or a run into whole slices
         if (K_full % split or (K_full // split) % vec_k
-                or any(g[t + "_k0"] != K_full and (K_full // split) % g[t + "_k0"] for t in ("a", "b"))):
+                or any(g[t + "_k0"] != K_full and (K_full // split) % g[t + "_k0"] and g[t + "_k0"] % (K_full // split) for t in ("a", "b"))):
             split = 1
     # ... or, with FUSEK (f32 template), folded inside the same launch by the slice that arrives last at the tile's
     # counter: one launch instead of two.
     fusek = 0
     if split > 1:
         KS = K_full // split
-        g = dict(g, K=KS, a_k0=KS if g["a_k0"] == K_full else g["a_k0"], b_k0=KS if g["b_k0"] == K_full else g["b_k0"])
+        run_full = dict(a=g["a_k0"], b=g["b_k0"])
+        # (a slice inside one run has a single stride, like a slice of a single-stride axis)
+        g = dict(g, K=KS, a_k0=KS if g["a_k0"] == K_full or g["a_k0"] > KS else g["a_k0"],
+                 b_k0=KS if g["b_k0"] == K_full or g["b_k0"] > KS else g["b_k0"])
         fusek = split if tile.get("FUSEK", 0) else 0
         if not fusek:
             out_t = "float"
@@ -786,9 +790,16 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     if split > 1:
         # a slice starts K elements further along k: K * sk for one stride, (K / k0) runs of sk1 for two
         # (whether the axis has two strides is the whole axis's property: a slice of exactly one run has k0 == K too)
-        a_step = g["K"] * g["a_sk"] if not two_stride["a"] else (g["K"] // g["a_k0"]) * g["a_sk1"]
-        b_step = g["K"] * g["b_sk"] if not two_stride["b"] else (g["K"] // g["b_k0"]) * g["b_sk1"]
-        lines.append(f"  a_base += (long long)blockIdx.y * {a_step}ll; b_base += (long long)blockIdx.y * {b_step}ll;"
+        # and for runs cut into r slices each, slice z is piece z % r of run z / r
+        def slice_offset(tag):
+            if not two_stride[tag]:
+                return f"(long long)blockIdx.y * {g['K'] * g[tag + '_sk']}ll"
+            if g["K"] % run_full[tag] == 0:
+                return f"(long long)blockIdx.y * {(g['K'] // run_full[tag]) * g[tag + '_sk1']}ll"
+            r = run_full[tag] // g["K"]
+            return f"((long long)(blockIdx.y / {r}) * {g[tag + '_sk1']}ll + (long long)(blockIdx.y % {r}) * {g['K'] * g[tag + '_sk']}ll)"
+
+        lines.append(f"  a_base += {slice_offset('a')}; b_base += {slice_offset('b')};"
                      + ("" if fusek else f" c_base += (long long)blockIdx.y * {pitch}ll;"))
         lines.append(f"  const int jh_k_off = (int)blockIdx.y * {g['K']};  // a gather loader is asked for k of the whole axis")
         for d in (gather_calls, gather_slow):

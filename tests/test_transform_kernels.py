@@ -443,7 +443,8 @@ def test_layer_sized_cotangent_plans():
     """Which templates and loaders the two cotangent convolutions of a 3x3 layer [8,64,56,56] -> 64 channels get (decided
     on the host): towards the activations the patch-in-LDS convolution template, its flipped and transposed filter read
     through the element loader by the weight pre-pass; towards the filter a GEMM over k = batch x positions in slices of
-    one image, the activations through the k-vector loader, the cotangent as a plain two-stride view."""
+    a quarter image (whole fractions of the cotangent's runs along k: one run is one image of one channel), the
+    activations through the k-vector loader, the cotangent as a plain two-stride view."""
     from jaxjs_hip.kernelgen import generate
     N, C, O, H = 8, 64, 64, 56
     p = ConvParams(0, [1, 1], [(1, 1), (1, 1)], [1, 1], [1, 1])
@@ -451,7 +452,7 @@ def test_layer_sized_cotangent_plans():
         pl = J.jit(lambda c, f: conv_transposed_to_lhs(c, f, [N, C, H, H], p), [ShapedArray((N, O, H, H), dt), ShapedArray((O, C, 3, 3), dt)])
         pr = J.jit(lambda a, c: conv_transposed_to_rhs(a, c, [O, C, 3, 3], p), [ShapedArray((N, C, H, H), dt), ShapedArray((N, O, H, H), dt)])
         kl, kr = generate(pl.kernels[0]), generate(pr.kernels[0])
-        assert kl.klass == "gemm" and kr.klass == "gemm+fold" and kr.info["splitk"] == N, (kl.klass, kr.klass, kr.info)
+        assert kl.klass == "gemm" and kr.klass == "gemm+fold" and kr.info["splitk"] == 4 * N, (kl.klass, kr.klass, kr.info)
         if dt == F16:
             assert kl.info["gather"] == {"a": "element (pre-pass)", "b": "patch"} and len(kl.steps) == 2, kl.info
             assert kr.info["gather"] == {"a": "k8", "b": "none"}, kr.info
