@@ -30,8 +30,8 @@ def choose_tile(g: dict) -> Dict[str, int]:
     CU = tuner.CU_COUNT
     # Slices of the k axis at most: 8, or 64 when the axis is very long (k = batch x positions of a filter cotangent:
     # 100352 against 9 output tiles), where the partial sums stay tiny next to the operands.
-    max_split = 64 if g["K"] >= 16384 else 8
     plain_k = not (g.get("a_gather") or g.get("b_gather")) and g["a_k0"] == g["K"] and g["b_k0"] == g["K"]
+    max_split = 64 if g["K"] >= (16384 if plain_k else 8192) else 8
     # A k axis that may be cut over workgroups: one stride per plain operand (a slice is a pointer offset), any gather
     # operand (a slice is an offset on the k its loader is asked for).
     # With exactly one gather operand and a short k axis the kernel is a forward convolution, whose stride-1 form has
@@ -656,12 +656,14 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                                       + "\n".join(mcg.take_lines()) + f"\n  return {mval};\n}}")
                     maskbit = f"jh_gmask_{tag}(row, e, k, b0, b1, b2)"
                 buf = names[gnode.arg[0]]
+                # (raw data + mask bits, the load unconditional: see the k-vector loader below)
                 gather_fns.append(
-                    f"static __device__ __forceinline__ jh_float4 jh_gather4_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
-                    f"  const int i0 = jh_gindex_{tag}(row, k, b0, b1, b2);\n  jh_float4 v;\n"
-                    f"  if ((unsigned)i0 <= (unsigned)({gnode.arg[1]} - 4)) {{\n    __builtin_memcpy(&v, {buf} + i0, 16);\n"
-                    f"#pragma unroll\n    for (int e = 0; e < 4; ++e) v[e] = {maskbit} ? v[e] : 0.0f;\n  }} else {{\n"
-                    f"#pragma unroll\n    for (int e = 0; e < 4; ++e) v[e] = jh_gather_{tag}(row + e, k, b0, b1, b2{epi_args});\n  }}\n  return v;\n}}")
+                    f"static __device__ __forceinline__ jh_g4 jh_gather4_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
+                    f"  const int i0 = jh_gindex_{tag}(row, k, b0, b1, b2);\n  jh_g4 out;\n  out.keep = 0u;\n"
+                    f"  const bool inb = (unsigned)i0 <= (unsigned)({gnode.arg[1]} - 4);\n  __builtin_memcpy(&out.v, {buf} + (inb ? i0 : 0), 16);\n"
+                    f"#pragma unroll\n  for (int e = 0; e < 4; ++e) out.keep |= ((inb && {maskbit}) ? 1u : 0u) << e;\n"
+                    f"  if (__builtin_amdgcn_ballot_w64(!inb) != 0) {{\n    if (!inb) {{\n"
+                    f"#pragma unroll\n      for (int e = 0; e < 4; ++e) out.v[e] = jh_gather_{tag}(row + e, k, b0, b1, b2{epi_args});\n      out.keep = 15u;\n    }}\n  }}\n  return out;\n}}")
                 gather_calls[tag] = f"jh_gather4_{tag}(row, k, jh_b0, jh_b1, jh_b2{epi_args})"
                 gather_flags[tag], gather_group[tag] = 5, 4
 
@@ -694,19 +696,40 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                 W = 8 if g["dtype"] == DType.Float16 else 4  # elements per chunk of the staging path
                 vec_t = "jh_half8" if g["dtype"] == DType.Float16 else "jh_float4"
                 zero = "(jh_f16)0.0f" if g["dtype"] == DType.Float16 else "0.0f"
-                gather_fns.append(
-                    f"typedef {in_t} jh_kpart_{tag} __attribute__((ext_vector_type({G})));\n"
-                    f"struct __attribute__((packed, aligned({2 if g['dtype'] == DType.Float16 else 4}))) jh_kpart_u_{tag} {{ jh_kpart_{tag} v; }};\n"
-                    f"static __device__ __forceinline__ {vec_t} jh_gatherk_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
-                    f"  {vec_t} out;\n#pragma unroll\n  for (int j = 0; j < {W // G}; ++j) {{\n    const int kk = k + j * {G};\n"
-                    f"    const int i0 = jh_kindex_{tag}(row, kk, b0, b1, b2);\n"
-                    f"    if ((unsigned)i0 <= (unsigned)({gnode.arg[1]} - {G})) {{\n"
-                    f"      const jh_kpart_{tag} part = reinterpret_cast<const jh_kpart_u_{tag}*>({buf} + i0)->v;\n"
-                    f"#pragma unroll\n      for (int e = 0; e < {G}; ++e) out[j * {G} + e] = {maskbit} ? part[e] : {zero};\n    }} else {{\n"
-                    f"#pragma unroll\n      for (int e = 0; e < {G}; ++e) out[j * {G} + e] = jh_gather_{tag}(row, kk + e, b0, b1, b2{epi_args});\n    }}\n  }}\n"
-                    f"  return out;\n}}")
+                part_t = (f"typedef {in_t} jh_kpart_{tag} __attribute__((ext_vector_type({G})));\n"
+                          f"struct __attribute__((packed, aligned({2 if g['dtype'] == DType.Float16 else 4}))) jh_kpart_u_{tag} {{ jh_kpart_{tag} v; }};\n")
+                if g["dtype"] == DType.Float16:
+                    # The f16 loader hands back the raw vector and the mask as bits (`jh_g8`), to be applied when the staged
+                    # registers are written to LDS, and its vector load is unconditional (a group that would leave the buffer
+                    # loads from the buffer's start instead).  A select right behind the load would wait for the data inside
+                    # the fetch, and a load under a branch makes the wait before the commit of the previous slab a wait for
+                    # everything (the counter of loads in flight is not known at the join): either way one slab's loads are
+                    # in flight instead of two.  Groups off the buffer are redone element by element under one wave-uniform
+                    # branch, which consumes its own loads before it ends.
+                    gather_fns.append(
+                        part_t + f"static __device__ __forceinline__ jh_g8 jh_gatherk_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
+                        f"  jh_g8 out;\n  out.keep = 0u;\n  unsigned off = 0u;\n#pragma unroll\n  for (int j = 0; j < {W // G}; ++j) {{\n    const int kk = k + j * {G};\n"
+                        f"    const int i0 = jh_kindex_{tag}(row, kk, b0, b1, b2);\n"
+                        f"    const bool inb = (unsigned)i0 <= (unsigned)({gnode.arg[1]} - {G});\n"
+                        f"    const jh_kpart_{tag} part = reinterpret_cast<const jh_kpart_u_{tag}*>({buf} + (inb ? i0 : 0))->v;\n"
+                        f"#pragma unroll\n    for (int e = 0; e < {G}; ++e) {{ out.v[j * {G} + e] = part[e]; out.keep |= ((inb && {maskbit}) ? 1u : 0u) << (j * {G} + e); }}\n"
+                        f"    off |= (inb ? 0u : 1u) << j;\n  }}\n"
+                        f"  if (__builtin_amdgcn_ballot_w64(off != 0u) != 0) {{\n#pragma unroll\n    for (int j = 0; j < {W // G}; ++j)\n      if ((off >> j) & 1u) {{\n"
+                        f"#pragma unroll\n        for (int e = 0; e < {G}; ++e) out.v[j * {G} + e] = jh_gather_{tag}(row, k + j * {G} + e, b0, b1, b2{epi_args});\n"
+                        f"        out.keep |= {(1 << G) - 1}u << (j * {G});\n      }}\n  }}\n"
+                        f"  return out;\n}}")
+                else:
+                    gather_fns.append(
+                        part_t + f"static __device__ __forceinline__ jh_g4 jh_gatherk_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
+                        f"  jh_g4 out;\n  out.keep = 0u;\n  const int i0 = jh_kindex_{tag}(row, k, b0, b1, b2);\n  const int kk = k;\n"
+                        f"  const bool inb = (unsigned)i0 <= (unsigned)({gnode.arg[1]} - 4);\n"
+                        f"  const jh_kpart_{tag} part = reinterpret_cast<const jh_kpart_u_{tag}*>({buf} + (inb ? i0 : 0))->v;\n"
+                        f"#pragma unroll\n  for (int e = 0; e < 4; ++e) {{ out.v[e] = part[e]; out.keep |= ((inb && {maskbit}) ? 1u : 0u) << e; }}\n"
+                        f"  if (__builtin_amdgcn_ballot_w64(!inb) != 0) {{\n    if (!inb) {{\n"
+                        f"#pragma unroll\n      for (int e = 0; e < 4; ++e) out.v[e] = jh_gather_{tag}(row, k + e, b0, b1, b2{epi_args});\n      out.keep = 15u;\n    }}\n  }}\n"
+                        f"  return out;\n}}")
                 gather_calls[tag] = f"jh_gatherk_{tag}(row, k, jh_b0, jh_b1, jh_b2{epi_args})"
-                gather_flags[tag] = 4 if g["dtype"] == DType.Float16 else 6
+                gather_flags[tag] = 7 if g["dtype"] == DType.Float16 else 6
                 gather_group[tag] = G
 
     # Tap-major k order (see `tap_major_form`): one gather operand whose k splits into (channel, tap), the other a plain
@@ -879,8 +902,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                      GATHER_A_SLOW=gather_slow.get("a", "jh_half8{0, 0, 0, 0, 0, 0, 0, 0}"), GATHER_B_SLOW=gather_slow.get("b", "jh_half8{0, 0, 0, 0, 0, 0, 0, 0}"))
     src = _prelude(numerics) + fill(template(tmpl), dict(sched, 
         M=g["M"], N=g["N"], K=g["K"], M_LOAD=load_rows["a"], N_LOAD=load_rows["b"], BM=BM, BN=BN, WM=WM, WN=WN,
-        A_KCONTIG=0 if gather_flags["a"] in (2, 3, 5) else (1 if g["a_sk"] == 1 or g["K"] == 1 or gather_flags["a"] in (1, 4, 6) else 0),
-        B_KCONTIG=0 if gather_flags["b"] in (2, 3, 5) else (1 if g["b_sk"] == 1 or g["K"] == 1 or gather_flags["b"] in (1, 4, 6) else 0),
+        A_KCONTIG=0 if gather_flags["a"] in (2, 3, 5) else (1 if g["a_sk"] == 1 or g["K"] == 1 or gather_flags["a"] in (1, 4, 6, 7) else 0),
+        B_KCONTIG=0 if gather_flags["b"] in (2, 3, 5) else (1 if g["b_sk"] == 1 or g["K"] == 1 or gather_flags["b"] in (1, 4, 6, 7) else 0),
         NBATCH=nbatch, EPILOGUE_FN=epi_fn, NAME=name, PARAMS=params,
         A_OFF=g["a_off"], B_OFF=g["b_off"], BATCH_DECODE="\n".join(lines),
         A_PTR="jh_repack_a" if "a" in (repack or "") else names[g["gid_a"]], B_PTR="jh_repack_b" if "b" in (repack or "") else names[g["gid_b"]],
@@ -905,7 +928,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         info.update(stages=sched["STAGES"], ring=sched["RING"])
     if any_gather:
         info["gather"] = {tag: {0: "none", 1: "element", 2: f"rows{gather_group.get(tag, 8)}", 3: f"tap-major rows{gather_group.get(tag, 8)}",
-                                4: "tap-major strided" if tap_major is not None else f"k{gather_group.get(tag, 8)}", 5: "rows4", 6: "k4"}[gather_flags[tag]] for tag in ("a", "b")}
+                                4: "tap-major strided" if tap_major is not None else f"k{gather_group.get(tag, 8)}", 5: "rows4", 6: "k4", 7: f"k{gather_group.get(tag, 8)}"}[gather_flags[tag]] for tag in ("a", "b")}
         if tap_major is not None:
             info["tap_major"] = tap_major
     if repack:
