@@ -405,6 +405,75 @@ def _affine_in(e: AluExp, name: str):
     return None
 
 
+def _conj_terms(c: AluExp):
+    """The terms of a conjunction (booleans multiply)."""
+    if c.op == AluOp.Mul and c.dtype == DType.Bool:
+        return _conj_terms(c.src[0]) + _conj_terms(c.src[1])
+    return [c]
+
+
+def interval_mask_form(cond: AluExp, name: str = "e"):
+    """`cond` as (terms without `name`, lower bounds, upper bounds): cond == all(terms) and lo <= name < hi for every
+    lower bound lo and upper bound hi (integer expressions without `name`); None when some term is not a comparison
+    that is affine in `name` with coefficient +-1.  The padding masks of window views have this form: along a run of
+    consecutive elements the elements inside the image are one interval."""
+    inv, lows, highs = [], [], []
+    for t in _conj_terms(cond):
+        if not _has_special(t, name):
+            inv.append(t)
+            continue
+        negated = False
+        while t.op == AluOp.Cmpne and t.src[0].dtype == DType.Bool and any(x.op == AluOp.Const for x in t.src):
+            c, x = (t.src[0], t.src[1]) if t.src[0].op == AluOp.Const else (t.src[1], t.src[0])
+            if bool(c.arg):
+                negated = not negated
+            t = x
+        if t.op != AluOp.Cmplt or t.src[0].dtype != DType.Int32:
+            return None
+        fa, fb = _affine_in(t.src[0], name), _affine_in(t.src[1], name)
+        if fa is None or fb is None:
+            return None
+        coef, rest = fa[0] - fb[0], AluExp.sub(fa[1], fb[1])  # the term reads coef * name + rest < 0
+        if coef == 1:  # name < -rest; negated: name >= -rest
+            (lows if negated else highs).append(AluExp.sub(AluExp.i32(0), rest).simplify())
+        elif coef == -1:  # name > rest, i.e. name >= rest + 1; negated: name <= rest, i.e. name < rest + 1
+            (highs if negated else lows).append(AluExp.add(rest, AluExp.i32(1)).simplify())
+        else:
+            return None
+    return inv, lows, highs
+
+
+def mask_bits_fn(cond_e, tag: str, G: int, names, numerics: str) -> str:
+    """C function `jh_mbits_<tag>(row, k, b0, b1, b2)`: bit e set when element e of the group of `G` that starts at
+    (row, k) is inside the operand's mask.  From the interval form where the mask has one (two bounds and a few compares
+    per group instead of a compare chain per element: the loaders of gather GEMMs are bound by such arithmetic), element
+    by element otherwise."""
+    head = f"static __device__ __forceinline__ unsigned jh_mbits_{tag}(int row, int k, int b0, int b1, int b2) {{\n"
+    if cond_e is None:
+        return head + f"  return {(1 << G) - 1}u;\n}}"
+    vnames = {"row": "row", "e": "e", "k": "k", "b0": "b0", "b1": "b1", "b2": "b2"}
+    form = interval_mask_form(cond_e)
+    cg = HipExpCodegen(names, vnames, "  ", prefix=f"mb{tag}", numerics=numerics)
+    if form is None:
+        cg.indent = "    "
+        cg.countReferences(cond_e)
+        val = strip_parens(cg.run(cond_e))
+        return (head + f"  unsigned bits = 0u;\n#pragma unroll\n  for (int e = 0; e < {G}; ++e) {{\n" + "\n".join(cg.take_lines())
+                + f"\n    bits |= (({val}) ? 1u : 0u) << e;\n  }}\n  return bits;\n}}")
+    inv, lows, highs = form
+    for x in inv + lows + highs:
+        cg.countReferences(x)
+    inv_c = [strip_parens(cg.run(x)) for x in inv]
+    lo_c = [strip_parens(cg.run(x)) for x in lows]
+    hi_c = [strip_parens(cg.run(x)) for x in highs]
+    body = "\n".join(cg.take_lines())
+    lo_s = "".join(f"  lo = lo > ({x}) ? lo : ({x});\n" for x in lo_c)
+    hi_s = "".join(f"  hi = hi < ({x}) ? hi : ({x});\n" for x in hi_c)
+    ok = " && ".join(["lo < hi"] + [f"({x})" for x in inv_c])
+    return (head + (body + "\n" if body else "") + f"  int lo = 0, hi = {G};\n{lo_s}{hi_s}"
+            f"  return ({ok}) ? (((1u << hi) - 1u) & ~((1u << lo) - 1u)) : 0u;\n}}")
+
+
 def tap_major_form(oexp: AluExp, K: int):
     """For a gather operand's expression in (row, k, batch coordinates): try k = c * T + tap for every T that the
     expression divides k by.  Returns dict(T, C, cs, exp) where `exp` is the operand re-expressed in (row, tap, batch
@@ -604,14 +673,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
             ilines = "\n".join(icg.take_lines())
             gather_fns.append(f"static __device__ __forceinline__ int jh_gindex_{tag}(int row, int k, int b0, int b1, int b2) {{\n"
                               f"{ilines}\n  return {ival};\n}}")
-            if cond_e is not None:
-                mcg = HipExpCodegen(names, vnames, "  ", prefix=f"m{tag}", numerics=numerics)
-                mcg.countReferences(cond_e)
-                mval = strip_parens(mcg.run(cond_e))
-                gather_fns.append(f"static __device__ __forceinline__ bool jh_gmask_{tag}(int row, int e, int k, int b0, int b1, int b2) {{\n"
-                                  + "\n".join(mcg.take_lines()) + f"\n  return {mval};\n}}")
+            gather_fns.append(mask_bits_fn(cond_e, tag, G, names, numerics))
             buf = names[gnode.arg[0]]
-            maskbit = f"jh_gmask_{tag}(r, e, k, b0, b1, b2)" if cond_e is not None else "true"
             # The loader only forms addresses and mask bits and issues the loads (no use of the loaded data, no
             # branches): the stager applies the mask when it writes the slab to LDS, one slab later, so the eight
             # loads of a block are in flight together.  A group that would leave the buffer loads from a clamped
@@ -627,7 +690,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                 f"    const bool inside = (unsigned)i0 <= (unsigned)({gnode.arg[1]} - {G});\n"
                 f"    if (!inside) out.keep |= 0x100u;\n"
                 f"    const jh_part_{tag} part = reinterpret_cast<const jh_part_u_{tag}*>({buf} + (inside ? i0 : 0))->v;\n"
-                f"#pragma unroll\n    for (int e = 0; e < {G}; ++e) {{ out.v[j * {G} + e] = part[e]; if ({maskbit}) out.keep |= 1u << (j * {G} + e); }}\n  }}\n"
+                f"#pragma unroll\n    for (int e = 0; e < {G}; ++e) out.v[j * {G} + e] = part[e];\n"
+                f"    out.keep |= jh_mbits_{tag}(r, k, b0, b1, b2) << (j * {G});\n  }}\n"
                 f"  return out;\n}}")
             gather_slow[tag] = f"jh_gather8_slow_{tag}(row, k, jh_b0, jh_b1, jh_b2{epi_args})"
             gather_calls[tag] = f"jh_gather8_{tag}(row, k, jh_b0, jh_b1, jh_b2{epi_args})"
@@ -647,21 +711,14 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                 ival = strip_parens(icg.run(idx0))
                 gather_fns.append(f"static __device__ __forceinline__ int jh_gindex_{tag}(int row, int k, int b0, int b1, int b2) {{\n"
                                   + "\n".join(icg.take_lines()) + f"\n  return {ival};\n}}")
-                maskbit = "true"
-                if cond_e is not None:
-                    mcg = HipExpCodegen(names, vnames, "  ", prefix=f"m{tag}", numerics=numerics)
-                    mcg.countReferences(cond_e)
-                    mval = strip_parens(mcg.run(cond_e))
-                    gather_fns.append(f"static __device__ __forceinline__ bool jh_gmask_{tag}(int row, int e, int k, int b0, int b1, int b2) {{\n"
-                                      + "\n".join(mcg.take_lines()) + f"\n  return {mval};\n}}")
-                    maskbit = f"jh_gmask_{tag}(row, e, k, b0, b1, b2)"
+                gather_fns.append(mask_bits_fn(cond_e, tag, 4, names, numerics))
                 buf = names[gnode.arg[0]]
                 # (raw data + mask bits, the load unconditional: see the k-vector loader below)
                 gather_fns.append(
                     f"static __device__ __forceinline__ jh_g4 jh_gather4_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
                     f"  const int i0 = jh_gindex_{tag}(row, k, b0, b1, b2);\n  jh_g4 out;\n  out.keep = 0u;\n"
                     f"  const bool inb = (unsigned)i0 <= (unsigned)({gnode.arg[1]} - 4);\n  __builtin_memcpy(&out.v, {buf} + (inb ? i0 : 0), 16);\n"
-                    f"#pragma unroll\n  for (int e = 0; e < 4; ++e) out.keep |= ((inb && {maskbit}) ? 1u : 0u) << e;\n"
+                    f"  out.keep = inb ? jh_mbits_{tag}(row, k, b0, b1, b2) : 0u;\n"
                     f"  if (__builtin_amdgcn_ballot_w64(!inb) != 0) {{\n    if (!inb) {{\n"
                     f"#pragma unroll\n      for (int e = 0; e < 4; ++e) out.v[e] = jh_gather_{tag}(row + e, k, b0, b1, b2{epi_args});\n      out.keep = 15u;\n    }}\n  }}\n  return out;\n}}")
                 gather_calls[tag] = f"jh_gather4_{tag}(row, k, jh_b0, jh_b1, jh_b2{epi_args})"
@@ -684,14 +741,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                 ival = strip_parens(icg.run(idx0))
                 gather_fns.append(f"static __device__ __forceinline__ int jh_kindex_{tag}(int row, int k, int b0, int b1, int b2) {{\n"
                                   + "\n".join(icg.take_lines()) + f"\n  return {ival};\n}}")
-                maskbit = "true"
-                if cond_e is not None:
-                    mcg = HipExpCodegen(names, vnames, "  ", prefix=f"km{tag}", numerics=numerics)
-                    mcg.countReferences(cond_e)
-                    mval = strip_parens(mcg.run(cond_e))
-                    gather_fns.append(f"static __device__ __forceinline__ bool jh_kmask_{tag}(int row, int e, int k, int b0, int b1, int b2) {{\n"
-                                      + "\n".join(mcg.take_lines()) + f"\n  return {mval};\n}}")
-                    maskbit = f"jh_kmask_{tag}(row, e, kk, b0, b1, b2)"
+                gather_fns.append(mask_bits_fn(cond_e, tag, G, names, numerics))
                 buf = names[gnode.arg[0]]
                 W = 8 if g["dtype"] == DType.Float16 else 4  # elements per chunk of the staging path
                 vec_t = "jh_half8" if g["dtype"] == DType.Float16 else "jh_float4"
@@ -712,7 +762,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                         f"    const int i0 = jh_kindex_{tag}(row, kk, b0, b1, b2);\n"
                         f"    const bool inb = (unsigned)i0 <= (unsigned)({gnode.arg[1]} - {G});\n"
                         f"    const jh_kpart_{tag} part = reinterpret_cast<const jh_kpart_u_{tag}*>({buf} + (inb ? i0 : 0))->v;\n"
-                        f"#pragma unroll\n    for (int e = 0; e < {G}; ++e) {{ out.v[j * {G} + e] = part[e]; out.keep |= ((inb && {maskbit}) ? 1u : 0u) << (j * {G} + e); }}\n"
+                        f"#pragma unroll\n    for (int e = 0; e < {G}; ++e) out.v[j * {G} + e] = part[e];\n"
+                        f"    if (inb) out.keep |= jh_mbits_{tag}(row, kk, b0, b1, b2) << (j * {G});\n"
                         f"    off |= (inb ? 0u : 1u) << j;\n  }}\n"
                         f"  if (__builtin_amdgcn_ballot_w64(off != 0u) != 0) {{\n#pragma unroll\n    for (int j = 0; j < {W // G}; ++j)\n      if ((off >> j) & 1u) {{\n"
                         f"#pragma unroll\n        for (int e = 0; e < {G}; ++e) out.v[j * {G} + e] = jh_gather_{tag}(row, k + j * {G} + e, b0, b1, b2{epi_args});\n"
@@ -724,7 +775,8 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                         f"  jh_g4 out;\n  out.keep = 0u;\n  const int i0 = jh_kindex_{tag}(row, k, b0, b1, b2);\n  const int kk = k;\n"
                         f"  const bool inb = (unsigned)i0 <= (unsigned)({gnode.arg[1]} - 4);\n"
                         f"  const jh_kpart_{tag} part = reinterpret_cast<const jh_kpart_u_{tag}*>({buf} + (inb ? i0 : 0))->v;\n"
-                        f"#pragma unroll\n  for (int e = 0; e < 4; ++e) {{ out.v[e] = part[e]; out.keep |= ((inb && {maskbit}) ? 1u : 0u) << e; }}\n"
+                        f"#pragma unroll\n  for (int e = 0; e < 4; ++e) out.v[e] = part[e];\n"
+                        f"  out.keep = inb ? jh_mbits_{tag}(row, k, b0, b1, b2) : 0u;\n"
                         f"  if (__builtin_amdgcn_ballot_w64(!inb) != 0) {{\n    if (!inb) {{\n"
                         f"#pragma unroll\n      for (int e = 0; e < 4; ++e) out.v[e] = jh_gather_{tag}(row, k + e, b0, b1, b2{epi_args});\n      out.keep = 15u;\n    }}\n  }}\n"
                         f"  return out;\n}}")
