@@ -116,3 +116,42 @@ def test_clamped_edge_loads_stay_inside_the_operand():
                         assert a == (r0 + r) * K + slab * bk + kk
                     if not k_contiguous and r + 7 <= last:
                         assert a == (slab * bk + kk) * extent + r0 + r
+
+
+def test_interval_form_of_a_mask_matches_the_mask_element_by_element():
+    """`gemm.interval_mask_form`: a conjunction of comparisons affine in `e` (coefficient +-1) and terms without `e` is
+    rewritten as invariant terms and bounds lo <= e < hi.  Checked against the condition itself on random values of the
+    other variables, for every e of a group; conditions outside the form (a coefficient of 2, a comparison of something
+    not affine in e) are refused."""
+    import random
+    from jaxjs_hip.alu import AluExp
+    from jaxjs_hip.gemm import interval_mask_form
+    I, S = AluExp.i32, AluExp.special
+    row, k, e = S(DType.Int32, "row", 4096), S(DType.Int32, "k", 100352), S(DType.Int32, "e", 8)
+    NOT = lambda c: AluExp.cmpne(c, AluExp.bool(True))
+    x = AluExp.add(AluExp.mod(k, I(56)), AluExp.mod(row, I(3)))          # column of a padded window, before e
+    y = AluExp.add(AluExp.mod(AluExp.idiv(k, I(56)), I(56)), AluExp.idiv(row, I(3)))
+    conds = {
+        "window": AluExp.mul(AluExp.mul(AluExp.cmplt(y, I(57)), NOT(AluExp.cmplt(y, I(1)))),
+                             AluExp.mul(AluExp.cmplt(AluExp.add(x, e), I(57)), NOT(AluExp.cmplt(AluExp.add(x, e), I(1))))),
+        "flipped": AluExp.mul(AluExp.cmplt(I(3), AluExp.sub(x, e)), NOT(AluExp.cmplt(I(40), AluExp.sub(x, e)))),   # 3 < x - e <= 40
+        "both sides": AluExp.cmplt(AluExp.add(e, I(2)), AluExp.sub(x, I(20))),
+        "double negation": NOT(NOT(AluExp.cmplt(AluExp.add(e, x), I(30)))),
+        "no e at all": AluExp.cmplt(y, I(20)),
+    }
+    rng = random.Random(5)
+    for name, cond in conds.items():
+        form = interval_mask_form(cond)
+        assert form is not None, name
+        inv, lows, highs = form
+        for _ in range(300):
+            ctx = {"row": rng.randrange(4096), "k": rng.randrange(100352)}
+            signed = lambda v: v - (1 << 32) if v >= (1 << 31) else v  # bounds are signed 32-bit values
+            lo = max([0] + [signed(b.evaluate(ctx)) for b in lows])
+            hi = min([8] + [signed(b.evaluate(ctx)) for b in highs])
+            ok = all(bool(t.evaluate(ctx)) for t in inv)
+            for ev in range(8):
+                want = bool(cond.evaluate(dict(ctx, e=ev)))
+                assert want == (ok and lo <= ev < hi), (name, ctx, ev)
+    assert interval_mask_form(AluExp.cmplt(AluExp.add(x, AluExp.mul(e, I(2))), I(57))) is None
+    assert interval_mask_form(AluExp.cmplt(AluExp.mod(AluExp.add(x, e), I(7)), I(3))) is None
