@@ -677,6 +677,27 @@ def test_gemm_f32_integer_exact_and_checker():
     np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("dt", [DType.Float16, DType.Float32], ids=lambda d: d.value)
+@pytest.mark.parametrize("split", [2, 4, 8, 16], ids=lambda n: "slices%d" % n)
+def test_gemm_k_slices_of_a_two_stride_axis(split, dt):
+    """A stored [H, M, D] contracted over (h, d): its k axis is H runs of D elements.  Slices of two runs, of one run, of
+    half and of a quarter of a run (a slice inside a run is piece z % r of run z / r) against B [K, N], which runs along
+    its rows.  Integer data: every slice count gives the same bits."""
+    H, D, M, N = 4, 512, 128, 128
+    K = H * D
+    npdt = np.float16 if dt == DType.Float16 else np.float32
+    A3 = RNG.integers(-2, 3, (H, M, D)).astype(npdt)
+    B = RNG.integers(-2, 3, (K, N)).astype(npdt)
+    full = [M, N, K]
+    stA = ShapeTracker.fromShape([H, M, D]).permute([1, 0, 2]).reshape([M, 1, K]).expand(full)
+    stB = ShapeTracker.fromShape([K, N]).permute([1, 0]).reshape([1, N, K]).expand(full)
+    k = reduceKernel(full, [(dt, stA), (dt, stB)], lambda a, b: AluExp.mul(a, b), AluOp.Add)
+    got, ks = device_run(k, [A3, B], gemm_tile=(("BM", 64), ("BN", 64), ("SPLITK", split)))
+    assert ks.klass.startswith("gemm") and ks.info["splitk"] == split, (ks.klass, ks.info)
+    A = np.ascontiguousarray(A3.transpose(1, 0, 2)).reshape(M, K)
+    np.testing.assert_array_equal(got.reshape(M, N).astype(np.float64), A.astype(np.float64) @ B.astype(np.float64))
+
+
 @pytest.mark.parametrize("H,D", [(4, 64), (3, 128), (2, 192)], ids=str)
 def test_gemm_f16_two_level_k_with_deep_slabs(H, D):
     """A stored [H, M, D] and contracted over (h, d) against B stored [N, H*D]: both operands run along k, A in runs of
