@@ -744,8 +744,6 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                 gather_fns.append(mask_bits_fn(cond_e, tag, G, names, numerics))
                 buf = names[gnode.arg[0]]
                 W = 8 if g["dtype"] == DType.Float16 else 4  # elements per chunk of the staging path
-                vec_t = "jh_half8" if g["dtype"] == DType.Float16 else "jh_float4"
-                zero = "(jh_f16)0.0f" if g["dtype"] == DType.Float16 else "0.0f"
                 part_t = (f"typedef {in_t} jh_kpart_{tag} __attribute__((ext_vector_type({G})));\n"
                           f"struct __attribute__((packed, aligned({2 if g['dtype'] == DType.Float16 else 4}))) jh_kpart_u_{tag} {{ jh_kpart_{tag} v; }};\n")
                 if g["dtype"] == DType.Float16:
@@ -772,7 +770,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
                 else:
                     gather_fns.append(
                         part_t + f"static __device__ __forceinline__ jh_g4 jh_gatherk_{tag}(int row, int k, int b0, int b1, int b2{epi_params}) {{\n"
-                        f"  jh_g4 out;\n  out.keep = 0u;\n  const int i0 = jh_kindex_{tag}(row, k, b0, b1, b2);\n  const int kk = k;\n"
+                        f"  jh_g4 out;\n  out.keep = 0u;\n  const int i0 = jh_kindex_{tag}(row, k, b0, b1, b2);\n"
                         f"  const bool inb = (unsigned)i0 <= (unsigned)({gnode.arg[1]} - 4);\n"
                         f"  const jh_kpart_{tag} part = reinterpret_cast<const jh_kpart_u_{tag}*>({buf} + (inb ? i0 : 0))->v;\n"
                         f"#pragma unroll\n  for (int e = 0; e < 4; ++e) out.v[e] = part[e];\n"
