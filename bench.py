@@ -489,11 +489,12 @@ def main():
     ap.add_argument("--no-settle", action="store_true", help="skip the clock-settling launches before the warm-up steps")
     ap.add_argument("--no-graphs", action="store_true", help="skip the HIP-graph replays of the C5 programs (for runs under a profiler "
                                                              "whose graph-launch tracing is not to be relied on)")
-    ap.add_argument("--only", choices=["all", "gemm", "copy", "hbm", "matvec"], default="all",
+    ap.add_argument("--only", choices=["all", "gemm", "copy", "hbm", "matvec", "attention"], default="all",
                     help="gemm: headline kernel only; copy: a plain f32 copy kernel of known size (counter calibration); "
                          "hbm: headline + the HBM-bound secondary workloads only (matvecs, row kernels, map); "
                          "matvec: the two f16 matvec layouts under the launch plans compared in profiles/ (each as its own "
-                         "named kernel, cache-resident and cold), nothing else")
+                         "named kernel, cache-resident and cold), nothing else; attention: the GPT-2 block with the fused "
+                         "attention routine and that launch (`jh_attention`) alone, nothing else")
     args = ap.parse_args()
     global USE_GRAPHS
     USE_GRAPHS = not args.no_graphs
@@ -551,6 +552,11 @@ def main():
             for s_ in ws + [xs, o]:
                 be.decRef(s_)
         print(json.dumps({"workload": "f16 matvec [11008,4096], both layouts, plans compared", "bytes_per_launch": mv_bytes, "rows": rows}))
+        return
+
+    if args.only == "attention":
+        print(json.dumps({"workload": "GPT-2-small block, batch 8 x 1024 tokens, f16, fused attention routine (causal, 12 heads of 64)",
+                          **bench_program_gpt2_fused(be, hostrand, timed)}))
         return
 
     # ---- headline: f16 GEMM n^3 -----------------------------------------------------------------
