@@ -77,9 +77,12 @@ def choose_tile(g: dict) -> Dict[str, int]:
             # The slices are folded inside the launch (1024^3: 30.2 -> 27.8 us, 128x14336x4096: 169 -> 166, same bits);
             # four waves stacked along m then measure another 1 % better than 2x2.
             return dict(BM=128, BN=64, BK=bk, SPLITK=split, **(dict(FUSEK=1, WM=4, WN=1) if split > 1 else {}))
-        # Fewer than 128 rows or 64 columns: 64x64 tiles, the k axis cut the same way when they are few.
+        # Fewer than 128 rows or 64 columns: 64x64 tiles, the k axis cut the same way when they are few.  Gather operands
+        # keep gaining up to four workgroups per CU (filter cotangents: [32,128,28,28] 143 us in 16 slices = 576
+        # workgroups, 115 us in 32; [8,64,56,56] 54 -> 49 us; [16,128,28,28] 78 -> 67 us; [32,256,14,14] 183 -> 162 us).
+        fill = 4.0 if not plain_k and g["K"] >= 8192 else 1.5
         split = 1
-        while cut_k and tiles(64, 64) * split < 1.5 * CU and split < max_split and g["K"] % (split * 2 * bk) == 0 and g["K"] // (split * 2) >= 256 and runs_ok(split * 2):
+        while cut_k and tiles(64, 64) * split < fill * CU and split < max_split and g["K"] % (split * 2 * bk) == 0 and g["K"] // (split * 2) >= 256 and runs_ok(split * 2):
             split *= 2
         return dict(BM=64, BN=64, BK=bk, **(dict(SPLITK=split, FUSEK=1 if plain_k else 0) if split > 1 else {}))
     # f16: estimated time = (tiles the busiest CU runs) x (tile area) x (K + fixed per-tile overhead) / efficiency.
@@ -88,11 +91,11 @@ def choose_tile(g: dict) -> Dict[str, int]:
     # 218 us against 180 us with 128x256), 0.64 alone with its deeper slabs.  The fixed
     # overhead (pipeline fill + epilogue) is about 100 k-steps.  This picks big tiles for big problems and
     # smaller ones when 256x256 would leave the last round of CUs nearly empty (e.g. 288 tiles on 256 CUs).
-    def k_split(count):
-        # Fewer workgroups than 1.5 per CU: cut the k axis (partial sums in scratch, fold kernel) while slices stay >= 512 deep.
+    def k_split(count, fill=1.5):
+        # Fewer workgroups than `fill` per CU: cut the k axis (partial sums in scratch, fold kernel) while slices stay >= 512 deep.
         split = 1
         gran = 64 if plain_k else 8  # whole slabs for the direct loads; the gather loaders take a ragged last slab
-        while cut_k and count * split < 1.5 * CU and split < max_split and g["K"] % (split * 2 * gran) == 0 and g["K"] // (split * 2) >= 512 and runs_ok(split * 2):
+        while cut_k and count * split < fill * CU and split < max_split and g["K"] % (split * 2 * gran) == 0 and g["K"] // (split * 2) >= 512 and runs_ok(split * 2):
             split *= 2
         return dict(SPLITK=split) if split > 1 else {}
 
@@ -132,9 +135,12 @@ def choose_tile(g: dict) -> Dict[str, int]:
     if not plain_k and cut_k and g["K"] >= 8192 and tiles(128, 128) * 8 <= CU:
         # A handful of tiles over a very long k axis read through gather loaders (the filter cotangent of a convolution:
         # 9 taps x 64 x 64 or 128 x 128 outputs, k = batch x positions): 64x64 tiles waste no half-empty MFMA tile and
-        # give the k slices four times as many workgroups ([32,64,56,56] 93 -> 72 us, [32,128,28,28] 187 -> 64 us); slices
-        # of half an image (a run of the cotangent's k axis cut in two) double them again: 72 -> 57 us.
-        return dict(BM=64, BN=64, **k_split(tiles(64, 64)))
+        # give the k slices four times as many workgroups ([32,64,56,56] 93 -> 72 us, [32,128,28,28] 187 -> 64 us).  With a
+        # gather loader on one side only, one workgroup per CU is where more slices stop paying ([32,64,56,56]: 48 us in
+        # 32 slices = 288 workgroups, 53 us in 64; [8,64,56,56]: 25 / 30 us); with one on both sides the loads are slower
+        # and 1.5 per CU still gain ([32,128,28,28]: 61 us in 8 slices = 288 workgroups, 51 in 16, 53 in 32).
+        both = bool(g.get("a_gather")) and bool(g.get("b_gather"))
+        return dict(BM=64, BN=64, **k_split(tiles(64, 64), 1.5 if both else 1.0))
     best = None
     for bm, bn, eff, extra in ((256, 256, 1.00, dict()), (128, 256, 0.84, dict(WM=1, WN=4)), (256, 128, 0.79, dict()),
                                 (128, 128, 0.62, dict())):
