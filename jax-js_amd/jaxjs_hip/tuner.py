@@ -525,6 +525,22 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
             w_col += weight
 
     row_major = w_row >= w_col and w_row > 0 and R >= 8
+    # A short fold whose only stream along the reduce axis is a small table, under many outputs (the first layer of a
+    # small CNN: 9 or 25 filter taps per output, one input channel, millions of outputs): one lane per output walks the
+    # taps, so that consecutive lanes read consecutive pixels, instead of a few lanes sharing every output's taps.
+    # (The image itself is unit-stride along both axes -- a window row is a few consecutive pixels --, so it is weighed
+    # here by its stride along the outputs.)
+    if row_major and R <= 64 and size >= CU_COUNT * 256:
+        w_g = w_r_only = 0
+        for node in loads:
+            fr, fg = lane_form(node.src[0], "ridx", 1), lane_form(node.src[0], "gidx", 1)
+            weight = node.arg[1] * byteWidth(node.dtype)
+            if fg is not None and 1 <= fg[0] <= 4:  # (a strided window walk reads every 2nd..4th pixel)
+                w_g += weight
+            elif fr is not None and fr[0] == 1:
+                w_r_only += weight
+        if w_g >= 8 * w_r_only and w_g > 0:
+            row_major = False
     if w_row == 0 and w_col == 0 and size < 4096 and R >= 1024:
         row_major = True  # few outputs, long fold, no coalescing either way: spread the fold over lanes
 

@@ -526,3 +526,54 @@ def test_f16_convolution_on_gpu_is_exact_on_small_integers(case, tap_major):
         pads = L.padtypeToPads(case["x"][2:], case["w"][2:], case["strides"], case.get("rd") or [1] * len(case["strides"]), pads)
     want = conv_reference(x.astype(np.float32), w.astype(np.float32), case["strides"], pads, None, case.get("rd"))
     np.testing.assert_array_equal(r.reshape(want.shape).astype(np.float64), want)  # |sums| < 2048: exact in f16
+
+
+# First layers of small CNNs: one (or three) input channels, a handful of taps per output, millions of outputs.  Too few
+# k for the matrix cores; the fold is short and its only stream along the reduce axis is the filter, so one lane per output
+# walks the taps (column class, unrolled whole) instead of a few lanes sharing each output's taps.
+FIRST_LAYER_CONVS = [
+    dict(x=(128, 1, 28, 28), w=(32, 1, 3, 3), strides=[1, 1], padding="VALID"),
+    dict(x=(256, 1, 28, 28), w=(8, 1, 5, 5), strides=[1, 1], padding="SAME"),
+    dict(x=(64, 1, 28, 28), w=(16, 1, 3, 3), strides=[2, 2], padding="SAME"),
+    dict(x=(96, 2, 20, 24), w=(24, 2, 3, 3), strides=[1, 1], padding="SAME", rd=[2, 2]),
+]
+
+
+@pytest.mark.parametrize("case", FIRST_LAYER_CONVS, ids=lambda c: "x".join(map(str, c["x"])) + "*" + "x".join(map(str, c["w"])))
+def test_first_layer_convolutions_take_one_lane_per_output(case):
+    from jaxjs_hip.kernelgen import generate
+    for dt in (F32, DType.Float16):
+        prog = J.jit(lambda a, b: L.convGeneralDilated(a, b, case["strides"], case["padding"], rhsDilation=case.get("rd")),
+                     [ShapedArray(case["x"], dt), ShapedArray(case["w"], dt)])
+        ks = generate(prog.kernels[0])
+        assert ks.klass == "reduce_col" and ks.info["T"] == 1 and ks.info["split"] == 1, (ks.klass, ks.info)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt,npdt", [(DType.Float16, np.float16), (DType.Float32, np.float32)], ids=["f16", "f32"])
+@pytest.mark.parametrize("case", FIRST_LAYER_CONVS, ids=lambda c: "x".join(map(str, c["x"])) + "*" + "x".join(map(str, c["w"])))
+def test_first_layer_convolutions_on_gpu_are_exact_on_small_integers(case, dt, npdt):
+    from gpu_util import WARM_ONLY, backend
+    prog = J.jit(lambda a, b: L.convGeneralDilated(a, b, case["strides"], case["padding"], rhsDilation=case.get("rd")),
+                 [ShapedArray(case["x"], dt), ShapedArray(case["w"], dt)])
+    if WARM_ONLY:
+        from jaxjs_hip.kernelgen import generate
+        from jaxjs_hip.runtime import compile_source
+        for src in generate(prog.kernels[0]).sources:
+            compile_source(src)
+        pytest.skip("warm-up run: compiled only")
+    rng = np.random.default_rng(17)
+    x = rng.integers(-2, 3, case["x"]).astype(npdt)
+    w = rng.integers(-2, 3, case["w"]).astype(npdt)
+    be = backend()
+    exe = be.prepareKernelSync(prog.kernels[0])
+    sx, sw, so = be.malloc(x.nbytes, x.tobytes()), be.malloc(w.nbytes, w.tobytes()), be.malloc(prog.kernels[0].bytes)
+    be.dispatch(exe, [sx, sw], [so])
+    r = np.frombuffer(be.readSync(so), npdt).copy()
+    for s_ in (sx, sw, so):
+        be.decRef(s_)
+    pads = case["padding"]
+    if isinstance(pads, str):
+        pads = L.padtypeToPads(case["x"][2:], case["w"][2:], case["strides"], case.get("rd") or [1] * len(case["strides"]), pads)
+    want = conv_reference(x.astype(np.float32), w.astype(np.float32), case["strides"], pads, None, case.get("rd"))
+    np.testing.assert_array_equal(r.reshape(want.shape).astype(np.float64), want, err_msg=str(exe.data.ks.info))
