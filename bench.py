@@ -746,6 +746,15 @@ def main():
                 [hostrand.normal(1007, cx, 1.0, np.float16), hostrand.normal(1007, cw, 0.05, np.float16, stream=1)],
                 2.0 * cx[0] * cw[0] * (cx[2] // st) * (cx[3] // st) * cw[1] * 9, "TFLOP/s", PEAK_F16_TFLOPS)
 
+        # The reference's own conv2d bench (website/src/routes/bench/conv2d/strategies.ts:13-19: fp32, one 64 x 256 x 256
+        # image, 128 filters of 3 x 3, SAME padding, `lax.convGeneralDilated`), and the same layer in f16.
+        for cdt, npdt, tag in ((DType.Float32, np.float32, "f32"), (DType.Float16, np.float16, "f16")):
+            cx, cw = (1, 64, 256, 256), (128, 64, 3, 3)
+            cprog = J.jit(lambda a, b: Lb.convGeneralDilated(a, b, [1, 1], "SAME"), [ShapedArray(cx, cdt), ShapedArray(cw, cdt)])
+            run(f"reference_conv2d_bench_{tag}[1,64,256,256]x[128,64,3,3]", cprog.kernels[0],
+                [hostrand.normal(1009, cx, 1.0, npdt), hostrand.normal(1009, cw, 0.05, npdt, stream=1)],
+                2.0 * 128 * 64 * 256 * 256 * 9, "TFLOP/s", PEAK_F32_MATRIX_TFLOPS if cdt == DType.Float32 else PEAK_F16_TFLOPS)
+
         # The two cotangent convolutions of the 56x56x64 layer (what the transpose rule of Conv binds,
         # src/frontend/linearize.ts:783-837): towards the activations and towards the filter (the latter followed by a
         # small transposing map kernel, timed with it).

@@ -404,7 +404,8 @@ def test_f16_convolution_loader_choice(case):
 # ---- the layer shapes the bench measures, at full size --------------------------------------------------------------
 
 LAYER_CONVS = [((32, 64, 56, 56), (64, 64, 3, 3), 1), ((32, 256, 28, 28), (256, 256, 3, 3), 1), ((32, 256, 14, 14), (256, 256, 3, 3), 1),
-               ((32, 64, 56, 56), (128, 64, 3, 3), 2)]
+               ((32, 64, 56, 56), (128, 64, 3, 3), 2),
+               ((1, 64, 256, 256), (128, 64, 3, 3), 1)]  # the reference's conv2d bench (website/src/routes/bench/conv2d/strategies.ts:13-19)
 
 
 @pytest.mark.gpu
