@@ -578,3 +578,32 @@ def test_first_layer_convolutions_on_gpu_are_exact_on_small_integers(case, dt, n
         pads = L.padtypeToPads(case["x"][2:], case["w"][2:], case["strides"], case.get("rd") or [1] * len(case["strides"]), pads)
     want = conv_reference(x.astype(np.float32), w.astype(np.float32), case["strides"], pads, None, case.get("rd"))
     np.testing.assert_array_equal(r.reshape(want.shape).astype(np.float64), want, err_msg=str(exe.data.ks.info))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt,npdt", [(DType.Float16, np.float16), (DType.Float32, np.float32)], ids=["f16", "f32"])
+@pytest.mark.parametrize("cx,cw,groups", [((8, 64, 56, 56), (64, 8, 3, 3), 8), ((4, 32, 40, 40), (32, 1, 3, 3), 32), ((2, 16, 64, 64), (16, 4, 5, 5), 4)],
+                         ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else f"g{v}")
+def test_grouped_and_depthwise_convolutions_on_gpu_are_exact_on_small_integers(cx, cw, groups, dt, npdt):
+    """Feature groups (lax.ts:252-343): a leading batch axis of the Conv primitive, k = C/G x taps per output -- too few rows
+    per group for the matrix cores.  One lane per output, the fold of up to 256 steps unrolled whole; checked group by group
+    against the host convolution."""
+    from gpu_util import WARM_ONLY, backend
+    from jit_util import run_program
+    prog = J.jit(lambda a, b: L.convGeneralDilated(a, b, [1, 1], "SAME", featureGroupCount=groups), [ShapedArray(cx, dt), ShapedArray(cw, dt)])
+    if WARM_ONLY:
+        from jaxjs_hip.kernelgen import generate
+        from jaxjs_hip.runtime import compile_source
+        for k in prog.kernels:
+            for src in generate(k).sources:
+                compile_source(src)
+        pytest.skip("warm-up run: compiled only")
+    rng = np.random.default_rng(19)
+    x = rng.integers(-2, 3, cx).astype(npdt)
+    w = rng.integers(-2, 3, cw).astype(npdt)
+    (got,) = run_program(backend(), prog, [x, w])
+    pads = L.padtypeToPads(cx[2:], cw[2:], [1, 1], [1, 1], "SAME")
+    cg, og = cx[1] // groups, cw[0] // groups
+    want = np.concatenate([conv_reference(x[:, g * cg:(g + 1) * cg].astype(np.float32), w[g * og:(g + 1) * og].astype(np.float32), [1, 1], pads)
+                           for g in range(groups)], axis=1)
+    np.testing.assert_array_equal(np.asarray(got).reshape(want.shape).astype(np.float64), want)
