@@ -208,6 +208,11 @@ def gen_conv(kernel, g: dict, oexp: AluExp, numerics: str, name: str, params: st
         return None
     # output rows a tile's BN consecutive positions span; the image rows behind them live in SY planes (by row % SY) of
     # RP rows each: plane rows from floor(-PH / SY) to floor((KH - 1 - PH) / SY) past the tile's first and last row
+    # The patch holds whole image rows: a row several times as wide as the tile (a long 1-D signal: 1500 positions against
+    # 256) would be filled again by every tile along it, slab after slab ([1,384,3000] * [384,384,3] stride 2: 500 us here,
+    # 49 us on the gather loaders).
+    if OWP > 4 * BN:
+        return None
     n_tiles = -(-NV // BN)
     spans = max((min(t * BN + BN - 1, NV - 1) // OWP) - ((t * BN) // OWP) + 1 for t in range(n_tiles))
     SX, SY = cv["SX"], cv["SY"]

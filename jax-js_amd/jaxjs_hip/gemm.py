@@ -141,6 +141,13 @@ def choose_tile(g: dict) -> Dict[str, int]:
         # and 1.5 per CU still gain ([32,128,28,28]: 61 us in 8 slices = 288 workgroups, 51 in 16, 53 in 32).
         both = bool(g.get("a_gather")) and bool(g.get("b_gather"))
         return dict(BM=64, BN=64, **k_split(tiles(64, 64), 1.5 if both else 1.0))
+    if (bool(g.get("a_gather")) != bool(g.get("b_gather")) and g["K"] < 8192 and g["M"] >= 128 and g["N"] >= 128
+            and g["a_k0"] == g["K"] and g["b_k0"] == g["K"] and tiles(128, 128) < CU):
+        # One gather operand, fewer 128x128 tiles than CUs (the convolutions of audio models: a few hundred channels
+        # against one long row of a few thousand positions): smaller tiles until the launch covers the chip.
+        # [1,512,1500] * [512,512,3]: 48 tiles, 40.5 us; 192 of 64x64, 33.5 us.  [1,384,3000] stride 2: 36 tiles, 46.5 us;
+        # 144 of 64x64, 24.3 us.  [1,256,8000] * [256,256,7]: 126 tiles, 50.5 us; 250 of 128x64, 42.3 us (64x64: 49.6).
+        return dict(BM=64, BN=64) if tiles(128, 128) * 4 <= 1.5 * CU else dict(BM=128, BN=64)
     best = None
     for bm, bn, eff, extra in ((256, 256, 1.00, dict()), (128, 256, 0.84, dict(WM=1, WN=4)), (256, 128, 0.79, dict()),
                                 (128, 128, 0.62, dict())):

@@ -607,3 +607,52 @@ def test_grouped_and_depthwise_convolutions_on_gpu_are_exact_on_small_integers(c
     want = np.concatenate([conv_reference(x[:, g * cg:(g + 1) * cg].astype(np.float32), w[g * og:(g + 1) * og].astype(np.float32), [1, 1], pads)
                            for g in range(groups)], axis=1)
     np.testing.assert_array_equal(np.asarray(got).reshape(want.shape).astype(np.float64), want)
+
+
+# Convolutions of audio models: a few hundred channels against one long row of a few thousand positions.
+LONG_ROW_CONVS = [
+    dict(x=(1, 80, 3000), w=(384, 80, 3), strides=[1], padding="SAME"),
+    dict(x=(1, 384, 3000), w=(384, 384, 3), strides=[2], padding="SAME"),
+    dict(x=(1, 512, 1500), w=(512, 512, 3), strides=[1], padding="SAME"),
+]
+
+
+def test_long_row_convolutions_keep_off_the_patch_template_and_cover_the_chip():
+    """The patch-in-LDS template holds whole image rows, so a row several times as wide as its tile would be filled again by
+    every tile along it ([1,384,3000] stride 2 took 500 us that way); such shapes run on the gather loaders, in tiles small
+    enough that the launch has at least half as many workgroups as the chip has CUs."""
+    from jaxjs_hip.kernelgen import generate
+    from jaxjs_hip import tuner
+    for case in LONG_ROW_CONVS:
+        prog = J.jit(lambda a, b: L.convGeneralDilated(a, b, case["strides"], case["padding"]),
+                     [ShapedArray(case["x"], DType.Float16), ShapedArray(case["w"], DType.Float16)])
+        ks = generate(prog.kernels[0])
+        assert ks.klass == "gemm" and ks.info["gather"]["b"] != "patch" and ks.info["tiles"] * 2 >= tuner.CU_COUNT, ks.info
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt,npdt", [(DType.Float16, np.float16), (DType.Float32, np.float32)], ids=["f16", "f32"])
+@pytest.mark.parametrize("case", LONG_ROW_CONVS, ids=lambda c: "x".join(map(str, c["x"])) + "*" + "x".join(map(str, c["w"])))
+def test_long_row_convolutions_on_gpu_are_exact_on_small_integers(case, dt, npdt):
+    from gpu_util import WARM_ONLY, backend
+    prog = J.jit(lambda a, b: L.convGeneralDilated(a, b, case["strides"], case["padding"]), [ShapedArray(case["x"], dt), ShapedArray(case["w"], dt)])
+    if WARM_ONLY:
+        from jaxjs_hip.kernelgen import generate
+        from jaxjs_hip.runtime import compile_source
+        for src in generate(prog.kernels[0]).sources:
+            compile_source(src)
+        pytest.skip("warm-up run: compiled only")
+    rng = np.random.default_rng(23)
+    x = rng.integers(-1, 2, case["x"]).astype(npdt)
+    w = rng.integers(-1, 2, case["w"]).astype(npdt)
+    be = backend()
+    exe = be.prepareKernelSync(prog.kernels[0])
+    sx, sw, so = be.malloc(x.nbytes, x.tobytes()), be.malloc(w.nbytes, w.tobytes()), be.malloc(prog.kernels[0].bytes)
+    be.dispatch(exe, [sx, sw], [so])
+    r = np.frombuffer(be.readSync(so), npdt).copy()
+    for s_ in (sx, sw, so):
+        be.decRef(s_)
+    pads = L.padtypeToPads(case["x"][2:], case["w"][2:], case["strides"], [1], case["padding"])
+    want = conv_reference(x.astype(np.float32), w.astype(np.float32), case["strides"], pads)
+    assert np.abs(want).max() < 2048
+    np.testing.assert_array_equal(r.reshape(want.shape).astype(np.float64), want, err_msg=str(exe.data.ks.info))
