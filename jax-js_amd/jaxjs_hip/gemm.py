@@ -42,8 +42,14 @@ def choose_tile(g: dict) -> Dict[str, int]:
     def runs_ok(slices):  # whole runs, or a whole fraction of one
         return all((g["K"] // slices) % k0 == 0 or k0 % (g["K"] // slices) == 0 for k0 in two_level)
 
+    # (float32 has no such template: its forward convolutions are cut like any other gather GEMM.  Nor is that template
+    # any use to a float16 convolution with a handful of tiles -- one small image, many channels: [1,512,7,7] * [512,512,3,3]
+    # is 8 tiles whatever the template -- which is cut as well and then runs on the gather loaders.)
+    one_gather = bool(g.get("a_gather")) != bool(g.get("b_gather"))
+    few_tiles = (one_gather and 1024 <= g["K"] < 8192 and g["M"] >= 64 and tiles(64, 128) * 4 <= CU
+                 and g["M"] * g["N"] * nb * g["K"] >= (1 << 26))  # (smaller than that, a launch is a launch)
     cut_k = (all(g["K"] % k0 == 0 for k0 in two_level)
-             and (bool(g.get("a_gather")) == bool(g.get("b_gather")) or g["K"] >= 8192))
+             and (not one_gather or g["K"] >= 8192 or g["dtype"] == DType.Float32 or few_tiles))
     repack = _repack_operand(g)  # that operand is read from an aligned copy (rows padded to whole groups)
     loose_ops = bool(g.get("a_loose") or g.get("b_loose")) and repack is None
 
@@ -141,6 +147,9 @@ def choose_tile(g: dict) -> Dict[str, int]:
         # and 1.5 per CU still gain ([32,128,28,28]: 61 us in 8 slices = 288 workgroups, 51 in 16, 53 in 32).
         both = bool(g.get("a_gather")) and bool(g.get("b_gather"))
         return dict(BM=64, BN=64, **k_split(tiles(64, 64), 1.5 if both else 1.0))
+    if few_tiles and cut_k:
+        # [1,512,7,7] * [512,512,3,3] f16: 47.9 us as 8 tiles of the patch template; [1,256,28,28] stride 2: 37.9 us.
+        return dict(BM=64, BN=64, **k_split(tiles(64, 64)))
     if (bool(g.get("a_gather")) != bool(g.get("b_gather")) and g["K"] < 8192 and g["M"] >= 128 and g["N"] >= 128
             and g["a_k0"] == g["K"] and g["b_k0"] == g["K"] and tiles(128, 128) < CU):
         # One gather operand, fewer 128x128 tiles than CUs (the convolutions of audio models: a few hundred channels

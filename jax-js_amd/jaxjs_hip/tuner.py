@@ -525,12 +525,13 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
             w_col += weight
 
     row_major = w_row >= w_col and w_row > 0 and R >= 8
-    # A short fold whose only stream along the reduce axis is a small table, under many outputs (the first layer of a
-    # small CNN: 9 or 25 filter taps per output, one input channel, millions of outputs): one lane per output walks the
+    # A short fold (up to 256 steps: what the column template unrolls whole) whose only stream along the reduce axis is a
+    # small table, under many outputs (the first layer of a small CNN: 9 or 25 or 75 filter taps per output, one or three
+    # input channels, millions of outputs): one lane per output walks the
     # taps, so that consecutive lanes read consecutive pixels, instead of a few lanes sharing every output's taps.
     # (The image itself is unit-stride along both axes -- a window row is a few consecutive pixels --, so it is weighed
     # here by its stride along the outputs.)
-    if row_major and R <= 64 and size >= CU_COUNT * 256:
+    if row_major and R <= 256 and size >= CU_COUNT * 256:
         w_g = w_r_only = 0
         for node in loads:
             fr, fg = lane_form(node.src[0], "ridx", 1), lane_form(node.src[0], "gidx", 1)
