@@ -173,6 +173,7 @@ class _Body:
     def lanes(self, loads: Dict[int, str]) -> Tuple[str, str]:
         cg = HipExpCodegen(self.args, self.names, self.indent + "  ", prefix=f"l{self.tag}", numerics=self.numerics)
         cg.loads = loads
+        cg.packed_lanes = self.V > 1
         cg.countReferences(self.exp)
         value = strip_parens(cg.run(self.exp))
         return "\n".join(cg.take_lines()), value
@@ -181,6 +182,7 @@ class _Body:
         """`lanes` for several expressions that share one statement list (the two factors of a product)."""
         cg = HipExpCodegen(self.args, self.names, self.indent + "  ", prefix=f"l{self.tag}", numerics=self.numerics)
         cg.loads = loads
+        cg.packed_lanes = self.V > 1
         for e in exps:
             cg.countReferences(e)
         values = [strip_parens(cg.run(e)) for e in exps]

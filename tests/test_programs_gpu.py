@@ -97,6 +97,24 @@ def test_row_softmax_argmax_program():
     np.testing.assert_allclose(y, bufs[prog.outputs[0]], rtol=1e-5 * math.sqrt(1000))
 
 
+@pytest.mark.parametrize("rows,cols", [(64, 1001), (16, 50257)], ids=str)
+def test_float16_log_softmax_over_rows_off_the_pack_width(rows, cols):
+    """`x - log(sum)` in float16 with rows that are not whole packs of eight: every lane of a pack reads its own row's
+    statistic, rounds the logarithm to float16 and negates it (a form the device compiler could not select before the
+    rounded value was made opaque to it); each kernel against the checker."""
+    from jaxjs_hip import jit as J, library as Lb
+    from jaxjs_hip.jit import ShapedArray
+    prog = J.jit(lambda x: Lb.logSoftmax(x, -1), [ShapedArray((rows, cols), DType.Float16)])
+    if WARM_ONLY:
+        warm(prog)
+    x = np.random.default_rng(rows).standard_normal((rows, cols)).astype(np.float16)
+    bufs = replay_on_oracle(prog, [x])
+    assert check_each_kernel(prog, bufs)[-1] == "map"
+    (y,) = run_program(backend(), prog, [x])
+    want = x.astype(np.float64) - np.log(np.exp(x.astype(np.float64)).sum(-1, keepdims=True))
+    np.testing.assert_allclose(y.astype(np.float64).reshape(rows, cols), want, rtol=1e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("heads,expect_out_proj", [(4, "gemm"), (2, "gemm")])
 def test_gpt2_block_small_f16(heads, expect_out_proj):
     """d=128: with 2 heads (H=64) the out-projection reads the attention output through a two-level k axis whose runs
