@@ -167,15 +167,22 @@ def _in_bounds(node: AluExp) -> bool:
     return idx.min >= 0 and idx.max < node.arg[1]
 
 
-def classify_loads(exp: Optional[AluExp], sym: str, V: int) -> Dict[int, str]:
+def classify_loads(exp: Optional[AluExp], sym: str, V: int, guarded: bool = False) -> Dict[int, str]:
     """id(GlobalIndex node) -> "vector" (V consecutive, aligned elements per lane group), "vector_u" (V consecutive
     elements whose first is not known to sit on a multiple of V: rows of odd length, views shifted by an element) or
-    "uniform" (same element for the whole group).  Loads needing a bounds guard stay scalar."""
+    "uniform" (same element for the whole group).  Loads needing a bounds guard stay scalar, except (`guarded`) the
+    ones whose groups are inside the buffer or outside it as a whole -- the first index a multiple of V, positive or
+    negative, and the buffer a multiple of V long: "vector_g", the pieces of a concatenation or of a padding along an
+    outer axis."""
     out: Dict[int, str] = {}
     if V <= 1:
         return out
     for node in _load_nodes(exp):
         if not _in_bounds(node):
+            if guarded and node.arg[1] % V == 0:
+                f = lane_form(node.src[0], sym, V)
+                if f is not None and f[0] == 1 and f[1] % V == 0:
+                    out[id(node)] = "vector_g"
             continue
         f = lane_form(node.src[0], sym, V)
         if f is None:
@@ -471,7 +478,7 @@ def tuneHip(kernel: Kernel, *, allow_gemm: bool = True, allow_split: bool = True
             return t
         V = _pick_vector_width(kernel, t, size)
         t.klass = "map"
-        t.vector_loads = classify_loads(t.exp, "gidx", V)
+        t.vector_loads = classify_loads(t.exp, "gidx", V, guarded=True)
         groups = max(size // V, 1)
         # Groups per lane (their loads all issued before the first is consumed).  One by default: with a block per 256
         # groups the resident waves already keep enough loads in flight, and 2-8 groups per lane measured 1-15 % slower

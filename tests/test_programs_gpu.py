@@ -115,6 +115,42 @@ def test_float16_log_softmax_over_rows_off_the_pack_width(rows, cols):
     np.testing.assert_allclose(y.astype(np.float64).reshape(rows, cols), want, rtol=1e-2, atol=2e-2)
 
 
+def _piece_cases():
+    from jaxjs_hip import library as Lb
+    cat = lambda axis: (lambda *xs: Lb.concatenate(list(xs), axis), lambda *xs: np.concatenate(xs, axis))  # noqa: E731
+    pad = lambda w: (lambda x: Lb.pad(x, w), lambda x: np.pad(x, w))  # noqa: E731
+    return {
+        "kv_append": (cat(1), [(2, 255, 4, 64), (2, 1, 4, 64)], True),
+        "three_pieces_axis0": (cat(0), [(100, 264), (3, 264), (50, 264)], True),
+        "last_axis_40_24": (cat(1), [(512, 40), (512, 24)], True),
+        "last_axis_5_7": (cat(1), [(512, 5), (512, 7)], False),  # pieces that are not whole lane groups: element loads
+        "pad_channels": (pad([(0, 0), (8, 8), (0, 0), (0, 0)]), [(2, 16, 12, 12)], True),
+        "pad_rows": (pad([(3, 73), (0, 0)]), [(128, 768)], True),
+        "pad_image": (pad([(0, 0), (0, 0), (1, 1), (1, 1)]), [(2, 16, 12, 12)], False),
+    }
+
+
+@pytest.mark.parametrize("dtype", [DType.Float16, DType.Float32], ids=lambda d: d.value)
+@pytest.mark.parametrize("name", list(_piece_cases()))
+def test_concatenations_and_paddings_move_whole_lane_groups(name, dtype):
+    """Pieces of a concatenation or a padding read their operand under a bounds guard; when every lane group lies
+    inside or outside the operand as a whole the group is one wide load.  Bit-exact against numpy, and the plan is the
+    one expected (a guarded wide load in the source, or none)."""
+    from jaxjs_hip import jit as J
+    from jaxjs_hip.jit import ShapedArray
+    from jaxjs_hip.kernelgen import generate
+    (fn, ref), shapes, wide = _piece_cases()[name]
+    prog = J.jit(fn, [ShapedArray(s, dtype) for s in shapes])
+    (k,) = prog.kernels
+    assert ("_in ? " in generate(k, gpu_util.NUMERICS).sources[0]) == wide
+    if WARM_ONLY:
+        warm(prog)
+    rng = np.random.default_rng(len(name))
+    arrs = [rng.standard_normal(s).astype(numpyDtype(dtype)) for s in shapes]
+    (y,) = run_program(backend(), prog, arrs)
+    np.testing.assert_array_equal(y.reshape(ref(*arrs).shape), ref(*arrs))
+
+
 @pytest.mark.parametrize("heads,expect_out_proj", [(4, "gemm"), (2, "gemm")])
 def test_gpt2_block_small_f16(heads, expect_out_proj):
     """d=128: with 2 heads (H=64) the out-projection reads the attention output through a two-level k axis whose runs
