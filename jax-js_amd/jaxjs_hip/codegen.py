@@ -17,6 +17,11 @@ import numpy as np
 from .alu import AluExp, AluGroup, AluOp, DType, isFloatDtype
 from .errors import UnsupportedOpError
 
+# A generated source may open with lines of this form; `runtime.compile_source` adds the named option (from a fixed
+# list) to the compiler's command line for that source alone.
+SOURCE_OPTION = "// hiprtc-option: "
+SOURCE_OPTIONS_ALLOWED = ("-fno-slp-vectorize",)
+
 CTYPE = {
     DType.Float32: "float",
     DType.Int32: "int",
@@ -83,8 +88,6 @@ class HipExpCodegen:
         self.numerics = numerics
         self.lines: List[str] = []
         self.loads: Dict[int, str] = {}
-        self.packed_lanes = False  # True: the statements run once per lane of a pack (a fully unrolled loop)
-        self._gathers_memo: Dict[int, bool] = {}
         self._refs: Dict[int, int] = {}
         self._seen: set = set()
         self._ctx: Dict[int, str] = {}
@@ -147,37 +150,6 @@ class HipExpCodegen:
             self.emit(f"const {CTYPE[node.dtype]} {name} = {text};")
             text = name
         self._ctx[id(node)] = text
-
-    def _gathers(self, node: AluExp) -> bool:
-        """Does the subtree read memory at an index of its own (a load that is not one of the hoisted ones)?"""
-        memo = self._gathers_memo
-        stack = [node]
-        while stack:
-            n = stack[-1]
-            if id(n) in memo:
-                stack.pop()
-                continue
-            if n.op == AluOp.GlobalIndex:
-                memo[id(n)] = id(n) not in self.loads
-                stack.pop()
-                continue
-            todo = [c for c in n.src if id(c) not in memo]
-            if todo:
-                stack.extend(todo)
-                continue
-            memo[id(n)] = any(memo[id(c)] for c in n.src)
-            stack.pop()
-        return memo[id(node)]
-
-    def _rounded_f16(self, node: AluExp, text: str) -> str:
-        """A float16 value that was rounded from float32.  In the per-lane statements of a pack, when the value comes
-        from a load at the lane's own index (a row statistic read at `gidx / row_length`), the value is passed through
-        an empty asm statement: the compiler otherwise pairs such lanes into half-filled two-float vectors, moves a
-        following float16 negation in front of the rounding, and aborts in instruction selection on the two-float
-        negation it made (packed float32 arithmetic is switched off for this target)."""
-        if not (self.packed_lanes and self._gathers(node)):
-            return text
-        return f'({{ jh_f16 jh_r = {text}; asm volatile("" : "+v"(jh_r)); jh_r; }})'
 
     def _unsupported(self, node: AluExp, arg=None):
         return UnsupportedOpError(node.op, node.dtype, "hip", arg)
@@ -249,8 +221,6 @@ class HipExpCodegen:
                     call = f"jh_{fns[op]}_f16((float)({a}))"  # hardware exp2/log2: float16 has no Wasm polynomial to follow
                 if dtype == DType.Float64 and self.numerics == "native" and op not in (AluOp.Erf, AluOp.Erfc):
                     return f"__ocml_{fns[op]}_f64({a})", False
-                if dtype == DType.Float16:
-                    return self._rounded_f16(node, f"({ct})({call})"), False
                 return (call if dtype == DType.Float32 else f"({ct})({call})"), False
             if op == AluOp.Sqrt:
                 if dtype == DType.Float64:
@@ -283,8 +253,6 @@ class HipExpCodegen:
                             and self._refs.get(id(s0), 0) <= 1):
                         x, y = (self._ctx[id(t)] for t in s0.src)
                         return f"(({ct})({x}) * ({ct})({y}))", False
-                    if dtype == DType.Float16 and sdt in (DType.Float32, DType.Float64):
-                        return self._rounded_f16(node, f"({ct})({a})"), False
                     return f"({ct})({a})", False
                 if isFloatDtype(sdt):
                     return f"{'jh_f2i_sat' if dtype == DType.Int32 else 'jh_f2u_sat'}({a})", False

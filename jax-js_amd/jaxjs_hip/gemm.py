@@ -13,7 +13,7 @@ from typing import Dict, List
 
 from .alu import AluExp, AluOp, DType, Kernel, byteWidth
 from .codegen import CTYPE, STORAGE_CTYPE, HipExpCodegen, strip_parens
-from .kernelgen import KernelSource, LaunchStep, _Body, _min_bytes, _prelude, _used_args, fill, template
+from .kernelgen import KernelSource, LaunchStep, _Body, _min_bytes, _prelude, _used_args, epilogue_compile_options, fill, template
 from . import tuner
 from .tuner import TuneResult, classify_loads
 
@@ -621,7 +621,9 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     epi_params = "".join(f", const {STORAGE_CTYPE[d or DType.Float32]}* __restrict__ {n}" for d, n in zip(used, names))
     epi_fn = (f"static __device__ __forceinline__ {out_t} jh_epilogue(float acc, int row, int col, int b0, int b1, int b2{epi_params}) {{\n"
               + "\n".join(cg.take_lines()) + f"\n  return ({out_t})({value});\n}}")
+    src_options = epilogue_compile_options(epilogue)
     if split > 1 and not fusek:  # the fold kernel applies the epilogue; a slice stores its raw accumulator
+        src_options = ""
         epi_fn = f"static __device__ __forceinline__ float jh_epilogue(float acc, int row, int col, int b0, int b1, int b2{epi_params}) {{\n  return acc;\n}}"
     epi_args = "".join(f", {n}" for n in names)
 
@@ -670,6 +672,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
             conv = gen_conv(kernel, g, oexp, numerics, name, params, names, epi_fn, epi_args, conv_need, tile,
                             a_gather_fns=element_fn["a"] if g.get("a_gather") else None)
             if conv is not None:
+                conv.sources[0] = src_options + conv.sources[0]
                 return conv
         gcg = HipExpCodegen(names, {"row": "row", "k": "k", "b0": "b0", "b1": "b1", "b2": "b2"}, "  ", prefix=f"g{tag}", numerics=numerics)
         gcg.countReferences(oexp)
@@ -974,7 +977,7 @@ def gen_gemm(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
         sched.update(GATHER_FNS="\n".join(gather_fns), A_GATHER=gather_flags["a"], B_GATHER=gather_flags["b"],
                      GATHER_A_CALL=gather_calls["a"], GATHER_B_CALL=gather_calls["b"],
                      GATHER_A_SLOW=gather_slow.get("a", "jh_half8{0, 0, 0, 0, 0, 0, 0, 0}"), GATHER_B_SLOW=gather_slow.get("b", "jh_half8{0, 0, 0, 0, 0, 0, 0, 0}"))
-    src = _prelude(numerics) + fill(template(tmpl), dict(sched, 
+    src = src_options + _prelude(numerics) + fill(template(tmpl), dict(sched, 
         M=g["M"], N=g["N"], K=g["K"], M_LOAD=load_rows["a"], N_LOAD=load_rows["b"], BM=BM, BN=BN, WM=WM, WN=WN,
         A_KCONTIG=0 if gather_flags["a"] in (2, 3, 5) else (1 if g["a_sk"] == 1 or g["K"] == 1 or gather_flags["a"] in (1, 4, 6, 7) else 0),
         B_KCONTIG=0 if gather_flags["b"] in (2, 3, 5) else (1 if g["b_sk"] == 1 or g["K"] == 1 or gather_flags["b"] in (1, 4, 6, 7) else 0),

@@ -13,7 +13,7 @@ from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Tuple
 
 from .alu import AluExp, AluOp, AluVar, DType, Kernel, Reduction, byteWidth
-from .codegen import CTYPE, STORAGE_CTYPE, HipExpCodegen, const_literal, strip_parens
+from .codegen import CTYPE, SOURCE_OPTION, STORAGE_CTYPE, HipExpCodegen, const_literal, strip_parens
 from .errors import UnsupportedOpError
 from .shape import prod
 from .tuner import TuneResult, tuneHip
@@ -181,7 +181,6 @@ class _Body:
     def lanes(self, loads: Dict[int, str]) -> Tuple[str, str]:
         cg = HipExpCodegen(self.args, self.names, self.indent + "  ", prefix=f"l{self.tag}", numerics=self.numerics)
         cg.loads = loads
-        cg.packed_lanes = self.V > 1
         cg.countReferences(self.exp)
         value = strip_parens(cg.run(self.exp))
         return "\n".join(cg.take_lines()), value
@@ -190,7 +189,6 @@ class _Body:
         """`lanes` for several expressions that share one statement list (the two factors of a product)."""
         cg = HipExpCodegen(self.args, self.names, self.indent + "  ", prefix=f"l{self.tag}", numerics=self.numerics)
         cg.loads = loads
-        cg.packed_lanes = self.V > 1
         for e in exps:
             cg.countReferences(e)
         values = [strip_parens(cg.run(e)) for e in exps]
@@ -215,6 +213,39 @@ def _prelude(numerics: str) -> str:
         raise ValueError(f"numerics must be one of {NUMERICS}")
     return (f"#define JH_WASM_NUMERICS {1 if numerics in ('wasm', 'fast') else 0}\n#define JH_FAST_NUMERICS {1 if numerics == 'fast' else 0}\n"
             + template("prelude.hip.inc") + "\n")
+
+
+def _compile_options_of(kernel: Kernel, t: TuneResult) -> str:
+    """Leading source lines that `runtime.compile_source` turns into compiler options.  Kernels that touch float16 are
+    compiled without the SLP vectorizer: it pairs the unrolled lanes' float32 intermediates (the argument of a
+    logarithm, a mean) into two-float vectors, the backend then moves a float16 negation or subtraction in front of
+    the rounding, and instruction selection aborts the process on the two-float negation it made itself (packed
+    float32 arithmetic is switched off for this target).  `logSigmoid`, `acos`, a variance along axis 0 and
+    log-softmax over rows of 50257 in float16 all ran into it."""
+    halves = kernel.dtype == DType.Float16 or any(
+        e is not None and e.collect(lambda n: n.dtype == DType.Float16) for e in (t.exp, t.epilogue))
+    return SOURCE_OPTION + "-fno-slp-vectorize\n" if halves else ""
+
+
+_F16_PLAIN = (AluOp.Add, AluOp.Mul, AluOp.Max, AluOp.Min, AluOp.Where, AluOp.Cast, AluOp.Const, AluOp.GlobalIndex)
+
+
+def epilogue_compile_options(epilogue: Optional[AluExp]) -> str:
+    """The same for the matrix templates, whose per-element epilogue is inlined once per accumulator register: only
+    when the epilogue does more in float16 than add, multiply by something that is not a negative constant, clamp,
+    select and cast (bias, residual and ReLU keep the vectorizer; `-(a @ b)`, GELU or `logSigmoid` behind a product do
+    not)."""
+    if epilogue is None:
+        return ""
+
+    def risky(n: AluExp) -> bool:
+        if n.dtype != DType.Float16 or n.op in (AluOp.Variable, AluOp.Special):
+            return False
+        if n.op == AluOp.Mul:
+            return any(c.op == AluOp.Const and float(c.arg) < 0 for c in n.src)
+        return n.op not in _F16_PLAIN
+
+    return SOURCE_OPTION + "-fno-slp-vectorize\n" if epilogue.collect(risky) else ""
 
 
 IDENT = {"gidx": "gidx", "ridx": "ridx"}
@@ -251,7 +282,7 @@ def _gen_map(kernel: Kernel, t: TuneResult, numerics: str, name: str) -> KernelS
     body.indent = "        "
     lane_body, lane_value = body.lanes(loads)
     scalar_body, scalar_value = body.scalar("    ")
-    src = _prelude(numerics) + fill(template("map.hip.inc"), dict(
+    src = _compile_options_of(kernel, t) + _prelude(numerics) + fill(template("map.hip.inc"), dict(
         SIZE=kernel.size, V=V, BLOCK=block, UNROLL=t.params.get("unroll", 1), NT_STORE=t.params.get("nt_store", 0), NAME=name, PARAMS=params, OUT_T=out_t,
         LOAD_FIELDS=load_fields, LOAD_PARAMS=_in_params(used)[0], LOAD_ARGS=_in_params(used)[1],
         VECTOR_LOADS=hoisted, LANE_BODY=lane_body, LANE_VALUE=lane_value,
@@ -283,7 +314,7 @@ def _gen_map_transposed(kernel: Kernel, t: TuneResult, numerics: str, name: str)
     for i in reversed(outer):
         decode.append(f"  {{ const long long d = rem % {shape[i]}ll; rem /= {shape[i]}ll; in_base += d * {strides[i]}ll; out_base += d * {ostr[i]}ll; }}")
     blocks = prod([shape[i] for i in outer]) * -(-shape[j] // 64) * -(-shape[-1] // 64)
-    src = _prelude(numerics) + fill(template("map_t.hip.inc"), dict(
+    src = _compile_options_of(kernel, t) + _prelude(numerics) + fill(template("map_t.hip.inc"), dict(
         NJ=shape[j], NC=shape[-1], SC=strides[-1], OSJ=ostr[j], NAME=name, PARAMS=params, OUT_T=out_t,
         IN_T=STORAGE_CTYPE[load.dtype], IN_PTR=args[p["gid"]], IN_OFF=p["offset"], OUTER_DECODE="\n".join(decode), BODY=body, VALUE=value))
     step = LaunchStep(name, (blocks, 1, 1), (256, 1, 1), 0, [("in", i) for i in range(kernel.nargs)] + [("out", 0)])
@@ -357,7 +388,7 @@ def _gen_reduce(kernel: Kernel, t: TuneResult, numerics: str, name: str, row: bo
         scalar_body, scalar_value = body.scalar("        ")
         epi = _Body(t.epilogue, args, {"gidx": "gidx", "acc": "acc"}, "gidx", "gidx", 1, {}, numerics, "      ", "e")
         epi_body, epi_value = epi.scalar("      ", "e") if split == 1 else ("", "0")
-        src = _prelude(numerics) + fill(template("reduce_row.hip.inc"), dict(
+        src = _compile_options_of(kernel, t) + _prelude(numerics) + fill(template("reduce_row.hip.inc"), dict(
             SIZE=size, R=R, V=V, T=T, BLOCK=p["block"], ROWS=p["rows"], SPLIT=split, SLICE=slice_len,
             UNROLL=p.get("unroll", 4), REDUCE=_reduce_text(re.op, re.dtype), NAME=name, PARAMS=params, ACC_T=acc_t, OUT_T=out_t,
             LOAD_FIELDS=load_fields, LOAD_PARAMS=_in_params(used)[0], LOAD_ARGS=_in_params(used)[1],
@@ -380,7 +411,7 @@ def _gen_reduce(kernel: Kernel, t: TuneResult, numerics: str, name: str, row: bo
         else:
             epi_hoisted = epi_body = tail_body = ""
             epi_value = tail_value = "0"
-        src = _prelude(numerics) + fill(template("reduce_col.hip.inc"), dict(
+        src = _compile_options_of(kernel, t) + _prelude(numerics) + fill(template("reduce_col.hip.inc"), dict(
             SIZE=size, R=R, V=V, T=T, LX=p["lx"], SPLIT=split, SLICE=slice_len, PITCH=_partial_pitch(size, V),
             UNROLL=p.get("unroll", 4), INTERLEAVE=p.get("interleave", 0),
             LOAD_FIELDS=load_fields, LOAD_PARAMS=_in_params(used)[0], LOAD_ARGS=_in_params(used)[1],

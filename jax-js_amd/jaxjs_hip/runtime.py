@@ -14,6 +14,7 @@ import threading
 import numpy as np
 from typing import List, Optional, Sequence, Tuple
 
+from .codegen import SOURCE_OPTION, SOURCE_OPTIONS_ALLOWED
 from .errors import HipRuntimeError
 
 _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -146,6 +147,13 @@ def compile_source(source: str, name: str = "kernel.hip", options: Optional[Sequ
     if use_cache is None:
         use_cache = DISK_CACHE
     opts = list(options if options is not None else COMPILE_OPTIONS)
+    for line in source.split("\n", 4)[:4]:  # options the generator asks for in the source's opening lines
+        if line.startswith(SOURCE_OPTION):
+            opt = line[len(SOURCE_OPTION):].strip()
+            if opt not in SOURCE_OPTIONS_ALLOWED:
+                raise HipRuntimeError(f"{name}: the source asks for a compiler option that is not on the list: {opt!r}")
+            if opt not in opts:
+                opts.append(opt)
     key = hashlib.sha256((toolchain_tag() + "\0" + "\0".join(opts) + "\0" + source).encode()).hexdigest()[:32]
     path = os.path.join(CACHE_DIR, key + ".hsaco")
     if use_cache and os.path.exists(path):

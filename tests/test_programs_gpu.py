@@ -115,6 +115,34 @@ def test_float16_log_softmax_over_rows_off_the_pack_width(rows, cols):
     np.testing.assert_allclose(y.astype(np.float64).reshape(rows, cols), want, rtol=1e-2, atol=2e-2)
 
 
+def _float16_cases():
+    from jaxjs_hip import jit as J, library as Lb
+    return {
+        "logSigmoid": (lambda x: Lb.logSigmoid(x), [(16, 1001)]),
+        "acos": (lambda x: Lb.acos(Lb.tanh(x)), [(16, 1001)]),
+        "var_axis0": (lambda x: Lb.var_(x, 0), [(3, 5, 77)]),
+        "negated_product": (lambda a, b: J.neg(Lb.matmul(a, b)), [(256, 256), (256, 256)]),
+        "logSigmoid_behind_a_product": (lambda a, b: Lb.logSigmoid(Lb.matmul(a, b)), [(256, 256), (256, 256)]),
+    }
+
+
+@pytest.mark.parametrize("name", list(_float16_cases()))
+def test_float16_programs_the_device_compiler_used_to_abort_on(name):
+    """Float16 kernels whose unrolled lanes round a float32 intermediate and then negate or subtract it: the device
+    compiler's SLP vectorizer paired those lanes and instruction selection aborted the process (such sources now ask
+    for compilation without that pass).  Every kernel against the checker."""
+    from jaxjs_hip import jit as J
+    from jaxjs_hip.jit import ShapedArray
+    fn, shapes = _float16_cases()[name]
+    prog = J.jit(fn, [ShapedArray(s, DType.Float16) for s in shapes])
+    if WARM_ONLY:
+        warm(prog)
+    rng = np.random.default_rng(len(name))
+    arrs = [(rng.standard_normal(s) * (0.1 if len(shapes) == 2 else 1.0)).astype(np.float16) for s in shapes]
+    bufs = replay_on_oracle(prog, arrs)
+    check_each_kernel(prog, bufs, f16_rtol=2e-2)
+
+
 def _piece_cases():
     from jaxjs_hip import library as Lb
     cat = lambda axis: (lambda *xs: Lb.concatenate(list(xs), axis), lambda *xs: np.concatenate(xs, axis))  # noqa: E731
