@@ -100,8 +100,8 @@ def test_row_softmax_argmax_program():
 @pytest.mark.parametrize("rows,cols", [(64, 1001), (16, 50257)], ids=str)
 def test_float16_log_softmax_over_rows_off_the_pack_width(rows, cols):
     """`x - log(sum)` in float16 with rows that are not whole packs of eight: every lane of a pack reads its own row's
-    statistic, rounds the logarithm to float16 and negates it (a form the device compiler could not select before the
-    rounded value was made opaque to it); each kernel against the checker."""
+    statistic, rounds the logarithm to float16 and negates it (the first form on which the device compiler was seen
+    to abort; see the test of such programs below); each kernel against the checker."""
     from jaxjs_hip import jit as J, library as Lb
     from jaxjs_hip.jit import ShapedArray
     prog = J.jit(lambda x: Lb.logSoftmax(x, -1), [ShapedArray((rows, cols), DType.Float16)])
