@@ -155,3 +155,33 @@ def test_interval_form_of_a_mask_matches_the_mask_element_by_element():
                 assert want == (ok and lo <= ev < hi), (name, ctx, ev)
     assert interval_mask_form(AluExp.cmplt(AluExp.add(x, AluExp.mul(e, I(2))), I(57))) is None
     assert interval_mask_form(AluExp.cmplt(AluExp.mod(AluExp.add(x, e), I(7)), I(3))) is None
+
+
+def test_float16_sources_carry_their_compiler_option_and_unknown_options_are_refused():
+    """Float16 map and reduce kernels, and matrix kernels with a float16 epilogue beyond bias / ReLU, open with the line
+    that switches the SLP vectorizer off for that source; float32 kernels and plain epilogues do not.  The line is
+    honoured only for options on the fixed list."""
+    import pytest
+    from jaxjs_hip import jit as J, library as Lb
+    from jaxjs_hip.codegen import SOURCE_OPTION
+    from jaxjs_hip.errors import HipRuntimeError
+    from jaxjs_hip.jit import ShapedArray
+    from jaxjs_hip.runtime import compile_source
+    line = SOURCE_OPTION + "-fno-slp-vectorize\n"
+
+    def sources(fn, shapes, dtype):
+        prog = J.jit(fn, [ShapedArray(s, dtype) for s in shapes])
+        return [generate(k, "fast") for k in prog.kernels]
+
+    for dtype, expect in ((DType.Float16, True), (DType.Float32, False)):
+        gens = sources(lambda x: Lb.logSoftmax(x, -1), [(16, 1001)], dtype)
+        assert {g.klass for g in gens} == {"reduce_row", "map"}
+        assert all(g.sources[0].startswith(line) == expect for g in gens)
+    mm = [(256, 256), (256, 256)]
+    (neg,) = sources(lambda a, b: J.neg(Lb.matmul(a, b)), mm, DType.Float16)
+    (relu,) = sources(lambda a, b: Lb.relu(Lb.matmul(a, b)), mm, DType.Float16)
+    (neg32,) = sources(lambda a, b: J.neg(Lb.matmul(a, b)), mm, DType.Float32)
+    assert neg.klass == relu.klass == neg32.klass == "gemm"
+    assert neg.sources[0].startswith(line) and not relu.sources[0].startswith(line) and not neg32.sources[0].startswith(line)
+    with pytest.raises(HipRuntimeError, match="not on the list"):
+        compile_source(SOURCE_OPTION + "-O0\nextern \"C\" __global__ void k() {}\n", use_cache=False)
