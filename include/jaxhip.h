@@ -102,7 +102,9 @@ int jh_host_free(void *ptr);
  * src/backend/webgpu.ts:705-744, `new WebAssembly.Module` in src/backend/wasm.ts:125-147).
  * Needs no GPU, so it can also run ahead of time.  On success `*code`/`*code_size` hold a
  * malloc'd code object to release with `jh_code_free`; on failure `log` (if non-NULL) receives
- * the compiler output, truncated to `log_size`.
+ * the compiler output, truncated to `log_size`.  A source may ask for options of its own in leading lines of the form
+ * `// hiprtc-option: <option>`: they are added to `options` when they are on the library's fixed list
+ * (`-fno-slp-vectorize`, which the generator puts on float16 kernels) and make the call fail when they are not.
  */
 int jh_compile(const char *source, const char *name, const char *const *options, int num_options,
                void **code, size_t *code_size, char *log, size_t log_size);

@@ -14,6 +14,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <string>
+#include <vector>
 
 // Scratch memory of `jh_launch_static_scratch`: one array per GPU, inside the library's own code object, so the entry
 // point never allocates.  In host code the array's name is only a stand-in: the device address is looked up once
@@ -259,7 +260,34 @@ int jh_compile(const char *source, const char *name, const char *const *options,
   hiprtcProgram prog;
   hiprtcResult r = hiprtcCreateProgram(&prog, source, name ? name : "kernel.hip", 0, nullptr, nullptr);
   if (r != HIPRTC_SUCCESS) return fail((int)r, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
-  r = hiprtcCompileProgram(prog, num_options, const_cast<const char **>(options));
+  // Options the source asks for itself: leading lines of the form "// hiprtc-option: <option>", honoured for the
+  // options on a fixed list (the generator marks float16 kernels that the SLP vectorizer makes the compiler abort on).
+  std::vector<std::string> asked;
+  {
+    static const char kMark[] = "// hiprtc-option: ";
+    static const char *const kAllowed[] = {"-fno-slp-vectorize"};
+    const char *line = source;
+    while (strncmp(line, kMark, sizeof(kMark) - 1) == 0) {
+      const char *begin = line + sizeof(kMark) - 1;
+      const char *end = strchr(begin, '\n');
+      std::string opt = end ? std::string(begin, end) : std::string(begin);
+      while (!opt.empty() && (opt.back() == ' ' || opt.back() == '\r')) opt.pop_back();
+      bool ok = false;
+      for (const char *a : kAllowed) ok = ok || opt == a;
+      if (!ok) {
+        hiprtcDestroyProgram(&prog);
+        return fail(-5, "the source asks for a compiler option that is not on the list: %s", opt.c_str());
+      }
+      bool present = false;
+      for (int i = 0; i < num_options; ++i) present = present || (options[i] && opt == options[i]);
+      if (!present) asked.push_back(opt);
+      if (!end) break;
+      line = end + 1;
+    }
+  }
+  std::vector<const char *> all_options(options, options + (options ? num_options : 0));
+  for (const std::string &o : asked) all_options.push_back(o.c_str());
+  r = hiprtcCompileProgram(prog, (int)all_options.size(), all_options.data());
   size_t n = 0;
   if (hiprtcGetProgramLogSize(prog, &n) == HIPRTC_SUCCESS && n > 1) {
     std::string text(n, '\0');

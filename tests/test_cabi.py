@@ -45,6 +45,27 @@ def test_calls_before_init_fail_loudly():
     assert lib.jh_sync() != 0
 
 
+def test_library_honours_option_lines_of_a_source_and_refuses_unknown_ones():
+    """`jh_compile` itself reads the leading `// hiprtc-option:` lines (a host that replays exported plans passes the
+    plan's common options only): a listed option compiles with no options passed at all, any other is an error."""
+    import ctypes
+    lib = load_library()
+
+    def compile_raw(text):
+        code, size = ctypes.c_void_p(), ctypes.c_size_t()
+        opts = (ctypes.c_char_p * 1)(b"--offload-arch=gfx950")
+        rc = lib.jh_compile(text.encode(), b"k.hip", opts, 1, ctypes.byref(code), ctypes.byref(size), None, 0)
+        if rc == 0:
+            lib.jh_code_free(code)
+        return rc, size.value
+
+    body = 'extern "C" __global__ void k(float* p) { p[0] = 1.0f; }\n'
+    rc, size = compile_raw("// hiprtc-option: -fno-slp-vectorize\n" + body)
+    assert rc == 0 and size > 1000
+    rc, _ = compile_raw("// hiprtc-option: -DANYTHING\n" + body)
+    assert rc != 0 and b"not on the list" in lib.jh_last_error()
+
+
 def test_compile_error_is_reported():
     with pytest.raises(HipRuntimeError, match="hiprtc failed"):
         compile_source("extern \"C\" __global__ void k() { this is not C++; }", use_cache=False)
