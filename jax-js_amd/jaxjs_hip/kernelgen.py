@@ -143,11 +143,14 @@ class _Body:
                 load = {"vector": "jh_vload", "vector_u": "jh_vload_u", "vector_nt": "jh_vload_nt"}[self.classes[id(n)]]
                 cg.emit(f"const jh_pack<{st}, {self.V}> {var} = {load}<{st}, {self.V}>({ptr} + ({idx}));")
                 loads[id(n)] = f"{var}.v[lane]"
-            elif self.classes[id(n)] == "vector_g":
+            elif self.classes[id(n)] in ("vector_g", "vector_gm"):
                 # a group that is inside the buffer or outside it as a whole: one load from the group's place, or from
                 # element 0 when it is outside, where every lane then holds element 0 as a guarded scalar load would
                 var = f"v{self.tag}{k}"
-                cg.emit(f"const bool {var}_in = (jh_u32)({idx}) < (jh_u32){n.arg[1]};")
+                sign = ""
+                if self.classes[id(n)] == "vector_gm":  # index x % C: a negative x puts the whole group outside
+                    sign = f"({strip_parens(cg.run(n.src[0].src[0]))}) >= 0 && "
+                cg.emit(f"const bool {var}_in = {sign}(jh_u32)({idx}) < (jh_u32){n.arg[1]};")
                 cg.emit(f"jh_pack<{st}, {self.V}> {var} = jh_vload<{st}, {self.V}>({ptr} + ({var}_in ? ({idx}) : 0));")
                 cg.emit(f"if (!{var}_in) {{ for (int jh_i = 1; jh_i < {self.V}; ++jh_i) {var}.v[jh_i] = {var}.v[0]; }}")
                 loads[id(n)] = f"{var}.v[lane]"

@@ -108,6 +108,16 @@ def known_divisor(e: AluExp) -> int:
     return 1
 
 
+def _may_wrap(e: AluExp) -> bool:
+    """Can the int32 arithmetic of e wrap around (it then holds a loaded value: index arithmetic alone stays in range)?"""
+    return not (e.min >= -(1 << 31) and e.max <= (1 << 31) - 1)
+
+
+def _wrapped(e: AluExp, divisor: int) -> int:
+    """What is left of a divisibility claim when e may have wrapped modulo 2^32: its power-of-two part."""
+    return (divisor & -divisor) if divisor and _may_wrap(e) else divisor
+
+
 def lane_form(e: AluExp, sym: str, V: int) -> Optional[Tuple[int, int]]:
     """Describe e when `sym = V*q + lane`, lane in [0,V): returns (stride, align) such that
     e == u + stride*lane with u independent of lane and u % align == 0 (align 0: u is 0), or None
@@ -115,26 +125,30 @@ def lane_form(e: AluExp, sym: str, V: int) -> Optional[Tuple[int, int]]:
     understood; everything else referencing `sym` is "unknown".
     """
     if not references(e, sym):
-        return (0, known_divisor(e))
+        return (0, _wrapped(e, known_divisor(e)))
     if _is_symbol(e, sym):
         return (1, V)
     if e.dtype not in (DType.Int32, DType.Uint32):
         return None
     op = e.op
+    if op == AluOp.GlobalIndex:
+        # a value loaded at an index the whole group shares (the row id of a table lookup): the same for every lane
+        f = lane_form(e.src[0], sym, V)
+        return (0, 1) if f is not None and f[0] == 0 else None
     if op in (AluOp.Add, AluOp.Sub):
         a, b = lane_form(e.src[0], sym, V), lane_form(e.src[1], sym, V)
         if a is None or b is None:
             return None
         stride = a[0] + b[0] if op == AluOp.Add else a[0] - b[0]
-        return (stride, math.gcd(a[1], b[1]))
+        return (stride, _wrapped(e, math.gcd(a[1], b[1])))
     if op == AluOp.Mul:
         for i in (0, 1):
             c = e.src[i]
             if c.op == AluOp.Const:
                 f = lane_form(e.src[1 - i], sym, V)
-                if f is None:
+                if f is None or (f[0] != 0 and _may_wrap(e)):
                     return None
-                return (f[0] * int(c.arg), f[1] * abs(int(c.arg)))
+                return (f[0] * int(c.arg), _wrapped(e, f[1] * abs(int(c.arg))))
         return None
     if op in (AluOp.Idiv, AluOp.Mod) and e.src[1].op == AluOp.Const:
         C = int(e.src[1].arg)
@@ -173,16 +187,25 @@ def classify_loads(exp: Optional[AluExp], sym: str, V: int, guarded: bool = Fals
     "uniform" (same element for the whole group).  Loads needing a bounds guard stay scalar, except (`guarded`) the
     ones whose groups are inside the buffer or outside it as a whole -- the first index a multiple of V, positive or
     negative, and the buffer a multiple of V long: "vector_g", the pieces of a concatenation or of a padding along an
-    outer axis."""
+    outer axis; "vector_gm" when that holds for x in an index x % C (the rows of a table lookup)."""
     out: Dict[int, str] = {}
     if V <= 1:
         return out
     for node in _load_nodes(exp):
         if not _in_bounds(node):
-            if guarded and node.arg[1] % V == 0:
-                f = lane_form(node.src[0], sym, V)
+            if guarded and node.arg[1] % V == 0 and V & (V - 1) == 0:
+                idx = node.src[0]
+                f = lane_form(idx, sym, V)
                 if f is not None and f[0] == 1 and f[1] % V == 0:
                     out[id(node)] = "vector_g"
+                elif (idx.op == AluOp.Mod and idx.dtype == DType.Int32 and idx.src[1].op == AluOp.Const
+                      and int(idx.src[1].arg) > 0 and int(idx.src[1].arg) % V == 0):
+                    # x % C with x = x0 + lane, x0 a multiple of V of either sign (a table row chosen by a loaded id):
+                    # for x0 >= 0 the remainders are x0 % C + lane; for x0 < 0 every lane's remainder is negative, or
+                    # zero in lane 0 alone, and under the guard all of them read element 0
+                    f = lane_form(idx.src[0], sym, V)
+                    if f is not None and f[0] == 1 and f[1] % V == 0:
+                        out[id(node)] = "vector_gm"
             continue
         f = lane_form(node.src[0], sym, V)
         if f is None:

@@ -185,3 +185,36 @@ def test_float16_sources_carry_their_compiler_option_and_unknown_options_are_ref
     assert neg.sources[0].startswith(line) and not relu.sources[0].startswith(line) and not neg32.sources[0].startswith(line)
     with pytest.raises(HipRuntimeError, match="not on the list"):
         compile_source(SOURCE_OPTION + "-O0\nextern \"C\" __global__ void k() {}\n", use_cache=False)
+
+
+def test_wide_load_of_a_looked_up_row_reads_what_the_guarded_element_loads_read():
+    """The claim behind the `vector_gm` load class, by brute force over int32 ids (extremes, multiples of the table
+    length of either sign, values whose product with the row width wraps): with x = wrap(wrap(id * W) + r0 + lane),
+    element loads read `x % C` (C remainder, sign of x) when it lies in [0, C) and element 0 otherwise; the wide load
+    reads `x0 % C + lane` when x0 >= 0 and the remainder is in range, element 0 in every lane otherwise."""
+    import numpy as np
+    from jaxjs_hip import jit as J, library as Lb
+    from jaxjs_hip.jit import ShapedArray
+
+    def wrap(v):
+        return (v + 2**31) % 2**32 - 2**31
+
+    def crem(a, b):
+        return a - b * int(a / b)  # truncating division, exact for |a| < 2^53
+
+    rng = np.random.default_rng(5)
+    for rows, W, V in ((50257, 768, 8), (77, 64, 8), (1000, 8, 4), (3, 16, 8)):
+        C = rows * W
+        ids = [0, 1, -1, rows - 1, rows, -rows, 2 * rows, -2 * rows, 2**31 - 1, -2**31, 2**31 // W, -(2**31 // W), 2**32 // W + 1]
+        ids += [int(v) for v in rng.integers(-2**31, 2**31, 200)] + [int(v) for v in rng.integers(-3 * rows, 3 * rows, 200)]
+        for i in ids:
+            for r0 in range(0, W, V):
+                x0 = wrap(wrap(i * W) + r0)
+                each = [crem(wrap(x0 + lane), C) for lane in range(V)]
+                each = [f if 0 <= f < C else 0 for f in each]
+                f0 = crem(x0, C)
+                inside = x0 >= 0 and 0 <= f0 < C
+                assert each == ([f0 + lane for lane in range(V)] if inside else [0] * V), (rows, W, i, r0)
+    prog = J.jit(lambda t, i: Lb.take(t, i, 0), [ShapedArray((1000, 768), DType.Float16), ShapedArray((64,), DType.Int32)])
+    from jaxjs_hip.tuner import tuneHip
+    assert "vector_gm" in tuneHip(prog.kernels[0]).vector_loads.values()

@@ -143,6 +143,31 @@ def test_float16_programs_the_device_compiler_used_to_abort_on(name):
     check_each_kernel(prog, bufs, f16_rtol=2e-2)
 
 
+@pytest.mark.parametrize("dtype", [DType.Float16, DType.Float32], ids=lambda d: d.value)
+@pytest.mark.parametrize("rows,width,wide", [(1000, 768, True), (77, 64, True), (1000, 61, False)], ids=str)
+def test_table_rows_by_loaded_ids_including_ids_outside_the_table(rows, width, wide, dtype):
+    """`take` along axis 0: a row of whole lane groups is fetched with one wide load per group.  Ids outside the table
+    go the way the lowered index arithmetic takes them (wrap modulo the table, then the guard's element 0): bit-exact
+    against the checker for ids -1, rows, -rows, 2^31 - 1, -2^31 and a multiple of rows beyond the table."""
+    from jaxjs_hip import jit as J, library as Lb
+    from jaxjs_hip.jit import ShapedArray
+    from jaxjs_hip.kernelgen import generate
+    n = 4096
+    prog = J.jit(lambda t, i: Lb.take(t, i, 0), [ShapedArray((rows, width), dtype), ShapedArray((n,), DType.Int32)])
+    (k,) = prog.kernels
+    assert ("_in ? " in generate(k, gpu_util.NUMERICS).sources[0]) == wide
+    if WARM_ONLY:
+        warm(prog)
+    rng = np.random.default_rng(rows + width)
+    table = rng.standard_normal((rows, width)).astype(numpyDtype(dtype))
+    ids = rng.integers(0, rows, n).astype(np.int32)
+    ids[:8] = [-1, rows, -rows, 2**31 - 1, -2**31, 3 * rows, -3 * rows, rows - 1]
+    want = oracle.run_kernel(k, [table, ids], oracle.MODE_WASM)
+    np.testing.assert_array_equal(want.reshape(n, width)[8:], table[ids[8:]])
+    (y,) = run_program(backend(), prog, [table, ids])
+    np.testing.assert_array_equal(y.ravel(), want.ravel())
+
+
 def _piece_cases():
     from jaxjs_hip import library as Lb
     cat = lambda axis: (lambda *xs: Lb.concatenate(list(xs), axis), lambda *xs: np.concatenate(xs, axis))  # noqa: E731
