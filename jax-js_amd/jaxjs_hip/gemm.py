@@ -125,12 +125,14 @@ def choose_tile(g: dict) -> Dict[str, int]:
         # A 128-wide tile would compute and store a half-empty block (attention's probabilities x V, N = head
         # size 64): measured 30 % faster with 128x64 tiles, which is then bound by reading A.
         return dict(BM=128, BN=64, WM=2, WN=2, **k_split(tiles(128, 64)))
-    if (g["K"] <= 128 and g["K"] % 32 == 0 and plain_k and g["M"] % 128 == 0 and g["N"] % 128 == 0 and tiles(128, 128) >= 4 * CU
+    if (g["K"] <= 128 and g["K"] % 32 == 0 and plain_k and edge_ok(128, 128) and tiles(128, 128) >= 4 * CU
             and not loose_ops and repack is None):
         # A k axis of one to four slabs (attention scores: q.k^T over a head size of 64): the launch is bound by writing
         # C, and a workgroup spends its life in prologue and epilogue.  128x128 tiles with two shallow stages leave
         # room for four workgroups per CU, so that one's stores overlap another's loads and MFMAs
         # (96 x 1024 x 1024 x 64: 47.5 us with 256x256 tiles in the deep pipeline, 41.3 us = 5.5 TB/s this way).
+        # Ragged lengths take it through clamped edge loads (scores of 128 heads over 577 positions: 48.9 us on the
+        # 128x256 tiles the estimate below picked, 26.1 us here; 384 heads over 197: 17.2 -> 15.1 us).
         return dict(BM=128, BN=128, BK=32, STAGES=2, PIPE=0)
     if (g["K"] <= 1024 and g["K"] % 32 == 0 and plain_k and g["M"] % 128 == 0 and g["N"] % 256 == 0 and tiles(128, 256) >= 2 * CU
             and not loose_ops and repack is None and not (g["a_sk"] == 1 and g["b_sk"] == 1)):

@@ -168,6 +168,25 @@ def test_table_rows_by_loaded_ids_including_ids_outside_the_table(rows, width, w
     np.testing.assert_array_equal(y.ravel(), want.ravel())
 
 
+def test_attention_scores_over_ragged_lengths_take_the_shallow_plan_and_are_exact():
+    """q.k^T over a head size of 64 with 300 positions (not a multiple of any tile): the plan for short k axes under
+    many tiles applies through clamped edge loads.  Small integers, so the float16 result is exact."""
+    from jaxjs_hip import jit as J, library as Lb
+    from jaxjs_hip.jit import ShapedArray
+    from jaxjs_hip.kernelgen import generate
+    B, L, N, H = 12, 300, 12, 64
+    prog = J.jit(lambda q, k: Lb.einsum("BLNH,BSNH->BNLS", q, k), [ShapedArray((B, L, N, H), DType.Float16)] * 2)
+    info = generate(prog.kernels[0], gpu_util.NUMERICS).info
+    assert (info["BM"], info["BN"], info["direct_lds"], info["stages"]) == (128, 128, True, 2), info
+    if WARM_ONLY:
+        warm(prog)
+    rng = np.random.default_rng(9)
+    q, k = [rng.integers(-2, 3, (B, L, N, H)).astype(np.float16) for _ in range(2)]
+    (y,) = run_program(backend(), prog, [q, k])
+    want = np.einsum("blnh,bsnh->bnls", q.astype(np.float32), k.astype(np.float32))
+    np.testing.assert_array_equal(y.astype(np.float32).reshape(want.shape), want)
+
+
 def _piece_cases():
     from jaxjs_hip import library as Lb
     cat = lambda axis: (lambda *xs: Lb.concatenate(list(xs), axis), lambda *xs: np.concatenate(xs, axis))  # noqa: E731
