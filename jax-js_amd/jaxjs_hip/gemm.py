@@ -63,9 +63,20 @@ def choose_tile(g: dict) -> Dict[str, int]:
         # second one hides the first one's staging latency).  Slabs are 32 deep (measured 3-6 % over 16 on
         # 2048^3 and 4096^3: half the barriers); gather operands keep the 16-deep slabs they were tuned with.
         bk = 32 if plain_k else 16
-        for bm, bn in ((128, 128), (128, 64), (64, 64)):
+        # Among the shapes that do, the cheapest by (rounds of two workgroups per CU) x (tile area) / (rate of the
+        # shape relative to 128x128: 0.97, 0.80): a last round that is nearly empty costs a whole one (products of
+        # attention weights and values over 577 positions, 640 tiles of 128x64: 85.1 us, 66.1 us in 1280 of 64x64; the
+        # scores of the same, 3200 tiles of 128x128: 84.9 us, 77.1 us in 6400 of 128x64; 512 x 11008 x 4096, 688 tiles of
+        # 128x64: 600 -> 488 us in 1376 of 64x64; 2048 x 2304 x 768: 106 -> 91 us; 2048 x 3072 x 768 pays 4-7 % for it).
+        # (16-deep slabs measured faster on some of these short k axes and slower on others: not taken.)
+        best = None
+        for bm, bn, rate in ((128, 128, 1.0), (128, 64, 0.97), (64, 64, 0.80)):
             if g["M"] >= bm and g["N"] >= bn and tiles(bm, bn) >= 2 * CU:
-                return dict(BM=bm, BN=bn, BK=bk)
+                cost = -(-tiles(bm, bn) // (2 * CU)) * bm * bn / rate
+                if best is None or cost < best[0]:
+                    best = (cost, dict(BM=bm, BN=bn, BK=bk))
+        if best is not None:
+            return best[1]
         # A handful of tiles (512^3 and smaller): the launch is as long as one workgroup's walk along k.  64x64 tiles and
         # up to 8 slices of at least 64 k, until every CU has a workgroup, folded inside the launch
         # (128^3 8.2 -> 5.4 us, 256^3 15.2 -> 6.3 us, 512^3 17.2 -> 9.1 us; the launch floor is 4.7 us).
