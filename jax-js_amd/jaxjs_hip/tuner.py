@@ -122,7 +122,10 @@ def lane_form(e: AluExp, sym: str, V: int) -> Optional[Tuple[int, int]]:
     """Describe e when `sym = V*q + lane`, lane in [0,V): returns (stride, align) such that
     e == u + stride*lane with u independent of lane and u % align == 0 (align 0: u is 0), or None
     if e is not affine in the lane.  Only index arithmetic (int32 +,-,*,/,% by constants) is
-    understood; everything else referencing `sym` is "unknown".
+    understood, plus int32 values loaded at an index the whole group shares (stride 0, no alignment known); everything
+    else referencing `sym` is "unknown".  Once a loaded value is involved the arithmetic may wrap modulo 2^32: the
+    form then holds modulo 2^32, `align` keeps only its power-of-two part, and a product with a nonzero stride is
+    "unknown".
     """
     if not references(e, sym):
         return (0, _wrapped(e, known_divisor(e)))
